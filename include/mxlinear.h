@@ -1,0 +1,129 @@
+/*
+ * mxlinear.h -- C ABI of the MI355X (gfx950) MX low-precision linear path.
+ *
+ * The reference (AMD-AGI/Primus) reaches this path through the Python operator
+ * surface of the external package `primus_turbo`; the entry points below are
+ * what a binding for that surface needs, one per kernel family.  Each
+ * declaration cites the reference call site it serves.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer on the current HIP device unless the
+ *     name ends in _host; `stream` is a hipStream_t passed as void*.
+ *   - calls are asynchronous on `stream`, re-entrant, keep no state between
+ *     calls, never allocate, never synchronise and never read device memory
+ *     from the host (group_lens stays on the device).
+ *   - return value: MXL_OK (0) or a negative MXL_E* code; nothing throws.
+ *   - bf16 tensors are row-major and contiguous.
+ *   - "codes" are FP8 E4M3 bytes (fmt MXL_FMT_E4M3) or packed FP4 E2M1 nibbles,
+ *     two per byte, element 2i in bits 3:0 (fmt MXL_FMT_E2M1); "scales" are
+ *     E8M0 bytes, one per 32 elements along the contraction dim, row-major
+ *     [rows, K/32].
+ */
+#ifndef MXLINEAR_H
+#define MXLINEAR_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXL_OK 0
+#define MXL_EINVAL (-1)  /* bad shape / alignment / enum / null pointer */
+#define MXL_ELAUNCH (-2) /* HIP reported an error at launch */
+#define MXL_ENODEV (-3)  /* current device is not gfx950 */
+
+#define MXL_FMT_E4M3 0
+#define MXL_FMT_E2M1 1
+
+/* E8M0 scale rule (explicit because the reference's kernel library is not in
+ * its tree): OCP MX v1.0 floor rule, round-up rule, AITER/Quark "even" rule. */
+#define MXL_SCALE_OCP_FLOOR 0
+#define MXL_SCALE_RCEIL 1
+#define MXL_SCALE_EVEN 2
+
+#define MXL_BLOCK 32      /* MX block size (fp8_utils.py:48, fp4_utils.py:79) */
+#define MXL_SEG_ALIGN 128 /* padding of each expert segment in the transposed layout */
+#define MXL_MAX_GROUPS 1024
+
+int mxl_version(void);
+const char* mxl_error_string(int code);
+
+/* Width (elements along the token dim) of the segment-padded transposed
+ * layout for `total_rows` tokens in `num_groups` experts; depends on sizes
+ * only, never on group_lens. */
+int64_t mxl_padded_width(int64_t total_rows, int num_groups);
+
+/* MX quantisation of a bf16 matrix x[rows, cols].
+ *
+ * Serves QuantizedTensor.quantize(x, axis=-1 / axis=-2)
+ * (primus_turbo.py:321-354) and quantize_mxfp4_dual
+ * (primus_turbo_mxfp4_local.py:147-161).
+ *
+ *   q_row / s_row : row-wise copy, blocks along cols: codes [rows, cols] (or
+ *                   cols/2 bytes for FP4), scales [rows, cols/32].  Pass NULL
+ *                   for both to skip it.
+ *   q_colT / s_colT: column-wise copy stored TRANSPOSED, blocks along rows:
+ *                   codes [cols, W] (W/2 bytes for FP4), scales [cols, W/32]
+ *                   with W = mxl_padded_width(rows, max(num_groups,1)).
+ *                   Blocks restart at every group boundary; group g occupies
+ *                   columns [poff_g, poff_g + len_g) where poff is the prefix
+ *                   sum of the lens rounded up to 128; padding holds zero
+ *                   codes.  Pass NULL for both to skip it.
+ *   group_lens    : int64[num_groups] on the device, sum == rows; NULL (and
+ *                   num_groups 0) means one group of `rows` rows.
+ * Requires cols % 32 == 0.
+ */
+int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int fmt, int scale_mode,
+                 const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                 void* s_colT, void* stream);
+
+/* 2-D (32x32 tile) MX quantisation of `batch` independent weight matrices
+ * w[batch, n, k] (weights use ScalingRecipe(use_2d_block=True):
+ * primus_turbo.py:313-317; grid definition weight_deosc.py:29-33,136-174).
+ * Row-wise copy: codes [batch, n, k], scales [batch, n, k/32]; transposed
+ * copy: codes [batch, k, n], scales [batch, k, n/32] (either pair may be
+ * NULL).  The tile scale is replicated so both copies carry per-row scales.
+ * Requires n % 32 == 0 and k % 32 == 0. */
+int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int fmt,
+                           int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
+                           void* stream);
+
+/* Row-wise dequantise to bf16 (QuantizedTensor.dequantize(),
+ * weight_deosc.py:155-168): out[rows, k] = decode(codes) * 2^(scale-127). */
+int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,
+                   void* out_bf16, void* stream);
+
+/* Dense NT GEMM on pre-quantised operands (gemm_fp8_impl / gemm_fp4_impl:
+ * primus_turbo_float8_local.py:239-250, primus_turbo_mxfp4_local.py:319-331):
+ *   c[m, n] (bf16) = dq(a)[m, k] . dq(b)[n, k]^T, fp32 accumulation.
+ * Requires k % 32 == 0 and n % 32 == 0. */
+int mxl_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                const void* b_scales, int b_fmt, void* c_bf16, int64_t m, int64_t n, int64_t k,
+                void* stream);
+
+/* Grouped NT GEMM for forward and dgrad (grouped_gemm_fp8_impl,
+ * zbpp_gemm.py:590-603; call site primus_turbo.py:2122-2129):
+ *   rows of a[total_m, k] are split by group_lens (int64[num_groups], device);
+ *   b is [num_groups, n, k]; c[total_m, n] (bf16).  Empty groups are skipped;
+ *   group_lens is consumed on the device. */
+int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                        const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                        int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream);
+
+/* Grouped variable-K GEMM for wgrad (grouped_gemm_fp8_variable_k_impl,
+ * zbpp_gemm.py:710-724): operands in the segment-padded transposed layout
+ * written by mxl_quantize(..., q_colT, s_colT):
+ *   a = dY^T codes [n, W], b = X^T codes [k, W], W = mxl_padded_width(total_m, G);
+ *   c[g, n, k] (bf16) = a[:, seg_g] . b[:, seg_g]^T; an empty group yields zeros.
+ * Requires n % 32 == 0 and k % 32 == 0.  num_groups == 0 / group_lens NULL
+ * means one dense group (dense wgrad). */
+int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
+                           const void* b_codes, const void* b_scales, int b_fmt, void* c_bf16,
+                           const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
+                           int64_t k, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXLINEAR_H */

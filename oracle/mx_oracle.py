@@ -1,0 +1,457 @@
+"""CPU oracle for the MX (microscaling) low-precision linear path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing under ``primus_amd/`` may import this file;
+only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` use it, and only as the checker.
+
+What it restates
+----------------
+The arithmetic of this path lives in the third-party package ``primus_turbo``
+(AMD-AGI/Primus-Turbo, pinned at commit 22e544d56820674fcc4c8faf64651af99a5cd686
+by /root/reference/.github/workflows/ci.yaml:43), which is not vendored in the
+reference tree.  The oracle therefore restates the published OCP Microscaling
+Formats (MX) v1.0 algorithm, anchored on the reference's call sites:
+
+* block size 32, E8M0 scales, E4M3 / E2M1 elements:
+  primus/backends/megatron/core/fp8_utils.py:162-168,
+  primus/backends/megatron/core/fp4_utils.py:144-150
+* row-wise copy = ``axis=-1``; column-wise copy = ``axis=-2`` which yields the
+  TRANSPOSED quantised tensor:
+  primus/backends/megatron/core/extensions/primus_turbo.py:321-354
+* weights use 2-D 32x32 blocks, experts are independent matrices:
+  primus/backends/megatron/core/extensions/primus_turbo.py:313-317,
+  primus/backends/megatron/core/optimizer/weight_deosc.py:29-33,136-174
+* every GEMM is NT with both operands quantised along the contraction dim
+  (fwd / dgrad / wgrad operand table):
+  primus/backends/megatron/core/extensions/primus_turbo_mxfp4_local.py:316-331,
+  :432-444, :447-459
+* grouped GEMM takes tokens-per-expert (``group_lens``), empty experts allowed:
+  primus/backends/megatron/core/extensions/primus_turbo.py:2122-2129
+
+Parity status
+-------------
+* ``cast_e4m3`` : pinned against ``torch.float8_e4m3fn`` (library routine) and
+  brute-force nearest-value search.
+* ``cast_e2m1`` : pinned by brute-force nearest-value search over the 8-entry
+  E2M1 table (ties to even code).
+* ``e8m0_scale_byte`` : pinned against the closed forms of the three published
+  scale rules in exact rational arithmetic, for every non-negative bf16 amax.
+* which of the three scale rules the shipped Primus-Turbo quantiser uses, its
+  ``amax == 0`` byte, its NaN/Inf handling and the FP4 nibble order are
+  **parity unpinned** (the package is absent); the rule is an explicit
+  ``scale_mode`` argument everywhere, default ``OCP_FLOOR``.
+* GEMM / grouped GEMM / wgrad: dequantise -> fp32 matmul -> bf16, pinned by
+  invariants (G=1 == dense, permutation of experts, exactly representable
+  integer products) in tests/.
+
+All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
+results are reproducible bit-for-bit on any host.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+BLOCK = 32
+
+# element formats
+FMT_E4M3 = 0
+FMT_E2M1 = 1
+
+# E8M0 scale rules
+SCALE_OCP_FLOOR = 0  # OCP MX v1.0: floor(log2 amax) - emax_elem
+SCALE_RCEIL = 1  # 2^ceil(log2(amax / max_normal))
+SCALE_EVEN = 2  # round amax to the element mantissa width first, then floor
+
+# emax of the element format (exponent of its largest normal)
+_EMAX = {FMT_E4M3: 8, FMT_E2M1: 2}
+# mantissa (fp32 field) of the largest normal: 448 = 1.75*2^8, 6 = 1.5*2^2
+_MAXMAN = {FMT_E4M3: 0x600000, FMT_E2M1: 0x400000}
+# explicit mantissa bits of the element format
+_MBITS = {FMT_E4M3: 3, FMT_E2M1: 1}
+_MAXNORM = {FMT_E4M3: 448.0, FMT_E2M1: 6.0}
+
+E2M1_VALUES = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=np.float32)
+
+
+# --------------------------------------------------------------------------
+# bf16 <-> fp32 helpers (bf16 carried as uint16 bit patterns)
+# --------------------------------------------------------------------------
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    """Exact widening of bf16 bit patterns (uint16) to float32."""
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even narrowing of float32 to bf16 bit patterns."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    r = u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))
+    out = (r >> np.uint32(16)).astype(np.uint16)
+    out[nan] = ((u[nan] >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16)
+    return out
+
+
+def to_bf16_bits(x) -> np.ndarray:
+    """Accept a torch bf16 tensor, a uint16 array or a float array."""
+    try:
+        import torch
+
+        if isinstance(x, torch.Tensor):
+            if x.dtype != torch.bfloat16:
+                x = x.to(torch.bfloat16)
+            return x.contiguous().cpu().view(torch.int16).numpy().view(np.uint16)
+    except ImportError:  # pragma: no cover
+        pass
+    x = np.asarray(x)
+    if x.dtype == np.uint16:
+        return x
+    return f32_to_bf16_bits(x.astype(np.float32))
+
+
+# --------------------------------------------------------------------------
+# E8M0 block scale
+# --------------------------------------------------------------------------
+def e8m0_scale_byte(amax_bits: np.ndarray, fmt: int, scale_mode: int = SCALE_OCP_FLOOR) -> np.ndarray:
+    """E8M0 byte for a block whose finite amax has fp32 bit pattern ``amax_bits``.
+
+    byte = clamp(E - emax_elem + bump, 0, 254) where E is the biased fp32
+    exponent field of amax (after the EVEN pre-rounding, if selected) and
+    bump is 1 only for RCEIL when amax's mantissa exceeds the mantissa of the
+    format's largest normal.  amax == 0 gives byte 0.  Non-finite blocks are
+    handled by the caller (byte 255).
+    """
+    b = amax_bits.astype(np.int64)
+    if scale_mode == SCALE_EVEN:
+        b = b + (1 << (23 - _MBITS[fmt] - 1))
+    e = b >> 23
+    bump = np.zeros_like(e)
+    if scale_mode == SCALE_RCEIL:
+        bump = ((b & 0x7FFFFF) > _MAXMAN[fmt]).astype(np.int64)
+    byte = np.clip(e - _EMAX[fmt] + bump, 0, 254)
+    return byte.astype(np.uint8)
+
+
+def inv_scale_f32(byte: np.ndarray) -> np.ndarray:
+    """2^(127 - byte) as float32 (always a normal number for byte in [0, 253]);
+    0.0 for the NaN byte 255 so finite lanes of a non-finite block become +-0."""
+    b = byte.astype(np.int64)
+    bits = (np.clip(254 - b, 0, 254) << 23).astype(np.uint32)
+    out = bits.view(np.float32).copy()
+    out[b == 255] = 0.0
+    # byte 254 (scale 2^127) is unreachable from bf16 data (largest byte is 253)
+    return out
+
+
+def scale_f32(byte: np.ndarray) -> np.ndarray:
+    """2^(byte - 127) as float32 (float64 exponentiation, then exact narrowing);
+    NaN for byte 255."""
+    b = byte.astype(np.float64)
+    out = np.exp2(b - 127.0).astype(np.float32)
+    out[byte == 255] = np.nan
+    return out
+
+
+# --------------------------------------------------------------------------
+# element casts (saturating, round-to-nearest-even), integer arithmetic
+# --------------------------------------------------------------------------
+def cast_e4m3(v: np.ndarray) -> np.ndarray:
+    """float32 -> OCP FP8 E4M3 (fn) code, RNE, saturating at +-448, sign kept
+    on zero results, NaN -> sign|0x7F, +-Inf saturates like any large value."""
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    u = v.view(np.uint32)
+    sign = ((u >> np.uint32(24)) & np.uint32(0x80)).astype(np.uint8)
+    a_bits = u & np.uint32(0x7FFFFFFF)
+    nan = a_bits > np.uint32(0x7F800000)
+    a = np.minimum(a_bits.view(np.float32), np.float32(448.0))
+    a = np.where(nan, np.float32(0.0), a).astype(np.float32)
+    ab = a.view(np.uint32).astype(np.int64)
+    # normal range of e4m3: >= 2^-6
+    rounded = (ab + 0x7FFFF + ((ab >> 20) & 1)) >> 20  # (exp32 << 3) | m3 after carry
+    code_n = rounded - ((127 - 7) << 3)
+    # subnormal range: multiples of 2^-9
+    code_s = np.rint(a.astype(np.float64) * 512.0).astype(np.int64)
+    code = np.where(a >= np.float32(2.0**-6), code_n, code_s)
+    code = np.minimum(code, 0x7E)
+    code = np.where(nan, 0x7F, code)
+    return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def cast_e2m1(v: np.ndarray) -> np.ndarray:
+    """float32 -> FP4 E2M1 code (4 bits: s e e m), RNE (ties to even code),
+    saturating at +-6, sign kept on zero results.  NaN saturates to sign|7."""
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    u = v.view(np.uint32)
+    sign = ((u >> np.uint32(28)) & np.uint32(0x8)).astype(np.uint8)
+    a_bits = u & np.uint32(0x7FFFFFFF)
+    nan = a_bits > np.uint32(0x7F800000)
+    a = np.minimum(a_bits.view(np.float32), np.float32(6.0))
+    a = np.where(nan, np.float32(6.0), a).astype(np.float32)
+    ab = a.view(np.uint32).astype(np.int64)
+    rounded = (ab + 0x1FFFFF + ((ab >> 22) & 1)) >> 22  # (exp32 << 1) | m1
+    code_n = rounded - ((127 - 1) << 1)
+    code_s = np.rint(a.astype(np.float64) * 2.0).astype(np.int64)
+    code = np.where(a >= np.float32(1.0), code_n, code_s)
+    code = np.minimum(code, 7)
+    return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def decode_e4m3(code: np.ndarray) -> np.ndarray:
+    c = code.astype(np.int64)
+    s = np.where(c & 0x80, -1.0, 1.0)
+    e = (c >> 3) & 0xF
+    m = c & 0x7
+    val = np.where(e == 0, m * 2.0**-9, (8 + m) * np.exp2(e.astype(np.float64) - 10.0))
+    val = np.where((c & 0x7F) == 0x7F, np.nan, val)
+    return (s * val).astype(np.float32)
+
+
+def decode_e2m1(code: np.ndarray) -> np.ndarray:
+    c = code.astype(np.int64)
+    s = np.where(c & 0x8, -1.0, 1.0)
+    return (s * E2M1_VALUES[c & 0x7]).astype(np.float32)
+
+
+def pack_fp4(codes: np.ndarray) -> np.ndarray:
+    """Pack 4-bit codes along the last axis: element 2i -> bits 3:0, element
+    2i+1 -> bits 7:4 (the ``float4_e2m1fn_x2`` convention)."""
+    assert codes.shape[-1] % 2 == 0
+    lo = codes[..., 0::2] & 0xF
+    hi = codes[..., 1::2] & 0xF
+    return (lo | (hi << 4)).astype(np.uint8)
+
+
+def unpack_fp4(packed: np.ndarray) -> np.ndarray:
+    out = np.empty(packed.shape[:-1] + (packed.shape[-1] * 2,), dtype=np.uint8)
+    out[..., 0::2] = packed & 0xF
+    out[..., 1::2] = packed >> 4
+    return out
+
+
+# --------------------------------------------------------------------------
+# MX quantise / dequantise
+# --------------------------------------------------------------------------
+def _block_scale_bytes(xb_blocks: np.ndarray, fmt: int, scale_mode: int) -> np.ndarray:
+    """xb_blocks: uint16 bf16 bits, reduction over the last axis."""
+    mag = (xb_blocks & np.uint16(0x7FFF)).astype(np.uint32)
+    amax = mag.max(axis=-1)  # bf16 magnitudes order like unsigned ints
+    nonfinite = amax >= 0x7F80
+    byte = e8m0_scale_byte(amax << np.uint32(16), fmt, scale_mode)
+    byte[nonfinite] = 255
+    return byte
+
+
+def _cast_scaled(xb: np.ndarray, byte_per_elem: np.ndarray, fmt: int) -> np.ndarray:
+    x = bf16_bits_to_f32(xb)
+    inv = inv_scale_f32(byte_per_elem)
+    with np.errstate(invalid="ignore", over="ignore"):
+        v = (x * inv).astype(np.float32)  # exact: power-of-two factor; inf*0 -> nan
+    finite = (xb & np.uint16(0x7FFF)) < np.uint16(0x7F80)
+    if fmt == FMT_E4M3:
+        code = cast_e4m3(v)
+        # non-finite inputs (NaN or Inf) become NaN codes with the input's sign
+        sign = ((xb >> np.uint16(8)) & np.uint16(0x80)).astype(np.uint8)
+        code = np.where(finite, code, sign | np.uint8(0x7F)).astype(np.uint8)
+    else:
+        code = cast_e2m1(v)
+        sign = ((xb >> np.uint16(12)) & np.uint16(0x8)).astype(np.uint8)
+        code = np.where(finite, code, sign | np.uint8(0x7)).astype(np.uint8)
+    return code
+
+
+def quantize_mx_rowwise(x, fmt: int = FMT_E4M3, scale_mode: int = SCALE_OCP_FLOOR):
+    """x[..., K] bf16 -> (codes[..., K] (fp8) or [..., K/2] (fp4, packed),
+    scales[..., K/32]); blocks of 32 along the last axis (``axis=-1``,
+    primus_turbo.py:321-331)."""
+    xb = to_bf16_bits(x)
+    K = xb.shape[-1]
+    assert K % BLOCK == 0, "last dim must be a multiple of 32"
+    blocks = xb.reshape(xb.shape[:-1] + (K // BLOCK, BLOCK))
+    byte = _block_scale_bytes(blocks, fmt, scale_mode)
+    code = _cast_scaled(blocks, np.broadcast_to(byte[..., None], blocks.shape), fmt)
+    code = code.reshape(xb.shape)
+    if fmt == FMT_E2M1:
+        code = pack_fp4(code)
+    return code, byte
+
+
+def quantize_mx_colwise(x, fmt: int = FMT_E4M3, scale_mode: int = SCALE_OCP_FLOOR):
+    """``axis=-2`` quantisation: blocks of 32 along the second-to-last axis and
+    a TRANSPOSED result (primus_turbo.py:346-354):
+    x[..., M, C] -> codes[..., C, M] (or [..., C, M/2]), scales[..., C, M/32].
+    Defined as row-wise quantisation of the transposed input."""
+    xb = to_bf16_bits(x)
+    xt = np.ascontiguousarray(np.swapaxes(xb, -1, -2))
+    return quantize_mx_rowwise(xt, fmt, scale_mode)
+
+
+def quantize_mx_2d(x, fmt: int = FMT_E4M3, scale_mode: int = SCALE_OCP_FLOOR):
+    """2-D 32x32 block quantisation for weights (``use_2d_block=True``,
+    primus_turbo.py:313-317; grid definition weight_deosc.py:29-33): one scale
+    per 32x32 tile of each [N, K] matrix (leading dims are independent
+    matrices).  Returns the row-wise copy and the transposed copy, each with
+    its per-row scale array (the tile scale replicated):
+      (codes[..., N, K], scales[..., N, K/32], codesT[..., K, N], scalesT[..., K, N/32]).
+    """
+    xb = to_bf16_bits(x)
+    N, K = xb.shape[-2], xb.shape[-1]
+    assert N % BLOCK == 0 and K % BLOCK == 0
+    lead = xb.shape[:-2]
+    t = xb.reshape(lead + (N // BLOCK, BLOCK, K // BLOCK, BLOCK))
+    t = np.moveaxis(t, -2, -3)  # [..., N/32, K/32, 32, 32]
+    byte = _block_scale_bytes(t.reshape(t.shape[:-2] + (BLOCK * BLOCK,)), fmt, scale_mode)
+    code_t = _cast_scaled(t, np.broadcast_to(byte[..., None, None], t.shape), fmt)
+    code = np.moveaxis(code_t, -3, -2).reshape(xb.shape)
+    codeT = np.ascontiguousarray(np.swapaxes(code, -1, -2))
+    s_row = np.repeat(byte, BLOCK, axis=-2)  # [..., N, K/32]
+    s_col = np.repeat(np.swapaxes(byte, -1, -2), BLOCK, axis=-2)  # [..., K, N/32]
+    if fmt == FMT_E2M1:
+        code = pack_fp4(code)
+        codeT = pack_fp4(codeT)
+    return code, s_row, codeT, s_col
+
+
+def dequantize_mx(codes: np.ndarray, scales: np.ndarray, fmt: int = FMT_E4M3) -> np.ndarray:
+    """Inverse of the row-wise layout: float32[..., K]."""
+    if fmt == FMT_E2M1:
+        vals = decode_e2m1(unpack_fp4(codes))
+    else:
+        vals = decode_e4m3(codes)
+    s = np.repeat(scale_f32(scales), BLOCK, axis=-1)
+    with np.errstate(invalid="ignore", over="ignore"):
+        return (vals * s).astype(np.float32)
+
+
+# --------------------------------------------------------------------------
+# ragged (per-expert) column-wise layout used by the wgrad GEMM
+# --------------------------------------------------------------------------
+SEG_ALIGN = 128
+
+
+def segment_layout(group_lens, align: int = SEG_ALIGN):
+    """Offsets of each group's rows in the token-major tensor (``offs``) and in
+    the padded transposed tensor (``poffs``); every group's padded length is
+    its length rounded up to ``align``."""
+    lens = np.asarray(group_lens, dtype=np.int64)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    plen = (lens + align - 1) // align * align
+    poffs = np.concatenate([[0], np.cumsum(plen)])
+    return offs, poffs
+
+
+def padded_width(total_rows: int, num_groups: int, align: int = SEG_ALIGN) -> int:
+    """Capacity (in elements along the contraction dim) of the padded
+    transposed tensor, computable without reading ``group_lens``."""
+    return (total_rows + (align - 1) * max(num_groups, 1)) // align * align
+
+
+def quantize_mx_colwise_segmented(x, group_lens, fmt: int = FMT_E4M3, scale_mode: int = SCALE_OCP_FLOOR):
+    """Column-wise (transposed) quantisation whose 32-blocks restart at every
+    expert boundary, for the ragged-contraction wgrad GEMM
+    (zbpp_gemm.py:633-639 describes the segment-aware requirement).
+
+    x[sum(M_g), C] -> codes[C, W], scales[C, W/32] with
+    W = padded_width(sum(M_g), G).  Group g occupies columns
+    [poffs[g], poffs[g] + M_g); the tail up to the next multiple of 128 holds
+    zero codes and a scale computed from the zero-padded block (byte 0 for an
+    all-padding block).  Columns past poffs[G] are zero / byte 0.
+    """
+    xb = to_bf16_bits(x)
+    lens = np.asarray(group_lens, dtype=np.int64)
+    total, C = xb.shape
+    assert lens.sum() == total
+    offs, poffs = segment_layout(lens)
+    W = padded_width(total, len(lens))
+    xp = np.zeros((W, C), dtype=np.uint16)
+    for g in range(len(lens)):
+        xp[poffs[g] : poffs[g] + lens[g]] = xb[offs[g] : offs[g + 1]]
+    return quantize_mx_colwise(xp, fmt, scale_mode)
+
+
+# --------------------------------------------------------------------------
+# GEMMs: dequantise -> fp32 matmul -> bf16
+# --------------------------------------------------------------------------
+def _matmul_nt_f32(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    return np.matmul(a.astype(np.float32), b.astype(np.float32).T).astype(np.float32)
+
+
+def gemm_nt_ref(a_codes, a_scales, b_codes, b_scales, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, out_bf16=True):
+    """C[M, N] = dq(A)[M, K] . dq(B)[N, K]^T, fp32 accumulate."""
+    a = dequantize_mx(a_codes, a_scales, a_fmt)
+    b = dequantize_mx(b_codes, b_scales, b_fmt)
+    c = _matmul_nt_f32(a, b)
+    return f32_to_bf16_bits(c) if out_bf16 else c
+
+
+def grouped_gemm_nt_ref(a_codes, a_scales, b_codes, b_scales, group_lens, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, out_bf16=True):
+    """Forward / dgrad grouped GEMM: rows of A are split by ``group_lens``;
+    B is [G, N, K].  Empty groups contribute no rows."""
+    lens = np.asarray(group_lens, dtype=np.int64)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    N = b_codes.shape[1]
+    out = np.zeros((a_codes.shape[0], N), dtype=np.float32)
+    for g in range(len(lens)):
+        if lens[g] == 0:
+            continue
+        sl = slice(offs[g], offs[g + 1])
+        out[sl] = gemm_nt_ref(a_codes[sl], a_scales[sl], b_codes[g], b_scales[g], a_fmt, b_fmt, out_bf16=False)
+    return f32_to_bf16_bits(out) if out_bf16 else out
+
+
+def grouped_gemm_wgrad_ref(a_codes, a_scales, b_codes, b_scales, group_lens, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, out_bf16=True):
+    """Variable-K (wgrad) grouped GEMM on the segmented transposed layout:
+    A = dY^T codes [N, W], B = X^T codes [K, W]; dW[g] = A[:, seg_g] . B[:, seg_g]^T.
+    Empty groups give an all-zero dW[g]."""
+    lens = np.asarray(group_lens, dtype=np.int64)
+    _, poffs = segment_layout(lens)
+    a_per = 2 if a_fmt == FMT_E2M1 else 1
+    b_per = 2 if b_fmt == FMT_E2M1 else 1
+    G = len(lens)
+    out = np.zeros((G, a_codes.shape[0], b_codes.shape[0]), dtype=np.float32)
+    for g in range(G):
+        lo, hi = int(poffs[g]), int(poffs[g + 1])
+        if hi == lo:
+            continue
+        out[g] = gemm_nt_ref(
+            a_codes[:, lo // a_per : hi // a_per],
+            a_scales[:, lo // BLOCK : hi // BLOCK],
+            b_codes[:, lo // b_per : hi // b_per],
+            b_scales[:, lo // BLOCK : hi // BLOCK],
+            a_fmt,
+            b_fmt,
+            out_bf16=False,
+        )
+    return f32_to_bf16_bits(out) if out_bf16 else out
+
+
+# --------------------------------------------------------------------------
+# end-to-end linear (what ops.gemm_fp8 / grouped_gemm_fp8 compute)
+# --------------------------------------------------------------------------
+def linear_fwd_ref(x, w, fmt_x=FMT_E4M3, fmt_w=FMT_E4M3, scale_mode=SCALE_OCP_FLOOR, w_2d=True):
+    """Y = Q(X) . Q(W)^T for bf16 x[M, K], w[N, K] (primus_turbo.py:1095-1103)."""
+    xq, xs = quantize_mx_rowwise(x, fmt_x, scale_mode)
+    if w_2d:
+        wq, ws, _, _ = quantize_mx_2d(w, fmt_w, scale_mode)
+    else:
+        wq, ws = quantize_mx_rowwise(w, fmt_w, scale_mode)
+    return gemm_nt_ref(xq, xs, wq, ws, fmt_x, fmt_w)
+
+
+def linear_bwd_ref(x, w, dy, fmt=FMT_E4M3, scale_mode=SCALE_OCP_FLOOR, group_lens=None):
+    """(dX, dW) of the dense or grouped linear on bf16 inputs.
+    dX = Q_row(dY) . Q_colT(W)^T (contraction N); dW = Q_colT(dY) . Q_colT(X)^T
+    (contraction M, segment-aware).  Weight copies use 2-D blocks."""
+    xb, wb, dyb = to_bf16_bits(x), to_bf16_bits(w), to_bf16_bits(dy)
+    dense = group_lens is None
+    if dense:
+        group_lens = [xb.shape[0]]
+        wb = wb[None]
+    dyq, dys = quantize_mx_rowwise(dyb, fmt, scale_mode)
+    _, _, wqT, wsT = quantize_mx_2d(wb, fmt, scale_mode)
+    dx = grouped_gemm_nt_ref(dyq, dys, wqT, wsT, group_lens, fmt, fmt)
+    dyT, dysT = quantize_mx_colwise_segmented(dyb, group_lens, fmt, scale_mode)
+    xT, xsT = quantize_mx_colwise_segmented(xb, group_lens, fmt, scale_mode)
+    dw = grouped_gemm_wgrad_ref(dyT, dysT, xT, xsT, group_lens, fmt, fmt)
+    if dense:
+        dw = dw[0]
+    return dx, dw

@@ -1,0 +1,92 @@
+"""ctypes binding of the C-ABI extension (include/mxlinear.h).
+
+The extension is the only compute path: if the shared library is missing or a
+call fails, an exception is raised -- there is no CPU or PyTorch fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+from . import build as _build
+
+_lock = threading.Lock()
+_lib = None
+
+FMT_E4M3 = 0
+FMT_E2M1 = 1
+SCALE_OCP_FLOOR = 0
+SCALE_RCEIL = 1
+SCALE_EVEN = 2
+BLOCK = 32
+SEG_ALIGN = 128
+MAX_GROUPS = 1024
+
+EXPORTS = (
+    "mxl_version",
+    "mxl_error_string",
+    "mxl_padded_width",
+    "mxl_quantize",
+    "mxl_quantize_weight_2d",
+    "mxl_dequantize",
+    "mxl_gemm_nt",
+    "mxl_grouped_gemm_nt",
+    "mxl_grouped_gemm_wgrad",
+)
+
+
+class MXLinearError(RuntimeError):
+    pass
+
+
+def lib_path() -> str:
+    return _build.LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load libmxlinear.so (built in-tree by ``primus_amd.build``)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = lib_path()
+        if not os.path.exists(path):
+            raise MXLinearError(
+                f"{path} is missing: build the HIP extension first (python -m primus_amd.build). "
+                "The MX linear path has no fallback implementation."
+            )
+        lib = ctypes.CDLL(path)
+        vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        lib.mxl_version.restype = i32
+        lib.mxl_error_string.restype = ctypes.c_char_p
+        lib.mxl_error_string.argtypes = [i32]
+        lib.mxl_padded_width.restype = i64
+        lib.mxl_padded_width.argtypes = [i64, i32]
+        lib.mxl_quantize.restype = i32
+        lib.mxl_quantize.argtypes = [vp, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, vp]
+        lib.mxl_quantize_weight_2d.restype = i32
+        lib.mxl_quantize_weight_2d.argtypes = [vp, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
+        lib.mxl_dequantize.restype = i32
+        lib.mxl_dequantize.argtypes = [vp, vp, i64, i64, i32, vp, vp]
+        lib.mxl_gemm_nt.restype = i32
+        lib.mxl_gemm_nt.argtypes = [vp, vp, i32, vp, vp, i32, vp, i64, i64, i64, vp]
+        lib.mxl_grouped_gemm_nt.restype = i32
+        lib.mxl_grouped_gemm_nt.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        lib.mxl_grouped_gemm_wgrad.restype = i32
+        lib.mxl_grouped_gemm_wgrad.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().mxl_error_string(rc).decode()
+        raise MXLinearError(f"{what} failed: {msg} (code {rc})")
+
+
+def padded_width(total_rows: int, num_groups: int) -> int:
+    return int(load().mxl_padded_width(int(total_rows), int(num_groups)))

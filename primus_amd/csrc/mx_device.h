@@ -1,0 +1,122 @@
+// Device-side helpers shared by the MX quantisers and GEMMs (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mxlinear.h"
+
+namespace mxl {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+
+constexpr int kFmtE4M3 = MXL_FMT_E4M3;
+constexpr int kFmtE2M1 = MXL_FMT_E2M1;
+
+// Exponent of the largest normal, its fp32 mantissa field, explicit mantissa bits.
+template <int FMT> struct Elem;
+template <> struct Elem<kFmtE4M3> {
+    static constexpr int emax = 8;
+    static constexpr uint32_t maxman = 0x600000u;  // 448 = 1.75 * 2^8
+    static constexpr int mbits = 3;
+};
+template <> struct Elem<kFmtE2M1> {
+    static constexpr int emax = 2;
+    static constexpr uint32_t maxman = 0x400000u;  // 6 = 1.5 * 2^2
+    static constexpr int mbits = 1;
+};
+
+// E8M0 byte of a block from the largest bf16 magnitude in it (15-bit pattern).
+// Integer arithmetic on the fp32 exponent field only; 255 marks a block that
+// holds a NaN or an infinity.
+template <int FMT, int SMODE>
+__device__ __forceinline__ uint32_t scale_byte(uint32_t amax16) {
+    uint32_t b = amax16 << 16;
+    if (SMODE == MXL_SCALE_EVEN) b += 1u << (23 - Elem<FMT>::mbits - 1);
+    int e = (int)(b >> 23);
+    if (SMODE == MXL_SCALE_RCEIL) e += ((b & 0x7FFFFFu) > Elem<FMT>::maxman) ? 1 : 0;
+    e -= Elem<FMT>::emax;
+    e = e < 0 ? 0 : (e > 254 ? 254 : e);
+    return amax16 >= 0x7F80u ? 255u : (uint32_t)e;
+}
+
+// 2^(127 - byte) for byte <= 253 (always a normal float).
+__device__ __forceinline__ float inv_scale(uint32_t byte) { return __uint_as_float((254u - byte) << 23); }
+// 2^(byte - 127) for byte in [1, 254]; byte 0 gives the subnormal 2^-127.
+__device__ __forceinline__ float fwd_scale(uint32_t byte) {
+    return byte ? __uint_as_float(byte << 23) : __uint_as_float(0x00400000u);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xFFFF0000u); }
+
+// Largest magnitude (as 15-bit patterns) of the two bf16 halves, lane-wise packed.
+__device__ __forceinline__ uint32_t pk_absmax(uint32_t acc, uint32_t pair) {
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    us2 a = __builtin_bit_cast(us2, acc);
+    us2 b = __builtin_bit_cast(us2, pair & 0x7FFF7FFFu);
+    us2 r = {(unsigned short)(a[0] > b[0] ? a[0] : b[0]), (unsigned short)(a[1] > b[1] ? a[1] : b[1])};
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pk_max16(uint32_t x, uint32_t y) {
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    us2 a = __builtin_bit_cast(us2, x);
+    us2 b = __builtin_bit_cast(us2, y);
+    us2 r = {(unsigned short)(a[0] > b[0] ? a[0] : b[0]), (unsigned short)(a[1] > b[1] ? a[1] : b[1])};
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t hmax16(uint32_t pk) {
+    uint32_t lo = pk & 0xFFFFu, hi = pk >> 16;
+    return lo > hi ? lo : hi;
+}
+
+// Two bf16 (packed) -> two E4M3 bytes in the low 16 bits.  `inv` is the
+// power-of-two factor; the clamp makes the hardware convert (round to nearest
+// even, NaN on overflow) saturating.
+__device__ __forceinline__ uint32_t cvt2_e4m3(uint32_t pair, float inv) {
+    float a = __builtin_amdgcn_fmed3f(bf16_lo(pair) * inv, -448.f, 448.f);
+    float b = __builtin_amdgcn_fmed3f(bf16_hi(pair) * inv, -448.f, 448.f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
+}
+// Four bf16 (two packed pairs) -> four E4M3 bytes.
+__device__ __forceinline__ uint32_t cvt4_e4m3(uint32_t p0, uint32_t p1, float inv) {
+    float a = __builtin_amdgcn_fmed3f(bf16_lo(p0) * inv, -448.f, 448.f);
+    float b = __builtin_amdgcn_fmed3f(bf16_hi(p0) * inv, -448.f, 448.f);
+    float c = __builtin_amdgcn_fmed3f(bf16_lo(p1) * inv, -448.f, 448.f);
+    float d = __builtin_amdgcn_fmed3f(bf16_hi(p1) * inv, -448.f, 448.f);
+    int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+    return (uint32_t)r;
+}
+// Slow path for a block that holds a NaN/Inf: finite lanes -> signed zero,
+// non-finite lanes -> NaN code with the input's sign.
+__device__ __forceinline__ uint32_t nonfinite1_e4m3(uint32_t h) {
+    uint32_t s = (h >> 8) & 0x80u;
+    return ((h & 0x7FFFu) >= 0x7F80u) ? (s | 0x7Fu) : s;
+}
+__device__ __forceinline__ uint32_t nonfinite4_e4m3(uint32_t p0, uint32_t p1) {
+    return nonfinite1_e4m3(p0 & 0xFFFFu) | (nonfinite1_e4m3(p0 >> 16) << 8) | (nonfinite1_e4m3(p1 & 0xFFFFu) << 16) |
+           (nonfinite1_e4m3(p1 >> 16) << 24);
+}
+
+// Two bf16 (packed) -> two E2M1 nibbles in bits 7:0 (element 0 in bits 3:0).
+// The hardware convert divides by `scale` (a power of two), rounds to nearest
+// even and saturates at +-6.
+__device__ __forceinline__ uint32_t cvt2_e2m1(uint32_t pair, float scale) {
+    v2bf h = __builtin_bit_cast(v2bf, pair);
+    return __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(0u, h, scale, 0) & 0xFFu;
+}
+__device__ __forceinline__ uint32_t nonfinite1_e2m1(uint32_t h) {
+    uint32_t s = (h >> 12) & 0x8u;
+    return ((h & 0x7FFFu) >= 0x7F80u) ? (s | 0x7u) : s;
+}
+__device__ __forceinline__ uint32_t nonfinite2_e2m1(uint32_t pair) {
+    return nonfinite1_e2m1(pair & 0xFFFFu) | (nonfinite1_e2m1(pair >> 16) << 4);
+}
+
+}  // namespace mxl

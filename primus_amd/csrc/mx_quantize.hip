@@ -1,0 +1,413 @@
+// MX quantisers for gfx950: bf16 -> {E4M3, E2M1} codes + E8M0 block scales.
+//
+// One kernel family covers the three layouts the linear path needs
+// (primus_turbo.py:321-354, primus_turbo_mxfp4_local.py:147-207):
+//   ROW  : blocks of 32 along the columns, output in the input's orientation;
+//   COL  : blocks of 32 along the rows, output TRANSPOSED, blocks restarting at
+//          every expert boundary, each expert segment padded to 128;
+//   TWOD : one scale per 32x32 tile (weights), both copies from one scale.
+//
+// A workgroup (256 threads, 4 waves) owns a 128x128 tile.  Wave w owns rows
+// [32w, 32w+32) -- exactly one column-wise MX block -- and each lane loads
+// 8 rows x 8 columns as eight 16-byte loads, so a 16-lane group reads 256
+// contiguous bytes.  Row-block maxima are reduced over 4 adjacent lanes with
+// DPP, column-block maxima in registers over the lane's 8 rows and then over
+// the 4 lane groups.  The transposed codes go through an LDS tile so that the
+// global stores are 128 contiguous bytes per output row.
+#include "mx_device.h"
+
+namespace mxl {
+
+constexpr int QT = 128;       // tile edge
+constexpr int QTHREADS = 256;
+
+__device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+}
+
+struct QuantArgs {
+    const uint16_t* x;
+    int64_t rows, cols;
+    const int64_t* group_lens;
+    int num_groups;
+    uint8_t* q_row;
+    uint8_t* s_row;
+    uint8_t* q_colT;
+    uint8_t* s_colT;
+    int64_t W;          // padded width of the transposed copy (elements)
+    int64_t mat_rows;   // TWOD: rows per matrix (n); otherwise unused
+};
+
+template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD>
+__global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
+    constexpr bool FP4 = (FMT == kFmtE2M1);
+    constexpr int TPITCH = FP4 ? (QT / 2 + 16) : (QT + 16);  // bytes per LDS row of the transposed tile
+    __shared__ __attribute__((aligned(16))) uint8_t t_tile[COL ? QT * TPITCH : 16];
+    __shared__ uint32_t srow_tile[QT];
+    __shared__ uint32_t scol_tile[QT];
+
+    const int t = threadIdx.x;
+    const int w = t >> 6, l = t & 63, c16 = l & 15, rg = l >> 4;
+    const int64_t col0 = (int64_t)blockIdx.y * QT;
+    const int pt = blockIdx.x;
+
+    // ---- which source rows does this tile hold? ----
+    int64_t src_row0 = 0;
+    int rows_valid = 0;
+    int64_t batch_off_rows = 0;  // TWOD: first row of this matrix in the flattened input
+    if (TWOD) {
+        // grid.x enumerates (matrix, row tile); matrices are independent.
+        const int tiles_per_mat = (int)((a.mat_rows + QT - 1) / QT);
+        const int mat = pt / tiles_per_mat, rt = pt % tiles_per_mat;
+        batch_off_rows = (int64_t)mat * a.mat_rows;
+        src_row0 = batch_off_rows + (int64_t)rt * QT;
+        int64_t rem = a.mat_rows - (int64_t)rt * QT;
+        rows_valid = rem < QT ? (int)rem : QT;
+    } else if (!COL || a.group_lens == nullptr) {
+        src_row0 = (int64_t)pt * QT;
+        int64_t rem = a.rows - src_row0;
+        rows_valid = rem <= 0 ? 0 : (rem < QT ? (int)rem : QT);
+    } else {
+        int64_t off = 0;
+        int pto = 0;
+        for (int g = 0; g < a.num_groups; ++g) {
+            const int64_t len = a.group_lens[g];
+            const int nt = (int)((len + QT - 1) / QT);
+            if (pt < pto + nt) {
+                const int64_t r = (int64_t)(pt - pto) * QT;
+                src_row0 = off + r;
+                rows_valid = (len - r) < QT ? (int)(len - r) : QT;
+                break;
+            }
+            off += len;
+            pto += nt;
+        }
+    }
+
+    const int64_t col = col0 + 8 * c16;
+    const bool col_ok = col < a.cols;
+
+    // ---- load 8 rows x 8 columns per lane ----
+    uint4 d[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int r = 32 * w + 8 * rg + it;
+        d[it] = make_uint4(0, 0, 0, 0);
+        if (col_ok && r < rows_valid) d[it] = *(const uint4*)(a.x + (src_row0 + r) * a.cols + col);
+    }
+
+    // ---- block maxima ----
+    uint32_t rmax[8];  // per row: max over the lane's 8 columns, then over the 32-column block
+    uint32_t cmax[4] = {0, 0, 0, 0};  // per column pair (packed): max over the lane's 8 rows
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const uint32_t p0 = d[it].x & 0x7FFF7FFFu, p1 = d[it].y & 0x7FFF7FFFu, p2 = d[it].z & 0x7FFF7FFFu,
+                       p3 = d[it].w & 0x7FFF7FFFu;
+        if (COL && !TWOD) {
+            cmax[0] = pk_max16(cmax[0], p0);
+            cmax[1] = pk_max16(cmax[1], p1);
+            cmax[2] = pk_max16(cmax[2], p2);
+            cmax[3] = pk_max16(cmax[3], p3);
+        }
+        uint32_t m = pk_max16(pk_max16(p0, p1), pk_max16(p2, p3));
+        m = hmax16(m);
+        m = max(m, dpp_xor1(m));
+        m = max(m, dpp_xor2(m));
+        rmax[it] = m;
+    }
+    uint32_t tile_byte = 0;
+    if (TWOD) {
+        uint32_t m = rmax[0];
+#pragma unroll
+        for (int it = 1; it < 8; ++it) m = max(m, rmax[it]);
+        m = max(m, (uint32_t)__shfl_xor((int)m, 16));
+        m = max(m, (uint32_t)__shfl_xor((int)m, 32));
+        tile_byte = scale_byte<FMT, SMODE>(m);
+    } else if (COL) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 16));
+            cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 32));
+        }
+    }
+
+    // ---- row-wise copy ----
+    if (ROW) {
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = 32 * w + 8 * rg + it;
+            const uint32_t byte = TWOD ? tile_byte : scale_byte<FMT, SMODE>(rmax[it]);
+            if ((c16 & 3) == 0) ((uint8_t*)srow_tile)[r * 4 + (c16 >> 2)] = (uint8_t)byte;
+            if (!FP4) {
+                uint2 o;
+                if (byte != 255u) {
+                    const float inv = inv_scale(byte);
+                    o.x = cvt4_e4m3(d[it].x, d[it].y, inv);
+                    o.y = cvt4_e4m3(d[it].z, d[it].w, inv);
+                } else {
+                    o.x = nonfinite4_e4m3(d[it].x, d[it].y);
+                    o.y = nonfinite4_e4m3(d[it].z, d[it].w);
+                }
+                if (col_ok && r < rows_valid) *(uint2*)(a.q_row + (src_row0 + r) * a.cols + col) = o;
+            } else {
+                uint32_t o;
+                if (byte != 255u) {
+                    const float sc = fwd_scale(byte);
+                    o = cvt2_e2m1(d[it].x, sc) | (cvt2_e2m1(d[it].y, sc) << 8) | (cvt2_e2m1(d[it].z, sc) << 16) |
+                        (cvt2_e2m1(d[it].w, sc) << 24);
+                } else {
+                    o = nonfinite2_e2m1(d[it].x) | (nonfinite2_e2m1(d[it].y) << 8) | (nonfinite2_e2m1(d[it].z) << 16) |
+                        (nonfinite2_e2m1(d[it].w) << 24);
+                }
+                if (col_ok && r < rows_valid) *(uint32_t*)(a.q_row + ((src_row0 + r) * a.cols + col) / 2) = o;
+            }
+        }
+    }
+
+    // ---- column-wise (transposed) copy into the LDS tile ----
+    if (COL) {
+        const uint32_t* dw = (const uint32_t*)d;  // dw[it*4 + j]: columns 2j, 2j+1 of row `it`
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t amax = (j & 1) ? (cmax[j >> 1] >> 16) : (cmax[j >> 1] & 0xFFFFu);
+            const uint32_t byte = TWOD ? tile_byte : scale_byte<FMT, SMODE>(amax);
+            const int c = 8 * c16 + j;
+            if (rg == 0) ((uint8_t*)scol_tile)[c * 4 + w] = (uint8_t)byte;
+            // the lane's 8 rows of column j, as 4 packed (row 2i, row 2i+1) pairs
+            uint32_t pr[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t lo = dw[(2 * i) * 4 + (j >> 1)], hi = dw[(2 * i + 1) * 4 + (j >> 1)];
+                pr[i] = (j & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
+            }
+            if (!FP4) {
+                uint2 o;
+                if (byte != 255u) {
+                    const float inv = inv_scale(byte);
+                    o.x = cvt4_e4m3(pr[0], pr[1], inv);
+                    o.y = cvt4_e4m3(pr[2], pr[3], inv);
+                } else {
+                    o.x = nonfinite4_e4m3(pr[0], pr[1]);
+                    o.y = nonfinite4_e4m3(pr[2], pr[3]);
+                }
+                *(uint2*)(t_tile + c * TPITCH + 32 * w + 8 * rg) = o;
+            } else {
+                uint32_t o;
+                if (byte != 255u) {
+                    const float sc = fwd_scale(byte);
+                    o = cvt2_e2m1(pr[0], sc) | (cvt2_e2m1(pr[1], sc) << 8) | (cvt2_e2m1(pr[2], sc) << 16) |
+                        (cvt2_e2m1(pr[3], sc) << 24);
+                } else {
+                    o = nonfinite2_e2m1(pr[0]) | (nonfinite2_e2m1(pr[1]) << 8) | (nonfinite2_e2m1(pr[2]) << 16) |
+                        (nonfinite2_e2m1(pr[3]) << 24);
+                }
+                *(uint32_t*)(t_tile + c * TPITCH + (32 * w + 8 * rg) / 2) = o;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- scales: one dword (4 blocks) per row / per column of the tile ----
+    if (ROW && t < QT && t < rows_valid) {
+        const int64_t sld = a.cols / 32;
+        const int64_t nb = (a.cols - col0) / 32;  // valid blocks in this tile row
+        uint8_t* dst = a.s_row + (src_row0 + t) * sld + col0 / 32;
+        const uint32_t v = srow_tile[t];
+        if (nb >= 4 && (sld & 3) == 0) {
+            *(uint32_t*)dst = v;
+        } else {
+            for (int b = 0; b < 4 && b < nb; ++b) dst[b] = (uint8_t)(v >> (8 * b));
+        }
+    }
+    if (COL) {
+        const int64_t out_rows_base = TWOD ? (batch_off_rows / a.mat_rows) * a.cols : 0;  // TWOD: matrix * k
+        const int64_t m0 = TWOD ? (src_row0 - batch_off_rows) : (int64_t)pt * QT;          // position along W
+        if (t < QT && col0 + t < a.cols) {
+            uint8_t* dst = a.s_colT + (out_rows_base + col0 + t) * (a.W / 32) + m0 / 32;
+            const uint32_t v = scol_tile[t];
+            const int64_t nb = (a.W - m0) / 32;
+            if (nb >= 4 && ((a.W / 32) & 3) == 0) {
+                *(uint32_t*)dst = v;
+            } else {
+                for (int b = 0; b < 4 && b < nb; ++b) dst[b] = (uint8_t)(v >> (8 * b));
+            }
+        }
+        constexpr int ROWB = FP4 ? QT / 2 : QT;  // bytes per transposed tile row
+        constexpr int LPR = ROWB / 16;           // lanes per row
+        const int64_t wbytes = FP4 ? a.W / 2 : a.W;
+        const int64_t m0b = FP4 ? m0 / 2 : m0;
+        const int64_t avail = wbytes - m0b;      // bytes left in the output row (TWOD tails)
+#pragma unroll
+        for (int i = 0; i < QT / (QTHREADS / LPR); ++i) {
+            const int c = t / LPR + i * (QTHREADS / LPR);
+            const int ch = t % LPR;
+            if (col0 + c < a.cols && 16 * ch < avail) {
+                const uint4 v = *(const uint4*)(t_tile + c * TPITCH + 16 * ch);
+                *(uint4*)(a.q_colT + (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch) = v;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dequantise: codes + scales -> bf16 (row-wise layout)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float dec_e4m3(uint32_t c) {
+    // exact decode through fp32 bit assembly
+    const uint32_t s = (c & 0x80u) << 24, e = (c >> 3) & 0xFu, m = c & 7u;
+    float v;
+    if (e == 0)
+        v = (float)m * 0.001953125f;  // m * 2^-9
+    else if ((c & 0x7Fu) == 0x7Fu)
+        v = __uint_as_float(0x7FC00000u);
+    else
+        v = __uint_as_float(((e + 120u) << 23) | (m << 20));
+    return __uint_as_float(__float_as_uint(v) | s);
+}
+__device__ __forceinline__ float dec_e2m1(uint32_t c) {
+    const uint32_t s = (c & 8u) << 28, e = (c >> 1) & 3u, m = c & 1u;
+    const uint32_t bits = e ? (((e + 126u) << 23) | (m << 22)) : (m ? 0x3F000000u : 0u);
+    return __uint_as_float(bits | s);
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t* q, const uint8_t* s, uint16_t* out,
+                                                         int64_t nblocks) {
+    // one lane per 8 elements; 4 lanes per MX block
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t blk = i >> 2;
+    if (blk >= nblocks) return;
+    const uint32_t byte = s[blk];
+    // fp32 holds 2^(byte-127) exactly (subnormal for byte 0); multiply in two steps to stay exact
+    const float sc = (byte == 255u) ? __uint_as_float(0x7FC00000u) : fwd_scale(byte);
+    float v[8];
+    if (FMT == kFmtE4M3) {
+        const uint2 c = *(const uint2*)(q + i * 8);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            v[k] = dec_e4m3((c.x >> (8 * k)) & 0xFFu);
+            v[4 + k] = dec_e4m3((c.y >> (8 * k)) & 0xFFu);
+        }
+    } else {
+        const uint32_t c = *(const uint32_t*)(q + i * 4);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = dec_e2m1((c >> (4 * k)) & 0xFu);
+    }
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        v2bf h = {(__bf16)(v[2 * k] * sc), (__bf16)(v[2 * k + 1] * sc)};
+        o[k] = __builtin_bit_cast(uint32_t, h);
+    }
+    *(uint4*)(out + i * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// ---------------------------------------------------------------------------
+// host-side dispatch
+// ---------------------------------------------------------------------------
+template <int FMT, int SMODE, bool TWOD>
+static int launch_quant(const QuantArgs& a, dim3 grid, hipStream_t st) {
+    const bool row = a.q_row != nullptr, col = a.q_colT != nullptr;
+    if (row && col)
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD>), grid, dim3(QTHREADS), 0, st, a);
+    else if (row)
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD>), grid, dim3(QTHREADS), 0, st, a);
+    else
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD>), grid, dim3(QTHREADS), 0, st, a);
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
+
+template <bool TWOD>
+static int dispatch_quant(int fmt, int smode, const QuantArgs& a, dim3 grid, hipStream_t st) {
+#define MXL_Q(F, S) \
+    if (fmt == F && smode == S) return launch_quant<F, S, TWOD>(a, grid, st);
+    MXL_Q(MXL_FMT_E4M3, MXL_SCALE_OCP_FLOOR)
+    MXL_Q(MXL_FMT_E4M3, MXL_SCALE_RCEIL)
+    MXL_Q(MXL_FMT_E4M3, MXL_SCALE_EVEN)
+    MXL_Q(MXL_FMT_E2M1, MXL_SCALE_OCP_FLOOR)
+    MXL_Q(MXL_FMT_E2M1, MXL_SCALE_RCEIL)
+    MXL_Q(MXL_FMT_E2M1, MXL_SCALE_EVEN)
+#undef MXL_Q
+    return MXL_EINVAL;
+}
+
+}  // namespace mxl
+
+using namespace mxl;
+
+extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
+    if (num_groups < 1) num_groups = 1;
+    return (total_rows + (int64_t)(MXL_SEG_ALIGN - 1) * num_groups) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
+}
+
+extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int fmt, int scale_mode,
+                            const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                            void* s_colT, void* stream) {
+    if (!x_bf16 || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
+    if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
+    if (!q_row && !q_colT) return MXL_EINVAL;
+    if (num_groups < 0 || num_groups > MXL_MAX_GROUPS || (num_groups > 0) != (group_lens != nullptr)) return MXL_EINVAL;
+    QuantArgs a;
+    a.x = (const uint16_t*)x_bf16;
+    a.rows = rows;
+    a.cols = cols;
+    a.group_lens = group_lens;
+    a.num_groups = num_groups;
+    a.q_row = (uint8_t*)q_row;
+    a.s_row = (uint8_t*)s_row;
+    a.q_colT = (uint8_t*)q_colT;
+    a.s_colT = (uint8_t*)s_colT;
+    a.W = mxl_padded_width(rows, num_groups);
+    a.mat_rows = 0;
+    const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
+    const int64_t gy = (cols + QT - 1) / QT;
+    if (gx == 0) return MXL_OK;
+    if (gx > 0x7FFFFFFF || gy > 65535) return MXL_EINVAL;
+    return dispatch_quant<false>(fmt, scale_mode, a, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream);
+}
+
+extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int fmt,
+                                      int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
+                                      void* stream) {
+    if (!w_bf16 || batch <= 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
+    if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
+    if (!q_row && !q_colT) return MXL_EINVAL;
+    QuantArgs a;
+    a.x = (const uint16_t*)w_bf16;
+    a.rows = batch * n;
+    a.cols = k;
+    a.group_lens = nullptr;
+    a.num_groups = 0;
+    a.q_row = (uint8_t*)q_row;
+    a.s_row = (uint8_t*)s_row;
+    a.q_colT = (uint8_t*)q_colT;
+    a.s_colT = (uint8_t*)s_colT;
+    a.W = n;  // transposed copy of each matrix is [k, n]
+    a.mat_rows = n;
+    const int64_t gx = batch * ((n + QT - 1) / QT);
+    const int64_t gy = (k + QT - 1) / QT;
+    if (gx > 0x7FFFFFFF || gy > 65535) return MXL_EINVAL;
+    return dispatch_quant<true>(fmt, scale_mode, a, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream);
+}
+
+extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,
+                              void* out_bf16, void* stream) {
+    if (!codes || !scales || !out_bf16 || rows < 0 || k <= 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
+    const int64_t nblocks = rows * (k / MXL_BLOCK);
+    if (nblocks == 0) return MXL_OK;
+    const int64_t threads = nblocks * 4;
+    const int64_t grid = (threads + 255) / 256;
+    if (grid > 0x7FFFFFFF) return MXL_EINVAL;
+    if (fmt == MXL_FMT_E4M3)
+        hipLaunchKernelGGL((mx_dequant_kernel<MXL_FMT_E4M3>), dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                           (const uint8_t*)codes, (const uint8_t*)scales, (uint16_t*)out_bf16, nblocks);
+    else if (fmt == MXL_FMT_E2M1)
+        hipLaunchKernelGGL((mx_dequant_kernel<MXL_FMT_E2M1>), dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                           (const uint8_t*)codes, (const uint8_t*)scales, (uint16_t*)out_bf16, nblocks);
+    else
+        return MXL_EINVAL;
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}

@@ -146,7 +146,7 @@ def inv_scale_f32(byte: np.ndarray) -> np.ndarray:
 def scale_f32(byte: np.ndarray) -> np.ndarray:
     """2^(byte - 127) as float32 (float64 exponentiation, then exact narrowing);
     NaN for byte 255."""
-    b = byte.astype(np.float64)
+    b = np.where(byte == 255, 127, byte).astype(np.float64)
     out = np.exp2(b - 127.0).astype(np.float32)
     out[byte == 255] = np.nan
     return out

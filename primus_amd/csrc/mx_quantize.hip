@@ -346,7 +346,7 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
 extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int fmt, int scale_mode,
                             const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                             void* s_colT, void* stream) {
-    if (!x_bf16 || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
+    if ((!x_bf16 && rows > 0) || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
     if (!q_row && !q_colT) return MXL_EINVAL;
     if (num_groups < 0 || num_groups > MXL_MAX_GROUPS || (num_groups > 0) != (group_lens != nullptr)) return MXL_EINVAL;

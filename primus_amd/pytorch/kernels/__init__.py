@@ -1,0 +1,318 @@
+"""Tensor-level wrappers of the C-ABI extension (include/mxlinear.h).
+
+The ``*_impl`` names follow the low-level entry points the reference calls
+directly (gemm_fp8_impl: primus_turbo_float8_local.py:239-250; gemm_fp4_impl:
+primus_turbo_mxfp4_local.py:319-331; grouped_gemm_fp8_impl /
+grouped_gemm_fp8_variable_k_impl / group_offs_from_lens:
+zbpp_gemm.py:585-603,710-724).  Every function launches on the current HIP
+stream, allocates only its outputs and never reads device data from the host.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from ... import _lib
+from ..core.low_precision import (
+    ScalingGranularity,
+    dtype_to_fmt_code,
+    float4_e2m1fn_x2,
+    float8_e4m3,
+    float8_e8m0,
+)
+
+BLOCK = _lib.BLOCK
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("the MX linear path runs on the GPU only: got a CPU tensor")
+        if not t.is_contiguous():
+            raise ValueError("operands must be contiguous")
+
+
+def _codes_u8(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.uint8 else t.view(torch.uint8)
+
+
+def _per_byte(fmt: int) -> int:
+    return 2 if fmt == _lib.FMT_E2M1 else 1
+
+
+def _code_dtype(fmt: int) -> torch.dtype:
+    return float4_e2m1fn_x2 if fmt == _lib.FMT_E2M1 else float8_e4m3
+
+
+def fmt_of(codes: torch.Tensor) -> int:
+    return dtype_to_fmt_code(codes.dtype)
+
+
+def padded_width(total_rows: int, num_groups: int) -> int:
+    """Width of the segment-padded transposed layout (see mxl_padded_width)."""
+    return _lib.padded_width(total_rows, num_groups)
+
+
+def group_offs_from_lens(group_lens: torch.Tensor) -> torch.Tensor:
+    """Exclusive prefix sum [G+1] of tokens-per-expert, on the device
+    (zbpp_gemm.py:585).  The kernels here rebuild it themselves from
+    ``group_lens``; it is provided for callers that keep it around."""
+    offs = torch.zeros(group_lens.numel() + 1, dtype=torch.int64, device=group_lens.device)
+    torch.cumsum(group_lens.to(torch.int64), dim=0, out=offs[1:])
+    return offs
+
+
+def _check_group_lens(group_lens: Optional[torch.Tensor], device) -> int:
+    if group_lens is None:
+        return 0
+    if group_lens.dtype != torch.int64 or group_lens.dim() != 1:
+        raise ValueError("group_lens must be a 1-D int64 tensor")
+    if group_lens.device != device:
+        raise ValueError("group_lens must live on the same device as the activations")
+    if not group_lens.is_contiguous():
+        raise ValueError("group_lens must be contiguous")
+    if group_lens.numel() < 1 or group_lens.numel() > _lib.MAX_GROUPS:
+        raise ValueError(f"number of groups must be in [1, {_lib.MAX_GROUPS}]")
+    return group_lens.numel()
+
+
+# --------------------------------------------------------------------------
+# quantise / dequantise
+# --------------------------------------------------------------------------
+def quantize_mx_impl(
+    x: torch.Tensor,
+    fmt: int,
+    scale_mode: int = _lib.SCALE_OCP_FLOOR,
+    *,
+    rowwise: bool = True,
+    colwise: bool = False,
+    group_lens: Optional[torch.Tensor] = None,
+):
+    """MX-quantise bf16 ``x[rows, cols]``.
+
+    Returns ``(q_row, s_row, q_colT, s_colT)``; the pair that was not requested
+    is ``None``.  ``q_row``: codes ``[rows, cols]`` (``cols/2`` bytes for FP4),
+    ``s_row``: E8M0 ``[rows, cols/32]``.  ``q_colT``: codes of the transposed
+    tensor ``[cols, W]`` with 32-blocks along the token dim that restart at
+    each group boundary, ``W = padded_width(rows, G)``; ``s_colT``:
+    ``[cols, W/32]``.
+    """
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise ValueError("quantize expects a 2-D bfloat16 tensor")
+    _require_cuda(x, group_lens)
+    rows, cols = x.shape
+    if cols % BLOCK != 0:
+        raise ValueError(f"the quantised dim ({cols}) must be a multiple of {BLOCK}")
+    if not (rowwise or colwise):
+        raise ValueError("nothing to quantise: rowwise and colwise are both False")
+    G = _check_group_lens(group_lens, x.device)
+    per = _per_byte(fmt)
+    dev = x.device
+    q_row = s_row = q_col = s_col = None
+    if rowwise:
+        q_row = torch.empty((rows, cols // per), dtype=torch.uint8, device=dev)
+        s_row = torch.empty((rows, cols // BLOCK), dtype=torch.uint8, device=dev)
+    if colwise:
+        W = padded_width(rows, G)
+        q_col = torch.empty((cols, W // per), dtype=torch.uint8, device=dev)
+        s_col = torch.empty((cols, W // BLOCK), dtype=torch.uint8, device=dev)
+    if rows > 0 or (q_col is not None and q_col.numel() > 0):
+        # with no tokens only the padding of the transposed copy is left to write
+        row_ok = rows > 0
+        rc = _lib.load().mxl_quantize(
+            _ptr(x) if row_ok else None, rows, cols, fmt, scale_mode, _ptr(group_lens), G,
+            _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col), _stream(),
+        )
+        _lib.check(rc, "mxl_quantize")
+    cd = _code_dtype(fmt)
+    v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
+    return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0)
+
+
+def quantize_mx_weight_2d_impl(
+    w: torch.Tensor,
+    fmt: int,
+    scale_mode: int = _lib.SCALE_OCP_FLOOR,
+    *,
+    rowwise: bool = True,
+    colwise: bool = True,
+):
+    """2-D (32x32 tile) MX quantisation of ``w[n, k]`` or ``w[G, n, k]``;
+    returns ``(q_row [.., n, k], s_row [.., n, k/32], q_colT [.., k, n],
+    s_colT [.., k, n/32])`` with ``None`` for a copy that was not requested."""
+    if w.dtype != torch.bfloat16 or w.dim() not in (2, 3):
+        raise ValueError("weight quantisation expects a 2-D or 3-D bfloat16 tensor")
+    _require_cuda(w)
+    lead = tuple(w.shape[:-2])
+    batch = 1 if not lead else lead[0]
+    n, k = w.shape[-2], w.shape[-1]
+    if n % BLOCK != 0 or k % BLOCK != 0:
+        raise ValueError(f"2-D block quantisation needs both weight dims to be multiples of {BLOCK}, got {n}x{k}")
+    if not (rowwise or colwise):
+        raise ValueError("nothing to quantise: rowwise and colwise are both False")
+    per = _per_byte(fmt)
+    dev = w.device
+    q_row = s_row = q_col = s_col = None
+    if rowwise:
+        q_row = torch.empty(lead + (n, k // per), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(lead + (n, k // BLOCK), dtype=torch.uint8, device=dev)
+    if colwise:
+        q_col = torch.empty(lead + (k, n // per), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(lead + (k, n // BLOCK), dtype=torch.uint8, device=dev)
+    rc = _lib.load().mxl_quantize_weight_2d(
+        _ptr(w), batch, n, k, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col), _stream()
+    )
+    _lib.check(rc, "mxl_quantize_weight_2d")
+    cd = _code_dtype(fmt)
+    v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
+    return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0)
+
+
+def dequantize_mx_impl(codes: torch.Tensor, scales: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Row-wise layout back to bf16: ``out[..., k] = decode(codes) * 2^(scale-127)``."""
+    _require_cuda(codes, scales)
+    fmt = fmt_of(codes)
+    per = _per_byte(fmt)
+    k = codes.shape[-1] * per
+    rows = codes.numel() // codes.shape[-1] if codes.numel() else 0
+    if scales.shape[-1] * BLOCK != k or scales.numel() * BLOCK != rows * k:
+        raise ValueError("scale shape does not match the codes (one E8M0 byte per 32 elements)")
+    out = torch.empty(tuple(codes.shape[:-1]) + (k,), dtype=torch.bfloat16, device=codes.device)
+    rc = _lib.load().mxl_dequantize(_ptr(codes), _ptr(scales), rows, k, fmt, _ptr(out), _stream())
+    _lib.check(rc, "mxl_dequantize")
+    return out if out_dtype == torch.bfloat16 else out.to(out_dtype)
+
+
+# --------------------------------------------------------------------------
+# GEMMs on pre-quantised operands
+# --------------------------------------------------------------------------
+def _check_out_dtype(out_dtype) -> None:
+    if out_dtype not in (None, torch.bfloat16):
+        raise ValueError("the MX GEMMs produce bfloat16 output")
+
+
+def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T."""
+    _check_out_dtype(out_dtype)
+    _require_cuda(a, a_scale, b, b_scale)
+    a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
+    n, kb = b.shape[0], b.shape[1] * _per_byte(b_fmt)
+    if k != kb:
+        raise ValueError(f"contraction dims differ: {k} vs {kb}")
+    if tuple(a_scale.shape) != (m, k // BLOCK) or tuple(b_scale.shape) != (n, k // BLOCK):
+        raise ValueError("scale shapes must be [rows, k/32]")
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    rc = _lib.load().mxl_gemm_nt(_ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), m, n, k, _stream())
+    _lib.check(rc, "mxl_gemm_nt")
+    return c
+
+
+def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Forward / dgrad grouped GEMM: rows of ``a[total_m, k]`` split by
+    ``group_lens``; ``b`` is ``[G, n, k]``."""
+    _check_out_dtype(out_dtype)
+    _require_cuda(a, a_scale, b, b_scale, group_lens)
+    G = _check_group_lens(group_lens, a.device)
+    a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if b.dim() != 3 or b.shape[0] != G:
+        raise ValueError("grouped GEMM expects weights of shape [num_groups, n, k]")
+    total_m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
+    n, kb = b.shape[1], b.shape[2] * _per_byte(b_fmt)
+    if k != kb:
+        raise ValueError(f"contraction dims differ: {k} vs {kb}")
+    if tuple(a_scale.shape) != (total_m, k // BLOCK) or tuple(b_scale.shape) != (G, n, k // BLOCK):
+        raise ValueError("scale shapes must be [rows, k/32]")
+    c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+    rc = _lib.load().mxl_grouped_gemm_nt(
+        _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
+    )
+    _lib.check(rc, "mxl_grouped_gemm_nt")
+    return c
+
+
+def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total_m, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Variable-K (wgrad) grouped GEMM on segment-padded transposed operands:
+    ``a_t`` = dY^T codes ``[n, W]``, ``b_t`` = X^T codes ``[k, W]``; returns
+    ``[G, n, k]`` (``[n, k]`` when ``group_lens`` is None).  An expert with no
+    tokens gets a zero gradient."""
+    _check_out_dtype(out_dtype)
+    _require_cuda(a_t, a_t_scale, b_t, b_t_scale, group_lens)
+    G = _check_group_lens(group_lens, a_t.device)
+    a_fmt, b_fmt = fmt_of(a_t), fmt_of(b_t)
+    W = padded_width(total_m, G)
+    n, k = a_t.shape[0], b_t.shape[0]
+    if a_t.shape[1] * _per_byte(a_fmt) != W or b_t.shape[1] * _per_byte(b_fmt) != W:
+        raise ValueError(f"transposed operands must have padded width {W}")
+    if tuple(a_t_scale.shape) != (n, W // BLOCK) or tuple(b_t_scale.shape) != (k, W // BLOCK):
+        raise ValueError("scale shapes must be [rows, W/32]")
+    shape = (n, k) if group_lens is None else (G, n, k)
+    c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
+    rc = _lib.load().mxl_grouped_gemm_wgrad(
+        _ptr(a_t), _ptr(a_t_scale), a_fmt, _ptr(b_t), _ptr(b_t_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
+    )
+    _lib.check(rc, "mxl_grouped_gemm_wgrad")
+    return c
+
+
+# --------------------------------------------------------------------------
+# reference-named low-level entry points (MX granularity only)
+# --------------------------------------------------------------------------
+def _require_mx(granularity) -> None:
+    val = getattr(granularity, "value", granularity)
+    if val != ScalingGranularity.MX_BLOCKWISE.value:
+        raise NotImplementedError("only ScalingGranularity.MX_BLOCKWISE has kernels in this build")
+
+
+def gemm_fp8_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity=None, default_backend=None):
+    """gemm_fp8_impl of the reference (primus_turbo_float8_local.py:239-250)
+    for MX operands: only the NT form (trans_a=False, trans_b=True,
+    trans_c=False) exists because MX operands are quantised along K."""
+    _require_mx(granularity)
+    if trans_a or not trans_b or trans_c:
+        raise ValueError("MX GEMM supports the NT layout only (trans_a=False, trans_b=True, trans_c=False)")
+    return gemm_mx_nt_impl(a, a_scale_inv, b, b_scale_inv, out_dtype)
+
+
+def gemm_fp4_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity=None, default_backend=None, preshuffled=False):
+    """gemm_fp4_impl of the reference (primus_turbo_mxfp4_local.py:319-331)."""
+    if preshuffled:
+        raise NotImplementedError("pre-shuffled FP4 layouts are not implemented")
+    return gemm_fp8_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity, default_backend)
+
+
+def grouped_gemm_fp8_impl(a, b, a_scale_inv, b_scale_inv, group_lens, group_offs, trans_a=False, trans_b=True, out_dtype=torch.bfloat16, granularity=None, num_cu=None, default_backend=None):
+    """grouped_gemm_fp8_impl of the reference (zbpp_gemm.py:590-603);
+    ``group_offs`` and ``num_cu`` are accepted and unused (the tile schedule
+    is derived from ``group_lens`` on the device)."""
+    _require_mx(granularity)
+    if trans_a or not trans_b:
+        raise ValueError("MX grouped GEMM supports the NT layout only (trans_a=False, trans_b=True)")
+    return grouped_gemm_mx_nt_impl(a, a_scale_inv, b, b_scale_inv, group_lens, out_dtype)
+
+
+def grouped_gemm_fp8_variable_k_impl(a, b, a_scale_inv, b_scale_inv, group_lens, group_offs, trans_a=True, trans_b=False, trans_c=True, out_dtype=torch.bfloat16, granularity=None, num_cu=None, default_backend=None, total_m=None):
+    """grouped_gemm_fp8_variable_k_impl of the reference (zbpp_gemm.py:710-724):
+    ``a`` = X col-wise copy ``[k, W]``, ``b`` = dY col-wise copy ``[n, W]``
+    (both transposed, segment-padded); with ``trans_c=True`` (weights stored
+    ``[n, k]``, i.e. trans_b=True in the forward) returns ``[G, n, k]``."""
+    _require_mx(granularity)
+    if not trans_a or trans_b:
+        raise ValueError("variable-K grouped GEMM expects trans_a=True, trans_b=False")
+    if total_m is None:
+        raise ValueError("total_m (number of tokens) is required: the padded width alone does not determine it")
+    if trans_c:
+        return grouped_gemm_mx_wgrad_impl(b, b_scale_inv, a, a_scale_inv, group_lens, total_m, out_dtype)
+    return grouped_gemm_mx_wgrad_impl(a, a_scale_inv, b, b_scale_inv, group_lens, total_m, out_dtype)

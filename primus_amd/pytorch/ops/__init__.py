@@ -1,0 +1,184 @@
+"""Differentiable operators of the MX linear path.
+
+Same entry points and argument meaning as the operators the reference's
+Megatron modules call:
+
+* ``gemm_fp8`` / ``gemm_fp4``: primus/backends/megatron/core/extensions/
+  primus_turbo.py:1095-1103, :1142-1150 (and indexer.py:166,208 positional use)
+* ``grouped_gemm_fp8`` / ``grouped_gemm_fp4``: primus_turbo.py:2122-2129,
+  :2171-2178; keyword ``group_lens=`` at
+  primus/backends/torchtitan/models/moe/moe.py:38-48
+
+Operand flow per GEMM (primus_turbo_mxfp4_local.py:316-331 fwd, :432-444
+dgrad, :447-459 wgrad): every GEMM is NT with both operands quantised along
+its contraction dim --
+  fwd   Y[M,N]  = Qrow(X)[M,K]   . Qrow(W)[N,K]^T
+  dgrad dX[M,K] = Qrow(dY)[M,N]  . QcolT(W)[K,N]^T
+  wgrad dW[N,K] = QcolT(dY)[N,M] . QcolT(X)[K,M]^T   (M ragged per expert)
+Activations and gradients use 1-D blocks of 32, weights 2-D 32x32 blocks.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from ... import _lib
+from .. import kernels as K
+from ..core.low_precision import (
+    Float4QuantConfig,
+    Float8QuantConfig,
+    Format,
+    ScalingGranularity,
+    fmt_code,
+)
+from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
+
+__all__ = ["gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4"]
+
+
+class _MXLinearFunction(torch.autograd.Function):
+    """Y = X . W^T on MX operands, dense (``group_lens is None``) or grouped."""
+
+    @staticmethod
+    def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode):
+        need_dgrad = a.requires_grad
+        need_wgrad = b.requires_grad
+        grouped = group_lens is not None
+        # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
+        a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
+            a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens
+        )
+        if isinstance(b, QuantizedTensor):
+            # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
+            if b.axis != -1:
+                raise ValueError("the forward weight copy must be quantised along axis=-1")
+            w_row, w_rs = b.codes, b.scales
+            w_col = w_cs = None
+            if need_dgrad:
+                if b_t is None:
+                    raise ValueError("dgrad needs the transposed weight copy (QuantizedTensorPair.data_t)")
+                if b_t.axis != -2:
+                    raise ValueError("QuantizedTensorPair.data_t must be quantised along axis=-2")
+                w_col, w_cs = b_t.codes, b_t.scales
+        else:
+            w_row, w_rs, w_col, w_cs = K.quantize_mx_weight_2d_impl(
+                b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad
+            )
+        if grouped:
+            y = K.grouped_gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, group_lens)
+        else:
+            y = K.gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs)
+        ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens)
+        ctx.cfg = (act_fmt, scale_mode, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape))
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        a_col, a_cs, w_col, w_cs, group_lens = ctx.saved_tensors
+        act_fmt, scale_mode, total_m, need_dgrad, need_wgrad, w_shape = ctx.cfg
+        grouped = group_lens is not None
+        dy = dy.contiguous()
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        d_row, d_rs, d_col, d_cs = K.quantize_mx_impl(
+            dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens
+        )
+        grad_a = grad_b = None
+        if need_dgrad:
+            if grouped:
+                grad_a = K.grouped_gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, group_lens)
+            else:
+                grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs)
+        if need_wgrad:
+            grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
+        return grad_a, grad_b, None, None, None, None, None
+
+
+def _formats(config, fp4: bool):
+    if fp4:
+        if not isinstance(config, Float4QuantConfig):
+            raise TypeError("gemm_fp4 / grouped_gemm_fp4 expect a Float4QuantConfig")
+        return fmt_code(config.activation_format), _lib.FMT_E2M1
+    if not isinstance(config, Float8QuantConfig):
+        raise TypeError("gemm_fp8 / grouped_gemm_fp8 expect a Float8QuantConfig")
+    if config.granularity != ScalingGranularity.MX_BLOCKWISE:
+        raise NotImplementedError(
+            f"only the MX_BLOCKWISE recipe has kernels in this build (got {config.granularity})"
+        )
+    if config.format == Format.E5M2:
+        raise NotImplementedError("the MXFP8 recipe uses E4M3 for every operand (primus_turbo.py:481-487)")
+    f = fmt_code(config.format)
+    return f, f
+
+
+def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4):
+    if trans_a or not trans_b:
+        raise ValueError("the MX linear path is NT only: trans_a=False, trans_b=True (primus_turbo.py:1095-1103)")
+    if fuse_bgrad_accum_pattern is not None:
+        # never set for MX / FP4 by the reference (primus_turbo.py:247-249,259-264)
+        raise NotImplementedError("fused wgrad accumulation is not available for MX recipes")
+    if out_dtype not in (None, torch.bfloat16):
+        raise ValueError("the MX GEMMs produce bfloat16 output")
+    if config is None:
+        raise ValueError("config (Float8QuantConfig / Float4QuantConfig) is required")
+    act_fmt, w_fmt = _formats(config, fp4)
+    if a.dim() != 2 or a.dtype != torch.bfloat16:
+        raise ValueError("activations must be a 2-D bfloat16 tensor (callers flatten to [tokens, K])")
+    if not a.is_contiguous():
+        raise ValueError("activations must be contiguous")
+    b_t = None
+    if isinstance(b, QuantizedTensorPair):
+        b, b_t = b.data, b.data_t
+        if b.fmt != w_fmt:
+            raise ValueError("cached weight format does not match the op")
+    elif isinstance(b, QuantizedTensor):
+        pass
+    else:
+        if b.dtype != torch.bfloat16:
+            raise ValueError("weights must be bfloat16 or a QuantizedTensorPair")
+        if not b.is_contiguous():
+            raise ValueError("weights must be contiguous")
+    want_dims = 2 if group_lens is None else 3
+    if b.dim() != want_dims:
+        raise ValueError(f"weights must have {want_dims} dims ([N, K] dense, [G, N, K] grouped)")
+    if b.shape[-1] != a.shape[-1]:
+        raise ValueError(f"contraction dims differ: activations K={a.shape[-1]}, weights K={b.shape[-1]}")
+    if group_lens is not None and group_lens.numel() != b.shape[0]:
+        raise ValueError("group_lens must have one entry per expert weight")
+    return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value)
+
+
+def gemm_fp8(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
+             config: Optional[Float8QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
+    """``a[M, K] @ b[N, K]^T`` with MXFP8 operands; ``b`` is a bf16 weight or a
+    ``QuantizedTensorPair`` of cached copies.  Differentiable in ``a`` and ``b``."""
+    return _run(a, b, None, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4=False)
+
+
+def gemm_fp4(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
+             config: Optional[Float4QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
+    """Same with MXFP4 weights (activations per ``config.activation_format``)."""
+    return _run(a, b, None, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4=True)
+
+
+def _lens(group_lens: torch.Tensor) -> torch.Tensor:
+    if group_lens is None:
+        raise ValueError("group_lens (tokens per expert) is required")
+    if group_lens.dtype != torch.int64:
+        group_lens = group_lens.to(torch.int64)
+    return group_lens.contiguous()
+
+
+def grouped_gemm_fp8(a, b, group_lens: torch.Tensor, trans_b: bool = True,
+                     config: Optional[Float8QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
+    """Per expert g: ``a[rows of g] @ b[g]^T``; ``group_lens`` is tokens per
+    expert (int64, on the device of ``a``, zeros allowed) and is never read
+    back to the host."""
+    return _run(a, b, _lens(group_lens), False, trans_b, None, config, fuse_bgrad_accum_pattern, fp4=False)
+
+
+def grouped_gemm_fp4(a, b, group_lens: torch.Tensor, trans_b: bool = True,
+                     config: Optional[Float4QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
+    return _run(a, b, _lens(group_lens), False, trans_b, None, config, fuse_bgrad_accum_pattern, fp4=True)

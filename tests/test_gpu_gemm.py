@@ -1,0 +1,225 @@
+"""HIP MX GEMMs (through the C ABI) against the CPU oracle: dense, grouped
+(ragged / empty experts), variable-K wgrad, FP8 and FP4 operands.
+
+Tolerance: max |got - want| <= 1e-2 * max |want| with bf16 output (the bound
+named for this path; the reference's own layout-agreement bar is 2e-2,
+tests/unit_tests/backends/megatron/test_native_fp8_layout.py:141-151).
+Operands whose products and sums are exact in fp32 must match bit for bit.
+"""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as o
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+TOL = 1e-2
+
+
+def _dt(fmt):
+    return torch.float8_e4m3fn if fmt == o.FMT_E4M3 else torch.float4_e2m1fn_x2
+
+
+def _dev(a, dev, dtype):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev).view(dtype)
+
+
+def _bf16_np(t):
+    return o.bf16_bits_to_f32(t.view(torch.int16).cpu().numpy().view(np.uint16))
+
+
+def _check(got, want, tol=TOL):
+    assert not np.isnan(got).any()
+    scale = max(np.abs(want).max(), 1e-30)
+    err = np.abs(got - want).max() / scale
+    assert err <= tol, f"max err {err:.3e} > {tol}"
+
+
+def _run_fwd(dev, x, w, lens, afmt, bfmt):
+    """x[M,K] bf16, w[G,N,K] bf16 (CPU) -> (gpu result, oracle result) as float arrays."""
+    from primus_amd.pytorch import kernels as K
+
+    aq, as_ = o.quantize_mx_rowwise(x, afmt)
+    bq, bs = o.quantize_mx_rowwise(w, bfmt)
+    want = o.grouped_gemm_nt_ref(aq, as_, bq, bs, lens, afmt, bfmt, out_bf16=False)
+    A, SA = _dev(aq, dev, _dt(afmt)), _dev(as_, dev, torch.float8_e8m0fnu)
+    B, SB = _dev(bq, dev, _dt(bfmt)), _dev(bs, dev, torch.float8_e8m0fnu)
+    if len(lens) == 1 and w.shape[0] == 1:
+        got = K.gemm_mx_nt_impl(A, SA, B[0], SB[0])
+    else:
+        got = K.grouped_gemm_mx_nt_impl(A, SA, B, SB, torch.tensor(lens, dtype=torch.int64, device=dev))
+    return _bf16_np(got), want
+
+
+@pytest.mark.parametrize(
+    "m,n,k",
+    [(256, 256, 128), (256, 256, 512), (300, 320, 384), (512, 512, 2880), (1, 32, 32), (257, 288, 160), (64, 1024, 4096)],
+)
+def test_dense_fp8(gpu, m, n, k):
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(1, n, k, generator=g) * 0.05).bfloat16()
+    got, want = _run_fwd(gpu, x, w, [m], o.FMT_E4M3, o.FMT_E4M3)
+    _check(got, want)
+
+
+@pytest.mark.parametrize("afmt,bfmt", [(0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("m,n,k", [(300, 320, 384), (130, 64, 2880)])
+def test_dense_fp4_mixes(gpu, afmt, bfmt, m, n, k):
+    g = torch.Generator().manual_seed(afmt * 2 + bfmt + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(1, n, k, generator=g) * 0.05).bfloat16()
+    got, want = _run_fwd(gpu, x, w, [m], afmt, bfmt)
+    _check(got, want)
+
+
+@pytest.mark.parametrize(
+    "lens,n,k",
+    [
+        ([300, 0, 5, 695], 512, 256),
+        ([0, 33, 1, 64], 96, 160),
+        ([0, 0, 0, 7], 64, 64),
+        ([256, 256], 256, 128),
+        ([1] * 32, 64, 96),
+        ([513, 0, 255, 257, 0, 1, 31, 1000], 320, 512),
+    ],
+)
+@pytest.mark.parametrize("afmt,bfmt", [(0, 0), (0, 1)])
+def test_grouped_ragged(gpu, lens, n, k, afmt, bfmt):
+    m = sum(lens)
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(len(lens), n, k, generator=g) * 0.05).bfloat16()
+    got, want = _run_fwd(gpu, x, w, lens, afmt, bfmt)
+    _check(got, want)
+
+
+def _int_operands(rng, rows, k):
+    vals = np.array([0x00, 0x38, 0x40, 0x44, 0x48, 0xB8, 0xC0, 0xC4], dtype=np.uint8)  # 0, +-1, +-2, +-3, 4
+    q = vals[rng.integers(0, len(vals), size=(rows, k))]
+    s = rng.integers(125, 130, size=(rows, k // 32)).astype(np.uint8)
+    return q, s
+
+
+def test_exact_integer_products_bit_exact(gpu):
+    """Small integers with power-of-two scales: every partial sum is exact in
+    fp32, so the result must equal the oracle bit for bit, whatever the
+    accumulation order."""
+    from primus_amd.pytorch import kernels as K
+
+    rng = np.random.default_rng(12)
+    lens = [300, 0, 77, 135]
+    m, n, k = sum(lens), 288, 384
+    aq, as_ = _int_operands(rng, m, k)
+    bq, bs = _int_operands(rng, 4 * n, k)
+    bq, bs = bq.reshape(4, n, k), bs.reshape(4, n, k // 32)
+    want = o.grouped_gemm_nt_ref(aq, as_, bq, bs, lens)
+    got = K.grouped_gemm_mx_nt_impl(
+        _dev(aq, gpu, torch.float8_e4m3fn), _dev(as_, gpu, torch.float8_e8m0fnu), _dev(bq, gpu, torch.float8_e4m3fn),
+        _dev(bs, gpu, torch.float8_e8m0fnu), torch.tensor(lens, dtype=torch.int64, device=gpu),
+    )
+    assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want)
+
+
+@pytest.mark.parametrize(
+    "lens,n,k",
+    [([300, 0, 5, 695], 320, 288), ([128], 256, 256), ([0, 33, 1, 64], 96, 160), ([0, 0], 64, 32), ([200, 200, 200], 512, 96)],
+)
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_wgrad_variable_k(gpu, lens, n, k, fmt):
+    from primus_amd.pytorch import kernels as K
+
+    m = sum(lens)
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(max(m, 1), k, generator=g).bfloat16()[:m]
+    dy = torch.randn(max(m, 1), n, generator=g).bfloat16()[:m]
+    dyT, dysT = o.quantize_mx_colwise_segmented(dy, lens, fmt)
+    xT, xsT = o.quantize_mx_colwise_segmented(x, lens, fmt)
+    want = o.grouped_gemm_wgrad_ref(dyT, dysT, xT, xsT, lens, fmt, fmt, out_bf16=False)
+    if dyT.shape[1] == 0:  # no tokens at all and G small enough that the padded width is 0
+        pytest.skip("degenerate: empty padded layout")
+    got = K.grouped_gemm_mx_wgrad_impl(
+        _dev(dyT, gpu, _dt(fmt)), _dev(dysT, gpu, torch.float8_e8m0fnu), _dev(xT, gpu, _dt(fmt)),
+        _dev(xsT, gpu, torch.float8_e8m0fnu), torch.tensor(lens, dtype=torch.int64, device=gpu), m,
+    )
+    got = _bf16_np(got)
+    assert got.shape == want.shape
+    for e, ln in enumerate(lens):
+        if ln == 0:
+            assert not got[e].any()  # an expert without tokens gets exactly zero
+    _check(got, want)
+
+
+def test_golden_ragged_case(gpu):
+    """The committed 4-expert case {0, 33, 1, 64}: forward from the stored codes,
+    then the whole linear (quantise + 3 GEMMs) from the stored bf16 tensors."""
+    from primus_amd.pytorch import kernels as K
+
+    r = np.load(os.path.join(GOLD, "ragged_gemm.npz"))
+    lens = torch.tensor(r["lens"], dtype=torch.int64, device=gpu)
+    e8 = torch.float8_e8m0fnu
+    y = K.grouped_gemm_mx_nt_impl(
+        _dev(r["xq"], gpu, torch.float8_e4m3fn), _dev(r["xs"], gpu, e8), _dev(r["wq"], gpu, torch.float8_e4m3fn), _dev(r["ws"], gpu, e8), lens
+    )
+    _check(_bf16_np(y), o.bf16_bits_to_f32(r["y"]))
+    m = int(r["lens"].sum())
+    dy = torch.from_numpy(r["dy"].view(np.int16)).to(gpu).view(torch.bfloat16)
+    x = torch.from_numpy(r["x"].view(np.int16)).to(gpu).view(torch.bfloat16)
+    d_row, d_rs, d_col, d_cs = K.quantize_mx_impl(dy, 0, 0, rowwise=True, colwise=True, group_lens=lens)
+    _, _, x_col, x_cs = K.quantize_mx_impl(x, 0, 0, rowwise=False, colwise=True, group_lens=lens)
+    dx = K.grouped_gemm_mx_nt_impl(d_row, d_rs, _dev(r["wqt"], gpu, torch.float8_e4m3fn), _dev(r["wst"], gpu, e8), lens)
+    dw = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, x_col, x_cs, lens, m)
+    _check(_bf16_np(dx), o.bf16_bits_to_f32(r["dx"]))
+    _check(_bf16_np(dw), o.bf16_bits_to_f32(r["dw"]))
+    assert not _bf16_np(dw)[0].any()
+
+
+def test_full_size_against_torch_fp32(gpu):
+    """Mixtral-shape fc2 slice at full K (14336) and N (4096) on 2048 ragged rows:
+    checked against a plain PyTorch fp32 matmul of the dequantised operands
+    (decoded with torch's own float8 view, not with this library)."""
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator(device=gpu).manual_seed(1003)
+    lens_l = [700, 0, 1, 600, 300, 447, 0, 0]
+    m, k, n, G = sum(lens_l), 14336, 4096, 8
+    x = torch.randn(m, k, generator=g, device=gpu).bfloat16()
+    w = (torch.randn(G, n, k, generator=g, device=gpu) * 0.02).bfloat16()
+    lens = torch.tensor(lens_l, dtype=torch.int64, device=gpu)
+    xq, xs, _, _ = K.quantize_mx_impl(x, 0, 0, rowwise=True, colwise=False)
+    wq, ws, _, _ = K.quantize_mx_weight_2d_impl(w, 0, 0, colwise=False)
+    y = K.grouped_gemm_mx_nt_impl(xq, xs, wq, ws, lens).float()
+
+    def deq(q, s):
+        sc = torch.exp2(s.view(torch.uint8).float() - 127.0).repeat_interleave(32, dim=-1)
+        return q.float() * sc
+
+    xd, wd = deq(xq, xs), deq(wq, ws)
+    offs = [0]
+    for ln in lens_l:
+        offs.append(offs[-1] + ln)
+    want = torch.cat([xd[offs[e] : offs[e + 1]] @ wd[e].t() for e in range(G)])
+    err = (y - want).abs().max() / want.abs().max()
+    assert float(err) <= TOL, float(err)
+
+
+def test_bad_arguments_return_errors(gpu):
+    from primus_amd.pytorch import kernels as K
+
+    a = torch.zeros(4, 64, dtype=torch.uint8, device=gpu).view(torch.float8_e4m3fn)
+    s = torch.zeros(4, 2, dtype=torch.uint8, device=gpu).view(torch.float8_e8m0fnu)
+    b = torch.zeros(32, 96, dtype=torch.uint8, device=gpu).view(torch.float8_e4m3fn)
+    sb = torch.zeros(32, 3, dtype=torch.uint8, device=gpu).view(torch.float8_e8m0fnu)
+    with pytest.raises(ValueError):
+        K.gemm_mx_nt_impl(a, s, b, sb)  # K mismatch
+    with pytest.raises(ValueError):
+        K.gemm_mx_nt_impl(a, s, b[:, :64].contiguous(), sb)  # scale shape mismatch
+    with pytest.raises(ValueError):
+        K.gemm_mx_nt_impl(a, s, b[:, :64].contiguous(), sb[:, :2].contiguous(), out_dtype=torch.float16)
+    lens = torch.tensor([4], dtype=torch.int32, device=gpu)
+    with pytest.raises(ValueError):
+        K.grouped_gemm_mx_nt_impl(a, s, b[None, :, :64].contiguous(), sb[None, :, :2].contiguous(), lens)  # int32 lens

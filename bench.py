@@ -1,0 +1,309 @@
+#!/usr/bin/env python3
+"""Benchmark of the MX low-precision linear path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: for both
+grouped linears of an MoE expert layer (fc1 and fc2), forward + backward
+through ``ops.grouped_gemm_fp8`` -- i.e. MX quantisation of activations,
+weights (2-D blocks, every step, as the reference does when there is a single
+microbatch: primus_turbo.py:1094-1103) and output gradients, the forward
+grouped GEMM, the dgrad grouped GEMM and the variable-K wgrad grouped GEMM.
+
+Default workload: the Mixtral-8x7B-shape MoE layer (8 experts, top-2, 16384
+tokens -> 32768 routed rows, hidden 4096, ffn 14336, gate+up fused 28672),
+routing from softmax of Gaussian logits plus a per-expert bias (skewed, ragged
+tokens-per-expert).  Inputs are generated on the GPU from fixed seeds and are
+resident in HBM before the timed region.
+
+Prints ONE JSON line:  metric = grouped-GEMM algorithmic TFLOP/s of the whole
+step (2*M*N*K per GEMM over all six GEMMs, divided by the wall time of the
+step including every quantiser), plus a roofline object for the dominant
+kernel and a CPU baseline (the C restatement of the oracle, timed on the host
+cores on a 1/64 row sample).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP8_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (experts, top_k, tokens, hidden, fc1_out, fc2_in, routing, seed, fp4)
+    "mixtral_8x7b_moe_mxfp8": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False),
+    "deepseek_v3_shard_mxfp8": dict(G=32, topk=8, tokens=8192, hidden=7168, fc1_out=4096, fc2_in=2048, routing="zipf", seed=1004, fp4=False),
+    "gpt_oss_120b_mxfp4": dict(G=128, topk=4, tokens=16384, hidden=2880, fc1_out=5760, fc2_in=2880, routing="uniform", seed=1005, fp4=True),
+    "llama3_8b_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False),
+}
+
+
+def route(spec):
+    """tokens-per-expert (python list) from seeded synthetic router logits."""
+    import torch
+
+    G, topk, tokens = spec["G"], spec["topk"], spec["tokens"]
+    if spec["routing"] == "dense":
+        return [tokens]
+    g = torch.Generator().manual_seed(spec["seed"])
+    logits = torch.randn(tokens, G, generator=g)
+    if spec["routing"] == "gauss_bias":
+        logits = logits + torch.randn(G, generator=g)
+    elif spec["routing"] == "zipf":
+        ranks = torch.randperm(G, generator=g).float() + 1.0
+        logits = logits + torch.log(ranks ** -1.2) * 3.0
+    probs = torch.softmax(logits, dim=-1)
+    idx = probs.topk(topk, dim=-1).indices.reshape(-1)
+    return torch.bincount(idx, minlength=G).tolist()
+
+
+class LaunchTimer:
+    """Brackets every C-ABI launch with events on the launch stream."""
+
+    def __init__(self):
+        self.records = []
+        self.enabled = False
+
+    def __call__(self, name, info):
+        return _Bracket(self, name, info)
+
+
+class _Bracket:
+    def __init__(self, owner, name, info):
+        self.o, self.name, self.info = owner, name, info
+
+    def __enter__(self):
+        if self.o.enabled:
+            import torch
+
+            self.e0 = torch.cuda.Event(enable_timing=True)
+            self.e1 = torch.cuda.Event(enable_timing=True)
+            self.e0.record(torch.cuda.current_stream())
+        return self
+
+    def __exit__(self, *exc):
+        if self.o.enabled:
+            import torch
+
+            self.e1.record(torch.cuda.current_stream())
+            self.o.records.append((self.name, self.info, self.e0, self.e1))
+        return False
+
+
+def quant_bytes(info):
+    """Algorithmic bytes of one quantiser launch: bf16 read + codes + 1 scale byte / 32."""
+    el = info["rows"] * info["cols"]
+    code = 0.5 if info["fmt"] == 1 else 1.0
+    copies = int(bool(info["rowwise"])) + int(bool(info["colwise"]))
+    return el * (2.0 + copies * (code + 1.0 / 32.0))
+
+
+def cpu_baseline(spec, lens, sample_div=64):
+    """The oracle's C restatement on the host cores, on 1/sample_div of the rows
+    (same experts and weights shapes): quantise -> dequantise -> fp32 matmul
+    (torch CPU) -> bf16, forward + dgrad + wgrad of both linears."""
+    import numpy as np
+    import torch
+
+    from oracle import c_oracle as C
+    from oracle import mx_oracle as o
+
+    C.load()
+    threads = len(os.sched_getaffinity(0))
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    torch.set_num_threads(threads)
+    fmt_w = o.FMT_E2M1 if spec["fp4"] else o.FMT_E4M3
+    G = spec["G"]
+    slens = [max(1, ln // sample_div) if ln else 0 for ln in lens]
+    m = sum(slens)
+    g = torch.Generator().manual_seed(spec["seed"])
+    flops = 0.0
+    t0 = time.perf_counter()
+    for (k, n) in ((spec["hidden"], spec["fc1_out"]), (spec["fc2_in"], spec["hidden"])):
+        x = o.to_bf16_bits(torch.randn(m, k, generator=g).bfloat16())
+        dy = o.to_bf16_bits(torch.randn(m, n, generator=g).bfloat16())
+        w = o.to_bf16_bits((torch.randn(G, n, k, generator=g) * 0.02).bfloat16())
+        xq, xs = C.quantize_rowwise(x, o.FMT_E4M3)
+        xt, xts = C.quantize_colwise_segmented(x, slens, o.FMT_E4M3)
+        dq, ds = C.quantize_rowwise(dy, o.FMT_E4M3)
+        dt, dts = C.quantize_colwise_segmented(dy, slens, o.FMT_E4M3)
+        wq, ws, wqt, wst = C.quantize_2d(w, fmt_w)
+        xf = torch.from_numpy(C.dequantize(xq, xs, o.FMT_E4M3))
+        df = torch.from_numpy(C.dequantize(dq, ds, o.FMT_E4M3))
+        xtf = torch.from_numpy(C.dequantize(xt, xts, o.FMT_E4M3))
+        dtf = torch.from_numpy(C.dequantize(dt, dts, o.FMT_E4M3))
+        offs = np.concatenate([[0], np.cumsum(slens)])
+        _, poffs = o.segment_layout(slens)
+        for e in range(G):
+            if slens[e] == 0:
+                continue
+            wf = torch.from_numpy(C.dequantize(wq[e], ws[e], fmt_w))
+            wtf = torch.from_numpy(C.dequantize(wqt[e], wst[e], fmt_w))
+            sl = slice(int(offs[e]), int(offs[e + 1]))
+            ps = slice(int(poffs[e]), int(poffs[e + 1]))
+            y = (xf[sl] @ wf.t()).bfloat16()
+            dx = (df[sl] @ wtf.t()).bfloat16()
+            dw = (dtf[:, ps] @ xtf[:, ps].t()).bfloat16()
+            del y, dx, dw
+            flops += 6.0 * slens[e] * n * k
+    dt_s = time.perf_counter() - t0
+    return {
+        "value": round(flops / dt_s / 1e12, 6),
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"same workload with tokens-per-expert divided by {sample_div} ({m} routed rows), full-size weights; "
+        f"C oracle quantise/dequantise + torch CPU fp32 matmul; {dt_s:.1f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="mixtral_8x7b_moe_mxfp8", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no expert all-to-all); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import primus_amd.pytorch as pt
+    from primus_amd.pytorch import kernels as K
+    from primus_amd.pytorch.core import Float4QuantConfig, Float8QuantConfig, Format, ScaleDtype, ScalingGranularity
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU: the MX linear path has no CPU fallback"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    spec = WORKLOADS[args.workload]
+    lens = route(spec)
+    G, M = spec["G"], sum(lens)
+    grouped = spec["routing"] != "dense"
+    if spec["fp4"]:
+        cfg = Float4QuantConfig(activation_format=Format.E4M3)
+        op = pt.ops.grouped_gemm_fp4
+    else:
+        cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0, block_size=32)
+        op = pt.ops.grouped_gemm_fp8 if grouped else None
+
+    gen = torch.Generator(device=dev).manual_seed(spec["seed"])
+    shapes = ((spec["hidden"], spec["fc1_out"]), (spec["fc2_in"], spec["hidden"]))
+    layers = []
+    for (k, n) in shapes:
+        x = torch.randn(M, k, generator=gen, device=dev).bfloat16().requires_grad_()
+        wshape = (G, n, k) if grouped else (n, k)
+        w = (torch.randn(*wshape, generator=gen, device=dev) * 0.02).bfloat16().requires_grad_()
+        dy = torch.randn(M, n, generator=gen, device=dev).bfloat16()
+        layers.append((x, w, dy, k, n))
+    gl = torch.tensor(lens, dtype=torch.int64, device=dev)
+    flops_step = sum(6.0 * M * n * k for (_, _, _, k, n) in layers)
+
+    def step():
+        for (x, w, dy, k, n) in layers:
+            if grouped:
+                y = op(x, w, gl, trans_b=True, config=cfg)
+            else:
+                y = pt.ops.gemm_fp8(x, w, trans_a=False, trans_b=True, out_dtype=None, config=cfg)
+            y.backward(dy)
+            x.grad = None
+            w.grad = None
+
+    timer = LaunchTimer()
+    K.set_launch_hook(timer)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.enabled = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    timer.enabled = False
+    K.set_launch_hook(None)
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = flops_step / (ms_per_step * 1e-3) / 1e12
+
+    # per-kernel accounting from the bracketed launches
+    acc = {}
+    for name, info, e0, e1 in timer.records:
+        d = e0.elapsed_time(e1) * 1e-3
+        a = acc.setdefault(name, dict(sec=0.0, n=0, flops=0.0, bytes=0.0))
+        a["sec"] += d
+        a["n"] += 1
+        if "gemm" in name:
+            a["flops"] += 2.0 * info["m"] * info["n"] * info["k"]
+        else:
+            a["bytes"] += quant_bytes(info)
+    fwd_name = "grouped_gemm_nt" if grouped else "gemm_nt"
+    gk = acc[fwd_name]
+    gemm_tflops = gk["flops"] / gk["sec"] / 1e12
+    roofline = {
+        "kernel": "mx_gemm_kernel<e4m3,%s,fwd/dgrad> (%s)" % ("e2m1" if spec["fp4"] else "e4m3", fwd_name),
+        "bound": "mfma",
+        "achieved": round(gemm_tflops, 2),
+        "peak": FP8_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(gemm_tflops / FP8_PEAK_TFLOPS, 4),
+        "avg_launch_ms": round(gk["sec"] / gk["n"] * 1e3, 4),
+        "flops_per_launch": gk["flops"] / gk["n"],
+        "traffic": None,
+    }
+    kernels = {}
+    for name, a in acc.items():
+        ent = {"launches_per_step": a["n"] // args.steps, "ms_per_step": round(a["sec"] * 1e3 / args.steps, 4)}
+        if a["flops"]:
+            ent["TFLOP/s"] = round(a["flops"] / a["sec"] / 1e12, 2)
+            ent["frac_fp8_mfma_peak"] = round(a["flops"] / a["sec"] / 1e12 / FP8_PEAK_TFLOPS, 4)
+        else:
+            ent["GB/s"] = round(a["bytes"] / a["sec"] / 1e9, 1)
+            ent["frac_hbm_peak"] = round(a["bytes"] / a["sec"] / 1e9 / HBM_PEAK_GBS, 4)
+        kernels[name] = ent
+    gemm_sec = sum(a["sec"] for nme, a in acc.items() if "gemm" in nme)
+    gemm_flops = sum(a["flops"] for nme, a in acc.items() if "gemm" in nme)
+
+    out = {
+        "metric": "MXFP8 grouped-GEMM TFLOPS (fwd+dgrad+wgrad, quantisers inside the timed step)",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"] else "mxfp8_e4m3 (E8M0 block scales), fp32 accumulate",
+        "data": "synthetic (seeded, generated on the GPU; random-init weights N(0,0.02))",
+        "config": {
+            "workload": args.workload,
+            "experts": G,
+            "routed_rows": M,
+            "tokens_per_expert": lens if G <= 32 else {"min": min(lens), "max": max(lens), "zeros": lens.count(0)},
+            "gemms_nk": [[n, k] for (_, _, _, k, n) in layers],
+            "flops_per_step": flops_step,
+        },
+        "frac_fp8_mfma_peak_whole_step": round(value / FP8_PEAK_TFLOPS, 4),
+        "gemm_only_TFLOP/s": round(gemm_flops / gemm_sec / 1e12, 2),
+        "gemm_only_frac_fp8_mfma_peak": round(gemm_flops / gemm_sec / 1e12 / FP8_PEAK_TFLOPS, 4),
+        "kernels": kernels,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(spec, lens)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

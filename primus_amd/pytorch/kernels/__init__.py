@@ -25,6 +25,31 @@ from ..core.low_precision import (
 
 BLOCK = _lib.BLOCK
 
+# Optional observer of kernel launches: ``hook(name, info)`` is entered as a
+# context manager around every C-ABI call (benchmarks use it to bracket the
+# launches with events on the launch stream).  None in normal operation.
+_launch_hook = None
+
+
+def set_launch_hook(hook) -> None:
+    global _launch_hook
+    _launch_hook = hook
+
+
+class _NoHook:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_HOOK = _NoHook()
+
+
+def _hooked(name: str, **info):
+    return _launch_hook(name, info) if _launch_hook is not None else _NO_HOOK
+
 
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None or t.numel() == 0 else t.data_ptr()
@@ -131,10 +156,11 @@ def quantize_mx_impl(
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
         row_ok = rows > 0
-        rc = _lib.load().mxl_quantize(
+        with _hooked("quantize", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
+          rc = _lib.load().mxl_quantize(
             _ptr(x) if row_ok else None, rows, cols, fmt, scale_mode, _ptr(group_lens), G,
             _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col), _stream(),
-        )
+          )
         _lib.check(rc, "mxl_quantize")
     cd = _code_dtype(fmt)
     v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
@@ -171,9 +197,10 @@ def quantize_mx_weight_2d_impl(
     if colwise:
         q_col = torch.empty(lead + (k, n // per), dtype=torch.uint8, device=dev)
         s_col = torch.empty(lead + (k, n // BLOCK), dtype=torch.uint8, device=dev)
-    rc = _lib.load().mxl_quantize_weight_2d(
-        _ptr(w), batch, n, k, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col), _stream()
-    )
+    with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
+        rc = _lib.load().mxl_quantize_weight_2d(
+            _ptr(w), batch, n, k, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col), _stream()
+        )
     _lib.check(rc, "mxl_quantize_weight_2d")
     cd = _code_dtype(fmt)
     v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
@@ -215,7 +242,8 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16) -> torch.T
     if tuple(a_scale.shape) != (m, k // BLOCK) or tuple(b_scale.shape) != (n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-    rc = _lib.load().mxl_gemm_nt(_ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), m, n, k, _stream())
+    with _hooked("gemm_nt", m=m, n=n, k=k):
+        rc = _lib.load().mxl_gemm_nt(_ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), m, n, k, _stream())
     _lib.check(rc, "mxl_gemm_nt")
     return c
 
@@ -236,9 +264,10 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
     if tuple(a_scale.shape) != (total_m, k // BLOCK) or tuple(b_scale.shape) != (G, n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
-    rc = _lib.load().mxl_grouped_gemm_nt(
-        _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
-    )
+    with _hooked("grouped_gemm_nt", m=total_m, n=n, k=k):
+        rc = _lib.load().mxl_grouped_gemm_nt(
+            _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
+        )
     _lib.check(rc, "mxl_grouped_gemm_nt")
     return c
 
@@ -260,9 +289,10 @@ def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total
         raise ValueError("scale shapes must be [rows, W/32]")
     shape = (n, k) if group_lens is None else (G, n, k)
     c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
-    rc = _lib.load().mxl_grouped_gemm_wgrad(
-        _ptr(a_t), _ptr(a_t_scale), a_fmt, _ptr(b_t), _ptr(b_t_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
-    )
+    with _hooked("grouped_gemm_wgrad", m=total_m, n=n, k=k):
+        rc = _lib.load().mxl_grouped_gemm_wgrad(
+            _ptr(a_t), _ptr(a_t_scale), a_fmt, _ptr(b_t), _ptr(b_t_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
+        )
     _lib.check(rc, "mxl_grouped_gemm_wgrad")
     return c
 

@@ -72,9 +72,15 @@ int64_t mxl_padded_width(int64_t total_rows, int num_groups);
  *                   codes.  Pass NULL for both to skip it.
  *   group_lens    : int64[num_groups] on the device, sum == rows; NULL (and
  *                   num_groups 0) means one group of `rows` rows.
+ *   row_ld        : number of columns of the row-wise copy, >= cols and a
+ *                   multiple of 32 (0 means cols).  Columns past `cols` are
+ *                   padding: zero codes, scale byte 0.  The GEMMs want the
+ *                   contraction dim in multiples of 128, so a caller pads here
+ *                   (the reference pads its MXFP4 operands to 128 as well,
+ *                   primus_turbo_mxfp4_local.py:119-124).
  * Requires cols % 32 == 0.
  */
-int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int fmt, int scale_mode,
+int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                  const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                  void* s_colT, void* stream);
 
@@ -84,9 +90,12 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int fmt, int sc
  * Row-wise copy: codes [batch, n, k], scales [batch, n, k/32]; transposed
  * copy: codes [batch, k, n], scales [batch, k, n/32] (either pair may be
  * NULL).  The tile scale is replicated so both copies carry per-row scales.
+ * k_ld / n_ld are the padded pitches of the two copies (>= k / >= n, multiples
+ * of 32, n_ld at most n rounded up to 128; 0 means no padding): codes
+ * [batch, n, k_ld] and [batch, k, n_ld], padding = zero codes, scale byte 0.
  * Requires n % 32 == 0 and k % 32 == 0. */
-int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int fmt,
-                           int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
+int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
+                           int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
                            void* stream);
 
 /* Row-wise dequantise to bf16 (QuantizedTensor.dequantize(),
@@ -97,7 +106,8 @@ int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t 
 /* Dense NT GEMM on pre-quantised operands (gemm_fp8_impl / gemm_fp4_impl:
  * primus_turbo_float8_local.py:239-250, primus_turbo_mxfp4_local.py:319-331):
  *   c[m, n] (bf16) = dq(a)[m, k] . dq(b)[n, k]^T, fp32 accumulation.
- * Requires k % 32 == 0 and n % 32 == 0. */
+ * Requires k % 128 == 0 (scale rows must be dword aligned; callers get there
+ * with the row_ld / k_ld padding of the quantisers) and n % 32 == 0. */
 int mxl_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                 const void* b_scales, int b_fmt, void* c_bf16, int64_t m, int64_t n, int64_t k,
                 void* stream);

@@ -22,6 +22,7 @@ SCALE_RCEIL = 1
 SCALE_EVEN = 2
 BLOCK = 32
 SEG_ALIGN = 128
+GEMM_K_ALIGN = 128  # the GEMM kernels take the contraction dim in multiples of this
 MAX_GROUPS = 1024
 
 EXPORTS = (
@@ -67,9 +68,9 @@ def load() -> ctypes.CDLL:
         lib.mxl_padded_width.restype = i64
         lib.mxl_padded_width.argtypes = [i64, i32]
         lib.mxl_quantize.restype = i32
-        lib.mxl_quantize.argtypes = [vp, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, vp]
+        lib.mxl_quantize.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, vp]
         lib.mxl_quantize_weight_2d.restype = i32
-        lib.mxl_quantize_weight_2d.argtypes = [vp, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
+        lib.mxl_quantize_weight_2d.argtypes = [vp, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         lib.mxl_dequantize.restype = i32
         lib.mxl_dequantize.argtypes = [vp, vp, i64, i64, i32, vp, vp]
         lib.mxl_gemm_nt.restype = i32

@@ -9,23 +9,27 @@
 // derived on the device from group_lens, so nothing is read back to the host
 // and empty experts cost nothing.  A workgroup (4 waves, 2x2) owns a 256x256
 // output tile; each wave a 128x128 sub-tile = 4x4 MFMA tiles of 32x32 with
-// fp32 accumulators.  K advances 128 elements (4 MX blocks) per stage through a
-// double-buffered LDS ring; 16-byte chunks are XOR-swizzled so the fragment
-// reads are bank-conflict free.
+// fp32 accumulators (256 accumulator registers per lane).  K advances 64
+// elements (2 MX blocks, one MFMA K step) per stage through a 4-stage LDS ring
+// that is filled by asynchronous global->LDS loads (buffer_load ... lds), three
+// stages ahead; fragments of stage s+1 are read from LDS while the MFMAs of
+// stage s run, so there is one barrier per stage and no register staging.
+// 16-byte chunks are XOR-swizzled so the fragment reads are bank-conflict free.
 //
 // MFMA operand layout (measured on gfx950): lane l holds row l%32; its 32
 // bytes are k = 16g + [0,16) and k = 32 + 16g + [0,16) with g = l/32; the
 // scale of (row r, block kb) is taken from lane r + 32*kb, byte `opsel` of the
 // scale register.  An FP4 operand instead holds k = 32g + [0,32) in its first
-// four registers (low nibble first).  The kernel feeds the N-side operand as MFMA source 0 so a
-// lane ends up with 4 consecutive output columns (one 8-byte bf16 store).
+// four registers (low nibble first).  The kernel feeds the N-side operand as
+// MFMA source 0 so a lane ends up with 4 consecutive output columns (one
+// 8-byte bf16 store).
 #include <atomic>
 
 #include "mx_device.h"
 
 namespace mxl {
 
-constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int BM = 256, BN = 256, BK = 64, NSTAGE = 4;
 constexpr int GTHREADS = 256;
 constexpr int MODE_FWD = 0;    // rows of A ragged by group; B = [G, N, K]
 constexpr int MODE_WGRAD = 1;  // contraction ragged by group; C = [G, M, N]
@@ -46,88 +50,84 @@ struct GemmArgs {
 };
 
 template <int FMT> struct Op {
-    static constexpr int kb = (FMT == kFmtE2M1) ? BK / 2 : BK;  // bytes per row per K stage
-    static constexpr int cpr = kb / 16;                         // 16-byte chunks per row
-    static constexpr int nld = 256 * cpr / GTHREADS;            // chunk loads per thread per stage
-    static constexpr int rows_per_ld = GTHREADS / cpr;          // tile rows covered by one load round
+    static constexpr bool fp4 = (FMT == kFmtE2M1);
+    static constexpr int kb = fp4 ? BK / 2 : BK;      // bytes per row per stage
+    static constexpr int cpr = kb / 16;               // 16-byte chunks per row (= loads per thread per stage)
+    static constexpr int rows_per_ld = GTHREADS / cpr;  // tile rows covered by one load round
+    static constexpr int tile_bytes = 256 * kb;
+    // XOR swizzle of the chunk index: 16 consecutive rows reading the same logical
+    // chunk hit 16 different 16-byte bank groups of the 256-byte LDS row.
+    static __device__ __forceinline__ int swz(int row) { return fp4 ? ((row >> 3) & 1) : ((row >> 2) & 3); }
 };
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-
-__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+// ---- asynchronous global -> LDS loads ------------------------------------
+// Written as inline assembly on purpose: the compiler then keeps no record of
+// LDS writes in flight and does not put a full vmcnt wait in front of every
+// LDS read; completion is waited for explicitly (wait_vm) before the barrier
+// that publishes a stage.  The hardware writes lane i's data to LDS address
+// M0 + size*i, so the XOR swizzle is applied on the global side: the lane that
+// owns physical chunk (row, pch) fetches logical chunk pch ^ swz(row).
+__device__ __forceinline__ v4i make_rsrc(const void* base, int64_t bytes) {
+    const uint64_t p = (uint64_t)base;
     const uint32_t n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)(bytes < 0 ? 0 : bytes);
-    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, n, 0x00020000);  // raw buffer, out-of-range reads give 0
+    v4i r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32) & 0xFFFF);  // stride 0: raw buffer
+    r[2] = __builtin_amdgcn_readfirstlane((int)n);                             // bytes; reads past it give 0
+    r[3] = 0x00020000;
+    return r;
 }
+__device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_off), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory");
+}
+// two scale bytes of one row, zero-extended into that lane's LDS dword
+__device__ __forceinline__ void dma2(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_off), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-// One operand stage, global -> LDS without passing through registers
-// (buffer_load_dwordx4 ... lds).  The hardware writes lane i of a wave to
-// LDS slot base + 16*i, so the XOR swizzle is applied on the global side:
-// the lane that owns physical chunk (row, pch) fetches logical chunk
-// pch ^ swz(row).  `voff` is that lane's byte offset inside the tile for load
-// round 0; later rounds only add a uniform row step.  In a partial last stage
-// the lanes past the end of K store zeros instead (their LDS slot is their own).
+// LDS -> MFMA fragment of one 32-row tile (one K step = one stage).
 template <int FMT>
-__device__ __forceinline__ void stage_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds, uint32_t voff, int64_t kbyte,
-                                             int64_t ld_bytes, int kbytes_left, int logical_ch, int w, int l) {
-    const bool ok = 16 * logical_ch < kbytes_left;
-#pragma unroll
-    for (int i = 0; i < Op<FMT>::nld; ++i) {
-        uint8_t* dst = lds + (i * 4 + w) * 1024;
-        const uint32_t soff = (uint32_t)(kbyte + (int64_t)i * Op<FMT>::rows_per_ld * ld_bytes);
-        if (ok)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 16, voff, soff, 0, 0);
-        else
-            *(uint4*)(dst + 16 * l) = make_uint4(0, 0, 0, 0);
-    }
-}
-
-// Scale dword (4 blocks of this K stage) of one row; blocks past the end read as 2^0.
-__device__ __forceinline__ uint32_t load_scale4(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_off, int64_t blk0,
-                                                int64_t blk_end, bool aligned) {
-    uint32_t v;
-    if (aligned && blk0 + 4 <= blk_end) {
-        v = __builtin_amdgcn_raw_buffer_load_b32(rsrc, row_off, (uint32_t)blk0, 0);
-    } else {
-        v = 0x7F7F7F7Fu;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (blk0 + j < blk_end) {
-                const uint32_t b = __builtin_amdgcn_raw_buffer_load_b8(rsrc, row_off, (uint32_t)(blk0 + j), 0);
-                v = (v & ~(0xFFu << (8 * j))) | (b << (8 * j));
-            }
-    }
-    return v;
-}
-
-// LDS -> MFMA fragment of one 32-row tile for K step ks (64 elements).
-template <int FMT>
-__device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int ks, int g) {
+__device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int g) {
     v8i f;
+    const int s = Op<FMT>::swz(row);
     if (FMT == kFmtE4M3) {
-        const int s = swz(row);
-        const uint4 lo = *(const uint4*)(lds + row * 128 + 16 * ((4 * ks + g) ^ s));
-        const uint4 hi = *(const uint4*)(lds + row * 128 + 16 * ((4 * ks + 2 + g) ^ s));
+        const uint4 lo = *(const uint4*)(lds + row * 64 + 16 * (g ^ s));
+        const uint4 hi = *(const uint4*)(lds + row * 64 + 16 * ((2 + g) ^ s));
         f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
         f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
     } else {
-        // FP4 operands are laid out differently (measured): the lane's 32 nibbles are the
-        // 32 consecutive k = 32g + [0,32) of the K step, i.e. one 16-byte chunk of the 64-byte row.
-        const int s = swz(row) & 3;
-        const uint4 v = *(const uint4*)(lds + row * 64 + 16 * ((2 * ks + g) ^ s));
+        const uint4 v = *(const uint4*)(lds + row * 32 + 16 * (g ^ s));
         f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
         f[4] = 0; f[5] = 0; f[6] = 0; f[7] = 0;
     }
     return f;
 }
 
+struct Frags {
+    v8i a[4], b[4];
+    int sa[4], sb[4];
+};
+
 template <int AFMT, int BFMT, int MODE>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
-    constexpr int A_BYTES = 256 * Op<AFMT>::kb, B_BYTES = 256 * Op<BFMT>::kb;
-    constexpr int STAGE = A_BYTES + B_BYTES + 2 * 256 * 4;
+    constexpr int A_BYTES = Op<AFMT>::tile_bytes, B_BYTES = Op<BFMT>::tile_bytes;
+    constexpr int STAGE = A_BYTES + B_BYTES;
+    constexpr int LPT = Op<AFMT>::cpr + Op<BFMT>::cpr;  // async data loads per thread per stage
+    // E8M0 scales travel in "panels": 16 bytes per row = the scales of 8 K stages
+    // (K = 512), one 16-byte request per row per operand, double-buffered.
+    constexpr int PANEL = 256 * 16;           // one operand
+    constexpr int PANELS = 2 * 2 * PANEL;     // 2 buffers x 2 operands
+    constexpr int CB = BFMT == kFmtE2M1 ? 4 : 0, BL = AFMT == kFmtE2M1 ? 4 : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    int* pre_tiles = (int*)(smem + 2 * STAGE);                       // [G+1] prefix of row tiles (FWD)
+    uint8_t* panels = smem + NSTAGE * STAGE;
+    int* pre_tiles = (int*)(panels + PANELS);                        // [G+1] prefix of row tiles (FWD)
     int64_t* pre_rows = (int64_t*)(pre_tiles + MXL_MAX_GROUPS + 2);  // [G+1] prefix of rows / padded cols
 
     const int t = threadIdx.x;
@@ -135,6 +135,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     const int l = t & 63, lr = l & 31, g = l >> 5;
     const int wm = w >> 1, wn = w & 1;
     const int G = p.num_groups;
+    const uint32_t smem_base = (uint32_t)(uintptr_t)smem;  // LDS byte address of the ring
 
     // ---- per-workgroup group tables (device-side, no host sync) ----
     if (t == 0) {
@@ -170,23 +171,30 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // each XCD a contiguous run of the tile order.
     const int nwg = gridDim.x;
     const int per_xcd = nwg >> 3;
+#ifdef EXP_NOREMAP
+    const int vwg = (int)blockIdx.x; (void)per_xcd;
+#else
     const int vwg = (nwg & 7) ? (int)blockIdx.x : ((int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3));
+#endif
 
-    const int64_t lda = (AFMT == kFmtE2M1) ? p.k / 2 : p.k;
-    const int64_t ldb = (BFMT == kFmtE2M1) ? p.k / 2 : p.k;
+    const int64_t lda = Op<AFMT>::fp4 ? p.k / 2 : p.k;
+    const int64_t ldb = Op<BFMT>::fp4 ? p.k / 2 : p.k;
     const int64_t ld_s = p.k / 32;  // scale row pitch (both operands)
-    const bool s_aligned = ((((uintptr_t)p.sa | (uintptr_t)p.sb | (uintptr_t)ld_s) & 3) == 0);
     const int64_t a_rows_total = (MODE == MODE_FWD) ? p.total_m : p.m;
     const int64_t b_rows_total = (MODE == MODE_FWD) ? (int64_t)G * p.n : p.n;
 
-    // per-thread constants of the global -> LDS mapping (see stage_to_lds)
-    const int a_row = t / Op<AFMT>::cpr, a_pch = t % Op<AFMT>::cpr;
-    const int a_lch = (AFMT == kFmtE2M1) ? (a_pch ^ (swz(a_row) & 3)) : (a_pch ^ swz(a_row));
-    const uint32_t a_voff = (uint32_t)(a_row * (int)lda + 16 * a_lch);
-    const int b_row = t / Op<BFMT>::cpr, b_pch = t % Op<BFMT>::cpr;
-    const int b_lch = (BFMT == kFmtE2M1) ? (b_pch ^ (swz(b_row) & 3)) : (b_pch ^ swz(b_row));
-    const uint32_t b_voff = (uint32_t)(b_row * (int)ldb + 16 * b_lch);
+    // per-thread constants of the global -> LDS mapping
+    const int a_row = t / Op<AFMT>::cpr, b_row = t / Op<BFMT>::cpr;
+    const uint32_t a_voff = (uint32_t)(a_row * (int)lda + 16 * ((t % Op<AFMT>::cpr) ^ Op<AFMT>::swz(a_row)));
+    const uint32_t b_voff = (uint32_t)(b_row * (int)ldb + 16 * ((t % Op<BFMT>::cpr) ^ Op<BFMT>::swz(b_row)));
     const uint32_t s_voff = (uint32_t)(t * (int)ld_s);
+#ifdef EXP_FULLLINE
+    // timing experiment only (wrong data): 8 lanes read 128 contiguous bytes of a row
+    const uint32_t a_voff_x = (uint32_t)((t / 8) * (int)lda + 16 * (t % 8));
+    const uint32_t b_voff_x = (uint32_t)((t / 8) * (int)ldb + 16 * (t % 8));
+#define a_voff a_voff_x
+#define b_voff b_voff_x
+#endif
 
     for (int tile = vwg; tile < total_tiles; tile += nwg) {
         // ---- decode tile -> (group, pid_m, pid_n) ----
@@ -233,15 +241,18 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         }
         const int64_t n0 = (int64_t)pid_n * BN;
         const int n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
-        const int kt_count = (int)((k1 - k0 + BK - 1) / BK);
+        const int kt_count = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BK));
 
         // Buffer descriptors anchored at the tile's first row: rows past the end
         // of the operand read as zero, rows of a neighbouring group are read but
         // never stored.
-        const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
-        const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
-        const __amdgpu_buffer_rsrc_t rsa = make_rsrc(p.sa + a_row0 * ld_s, (a_rows_total - a_row0) * ld_s);
-        const __amdgpu_buffer_rsrc_t rsb = make_rsrc(p.sb + b_row0 * ld_s, (b_rows_total - b_row0) * ld_s);
+        const v4i ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
+        const v4i rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
+        const v4i rsa = make_rsrc(p.sa + a_row0 * ld_s, (a_rows_total - a_row0) * ld_s);
+        const v4i rsb = make_rsrc(p.sb + b_row0 * ld_s, (b_rows_total - b_row0) * ld_s);
+        const uint32_t ka0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<AFMT>::fp4 ? k0 / 2 : k0));
+        const uint32_t kb0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<BFMT>::fp4 ? k0 / 2 : k0));
+        const uint32_t ks0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(k0 / 32));
 
         v16f acc[4][4];
 #pragma unroll
@@ -251,73 +262,106 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-        uint32_t vsa = 0, vsb = 0;
-        auto issue = [&](int kt, int stage) {
-            const int64_t ke = k0 + (int64_t)kt * BK;
-            const int left = (int)((k1 - ke) < BK ? (k1 - ke) : BK);
-            uint8_t* s = smem + stage * STAGE;
-            stage_to_lds<AFMT>(ra, s, a_voff, (AFMT == kFmtE2M1) ? ke / 2 : ke, lda, (AFMT == kFmtE2M1) ? left / 2 : left,
-                               a_lch, w, l);
-            stage_to_lds<BFMT>(rb, s + A_BYTES, b_voff, (BFMT == kFmtE2M1) ? ke / 2 : ke, ldb,
-                               (BFMT == kFmtE2M1) ? left / 2 : left, b_lch, w, l);
-            vsa = load_scale4(rsa, s_voff, ke / 32, k1 / 32, s_aligned);
-            vsb = load_scale4(rsb, s_voff, ke / 32, k1 / 32, s_aligned);
+        // async loads of K stage kt into ring slot `slot`, in three parts so they can be
+        // slotted between MFMAs
+        auto issue_a = [&](int kt, int slot) {
+            const uint32_t base = smem_base + slot * STAGE;
+#pragma unroll
+            for (int i = 0; i < Op<AFMT>::cpr; ++i)
+                dma16(ra, base + (i * 4 + w) * 1024, a_voff,
+                      ka0 + kt * Op<AFMT>::kb + (uint32_t)(i * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
         };
-        auto put_scales = [&](int stage) {
-            uint32_t* s = (uint32_t*)(smem + stage * STAGE + A_BYTES + B_BYTES);
-            s[t] = vsa;
-            s[256 + t] = vsb;
+        auto issue_b = [&](int kt, int slot) {
+            const uint32_t base = smem_base + slot * STAGE;
+#pragma unroll
+            for (int i = 0; i < Op<BFMT>::cpr; ++i)
+                dma16(rb, base + A_BYTES + (i * 4 + w) * 1024, b_voff,
+                      kb0 + kt * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb);
         };
-
-        if (kt_count > 0) {
-            issue(0, 0);
-            put_scales(0);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-
-        for (int kt = 0; kt < kt_count; ++kt) {
-            const bool more = kt + 1 < kt_count;
-            if (more) issue(kt + 1, (kt + 1) & 1);
-            const uint8_t* s = smem + (kt & 1) * STAGE;
-            const uint8_t* sA = s;
-            const uint8_t* sB = s + A_BYTES;
-            const uint32_t* sSA = (const uint32_t*)(s + A_BYTES + B_BYTES);
-            const uint32_t* sSB = sSA + 256;
-            int sca[4], scb[4];
+        // scale panel pn (K stages 8pn .. 8pn+7) into panel buffer pn & 1
+        auto issue_s = [&](int pn) {
+            const uint32_t base = smem_base + NSTAGE * STAGE + (pn & 1) * 2 * PANEL;
+            dma16(rsa, base + w * 1024, s_voff, ks0 + 16 * pn);
+            dma16(rsb, base + PANEL + w * 1024, s_voff, ks0 + 16 * pn);
+        };
+        // fragments and scale bytes of K stage kt (ring slot `slot`)
+        auto read_frags = [&](Frags& f, int kt, int slot) {
+            const uint8_t* s = smem + slot * STAGE;
+            const uint8_t* pan = panels + ((kt >> 3) & 1) * 2 * PANEL + 2 * (kt & 7) + g;  // byte of (stage, block g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) f.b[i] = read_frag<BFMT>(s + A_BYTES, wn * 128 + i * 32 + lr, g);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) f.a[i] = read_frag<AFMT>(s, wm * 128 + i * 32 + lr, g);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                sca[i] = (int)(sSA[wm * 128 + i * 32 + lr] >> (8 * g));
-                scb[i] = (int)(sSB[wn * 128 + i * 32 + lr] >> (8 * g));
+                f.sb[i] = pan[PANEL + 16 * (wn * 128 + i * 32 + lr)];
+                f.sa[i] = pan[16 * (wm * 128 + i * 32 + lr)];
             }
+        };
+#define MXL_MFMA(F, I, J) \
+    acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I])
+
+        Frags f0, f1;
+        __syncthreads();  // every wave is done reading the ring for the previous tile
+        // Stages past the end of K are requested as well (their data is never used):
+        // it keeps every step of the pipeline identical and free of branches.
+        issue_s(0);
+        issue_a(0, 0); issue_b(0, 0);
+        issue_a(1, 1); issue_b(1, 1);
+        issue_a(2, 2); issue_b(2, 2);
+        wait_vm<2 * LPT>();
+        __syncthreads();
+        read_frags(f0, 0, 0);
+        // One K stage: MFMAs of stage kt from registers `cur`; meanwhile stage kt+3
+        // is requested from memory and the fragments of stage kt+1 are read from LDS.
+        auto stage_body = [&](int kt, int sub, Frags& cur, Frags& nxt) {
+            const int slot = sub & 3;
+            MXL_MFMA(cur, 0, 0);
+#ifndef EXP_NOSCALE
+            if (sub == 0) issue_s((kt >> 3) + 1);  // next panel; its buffer was last read two stages ago
+#endif
+#ifndef EXP_NODMA
+            issue_a(kt + 3, (slot + 3) & 3);
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+            MXL_MFMA(cur, 1, 0);
+#ifndef EXP_NODMA
+            issue_b(kt + 3, (slot + 3) & 3);
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+            MXL_MFMA(cur, 2, 0);
+            MXL_MFMA(cur, 3, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<2 * LPT>();  // stage kt+1 has landed (kt+2, kt+3 may still be in flight)
+#ifndef EXP_NOBAR
+            __syncthreads();     // ... for every wave, and every wave is done reading slot of stage kt-1
+#endif
+#ifndef EXP_NOLDS
+            read_frags(nxt, kt + 1, (slot + 1) & 3);
+#endif
+            MXL_MFMA(cur, 0, 1); MXL_MFMA(cur, 1, 1); MXL_MFMA(cur, 2, 1); MXL_MFMA(cur, 3, 1);
+            MXL_MFMA(cur, 0, 2); MXL_MFMA(cur, 1, 2); MXL_MFMA(cur, 2, 2); MXL_MFMA(cur, 3, 2);
+            MXL_MFMA(cur, 0, 3); MXL_MFMA(cur, 1, 3); MXL_MFMA(cur, 2, 3); MXL_MFMA(cur, 3, 3);
+            // interleave: one MFMA, then two LDS reads, twelve times
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                v8i fa[4], fb[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    fa[i] = read_frag<AFMT>(sA, wm * 128 + i * 32 + lr, ks, g);
-                    fb[i] = read_frag<BFMT>(sB, wn * 128 + i * 32 + lr, ks, g);
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        // source 0 = N side (format cbsz), source 1 = M side (format blgp)
-                        if (ks == 0)
-                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                                fb[j], fa[i], acc[i][j], BFMT == kFmtE2M1 ? 4 : 0, AFMT == kFmtE2M1 ? 4 : 0, 0, scb[j], 0,
-                                sca[i]);
-                        else
-                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                                fb[j], fa[i], acc[i][j], BFMT == kFmtE2M1 ? 4 : 0, AFMT == kFmtE2M1 ? 4 : 0, 2, scb[j], 2,
-                                sca[i]);
-                    }
+            for (int r = 0; r < 12; ++r) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the wait: loads overlap with them
-            if (more) put_scales((kt + 1) & 1);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        for (int kt = 0; kt < kt_count; kt += 8) {
+            stage_body(kt, 0, f0, f1);
+            if (kt + 1 < kt_count) stage_body(kt + 1, 1, f1, f0);
+            if (kt + 2 < kt_count) stage_body(kt + 2, 2, f0, f1);
+            if (kt + 3 < kt_count) stage_body(kt + 3, 3, f1, f0);
+            if (kt + 4 < kt_count) stage_body(kt + 4, 4, f0, f1);
+            if (kt + 5 < kt_count) stage_body(kt + 5, 5, f1, f0);
+            if (kt + 6 < kt_count) stage_body(kt + 6, 6, f0, f1);
+            if (kt + 7 < kt_count) stage_body(kt + 7, 7, f1, f0);
         }
+        wait_vm<0>();  // drain the look-ahead requests before the ring is reused
+#undef MXL_MFMA
 
         // ---- epilogue: fp32 -> bf16, 4 consecutive columns per lane ----
 #pragma unroll
@@ -330,7 +374,11 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int ncol = wn * 128 + j * 32 + 8 * q + 4 * g;
+#ifdef EXP_NOSTORE
+                        if (ncol < n_valid && acc[i][j][4*q] == 1234.5f) {
+#else
                         if (ncol < n_valid) {
+#endif
                             v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1],
                                       (__bf16)acc[i][j][4 * q + 2], (__bf16)acc[i][j][4 * q + 3]};
                             *(v4bf*)(crow + ncol) = o;
@@ -342,7 +390,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 }
 
 constexpr int gemm_lds_bytes(int afmt, int bfmt) {
-    return 2 * (256 * (afmt == kFmtE2M1 ? 64 : 128) + 256 * (bfmt == kFmtE2M1 ? 64 : 128) + 2048) +
+    return NSTAGE * (256 * (afmt == kFmtE2M1 ? BK / 2 : BK) + 256 * (bfmt == kFmtE2M1 ? BK / 2 : BK)) + 4 * 256 * 16 +
            (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
 }
 
@@ -391,7 +439,7 @@ extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, in
                                    const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                                    int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
     if (!a_codes || !a_scales || !b_codes || !b_scales || !c_bf16) return MXL_EINVAL;
-    if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
+    if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if (num_groups > 1 && !group_lens) return MXL_EINVAL;
     if (total_m == 0) return MXL_OK;

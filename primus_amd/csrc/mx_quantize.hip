@@ -37,6 +37,7 @@ struct QuantArgs {
     uint8_t* s_row;
     uint8_t* q_colT;
     uint8_t* s_colT;
+    int64_t row_ld;     // columns of the row-wise copy (>= cols; the excess is zero-filled padding)
     int64_t W;          // padded width of the transposed copy (elements)
     int64_t mat_rows;   // TWOD: rows per matrix (n); otherwise unused
 };
@@ -88,7 +89,8 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     }
 
     const int64_t col = col0 + 8 * c16;
-    const bool col_ok = col < a.cols;
+    const bool col_ok = col < a.cols;      // source column exists
+    const bool out_ok = col < a.row_ld;    // row-wise output column exists (padding is written as zeros)
 
     // ---- load 8 rows x 8 columns per lane ----
     uint4 d[8];
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o.x = nonfinite4_e4m3(d[it].x, d[it].y);
                     o.y = nonfinite4_e4m3(d[it].z, d[it].w);
                 }
-                if (col_ok && r < rows_valid) *(uint2*)(a.q_row + (src_row0 + r) * a.cols + col) = o;
+                if (out_ok && r < rows_valid) *(uint2*)(a.q_row + (src_row0 + r) * a.row_ld + col) = o;
             } else {
                 uint32_t o;
                 if (byte != 255u) {
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o = nonfinite2_e2m1(d[it].x) | (nonfinite2_e2m1(d[it].y) << 8) | (nonfinite2_e2m1(d[it].z) << 16) |
                         (nonfinite2_e2m1(d[it].w) << 24);
                 }
-                if (col_ok && r < rows_valid) *(uint32_t*)(a.q_row + ((src_row0 + r) * a.cols + col) / 2) = o;
+                if (out_ok && r < rows_valid) *(uint32_t*)(a.q_row + ((src_row0 + r) * a.row_ld + col) / 2) = o;
             }
         }
     }
@@ -212,8 +214,8 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 
     // ---- scales: one dword (4 blocks) per row / per column of the tile ----
     if (ROW && t < QT && t < rows_valid) {
-        const int64_t sld = a.cols / 32;
-        const int64_t nb = (a.cols - col0) / 32;  // valid blocks in this tile row
+        const int64_t sld = a.row_ld / 32;
+        const int64_t nb = (a.row_ld - col0) / 32;  // valid blocks in this tile row
         uint8_t* dst = a.s_row + (src_row0 + t) * sld + col0 / 32;
         const uint32_t v = srow_tile[t];
         if (nb >= 4 && (sld & 3) == 0) {
@@ -343,9 +345,11 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
     return (total_rows + (int64_t)(MXL_SEG_ALIGN - 1) * num_groups) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
 }
 
-extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int fmt, int scale_mode,
+extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                             const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                             void* s_colT, void* stream) {
+    if (row_ld == 0) row_ld = cols;
+    if (row_ld < cols || row_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((!x_bf16 && rows > 0) || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
     if (!q_row && !q_colT) return MXL_EINVAL;
@@ -360,18 +364,23 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int 
     a.s_row = (uint8_t*)s_row;
     a.q_colT = (uint8_t*)q_colT;
     a.s_colT = (uint8_t*)s_colT;
+    a.row_ld = row_ld;
     a.W = mxl_padded_width(rows, num_groups);
     a.mat_rows = 0;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
-    const int64_t gy = (cols + QT - 1) / QT;
+    const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
     if (gx == 0) return MXL_OK;
     if (gx > 0x7FFFFFFF || gy > 65535) return MXL_EINVAL;
     return dispatch_quant<false>(fmt, scale_mode, a, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream);
 }
 
-extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int fmt,
-                                      int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
-                                      void* stream) {
+extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
+                                      int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
+                                      void* s_colT, void* stream) {
+    if (k_ld == 0) k_ld = k;
+    if (n_ld == 0) n_ld = n;
+    if (k_ld < k || n_ld < n || k_ld % MXL_BLOCK != 0 || n_ld % MXL_BLOCK != 0) return MXL_EINVAL;
+    if (n_ld > (n + QT - 1) / QT * QT) return MXL_EINVAL;  // padding of the transposed copy stays inside the last tile
     if (!w_bf16 || batch <= 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
     if (!q_row && !q_colT) return MXL_EINVAL;
@@ -385,10 +394,11 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
     a.s_row = (uint8_t*)s_row;
     a.q_colT = (uint8_t*)q_colT;
     a.s_colT = (uint8_t*)s_colT;
-    a.W = n;  // transposed copy of each matrix is [k, n]
+    a.row_ld = k_ld;
+    a.W = n_ld;  // transposed copy of each matrix is [k, n_ld]
     a.mat_rows = n;
     const int64_t gx = batch * ((n + QT - 1) / QT);
-    const int64_t gy = (k + QT - 1) / QT;
+    const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
     if (gx > 0x7FFFFFFF || gy > 65535) return MXL_EINVAL;
     return dispatch_quant<true>(fmt, scale_mode, a, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream);
 }

@@ -165,11 +165,10 @@ class QuantizedTensor(torch.Tensor):
         """Back to the original dtype in the payload's orientation.  For a
         transposed copy of ``rows`` tokens the padding columns are dropped."""
         out = K.dequantize_mx_impl(self._codes, self._scales, self.dtype)
-        if self._axis == -2 and not self._use_2d_block:
-            if self._segment_lens is not None:
-                raise NotImplementedError("dequantize of a segment-padded activation copy")
-            out = out[..., : self._total_rows]
-        return out
+        if self._axis == -2 and not self._use_2d_block and self._segment_lens is not None:
+            raise NotImplementedError("dequantize of a segment-padded activation copy")
+        # drop the padding of the contraction dim (GEMM granularity / token padding)
+        return out[..., : self.shape[-1]]
 
     def transpose(self, dim0: int, dim1: int):  # noqa: D102
         raise NotImplementedError(
@@ -209,7 +208,7 @@ def create_quantized_weight(
         raise ValueError("create_quantized_weight expects a bfloat16 weight")
     mode = quant_config.scale_mode
     q_row, s_row, q_col, s_col = K.quantize_mx_weight_2d_impl(
-        w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache
+        w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN
     )
     row = QuantizedTensor(q_row, s_row, logical_shape=w.shape, orig_dtype=w.dtype, axis=-1, use_2d_block=True,
                           scale_mode=mode)

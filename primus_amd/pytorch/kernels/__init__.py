@@ -51,6 +51,10 @@ def _hooked(name: str, **info):
     return _launch_hook(name, info) if _launch_hook is not None else _NO_HOOK
 
 
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None or t.numel() == 0 else t.data_ptr()
 
@@ -124,8 +128,13 @@ def quantize_mx_impl(
     rowwise: bool = True,
     colwise: bool = False,
     group_lens: Optional[torch.Tensor] = None,
+    pad_to: int = 1,
 ):
     """MX-quantise bf16 ``x[rows, cols]``.
+
+    ``pad_to`` rounds the column count of the row-wise copy up to a multiple
+    (zero codes, scale byte 0 in the padding) so that it can feed a GEMM,
+    whose contraction dim must be a multiple of 128.
 
     Returns ``(q_row, s_row, q_colT, s_colT)``; the pair that was not requested
     is ``None``.  ``q_row``: codes ``[rows, cols]`` (``cols/2`` bytes for FP4),
@@ -146,9 +155,10 @@ def quantize_mx_impl(
     per = _per_byte(fmt)
     dev = x.device
     q_row = s_row = q_col = s_col = None
+    row_ld = _round_up(cols, pad_to)
     if rowwise:
-        q_row = torch.empty((rows, cols // per), dtype=torch.uint8, device=dev)
-        s_row = torch.empty((rows, cols // BLOCK), dtype=torch.uint8, device=dev)
+        q_row = torch.empty((rows, row_ld // per), dtype=torch.uint8, device=dev)
+        s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
         q_col = torch.empty((cols, W // per), dtype=torch.uint8, device=dev)
@@ -158,7 +168,7 @@ def quantize_mx_impl(
         row_ok = rows > 0
         with _hooked("quantize", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
           rc = _lib.load().mxl_quantize(
-            _ptr(x) if row_ok else None, rows, cols, fmt, scale_mode, _ptr(group_lens), G,
+            _ptr(x) if row_ok else None, rows, cols, row_ld, fmt, scale_mode, _ptr(group_lens), G,
             _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col), _stream(),
           )
         _lib.check(rc, "mxl_quantize")
@@ -174,10 +184,12 @@ def quantize_mx_weight_2d_impl(
     *,
     rowwise: bool = True,
     colwise: bool = True,
+    pad_to: int = 1,
 ):
     """2-D (32x32 tile) MX quantisation of ``w[n, k]`` or ``w[G, n, k]``;
     returns ``(q_row [.., n, k], s_row [.., n, k/32], q_colT [.., k, n],
-    s_colT [.., k, n/32])`` with ``None`` for a copy that was not requested."""
+    s_colT [.., k, n/32])`` with ``None`` for a copy that was not requested.
+    ``pad_to`` rounds the last dim of both copies up (zero padding)."""
     if w.dtype != torch.bfloat16 or w.dim() not in (2, 3):
         raise ValueError("weight quantisation expects a 2-D or 3-D bfloat16 tensor")
     _require_cuda(w)
@@ -191,15 +203,16 @@ def quantize_mx_weight_2d_impl(
     per = _per_byte(fmt)
     dev = w.device
     q_row = s_row = q_col = s_col = None
+    k_ld, n_ld = _round_up(k, pad_to), _round_up(n, pad_to)
     if rowwise:
-        q_row = torch.empty(lead + (n, k // per), dtype=torch.uint8, device=dev)
-        s_row = torch.empty(lead + (n, k // BLOCK), dtype=torch.uint8, device=dev)
+        q_row = torch.empty(lead + (n, k_ld // per), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
-        q_col = torch.empty(lead + (k, n // per), dtype=torch.uint8, device=dev)
-        s_col = torch.empty(lead + (k, n // BLOCK), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(lead + (k, n_ld // per), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_2d(
-            _ptr(w), batch, n, k, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col), _stream()
+            _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col), _stream()
         )
     _lib.check(rc, "mxl_quantize_weight_2d")
     cd = _code_dtype(fmt)
@@ -225,6 +238,22 @@ def dequantize_mx_impl(codes: torch.Tensor, scales: torch.Tensor, out_dtype: tor
 # --------------------------------------------------------------------------
 # GEMMs on pre-quantised operands
 # --------------------------------------------------------------------------
+GEMM_K_ALIGN = _lib.GEMM_K_ALIGN
+
+
+def _pad_k(codes: torch.Tensor, scales: torch.Tensor, fmt: int):
+    """The GEMM kernels take K in multiples of 128.  Operands produced with
+    ``pad_to=128`` already are; anything else gets all-zero MX blocks (zero
+    codes, scale 2^0) appended to every row, at the cost of a copy."""
+    k = codes.shape[-1] * _per_byte(fmt)
+    if k % GEMM_K_ALIGN == 0:
+        return codes, scales, k
+    kp = _round_up(k, GEMM_K_ALIGN)
+    c = torch.nn.functional.pad(codes.view(torch.uint8), (0, (kp - k) // _per_byte(fmt)), value=0).view(codes.dtype)
+    s = torch.nn.functional.pad(scales.view(torch.uint8), (0, (kp - k) // BLOCK), value=127).view(scales.dtype)
+    return c, s, kp
+
+
 def _check_out_dtype(out_dtype) -> None:
     if out_dtype not in (None, torch.bfloat16):
         raise ValueError("the MX GEMMs produce bfloat16 output")
@@ -242,6 +271,8 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16) -> torch.T
     if tuple(a_scale.shape) != (m, k // BLOCK) or tuple(b_scale.shape) != (n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    a, a_scale, _ = _pad_k(a, a_scale, a_fmt)
+    b, b_scale, k = _pad_k(b, b_scale, b_fmt)
     with _hooked("gemm_nt", m=m, n=n, k=k):
         rc = _lib.load().mxl_gemm_nt(_ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), m, n, k, _stream())
     _lib.check(rc, "mxl_gemm_nt")
@@ -264,6 +295,8 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
     if tuple(a_scale.shape) != (total_m, k // BLOCK) or tuple(b_scale.shape) != (G, n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+    a, a_scale, _ = _pad_k(a, a_scale, a_fmt)
+    b, b_scale, k = _pad_k(b, b_scale, b_fmt)
     with _hooked("grouped_gemm_nt", m=total_m, n=n, k=k):
         rc = _lib.load().mxl_grouped_gemm_nt(
             _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()

@@ -47,8 +47,10 @@ class _MXLinearFunction(torch.autograd.Function):
         need_wgrad = b.requires_grad
         grouped = group_lens is not None
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
+        # (row-wise copies are padded to the GEMM's K granularity, like the reference pads its
+        # MXFP4 operands to 128: primus_turbo_mxfp4_local.py:119-124)
         a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
-            a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens
+            a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
         )
         if isinstance(b, QuantizedTensor):
             # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
@@ -64,7 +66,7 @@ class _MXLinearFunction(torch.autograd.Function):
                 w_col, w_cs = b_t.codes, b_t.scales
         else:
             w_row, w_rs, w_col, w_cs = K.quantize_mx_weight_2d_impl(
-                b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad
+                b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN
             )
         if grouped:
             y = K.grouped_gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, group_lens)
@@ -83,7 +85,7 @@ class _MXLinearFunction(torch.autograd.Function):
         if dy.dtype != torch.bfloat16:
             dy = dy.to(torch.bfloat16)
         d_row, d_rs, d_col, d_cs = K.quantize_mx_impl(
-            dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens
+            dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
         )
         grad_a = grad_b = None
         if need_dgrad:

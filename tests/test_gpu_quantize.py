@@ -118,6 +118,32 @@ def test_weight_2d_vs_oracle(gpu, fmt, fn, mode, mn, shape):
 
 
 @pytest.mark.parametrize("fmt,fn", FMTS)
+def test_padded_pitch_for_gemm(gpu, fmt, fn):
+    """Row-wise copies padded to the GEMM's K granularity: the real columns match
+    the oracle, the padding is zero codes with scale byte 0."""
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(70, 2880, generator=g).bfloat16()
+    q, s, qc, sc = [_np(t) for t in K.quantize_mx_impl(x.to(gpu), fmt, 0, rowwise=True, colwise=True, pad_to=128)]
+    per = 2 if fmt == o.FMT_E2M1 else 1
+    rq, rs = o.quantize_mx_rowwise(x, fmt)
+    assert q.shape == (70, 2944 // per) and s.shape == (70, 92)
+    assert np.array_equal(q[:, : 2880 // per], rq) and np.array_equal(s[:, :90], rs)
+    assert not q[:, 2880 // per :].any() and not s[:, 90:].any()
+    cq, cs = o.quantize_mx_colwise_segmented(x, [70], fmt)
+    assert np.array_equal(qc, cq) and np.array_equal(sc, cs)
+    w = (torch.randn(2, 96, 160, generator=g) * 0.02).bfloat16()
+    got = [_np(t) for t in K.quantize_mx_weight_2d_impl(w.to(gpu), fmt, 0, pad_to=128)]
+    want = o.quantize_mx_2d(w, fmt)
+    assert got[0].shape == (2, 96, 256 // per) and got[2].shape == (2, 160, 128 // per)
+    assert np.array_equal(got[0][..., : 160 // per], want[0]) and np.array_equal(got[1][..., :5], want[1])
+    assert np.array_equal(got[2][..., : 96 // per], want[2]) and np.array_equal(got[3][..., :3], want[3])
+    assert not got[0][..., 160 // per :].any() and not got[2][..., 96 // per :].any()
+    assert not got[1][..., 5:].any() and not got[3][..., 3:].any()
+
+
+@pytest.mark.parametrize("fmt,fn", FMTS)
 def test_special_values(gpu, fmt, fn):
     x = torch.zeros(8, 64).bfloat16()
     x[0, 3] = float("inf")
@@ -190,6 +216,7 @@ def test_error_codes_not_aborts(gpu):
     with pytest.raises(ValueError):
         K.quantize_mx_impl(torch.zeros(4, 64, dtype=torch.bfloat16), 0)  # CPU tensor
     L = _lib.load()
-    assert L.mxl_quantize(x.data_ptr(), 4, 48, 0, 0, None, 0, x.data_ptr(), x.data_ptr(), None, None, None) == -1
-    assert L.mxl_quantize(x.data_ptr(), 4, 64, 7, 0, None, 0, x.data_ptr(), x.data_ptr(), None, None, None) == -1
+    assert L.mxl_quantize(x.data_ptr(), 4, 48, 0, 0, 0, None, 0, x.data_ptr(), x.data_ptr(), None, None, None) == -1
+    assert L.mxl_quantize(x.data_ptr(), 4, 64, 0, 7, 0, None, 0, x.data_ptr(), x.data_ptr(), None, None, None) == -1
+    assert L.mxl_quantize(x.data_ptr(), 4, 64, 32, 0, 0, None, 0, x.data_ptr(), x.data_ptr(), None, None, None) == -1  # row_ld < cols
     assert L.mxl_gemm_nt(None, None, 0, None, None, 0, None, 1, 32, 32, None) == -1

@@ -24,12 +24,16 @@
 // MFMA source 0 so a lane ends up with 4 consecutive output columns (one
 // 8-byte bf16 store).
 #include <atomic>
+#include <type_traits>
 
 #include "mx_device.h"
 
 namespace mxl {
 
-constexpr int BM = 256, BN = 256, BK = 64, NSTAGE = 4;
+constexpr int BM = 256, BN = 256;
+constexpr int BK = 64;     // one MFMA K step (two MX blocks)
+constexpr int BKP = 128;   // K per LDS slot: two K steps, one full 128-byte line per FP8 row
+constexpr int NSLOT = 2;
 constexpr int GTHREADS = 256;
 constexpr int MODE_FWD = 0;    // rows of A ragged by group; B = [G, N, K]
 constexpr int MODE_WGRAD = 1;  // contraction ragged by group; C = [G, M, N]
@@ -51,13 +55,13 @@ struct GemmArgs {
 
 template <int FMT> struct Op {
     static constexpr bool fp4 = (FMT == kFmtE2M1);
-    static constexpr int kb = fp4 ? BK / 2 : BK;      // bytes per row per stage
-    static constexpr int cpr = kb / 16;               // 16-byte chunks per row (= loads per thread per stage)
+    static constexpr int kb = fp4 ? BKP / 2 : BKP;      // bytes per row per slot (128 or 64)
+    static constexpr int cpr = kb / 16;                 // 16-byte chunks per row (= loads per thread per slot)
     static constexpr int rows_per_ld = GTHREADS / cpr;  // tile rows covered by one load round
     static constexpr int tile_bytes = 256 * kb;
-    // XOR swizzle of the chunk index: 16 consecutive rows reading the same logical
-    // chunk hit 16 different 16-byte bank groups of the 256-byte LDS row.
-    static __device__ __forceinline__ int swz(int row) { return fp4 ? ((row >> 3) & 1) : ((row >> 2) & 3); }
+    // XOR swizzle of the chunk index (both measured conflict-free for 16-byte reads by
+    // 32 consecutive rows): 8 chunks per 128-byte row, 4 chunks per 64-byte row.
+    static __device__ __forceinline__ int swz(int row) { return fp4 ? ((row >> 2) & 3) : ((row >> 1) & 7); }
 };
 
 // ---- asynchronous global -> LDS loads ------------------------------------
@@ -92,18 +96,18 @@ __device__ __forceinline__ void dma2(v4i rsrc, uint32_t lds_off, uint32_t voff, 
 }
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-// LDS -> MFMA fragment of one 32-row tile (one K step = one stage).
+// LDS -> MFMA fragment of one 32-row tile for K step ks (0 or 1) of a slot.
 template <int FMT>
-__device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int g) {
+__device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int ks, int g) {
     v8i f;
     const int s = Op<FMT>::swz(row);
     if (FMT == kFmtE4M3) {
-        const uint4 lo = *(const uint4*)(lds + row * 64 + 16 * (g ^ s));
-        const uint4 hi = *(const uint4*)(lds + row * 64 + 16 * ((2 + g) ^ s));
+        const uint4 lo = *(const uint4*)(lds + row * 128 + 16 * ((4 * ks + g) ^ s));
+        const uint4 hi = *(const uint4*)(lds + row * 128 + 16 * ((4 * ks + 2 + g) ^ s));
         f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
         f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
     } else {
-        const uint4 v = *(const uint4*)(lds + row * 32 + 16 * (g ^ s));
+        const uint4 v = *(const uint4*)(lds + row * 64 + 16 * ((2 * ks + g) ^ s));
         f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
         f[4] = 0; f[5] = 0; f[6] = 0; f[7] = 0;
     }
@@ -118,15 +122,16 @@ struct Frags {
 template <int AFMT, int BFMT, int MODE>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     constexpr int A_BYTES = Op<AFMT>::tile_bytes, B_BYTES = Op<BFMT>::tile_bytes;
-    constexpr int STAGE = A_BYTES + B_BYTES;
-    constexpr int LPT = Op<AFMT>::cpr + Op<BFMT>::cpr;  // async data loads per thread per stage
+    constexpr int STAGE = A_BYTES + B_BYTES;            // one slot: K = 128 of both operands
+    constexpr int LPA = Op<AFMT>::cpr, LPB = Op<BFMT>::cpr;
+    constexpr int LPT = LPA + LPB;                      // async data loads per thread per slot
     // E8M0 scales travel in "panels": 16 bytes per row = the scales of 8 K stages
     // (K = 512), one 16-byte request per row per operand, double-buffered.
     constexpr int PANEL = 256 * 16;           // one operand
     constexpr int PANELS = 2 * 2 * PANEL;     // 2 buffers x 2 operands
     constexpr int CB = BFMT == kFmtE2M1 ? 4 : 0, BL = AFMT == kFmtE2M1 ? 4 : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint8_t* panels = smem + NSTAGE * STAGE;
+    uint8_t* panels = smem + NSLOT * STAGE;
     int* pre_tiles = (int*)(panels + PANELS);                        // [G+1] prefix of row tiles (FWD)
     int64_t* pre_rows = (int64_t*)(pre_tiles + MXL_MAX_GROUPS + 2);  // [G+1] prefix of rows / padded cols
 
@@ -241,7 +246,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         }
         const int64_t n0 = (int64_t)pid_n * BN;
         const int n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
-        const int kt_count = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BK));
+        const int np = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BKP));  // K slots of 128 ("pairs" of K steps)
 
         // Buffer descriptors anchored at the tile's first row: rows past the end
         // of the operand read as zero, rows of a neighbouring group are read but
@@ -262,106 +267,128 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-        // async loads of K stage kt into ring slot `slot`, in three parts so they can be
-        // slotted between MFMAs
-        auto issue_a = [&](int kt, int slot) {
-            const uint32_t base = smem_base + slot * STAGE;
-#pragma unroll
-            for (int i = 0; i < Op<AFMT>::cpr; ++i)
-                dma16(ra, base + (i * 4 + w) * 1024, a_voff,
-                      ka0 + kt * Op<AFMT>::kb + (uint32_t)(i * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
+        // One async load of K slot `kp` (K = 128) into ring slot `slot`: round i covers tile rows
+        // [i * rows_per_ld, (i+1) * rows_per_ld).  Rounds 0 .. LPA-1 are the M-side operand, the
+        // rest the N-side operand; a round past the end is a no-op.
+        auto issue_1 = [&](int kp, int slot, int r) __attribute__((always_inline)) {
+#ifdef EXP_NODMA
+            return;
+#endif
+            if (r < LPA) {
+                dma16(ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff,
+                      ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
+            } else if (r < LPT) {
+                const int i = r - LPA;
+                dma16(rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff,
+                      kb0 + kp * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb);
+            }
         };
-        auto issue_b = [&](int kt, int slot) {
-            const uint32_t base = smem_base + slot * STAGE;
-#pragma unroll
-            for (int i = 0; i < Op<BFMT>::cpr; ++i)
-                dma16(rb, base + A_BYTES + (i * 4 + w) * 1024, b_voff,
-                      kb0 + kt * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb);
-        };
-        // scale panel pn (K stages 8pn .. 8pn+7) into panel buffer pn & 1
-        auto issue_s = [&](int pn) {
-            const uint32_t base = smem_base + NSTAGE * STAGE + (pn & 1) * 2 * PANEL;
+        // scale panel pn (K slots 4pn .. 4pn+3) into panel buffer pn & 1
+        auto issue_s = [&](int pn) __attribute__((always_inline)) {
+            const uint32_t base = smem_base + NSLOT * STAGE + (pn & 1) * 2 * PANEL;
             dma16(rsa, base + w * 1024, s_voff, ks0 + 16 * pn);
             dma16(rsb, base + PANEL + w * 1024, s_voff, ks0 + 16 * pn);
         };
-        // fragments and scale bytes of K stage kt (ring slot `slot`)
-        auto read_frags = [&](Frags& f, int kt, int slot) {
-            const uint8_t* s = smem + slot * STAGE;
-            const uint8_t* pan = panels + ((kt >> 3) & 1) * 2 * PANEL + 2 * (kt & 7) + g;  // byte of (stage, block g)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) f.b[i] = read_frag<BFMT>(s + A_BYTES, wn * 128 + i * 32 + lr, g);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) f.a[i] = read_frag<AFMT>(s, wm * 128 + i * 32 + lr, g);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                f.sb[i] = pan[PANEL + 16 * (wn * 128 + i * 32 + lr)];
-                f.sa[i] = pan[16 * (wm * 128 + i * 32 + lr)];
-            }
-        };
 #define MXL_MFMA(F, I, J) \
     acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I])
+#define MXL_PIN __builtin_amdgcn_sched_barrier(0)
+        // read one fragment (+ its scale byte) of K step `st` (global K-step index) from slot `slot`
+#define MXL_RD_A(F, I) \
+    F.a[I] = read_frag<AFMT>(sn, wm * 128 + (I) * 32 + lr, ks_n, g); \
+    F.sa[I] = pan[16 * (wm * 128 + (I) * 32 + lr)]
+#define MXL_RD_B(F, J) \
+    F.b[J] = read_frag<BFMT>(sn + A_BYTES, wn * 128 + (J) * 32 + lr, ks_n, g); \
+    F.sb[J] = pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]
 
         Frags f0, f1;
         __syncthreads();  // every wave is done reading the ring for the previous tile
-        // Stages past the end of K are requested as well (their data is never used):
-        // it keeps every step of the pipeline identical and free of branches.
+        // K slots past the end are requested as well (their data is never used): it keeps every
+        // step of the pipeline identical and free of branches.
         issue_s(0);
-        issue_a(0, 0); issue_b(0, 0);
-        issue_a(1, 1); issue_b(1, 1);
-        issue_a(2, 2); issue_b(2, 2);
-        wait_vm<2 * LPT>();
-        __syncthreads();
-        read_frags(f0, 0, 0);
-        // One K stage: MFMAs of stage kt from registers `cur`; meanwhile stage kt+3
-        // is requested from memory and the fragments of stage kt+1 are read from LDS.
-        auto stage_body = [&](int kt, int sub, Frags& cur, Frags& nxt) {
-            const int slot = sub & 3;
-            MXL_MFMA(cur, 0, 0);
-#ifndef EXP_NOSCALE
-            if (sub == 0) issue_s((kt >> 3) + 1);  // next panel; its buffer was last read two stages ago
-#endif
-#ifndef EXP_NODMA
-            issue_a(kt + 3, (slot + 3) & 3);
-#endif
-            __builtin_amdgcn_sched_barrier(0);
-            MXL_MFMA(cur, 1, 0);
-#ifndef EXP_NODMA
-            issue_b(kt + 3, (slot + 3) & 3);
-#endif
-            __builtin_amdgcn_sched_barrier(0);
-            MXL_MFMA(cur, 2, 0);
-            MXL_MFMA(cur, 3, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            wait_vm<2 * LPT>();  // stage kt+1 has landed (kt+2, kt+3 may still be in flight)
-#ifndef EXP_NOBAR
-            __syncthreads();     // ... for every wave, and every wave is done reading slot of stage kt-1
-#endif
-#ifndef EXP_NOLDS
-            read_frags(nxt, kt + 1, (slot + 1) & 3);
-#endif
-            MXL_MFMA(cur, 0, 1); MXL_MFMA(cur, 1, 1); MXL_MFMA(cur, 2, 1); MXL_MFMA(cur, 3, 1);
-            MXL_MFMA(cur, 0, 2); MXL_MFMA(cur, 1, 2); MXL_MFMA(cur, 2, 2); MXL_MFMA(cur, 3, 2);
-            MXL_MFMA(cur, 0, 3); MXL_MFMA(cur, 1, 3); MXL_MFMA(cur, 2, 3); MXL_MFMA(cur, 3, 3);
-            // interleave: one MFMA, then two LDS reads, twelve times
 #pragma unroll
-            for (int r = 0; r < 12; ++r) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        };
-        for (int kt = 0; kt < kt_count; kt += 8) {
-            stage_body(kt, 0, f0, f1);
-            if (kt + 1 < kt_count) stage_body(kt + 1, 1, f1, f0);
-            if (kt + 2 < kt_count) stage_body(kt + 2, 2, f0, f1);
-            if (kt + 3 < kt_count) stage_body(kt + 3, 3, f1, f0);
-            if (kt + 4 < kt_count) stage_body(kt + 4, 4, f0, f1);
-            if (kt + 5 < kt_count) stage_body(kt + 5, 5, f1, f0);
-            if (kt + 6 < kt_count) stage_body(kt + 6, 6, f0, f1);
-            if (kt + 7 < kt_count) stage_body(kt + 7, 7, f1, f0);
+        for (int r = 0; r < LPT; ++r) issue_1(0, 0, r);
+#pragma unroll
+        for (int r = 0; r < LPT - 4; ++r) issue_1(1, 1, r);  // the last four go out with the first MFMAs
+        wait_vm<(LPT > 4 ? LPT - 4 : 0)>();
+        __syncthreads();
+        {
+            const uint8_t* sn = smem;
+            const uint8_t* pan = panels + g;
+            constexpr int ks_n = 0;
+            MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
+            MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
         }
-        wait_vm<0>();  // drain the look-ahead requests before the ring is reused
+        // One K step (16 MFMAs) of K slot kp.  KS = 0: first half of the slot; its data landed a
+        // step ago; the last 4 loads of slot kp+1 go out.  KS = 1: second half; after its barrier
+        // the slot of kp-1... (= slot of kp+1) has landed and this slot's first half is dead, and
+        // the first LPT-4 loads of slot kp+2 go out, one per MFMA.
+        // The body is written in its final instruction order and pinned with scheduling barriers:
+        // memory requests are spread (a burst fills the texture-addresser queue and stalls the
+        // issuing wave, MFMAs included) and each LDS fragment read sits next to an MFMA.
+        auto kstep = [&](auto ks_tag, auto sub_tag, int kp, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
+            constexpr int KS = decltype(ks_tag)::value;
+            constexpr int SUB = decltype(sub_tag)::value;      // kp & 3, known at compile time
+            constexpr int slot = SUB & 1;
+            constexpr int ks_n = 1 - KS;                       // K step (within its slot) of the fragments read here
+            const int st_n = 2 * kp + KS + 1;                  // its global K-step index
+            const uint8_t* sn = smem + (KS == 0 ? slot : (slot ^ 1)) * STAGE;
+            const uint8_t* pan = panels + ((st_n >> 3) & 1) * 2 * PANEL + 2 * (st_n & 7) + g;
+            MXL_MFMA(cur, 0, 0);
+            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 4);
+            MXL_PIN;
+            MXL_MFMA(cur, 1, 0);
+            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 3);
+            MXL_PIN;
+            MXL_MFMA(cur, 2, 0);
+            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 2);
+            MXL_PIN;
+            MXL_MFMA(cur, 3, 0);
+            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 1);
+            MXL_PIN;
+            if (KS == 1) wait_vm<0>();  // K slot kp+1 has landed (every request was issued at least a K step ago)
+#ifndef EXP_NOBAR
+            __syncthreads();
+#endif
+            MXL_PIN;
+            if (KS == 1 && SUB == 0) issue_s((kp >> 2) + 1);  // next scale panel; its buffer is dead since slot kp-1
+            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1); if (KS == 1) issue_1(kp + 2, slot, 0); MXL_PIN;
+            MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1); if (KS == 1) issue_1(kp + 2, slot, 1); MXL_PIN;
+            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1); if (KS == 1) issue_1(kp + 2, slot, 2); MXL_PIN;
+            MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1); if (KS == 1) issue_1(kp + 2, slot, 3); MXL_PIN;
+            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2); if (KS == 1) issue_1(kp + 2, slot, 4); MXL_PIN;
+            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2); if (KS == 1) issue_1(kp + 2, slot, 5); MXL_PIN;
+            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2); if (KS == 1) issue_1(kp + 2, slot, 6); MXL_PIN;
+            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2); if (KS == 1) issue_1(kp + 2, slot, 7); MXL_PIN;
+            MXL_MFMA(cur, 0, 3); if (KS == 1) issue_1(kp + 2, slot, 8); MXL_PIN;
+            MXL_MFMA(cur, 1, 3); if (KS == 1) issue_1(kp + 2, slot, 9); MXL_PIN;
+            MXL_MFMA(cur, 2, 3); if (KS == 1) issue_1(kp + 2, slot, 10); MXL_PIN;
+            MXL_MFMA(cur, 3, 3); if (KS == 1) issue_1(kp + 2, slot, 11); MXL_PIN;
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        for (int kp = 0; kp < np; kp += 4) {
+            kstep(I0{}, I0{}, kp, f0, f1);
+            kstep(I1{}, I0{}, kp, f1, f0);
+            if (kp + 1 < np) {
+                kstep(I0{}, I1{}, kp + 1, f0, f1);
+                kstep(I1{}, I1{}, kp + 1, f1, f0);
+            }
+            if (kp + 2 < np) {
+                kstep(I0{}, I2{}, kp + 2, f0, f1);
+                kstep(I1{}, I2{}, kp + 2, f1, f0);
+            }
+            if (kp + 3 < np) {
+                kstep(I0{}, I3{}, kp + 3, f0, f1);
+                kstep(I1{}, I3{}, kp + 3, f1, f0);
+            }
+        }
 #undef MXL_MFMA
+#undef MXL_PIN
+#undef MXL_RD_A
+#undef MXL_RD_B
+        wait_vm<0>();  // drain the look-ahead requests before the ring is reused
 
         // ---- epilogue: fp32 -> bf16, 4 consecutive columns per lane ----
 #pragma unroll
@@ -390,7 +417,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 }
 
 constexpr int gemm_lds_bytes(int afmt, int bfmt) {
-    return NSTAGE * (256 * (afmt == kFmtE2M1 ? BK / 2 : BK) + 256 * (bfmt == kFmtE2M1 ? BK / 2 : BK)) + 4 * 256 * 16 +
+    return NSLOT * (256 * (afmt == kFmtE2M1 ? BKP / 2 : BKP) + 256 * (bfmt == kFmtE2M1 ? BKP / 2 : BKP)) + 4 * 256 * 16 +
            (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
 }
 

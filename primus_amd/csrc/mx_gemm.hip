@@ -114,6 +114,26 @@ __device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int ks, in
     return f;
 }
 
+// Which async load (0 .. 15, -1 = none) goes out in MFMA position q of the 32 positions between
+// the moment a ring slot becomes free (barrier of the second K step of slot kp) and the barrier
+// that needs its new contents (second K step of slot kp+1).  Requests are spread: four waves
+// issuing one 1 KiB request each per MFMA keeps the texture addresser saturated and its queue
+// full, which stalls the issuing waves, MFMAs included.
+#ifndef EXP_SCHED
+#define EXP_SCHED 1
+#endif
+__host__ __device__ constexpr int load_at(int q) {
+#if EXP_SCHED == 0
+    return q < 16 ? q : -1;                                   // back to back
+#elif EXP_SCHED == 1
+    return (q < 24 && q % 3 != 2) ? q - q / 3 : -1;           // two out of three positions, done by q = 22
+#elif EXP_SCHED == 2
+    return (q % 2 == 0) ? q / 2 : -1;                         // every other position, done by q = 30
+#elif EXP_SCHED == 3
+    return (q < 20 && q % 5 != 4) ? q - q / 5 : -1;           // four out of five, done by q = 18
+#endif
+}
+
 struct Frags {
     v8i a[4], b[4];
     int sa[4], sb[4];
@@ -136,6 +156,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     int64_t* pre_rows = (int64_t*)(pre_tiles + MXL_MAX_GROUPS + 2);  // [G+1] prefix of rows / padded cols
 
     const int t = threadIdx.x;
+#ifdef EXP_CLK
+    const uint64_t clk0 = clock64(), wall0 = wall_clock64();
+#endif
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l = t & 63, lr = l & 31, g = l >> 5;
     const int wm = w >> 1, wn = w & 1;
@@ -201,8 +224,16 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #define b_voff b_voff_x
 #endif
 
-    for (int tile = vwg; tile < total_tiles; tile += nwg) {
-        // ---- decode tile -> (group, pid_m, pid_n) ----
+    // Everything a tile needs, decoded from its index on the device.
+    struct Tile {
+        v4i ra, rb, rsa, rsb;      // buffer descriptors anchored at the tile's first rows
+        uint32_t ka0, kb0, ks0;    // byte / block offsets of the contraction range
+        int np;                    // K slots of 128
+        int m_valid, n_valid;
+        int64_t c_off;             // element offset of the tile's first output
+    };
+    auto decode = [&](int tile) __attribute__((always_inline)) {
+        Tile d;
         int grp = 0, pid_m, pid_n;
         int tl = tile;
         if (MODE == MODE_WGRAD) {
@@ -217,9 +248,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             pid_m = first + (tl % width) % gsz;
             pid_n = (tl % width) / gsz;
         }
-        int64_t a_row0, b_row0, c_row0;
-        int m_valid;
-        int64_t k0, k1;  // contraction range in elements
+        int64_t a_row0, b_row0, c_row0, k0, k1;
         if (MODE == MODE_FWD) {
             // binary search: largest grp with pre_tiles[grp] <= pid_m
             int lo = 0, hi = G;
@@ -231,34 +260,79 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             const int64_t g_row0 = pre_rows[grp], g_rows = pre_rows[grp + 1] - g_row0;
             const int64_t r = (int64_t)(pid_m - pre_tiles[grp]) * BM;
             a_row0 = g_row0 + r;
-            m_valid = (g_rows - r) < BM ? (int)(g_rows - r) : BM;
+            d.m_valid = (g_rows - r) < BM ? (int)(g_rows - r) : BM;
             b_row0 = (int64_t)grp * p.n + (int64_t)pid_n * BN;
             c_row0 = a_row0;
             k0 = 0;
             k1 = p.k;
         } else {
             a_row0 = (int64_t)pid_m * BM;
-            m_valid = (p.m - a_row0) < BM ? (int)(p.m - a_row0) : BM;
+            d.m_valid = (p.m - a_row0) < BM ? (int)(p.m - a_row0) : BM;
             b_row0 = (int64_t)pid_n * BN;
             c_row0 = (int64_t)grp * p.m + a_row0;
             k0 = pre_rows[grp];
             k1 = pre_rows[grp + 1];
         }
         const int64_t n0 = (int64_t)pid_n * BN;
-        const int n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
-        const int np = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BKP));  // K slots of 128 ("pairs" of K steps)
+        d.n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
+        d.c_off = c_row0 * p.n + n0;
+        d.np = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BKP));
+        // Rows past the end of the operand read as zero; rows of a neighbouring group are read
+        // but never stored.
+        d.ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
+        d.rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
+        d.rsa = make_rsrc(p.sa + a_row0 * ld_s, (a_rows_total - a_row0) * ld_s);
+        d.rsb = make_rsrc(p.sb + b_row0 * ld_s, (b_rows_total - b_row0) * ld_s);
+        d.ka0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<AFMT>::fp4 ? k0 / 2 : k0));
+        d.kb0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<BFMT>::fp4 ? k0 / 2 : k0));
+        d.ks0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(k0 / 32));
+        return d;
+    };
+    // One async load of K slot `kp` (K = 128) of tile d into ring slot `slot`: round r covers
+    // tile rows [r * rows_per_ld, (r+1) * rows_per_ld) of the M-side operand for r < LPA, of
+    // the N-side operand for LPA <= r < LPT; a round past the end is a no-op.
+    auto issue_1 = [&](const Tile& d, int kp, int slot, int r) __attribute__((always_inline)) {
+#ifdef EXP_NODMA
+        return;
+#endif
+        if (r < LPA) {
+            dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff,
+                  d.ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
+        } else if (r < LPT) {
+            const int i = r - LPA;
+            dma16(d.rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff,
+                  d.kb0 + kp * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb);
+        }
+    };
+    // scale panel pn (K slots 4pn .. 4pn+3) into panel buffer pn & 1
+    auto issue_s = [&](const Tile& d, int pn) __attribute__((always_inline)) {
+        const uint32_t base = smem_base + NSLOT * STAGE + (pn & 1) * 2 * PANEL;
+        dma16(d.rsa, base + w * 1024, s_voff, d.ks0 + 16 * pn);
+        dma16(d.rsb, base + PANEL + w * 1024, s_voff, d.ks0 + 16 * pn);
+    };
+    // first requests of a tile: scale panel 0 and all of K slot 0
+    auto issue_head = [&](const Tile& d) __attribute__((always_inline)) {
+        issue_s(d, 0);
+#pragma unroll
+        for (int r = 0; r < LPT; ++r) issue_1(d, 0, 0, r);
+    };
 
-        // Buffer descriptors anchored at the tile's first row: rows past the end
-        // of the operand read as zero, rows of a neighbouring group are read but
-        // never stored.
-        const v4i ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
-        const v4i rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
-        const v4i rsa = make_rsrc(p.sa + a_row0 * ld_s, (a_rows_total - a_row0) * ld_s);
-        const v4i rsb = make_rsrc(p.sb + b_row0 * ld_s, (b_rows_total - b_row0) * ld_s);
-        const uint32_t ka0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<AFMT>::fp4 ? k0 / 2 : k0));
-        const uint32_t kb0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<BFMT>::fp4 ? k0 / 2 : k0));
-        const uint32_t ks0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(k0 / 32));
+#define MXL_MFMA(F, I, J) \
+    acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I])
+#define MXL_PIN __builtin_amdgcn_sched_barrier(0)
+    // read one fragment (+ its scale byte) of the K step described by (sn, pan, ks_n)
+#define MXL_RD_A(F, I) \
+    F.a[I] = read_frag<AFMT>(sn, wm * 128 + (I) * 32 + lr, ks_n, g); \
+    F.sa[I] = pan[16 * (wm * 128 + (I) * 32 + lr)]
+#define MXL_RD_B(F, J) \
+    F.b[J] = read_frag<BFMT>(sn + A_BYTES, wn * 128 + (J) * 32 + lr, ks_n, g); \
+    F.sb[J] = pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]
 
+    int tile = vwg;
+    if (tile >= total_tiles) return;
+    Tile d = decode(tile);
+    issue_head(d);
+    while (tile < total_tiles) {
         v16f acc[4][4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -267,50 +341,16 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-        // One async load of K slot `kp` (K = 128) into ring slot `slot`: round i covers tile rows
-        // [i * rows_per_ld, (i+1) * rows_per_ld).  Rounds 0 .. LPA-1 are the M-side operand, the
-        // rest the N-side operand; a round past the end is a no-op.
-        auto issue_1 = [&](int kp, int slot, int r) __attribute__((always_inline)) {
-#ifdef EXP_NODMA
-            return;
-#endif
-            if (r < LPA) {
-                dma16(ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff,
-                      ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
-            } else if (r < LPT) {
-                const int i = r - LPA;
-                dma16(rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff,
-                      kb0 + kp * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb);
-            }
-        };
-        // scale panel pn (K slots 4pn .. 4pn+3) into panel buffer pn & 1
-        auto issue_s = [&](int pn) __attribute__((always_inline)) {
-            const uint32_t base = smem_base + NSLOT * STAGE + (pn & 1) * 2 * PANEL;
-            dma16(rsa, base + w * 1024, s_voff, ks0 + 16 * pn);
-            dma16(rsb, base + PANEL + w * 1024, s_voff, ks0 + 16 * pn);
-        };
-#define MXL_MFMA(F, I, J) \
-    acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I])
-#define MXL_PIN __builtin_amdgcn_sched_barrier(0)
-        // read one fragment (+ its scale byte) of K step `st` (global K-step index) from slot `slot`
-#define MXL_RD_A(F, I) \
-    F.a[I] = read_frag<AFMT>(sn, wm * 128 + (I) * 32 + lr, ks_n, g); \
-    F.sa[I] = pan[16 * (wm * 128 + (I) * 32 + lr)]
-#define MXL_RD_B(F, J) \
-    F.b[J] = read_frag<BFMT>(sn + A_BYTES, wn * 128 + (J) * 32 + lr, ks_n, g); \
-    F.sb[J] = pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]
-
         Frags f0, f1;
-        __syncthreads();  // every wave is done reading the ring for the previous tile
-        // K slots past the end are requested as well (their data is never used): it keeps every
-        // step of the pipeline identical and free of branches.
-        issue_s(0);
-#pragma unroll
-        for (int r = 0; r < LPT; ++r) issue_1(0, 0, r);
-#pragma unroll
-        for (int r = 0; r < LPT - 4; ++r) issue_1(1, 1, r);  // the last four go out with the first MFMAs
-        wait_vm<(LPT > 4 ? LPT - 4 : 0)>();
+        // K slot 0 and scale panel 0 of this tile were requested before the previous tile's
+        // epilogue.  K slots past the end are requested as well (their data is never used):
+        // it keeps every step of the pipeline identical and free of branches.
+        wait_vm<0>();
         __syncthreads();
+        // K slot 1: the part of its request window that lies before the first K step
+#pragma unroll
+        for (int q = 0; q < 12; ++q)
+            if (load_at(q) >= 0) issue_1(d, 1, 1, load_at(q));
         {
             const uint8_t* sn = smem;
             const uint8_t* pan = panels + g;
@@ -318,13 +358,11 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
             MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
         }
-        // One K step (16 MFMAs) of K slot kp.  KS = 0: first half of the slot; its data landed a
-        // step ago; the last 4 loads of slot kp+1 go out.  KS = 1: second half; after its barrier
-        // the slot of kp-1... (= slot of kp+1) has landed and this slot's first half is dead, and
-        // the first LPT-4 loads of slot kp+2 go out, one per MFMA.
-        // The body is written in its final instruction order and pinned with scheduling barriers:
-        // memory requests are spread (a burst fills the texture-addresser queue and stalls the
-        // issuing wave, MFMAs included) and each LDS fragment read sits next to an MFMA.
+        // One K step (16 MFMAs) of K slot kp.  KS = 0: first half of the slot.  KS = 1: second
+        // half; after its barrier K slot kp+1 has landed in the other ring slot and this ring
+        // slot is dead, so the requests for K slot kp+2 start to go out.
+        // The body is written in its final instruction order and pinned with scheduling
+        // barriers; each LDS fragment read sits next to an MFMA that hides it.
         auto kstep = [&](auto ks_tag, auto sub_tag, int kp, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
             constexpr int KS = decltype(ks_tag)::value;
             constexpr int SUB = decltype(sub_tag)::value;      // kp & 3, known at compile time
@@ -333,41 +371,48 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             const int st_n = 2 * kp + KS + 1;                  // its global K-step index
             const uint8_t* sn = smem + (KS == 0 ? slot : (slot ^ 1)) * STAGE;
             const uint8_t* pan = panels + ((st_n >> 3) & 1) * 2 * PANEL + 2 * (st_n & 7) + g;
-            MXL_MFMA(cur, 0, 0);
-            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 4);
-            MXL_PIN;
-            MXL_MFMA(cur, 1, 0);
-            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 3);
-            MXL_PIN;
-            MXL_MFMA(cur, 2, 0);
-            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 2);
-            MXL_PIN;
-            MXL_MFMA(cur, 3, 0);
-            if (KS == 0) issue_1(kp + 1, slot ^ 1, LPT - 1);
-            MXL_PIN;
-            if (KS == 1) wait_vm<0>();  // K slot kp+1 has landed (every request was issued at least a K step ago)
+            // position m of this K step in the 32-position window of the slot being refilled:
+            //   KS = 1, m >= 4 : q = m - 4   (K slot kp+2 -> this ring slot, free after the barrier below)
+            //   KS = 0         : q = 12 + m  (K slot kp+1 -> the other ring slot)
+            //   KS = 1, m <  4 : q = 28 + m  (K slot kp+1 -> the other ring slot)
+#define MXL_LD(M) \
+    do { \
+        constexpr int q_ = (KS == 1) ? ((M) >= 4 ? (M) - 4 : 28 + (M)) : 12 + (M); \
+        constexpr int r_ = load_at(q_); \
+        if (r_ >= 0) { \
+            if (KS == 1 && (M) >= 4) issue_1(d, kp + 2, slot, r_); \
+            else issue_1(d, kp + 1, slot ^ 1, r_); \
+        } \
+    } while (0)
+            MXL_MFMA(cur, 0, 0); MXL_LD(0); MXL_PIN;
+            MXL_MFMA(cur, 1, 0); MXL_LD(1); MXL_PIN;
+            MXL_MFMA(cur, 2, 0); MXL_LD(2); MXL_PIN;
+            MXL_MFMA(cur, 3, 0); MXL_LD(3); MXL_PIN;
+            if (KS == 1) wait_vm<0>();  // K slot kp+1 has landed (its last request went out several MFMAs ago)
 #ifndef EXP_NOBAR
             __syncthreads();
 #endif
             MXL_PIN;
-            if (KS == 1 && SUB == 0) issue_s((kp >> 2) + 1);  // next scale panel; its buffer is dead since slot kp-1
-            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1); if (KS == 1) issue_1(kp + 2, slot, 0); MXL_PIN;
-            MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1); if (KS == 1) issue_1(kp + 2, slot, 1); MXL_PIN;
-            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1); if (KS == 1) issue_1(kp + 2, slot, 2); MXL_PIN;
-            MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1); if (KS == 1) issue_1(kp + 2, slot, 3); MXL_PIN;
-            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2); if (KS == 1) issue_1(kp + 2, slot, 4); MXL_PIN;
-            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2); if (KS == 1) issue_1(kp + 2, slot, 5); MXL_PIN;
-            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2); if (KS == 1) issue_1(kp + 2, slot, 6); MXL_PIN;
-            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2); if (KS == 1) issue_1(kp + 2, slot, 7); MXL_PIN;
-            MXL_MFMA(cur, 0, 3); if (KS == 1) issue_1(kp + 2, slot, 8); MXL_PIN;
-            MXL_MFMA(cur, 1, 3); if (KS == 1) issue_1(kp + 2, slot, 9); MXL_PIN;
-            MXL_MFMA(cur, 2, 3); if (KS == 1) issue_1(kp + 2, slot, 10); MXL_PIN;
-            MXL_MFMA(cur, 3, 3); if (KS == 1) issue_1(kp + 2, slot, 11); MXL_PIN;
+            if (KS == 1 && SUB == 0) issue_s(d, (kp >> 2) + 1);  // next scale panel; its buffer is dead since K slot kp-1
+            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1); MXL_LD(4); MXL_PIN;
+            MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1); MXL_LD(5); MXL_PIN;
+            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1); MXL_LD(6); MXL_PIN;
+            MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1); MXL_LD(7); MXL_PIN;
+            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2); MXL_LD(8); MXL_PIN;
+            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2); MXL_LD(9); MXL_PIN;
+            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2); MXL_LD(10); MXL_PIN;
+            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2); MXL_LD(11); MXL_PIN;
+            MXL_MFMA(cur, 0, 3); MXL_LD(12); MXL_PIN;
+            MXL_MFMA(cur, 1, 3); MXL_LD(13); MXL_PIN;
+            MXL_MFMA(cur, 2, 3); MXL_LD(14); MXL_PIN;
+            MXL_MFMA(cur, 3, 3); MXL_LD(15); MXL_PIN;
+#undef MXL_LD
         };
         using I0 = std::integral_constant<int, 0>;
         using I1 = std::integral_constant<int, 1>;
         using I2 = std::integral_constant<int, 2>;
         using I3 = std::integral_constant<int, 3>;
+        const int np = d.np;
         for (int kp = 0; kp < np; kp += 4) {
             kstep(I0{}, I0{}, kp, f0, f1);
             kstep(I1{}, I0{}, kp, f1, f0);
@@ -384,36 +429,78 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
                 kstep(I1{}, I3{}, kp + 3, f1, f0);
             }
         }
-#undef MXL_MFMA
-#undef MXL_PIN
-#undef MXL_RD_A
-#undef MXL_RD_B
-        wait_vm<0>();  // drain the look-ahead requests before the ring is reused
+        // Drain the look-ahead requests (they target the ring) and make sure every wave is done
+        // reading it; then the next tile's first requests go out and overlap with the epilogue.
+        wait_vm<0>();
+        __syncthreads();
+        const int m_valid = d.m_valid, n_valid = d.n_valid;
+        uint16_t* ctile = p.c + d.c_off;
+        tile += nwg;
+        // (past the last tile the requests are still sent, for the last tile again: nobody reads them)
+        d = decode(tile < total_tiles ? tile : total_tiles - 1);
+        issue_head(d);
+        MXL_PIN;  // keep the accumulator read-out below: it would otherwise be hoisted and spill
 
-        // ---- epilogue: fp32 -> bf16, 4 consecutive columns per lane ----
+        // ---- epilogue: fp32 -> bf16 through a wave-private LDS patch (in ring slot 1, which the
+        // requests above do not touch), so that the global stores are 16 bytes per lane and each
+        // store instruction covers 4 rows x 256 contiguous bytes ----
+#ifdef EXP_NOSTORE
+        if (acc[0][0][0] == 1234.5f)
+#endif
+        {
+            constexpr int SP = 272;  // bytes per staged row (256 + 16: spreads the rows over the banks)
+            uint8_t* stg = smem + STAGE + w * (32 * SP);
+            uint8_t* wr = stg + lr * SP + 8 * g;                   // this lane's row while writing
+            const uint8_t* rd = stg + (l >> 4) * SP + (l & 15) * 16;  // this lane's 16 bytes while reading
+            const int rr = l >> 4, cc = wn * 128 + (l & 15) * 8;
+            const uint32_t lane_off = (uint32_t)((rr * (int)p.n + (l & 15) * 8) * 2);
+            const bool full = (m_valid == BM) && (n_valid == BN);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int mrow = wm * 128 + i * 32 + lr;
-            if (mrow < m_valid) {
-                uint16_t* crow = p.c + (c_row0 + mrow) * p.n + n0;
+            for (int i = 0; i < 4; ++i) {
+                // lane (lr, g) holds row lr of this 32-row block: columns j*32 + 8q + 4g .. +3
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const int ncol = wn * 128 + j * 32 + 8 * q + 4 * g;
-#ifdef EXP_NOSTORE
-                        if (ncol < n_valid && acc[i][j][4*q] == 1234.5f) {
-#else
-                        if (ncol < n_valid) {
-#endif
-                            v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1],
-                                      (__bf16)acc[i][j][4 * q + 2], (__bf16)acc[i][j][4 * q + 3]};
-                            *(v4bf*)(crow + ncol) = o;
-                        }
+                        v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
+                                  (__bf16)acc[i][j][4 * q + 3]};
+                        *(v4bf*)(wr + (j * 32 + 8 * q) * 2) = o;
                     }
+                // 16 lanes per row, 4 rows per store instruction; the row base is uniform
+                uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32) * p.n + wn * 128);
+                if (full) {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const uint4 v = *(const uint4*)(rd + 4 * u * SP);
+#ifdef EXP_NOGSTORE
+                        if (v.x == 0x12345678u)
+#endif
+                        *(uint4*)(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off) = v;
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const uint4 v = *(const uint4*)(rd + 4 * u * SP);
+                        if (wm * 128 + i * 32 + 4 * u + rr < m_valid && cc < n_valid)
+                            *(uint4*)(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off) = v;
+                    }
+                }
+                MXL_PIN;  // one 32-row block at a time: 64 accumulators live, not 256
             }
         }
     }
+#undef MXL_MFMA
+#undef MXL_PIN
+#undef MXL_RD_A
+#undef MXL_RD_B
+#ifdef EXP_CLK
+    if (t == 0 && blockIdx.x < 64) {
+        const uint64_t clk1 = clock64(), wall1 = wall_clock64();
+        uint64_t* dbg = (uint64_t*)p.c;
+        dbg[2 * blockIdx.x] = clk1 - clk0;
+        dbg[2 * blockIdx.x + 1] = wall1 - wall0;
+    }
+#endif
 }
 
 constexpr int gemm_lds_bytes(int afmt, int bfmt) {

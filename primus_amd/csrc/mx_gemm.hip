@@ -119,19 +119,8 @@ __device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int ks, in
 // that needs its new contents (second K step of slot kp+1).  Requests are spread: four waves
 // issuing one 1 KiB request each per MFMA keeps the texture addresser saturated and its queue
 // full, which stalls the issuing waves, MFMAs included.
-#ifndef EXP_SCHED
-#define EXP_SCHED 1
-#endif
 __host__ __device__ constexpr int load_at(int q) {
-#if EXP_SCHED == 0
-    return q < 16 ? q : -1;                                   // back to back
-#elif EXP_SCHED == 1
     return (q < 24 && q % 3 != 2) ? q - q / 3 : -1;           // two out of three positions, done by q = 22
-#elif EXP_SCHED == 2
-    return (q % 2 == 0) ? q / 2 : -1;                         // every other position, done by q = 30
-#elif EXP_SCHED == 3
-    return (q < 20 && q % 5 != 4) ? q - q / 5 : -1;           // four out of five, done by q = 18
-#endif
 }
 
 struct Frags {
@@ -156,9 +145,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     int64_t* pre_rows = (int64_t*)(pre_tiles + MXL_MAX_GROUPS + 2);  // [G+1] prefix of rows / padded cols
 
     const int t = threadIdx.x;
-#ifdef EXP_CLK
-    const uint64_t clk0 = clock64(), wall0 = wall_clock64();
-#endif
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l = t & 63, lr = l & 31, g = l >> 5;
     const int wm = w >> 1, wn = w & 1;
@@ -199,11 +185,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // each XCD a contiguous run of the tile order.
     const int nwg = gridDim.x;
     const int per_xcd = nwg >> 3;
-#ifdef EXP_NOREMAP
-    const int vwg = (int)blockIdx.x; (void)per_xcd;
-#else
     const int vwg = (nwg & 7) ? (int)blockIdx.x : ((int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3));
-#endif
 
     const int64_t lda = Op<AFMT>::fp4 ? p.k / 2 : p.k;
     const int64_t ldb = Op<BFMT>::fp4 ? p.k / 2 : p.k;
@@ -216,13 +198,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     const uint32_t a_voff = (uint32_t)(a_row * (int)lda + 16 * ((t % Op<AFMT>::cpr) ^ Op<AFMT>::swz(a_row)));
     const uint32_t b_voff = (uint32_t)(b_row * (int)ldb + 16 * ((t % Op<BFMT>::cpr) ^ Op<BFMT>::swz(b_row)));
     const uint32_t s_voff = (uint32_t)(t * (int)ld_s);
-#ifdef EXP_FULLLINE
-    // timing experiment only (wrong data): 8 lanes read 128 contiguous bytes of a row
-    const uint32_t a_voff_x = (uint32_t)((t / 8) * (int)lda + 16 * (t % 8));
-    const uint32_t b_voff_x = (uint32_t)((t / 8) * (int)ldb + 16 * (t % 8));
-#define a_voff a_voff_x
-#define b_voff b_voff_x
-#endif
 
     // Everything a tile needs, decoded from its index on the device.
     struct Tile {
@@ -292,9 +267,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // tile rows [r * rows_per_ld, (r+1) * rows_per_ld) of the M-side operand for r < LPA, of
     // the N-side operand for LPA <= r < LPT; a round past the end is a no-op.
     auto issue_1 = [&](const Tile& d, int kp, int slot, int r) __attribute__((always_inline)) {
-#ifdef EXP_NODMA
-        return;
-#endif
         if (r < LPA) {
             dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff,
                   d.ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
@@ -389,9 +361,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             MXL_MFMA(cur, 2, 0); MXL_LD(2); MXL_PIN;
             MXL_MFMA(cur, 3, 0); MXL_LD(3); MXL_PIN;
             if (KS == 1) wait_vm<0>();  // K slot kp+1 has landed (its last request went out several MFMAs ago)
-#ifndef EXP_NOBAR
             __syncthreads();
-#endif
             MXL_PIN;
             if (KS == 1 && SUB == 0) issue_s(d, (kp >> 2) + 1);  // next scale panel; its buffer is dead since K slot kp-1
             MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1); MXL_LD(4); MXL_PIN;
@@ -444,9 +414,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         // ---- epilogue: fp32 -> bf16 through a wave-private LDS patch (in ring slot 1, which the
         // requests above do not touch), so that the global stores are 16 bytes per lane and each
         // store instruction covers 4 rows x 256 contiguous bytes ----
-#ifdef EXP_NOSTORE
-        if (acc[0][0][0] == 1234.5f)
-#endif
         {
             constexpr int SP = 272;  // bytes per staged row (256 + 16: spreads the rows over the banks)
             uint8_t* stg = smem + STAGE + w * (32 * SP);
@@ -472,9 +439,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
                         const uint4 v = *(const uint4*)(rd + 4 * u * SP);
-#ifdef EXP_NOGSTORE
-                        if (v.x == 0x12345678u)
-#endif
                         *(uint4*)(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off) = v;
                     }
                 } else {
@@ -493,14 +457,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #undef MXL_PIN
 #undef MXL_RD_A
 #undef MXL_RD_B
-#ifdef EXP_CLK
-    if (t == 0 && blockIdx.x < 64) {
-        const uint64_t clk1 = clock64(), wall1 = wall_clock64();
-        uint64_t* dbg = (uint64_t*)p.c;
-        dbg[2 * blockIdx.x] = clk1 - clk0;
-        dbg[2 * blockIdx.x + 1] = wall1 - wall0;
-    }
-#endif
 }
 
 constexpr int gemm_lds_bytes(int afmt, int bfmt) {

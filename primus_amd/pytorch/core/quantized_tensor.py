@@ -105,6 +105,9 @@ class QuantizedTensor(torch.Tensor):
     def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
         if func in _pass_through_ops():
             return args[0]._rewrap()
+        if func is torch.ops.aten.view.default and tuple(args[1]) == tuple(args[0].shape):
+            # autograd aliases a tensor that a Function returns unchanged with a same-shape view
+            return args[0]._rewrap()
         raise NotImplementedError(
             f"{func} is not defined on a QuantizedTensor; call .dequantize() first or hand it to a gemm op"
         )

@@ -35,7 +35,7 @@ from ..core.low_precision import (
 )
 from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
-__all__ = ["gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4"]
+__all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4"]
 
 
 class _MXLinearFunction(torch.autograd.Function):
@@ -184,3 +184,34 @@ def grouped_gemm_fp8(a, b, group_lens: torch.Tensor, trans_b: bool = True,
 def grouped_gemm_fp4(a, b, group_lens: torch.Tensor, trans_b: bool = True,
                      config: Optional[Float4QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
     return _run(a, b, _lens(group_lens), False, trans_b, None, config, fuse_bgrad_accum_pattern, fp4=True)
+
+
+# ---------------------------------------------------------------------------
+# Unquantised operators.  The reference's modules fall back to them outside a
+# low-precision autocast (primus_turbo.py:1180-1188, :2210-2216).  They are not
+# part of the MX path and have no kernels of their own here: the dense one is
+# the library GEMM behind ``torch.matmul``, the grouped one a loop of those
+# (which reads ``group_lens`` back to the host).
+# ---------------------------------------------------------------------------
+def gemm(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
+         fuse_bgrad_accum_pattern: Optional[str] = None):
+    if fuse_bgrad_accum_pattern is not None:
+        raise NotImplementedError("fused wgrad accumulation is not implemented")
+    a2 = a.transpose(-2, -1) if trans_a else a
+    b2 = b.transpose(-2, -1) if trans_b else b
+    out = torch.matmul(a2, b2)
+    return out if out_dtype is None else out.to(out_dtype)
+
+
+def grouped_gemm(a, b, group_lens: torch.Tensor, trans_b: bool = True,
+                 fuse_bgrad_accum_pattern: Optional[str] = None):
+    if fuse_bgrad_accum_pattern is not None:
+        raise NotImplementedError("fused wgrad accumulation is not implemented")
+    lens = [int(v) for v in _lens(group_lens).tolist()]
+    if sum(lens) != a.shape[0]:
+        raise ValueError("group_lens must sum to the number of rows of a")
+    outs = []
+    for g, rows in enumerate(torch.split(a, lens, dim=0)):
+        w = b[g].transpose(-2, -1) if trans_b else b[g]
+        outs.append(torch.matmul(rows, w))
+    return torch.cat(outs, dim=0)

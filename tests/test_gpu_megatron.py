@@ -1,0 +1,290 @@
+"""The Megatron-side modules on the real kernels: linear / grouped linear /
+expert MLP under the MXFP8 and MXFP4 autocasts, cached quantised weights with
+``main_grad`` accumulation, the MXFP4 local function and the optimizer's
+quantisation grid -- against the oracle where it restates the arithmetic, and
+against the reference's own acceptance bars where it states them (MXFP8 MoE
+cosine >= 0.90 vs bf16: tests/unit_tests/megatron/moe/test_mega_moe.py:243-280;
+MXFP4 gradient SNR > 10 dB vs bf16: test_primus_turbo_mxfp4_local.py:182-189)."""
+
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as o
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2  # max abs error / max abs value of the oracle's result
+
+
+def _f(t):
+    return o.bf16_bits_to_f32(t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16))
+
+
+def _close(got, want_bits, tol=TOL):
+    want = o.bf16_bits_to_f32(want_bits)
+    err = np.abs(_f(got).reshape(want.shape) - want).max() / max(np.abs(want).max(), 1e-30)
+    assert err <= tol, err
+
+
+def _snr_db(got, truth):
+    got, truth = got.float(), truth.float()
+    return (10 * torch.log10(truth.pow(2).sum() / (got - truth).pow(2).sum())).item()
+
+
+def _cos(a, b):
+    return torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item()
+
+
+@pytest.fixture
+def mg(gpu):
+    from primus_amd.megatron import runtime
+    from primus_amd.megatron.extensions import primus_turbo as pt
+
+    pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+    runtime.bind()
+    runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                     turbo_grouped_gemm_without_padding=True)
+    runtime.set_num_microbatches(1)
+    yield pt
+    pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+    runtime.set_args()
+    runtime.set_num_microbatches(1)
+
+
+def _cfg(**kw):
+    values = dict(params_dtype=torch.bfloat16, use_cpu_initialization=False, perform_initialization=True,
+                  tensor_model_parallel_size=1, gradient_accumulation_fusion=False, normalization="RMSNorm",
+                  layernorm_epsilon=1e-5)
+    values.update(kw)
+    return SimpleNamespace(**values)
+
+
+def _mxfp8(pt):
+    from primus_amd.pytorch.core import Format, ScaleDtype, ScalingGranularity
+
+    return pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.MX_BLOCKWISE, format=Format.E4M3, block_size=32,
+                                     scale_dtype=ScaleDtype.E8M0)
+
+
+def _mxfp4(pt, **kw):
+    from primus_amd.pytorch.core import Format, ScaleDtype, ScalingGranularity
+
+    return pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.MX_BLOCKWISE, format=Format.E2M1_X2, block_size=32,
+                                     scale_dtype=ScaleDtype.E8M0, use_gradient_sr=False, **kw)
+
+
+def test_linear_mxfp8_forward_backward_matches_oracle(mg, gpu):
+    pt = mg
+    torch.manual_seed(3)
+    lin = pt.PrimusTurboLinear(256, 160, parallel_mode=None, config=_cfg(), bias=True, skip_bias_add=False)
+    with torch.no_grad():
+        lin.bias.copy_(torch.linspace(-1, 1, 160))
+    x = torch.randn(25, 8, 256, device=gpu).bfloat16().requires_grad_()
+    dy = torch.randn(25, 8, 160, device=gpu).bfloat16()
+    with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt)):
+        y, bias = lin(x)
+    assert bias is None and y.shape == (25, 8, 160) and y.dtype == torch.bfloat16
+    y.backward(dy)
+    x2, w = x.detach().cpu().view(-1, 256), lin.weight.detach().cpu()
+    y_ref = o.bf16_bits_to_f32(o.linear_fwd_ref(x2, w)) + lin.bias.detach().float().cpu().numpy()
+    err = np.abs(_f(y).reshape(y_ref.shape) - y_ref).max() / np.abs(y_ref).max()
+    assert err <= TOL, err
+    dx, dw = o.linear_bwd_ref(x2, w, dy.cpu().view(-1, 160))
+    _close(x.grad, dx)
+    _close(lin.weight.grad, dw)
+    torch.testing.assert_close(lin.bias.grad.float(), dy.float().sum((0, 1)), rtol=2e-2, atol=2e-1)
+    # outside the autocast the same module is a plain bf16 linear
+    y_bf16, _ = lin(x.detach())
+    want = torch.nn.functional.linear(x.detach(), lin.weight, lin.bias)
+    torch.testing.assert_close(y_bf16.float(), want.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_cached_weights_accumulate_into_main_grad_over_microbatches(mg, gpu):
+    pt = mg
+    from primus_amd.megatron import runtime
+
+    runtime.set_num_microbatches(3)
+    torch.manual_seed(4)
+    lin = pt.PrimusTurboColumnParallelLinear(128, 96, config=_cfg(), bias=False)
+    lin.weight.main_grad = torch.zeros(96, 128, dtype=torch.float32, device=gpu)
+    lin.weight.grad_added_to_main_grad = False
+    xs = [torch.randn(40, 1, 128, device=gpu).bfloat16().requires_grad_() for _ in range(3)]
+    dys = [torch.randn(40, 1, 96, device=gpu).bfloat16() for _ in range(3)]
+    want = np.zeros((96, 128), dtype=np.float32)
+    w_cpu = lin.weight.detach().cpu()
+    with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt)):
+        for i, (x, dy) in enumerate(zip(xs, dys)):
+            y, _ = lin(x)
+            if i == 0:
+                first_codes = lin.quantized_weight_buffer.codes
+            assert lin.quantized_weight_buffer.codes.data_ptr() == first_codes.data_ptr()  # quantised once
+            lin.weight.grad_added_to_main_grad = False  # what the DDP wrapper does per microbatch
+            y.backward(dy)
+            _close(y, o.linear_fwd_ref(x.detach().cpu().view(-1, 128), w_cpu))
+            dx, dw = o.linear_bwd_ref(x.detach().cpu().view(-1, 128), w_cpu, dy.cpu().view(-1, 96))
+            _close(x.grad, dx)
+            want += o.bf16_bits_to_f32(dw)
+    got = lin.weight.main_grad.cpu().numpy()
+    assert np.abs(got - want).max() / np.abs(want).max() <= TOL
+    assert lin.weight.grad_added_to_main_grad is True
+    assert lin.weight.grad is not None and lin.weight.grad.shape == lin.weight.shape  # placeholder fired the hooks
+    assert lin.quantized_weight_t_buffer.axis == -2 and tuple(lin.quantized_weight_t_buffer.shape) == (128, 96)
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+def test_grouped_linear_ragged_groups(mg, gpu, fp4):
+    pt = mg
+    torch.manual_seed(5)
+    lens = [33, 0, 130, 1, 92]
+    gl = pt.PrimusTurboColumnParallelGroupedLinear(5, 128, 96, config=_cfg())
+    x = torch.randn(sum(lens), 128, device=gpu).bfloat16().requires_grad_()
+    dy = torch.randn(sum(lens), 96, device=gpu).bfloat16()
+    splits = torch.tensor(lens)  # on the host on purpose: the module moves it to the device
+    if fp4:
+        ctx = pt.primus_turbo_fp4_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp4(pt))
+        fmt = o.FMT_E2M1
+    else:
+        ctx = pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt))
+        fmt = o.FMT_E4M3
+    with ctx:
+        y, _ = gl(x, splits)
+    y.backward(dy)
+    xc, wc = x.detach().cpu(), gl.weights.detach().cpu()
+    xq, xs = o.quantize_mx_rowwise(xc, fmt)
+    wq, ws, _, _ = o.quantize_mx_2d(wc, fmt)
+    tol = 3e-2 if fp4 else TOL  # FP4 sums carry larger bf16 rounding of larger partials; still the reference's 3e-2 bar
+    _close(y, o.grouped_gemm_nt_ref(xq, xs, wq, ws, lens, fmt, fmt), tol)
+    dx, dw = o.linear_bwd_ref(xc, wc, dy.cpu(), fmt=fmt, group_lens=lens)
+    _close(x.grad, dx, tol)
+    _close(gl.weights.grad, dw, tol)
+    assert not gl.weights.grad[1].any()  # expert without tokens
+
+
+def _mlp(pt, gpu, experts, hidden, ffn, **cfg):
+    from primus_amd.megatron.transformer.experts import PrimusGroupedMLP
+
+    return PrimusGroupedMLP(experts, _cfg(hidden_size=hidden, ffn_hidden_size=ffn, moe_ffn_hidden_size=ffn,
+                                          gated_linear_unit=True, fp8="e4m3", fp8_recipe="mxfp8", fp4=None,
+                                          add_bias_linear=False, **cfg))
+
+
+def test_grouped_mlp_mxfp8_close_to_bf16(mg, gpu):
+    """Forward, dX and dW of the expert MLP in MXFP8 against the same module in bf16."""
+    pt = mg
+    torch.manual_seed(6)
+    mlp = _mlp(pt, gpu, 4, 256, 512)
+    lens = [100, 0, 257, 27]
+    x = torch.randn(sum(lens), 256, device=gpu).bfloat16()
+    probs = torch.rand(sum(lens), device=gpu).bfloat16()
+    tpe = torch.tensor(lens, device=gpu)
+    dy = torch.randn(sum(lens), 256, device=gpu).bfloat16()
+
+    def run(ctx):
+        mlp.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_()
+        with ctx:
+            out, _ = mlp(xi, tpe, probs)
+        out.backward(dy)
+        return out.detach(), xi.grad, mlp.linear_fc1.weights.grad.clone(), mlp.linear_fc2.weights.grad.clone()
+
+    import contextlib
+
+    ref = run(contextlib.nullcontext())
+    got = run(pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt)))
+    for name, a, b in zip(("y", "dx", "dw1", "dw2"), got, ref):
+        assert torch.isfinite(a.float()).all(), name
+        assert _cos(a, b) >= 0.99, (name, _cos(a, b))  # the reference's bar is 0.90
+
+
+def test_grouped_mlp_explicit_padding_gives_the_same_forward(mg, gpu):
+    """Padding rows are zeros and row-wise blocks never mix rows, so the padded
+    and the ragged path quantise every real row identically."""
+    pt = mg
+    from primus_amd.megatron import runtime
+
+    torch.manual_seed(7)
+    lens = [5, 0, 33, 64]
+    x = torch.randn(sum(lens), 128, device=gpu).bfloat16()
+    probs = torch.rand(sum(lens), device=gpu).bfloat16()
+    tpe = torch.tensor(lens, device=gpu)
+    ragged = _mlp(pt, gpu, 4, 128, 256)
+    runtime.set_args(enable_primus_turbo=True, use_turbo_grouped_gemm=True, turbo_grouped_gemm_without_padding=False)
+    padded = _mlp(pt, gpu, 4, 128, 256)
+    padded.load_state_dict(ragged.state_dict())
+    assert padded._use_explicit_quantization_padding() and not ragged._use_explicit_quantization_padding()
+    with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt)):
+        a, _ = ragged(x, tpe, probs)
+        b, _ = padded(x, tpe, probs)
+    assert a.shape == b.shape == (sum(lens), 128)
+    assert torch.equal(a, b)
+
+
+def test_mxfp4_dual_quantize_op_matches_oracle_bytes(mg, gpu):
+    from primus_amd.megatron.extensions import primus_turbo_mxfp4_local as m4
+
+    torch.manual_seed(8)
+    x = torch.randn(100, 96, device=gpu).bfloat16()        # activation recipe: 1-D blocks
+    row, row_s, col, col_s = m4._quantize_input_dual(x)
+    assert tuple(row.shape) == (100, 64) and tuple(row_s.shape) == (100, 4)
+    assert tuple(col.shape) == (96, 64) and tuple(col_s.shape) == (96, 4)
+    q, s = o.quantize_mx_rowwise(x.cpu(), o.FMT_E2M1)
+    assert np.array_equal(row.view(torch.uint8).cpu().numpy()[:, :48], q)
+    assert np.array_equal(row_s.view(torch.uint8).cpu().numpy()[:, :3], s)
+    assert not row.view(torch.uint8)[:, 48:].any() and not row_s.view(torch.uint8)[:, 3:].any()
+    qT, sT = o.quantize_mx_colwise_segmented(x.cpu(), [100], o.FMT_E2M1)
+    assert np.array_equal(col.view(torch.uint8).cpu().numpy(), qT)
+    assert np.array_equal(col_s.view(torch.uint8).cpu().numpy(), sT)
+
+    w = (torch.randn(64, 96, device=gpu) * 0.05).bfloat16()  # weight recipe: 2-D blocks
+    wr, wrs, wc, wcs = m4._quantize_weight_dual(w)
+    q, s, qt, st = o.quantize_mx_2d(w.cpu(), o.FMT_E2M1)
+    assert np.array_equal(wr.view(torch.uint8).cpu().numpy()[:, :48], q)
+    assert np.array_equal(wrs.view(torch.uint8).cpu().numpy()[:, :3], s)
+    assert np.array_equal(wc.view(torch.uint8).cpu().numpy()[:, :32], qt)
+    assert np.array_equal(wcs.view(torch.uint8).cpu().numpy()[:, :2], st)
+    with pytest.raises(NotImplementedError, match="colwise_use_rht"):
+        m4._quantize_input_dual(x, use_rht=True)
+    with pytest.raises(NotImplementedError, match="rowwise_use_sr"):
+        m4._quantize_grad_dual(x, use_sr=True)
+
+
+def test_mxfp4_linear_function_snr_against_bf16(mg, gpu):
+    """Shapes of the reference's test (x[128, 256], w[512, 256]); its bar is SNR > 10 dB."""
+    from primus_amd.megatron.extensions.primus_turbo_mxfp4_local import MXFP4LinearFunction
+
+    torch.manual_seed(9)
+    x = torch.randn(128, 256, device=gpu).bfloat16().requires_grad_()
+    w = (torch.randn(512, 256, device=gpu) * 0.05).bfloat16().requires_grad_()
+    dy = torch.randn(128, 512, device=gpu).bfloat16()
+    y = MXFP4LinearFunction.apply(x, w)
+    y.backward(dy)
+    xr, wr = x.detach().float().requires_grad_(), w.detach().float().requires_grad_()
+    yr = xr @ wr.T
+    yr.backward(dy.float())
+    assert y.shape == (128, 512) and x.grad.shape == x.shape and w.grad.shape == w.shape
+    for name, a, b in (("y", y, yr), ("dx", x.grad, xr.grad), ("dw", w.grad, wr.grad)):
+        assert _snr_db(a.detach(), b.detach()) > 10.0, (name, _snr_db(a.detach(), b.detach()))
+    # and the forward equals the oracle's MXFP4 linear
+    _close(y, o.linear_fwd_ref(x.detach().cpu(), w.detach().cpu(), o.FMT_E2M1, o.FMT_E2M1), 3e-2)
+
+
+def test_qdq_mxfp4_is_the_forward_weight_grid(mg, gpu):
+    from primus_amd.megatron.optimizer.weight_deosc import qdq_mxfp4, qdq_mxfp4_local_shard
+
+    torch.manual_seed(10)
+    w = (torch.randn(3, 64, 96, device=gpu) * 0.05).bfloat16()
+    got = qdq_mxfp4(w)
+    q, s, _, _ = o.quantize_mx_2d(w.cpu(), o.FMT_E2M1)
+    want = o.dequantize_mx(q, s, o.FMT_E2M1)
+    assert got.shape == w.shape and got.dtype == w.dtype
+    assert np.array_equal(_f(got), want.astype(np.float32).reshape(_f(got).shape))
+    assert torch.equal(qdq_mxfp4(w[1]), got[1])             # experts are independent 2-D matrices
+    assert torch.equal(qdq_mxfp4(got), got)                 # idempotent: grid points stay put
+    # a shard that covers whole tile rows of expert 1 reproduces the full result there
+    per = 64 * 96
+    start, end = per + 32 * 96, per + 64 * 96
+    shard = w.reshape(-1)[start:end].float()
+    local = qdq_mxfp4_local_shard(shard, tuple(w.shape), start, end, torch.bfloat16)
+    assert torch.equal(local, got.reshape(-1)[start:end])

@@ -45,6 +45,15 @@ WORKLOADS = {
 }
 
 
+# HBM bytes per launch of the forward/dgrad grouped GEMM, measured with hardware counters
+# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; KiB per dispatch averaged over the four launches of a
+# step, each scaled by what the same counter reads for a 1 GiB -> 1 GiB elementwise kernel: 2.000 and
+# 1.000).  The counter summary is committed as profiles/bench_mixtral_mxfp8_hbm_traffic.txt.
+TRAFFIC_BYTES_PER_LAUNCH = {
+    "mixtral_8x7b_moe_mxfp8": (2889349.2 * 2.000 + 835472.0 * 1.000) * 1024,
+}
+
+
 def route(spec):
     """tokens-per-expert (python list) from seeded synthetic router logits."""
     import torch
@@ -171,6 +180,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="mixtral_8x7b_moe_mxfp8", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-traffic", action="store_true",
+                    help="launch one plain 1 GiB-in / 1 GiB-out elementwise kernel first, so that a hardware-counter "
+                         "run of this command also reads the counters for a kernel of known HBM traffic")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no expert all-to-all); use --gpus 1", file=sys.stderr)
@@ -218,6 +230,13 @@ def main():
             x.grad = None
             w.grad = None
 
+    if args.calibrate_traffic:
+        src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)   # 1 GiB
+        dst = torch.empty_like(src)
+        torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
     timer = LaunchTimer()
     K.set_launch_hook(timer)
     for _ in range(args.warmup):
@@ -258,7 +277,7 @@ def main():
         "frac": round(gemm_tflops / FP8_PEAK_TFLOPS, 4),
         "avg_launch_ms": round(gk["sec"] / gk["n"] * 1e3, 4),
         "flops_per_launch": gk["flops"] / gk["n"],
-        "traffic": None,
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
     }
     kernels = {}
     for name, a in acc.items():

@@ -40,7 +40,27 @@ struct QuantArgs {
     int64_t row_ld;     // columns of the row-wise copy (>= cols; the excess is zero-filled padding)
     int64_t W;          // padded width of the transposed copy (elements)
     int64_t mat_rows;   // TWOD: rows per matrix (n); otherwise unused
+    int tiles_r, tiles_c;   // tile grid: row tiles (upper bound when grouped) x column tiles
+    int super_c, n_super;   // 8x8-tile supertiles: count along the columns, total
 };
+
+// Workgroup -> tile.  Workgroups are dealt to the 8 XCDs round robin, so workgroup L is the
+// (L / 8)-th one of XCD L % 8.  Each XCD walks whole 8x8-tile supertiles, column tile fastest:
+//  - the 4-byte scale pieces that 8 neighbouring tiles write (32 contiguous bytes, along the columns
+//    for the row-wise copy and along the rows for the transposed one) meet in one L2 and leave it as
+//    one write instead of eight partial ones;
+//  - the workgroups resident at any moment cover long contiguous row spans instead of one 256-byte
+//    column slice at a power-of-two stride, which would camp on a few memory channels.
+constexpr int QSUPER = 8;
+__device__ __forceinline__ bool quant_tile_of_workgroup(const QuantArgs& a, int& pt, int& ct) {
+    const int L = blockIdx.x, xcd = L & 7, k = L >> 3;
+    const int s = (k / (QSUPER * QSUPER)) * 8 + xcd;
+    if (s >= a.n_super) return false;
+    const int within = k % (QSUPER * QSUPER);
+    pt = (s / a.super_c) * QSUPER + within / QSUPER;
+    ct = (s % a.super_c) * QSUPER + within % QSUPER;
+    return pt < a.tiles_r && ct < a.tiles_c;
+}
 
 template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
@@ -52,8 +72,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 
     const int t = threadIdx.x;
     const int w = t >> 6, l = t & 63, c16 = l & 15, rg = l >> 4;
-    const int64_t col0 = (int64_t)blockIdx.y * QT;
-    const int pt = blockIdx.x;
+    int pt, ct;
+    if (!quant_tile_of_workgroup(a, pt, ct)) return;   // uniform over the workgroup
+    const int64_t col0 = (int64_t)ct * QT;
 
     // ---- which source rows does this tile hold? ----
     int64_t src_row0 = 0;
@@ -311,7 +332,16 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t* q, const
 // host-side dispatch
 // ---------------------------------------------------------------------------
 template <int FMT, int SMODE, bool TWOD>
-static int launch_quant(const QuantArgs& a, dim3 grid, hipStream_t st) {
+static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
+    const int64_t super_r = (tiles_r + QSUPER - 1) / QSUPER, super_c = (tiles_c + QSUPER - 1) / QSUPER;
+    const int64_t n_super = super_r * super_c;
+    const int64_t wgs = (n_super + 7) / 8 * 8 * QSUPER * QSUPER;
+    if (tiles_r > 0x7FFFFFFF || tiles_c > 0x7FFFFFFF || wgs > 0x7FFFFFFF) return MXL_EINVAL;
+    a.tiles_r = (int)tiles_r;
+    a.tiles_c = (int)tiles_c;
+    a.super_c = (int)super_c;
+    a.n_super = (int)n_super;
+    const dim3 grid((unsigned)wgs);
     const bool row = a.q_row != nullptr, col = a.q_colT != nullptr;
     if (row && col)
         hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD>), grid, dim3(QTHREADS), 0, st, a);
@@ -323,9 +353,9 @@ static int launch_quant(const QuantArgs& a, dim3 grid, hipStream_t st) {
 }
 
 template <bool TWOD>
-static int dispatch_quant(int fmt, int smode, const QuantArgs& a, dim3 grid, hipStream_t st) {
+static int dispatch_quant(int fmt, int smode, QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
 #define MXL_Q(F, S) \
-    if (fmt == F && smode == S) return launch_quant<F, S, TWOD>(a, grid, st);
+    if (fmt == F && smode == S) return launch_quant<F, S, TWOD>(a, tiles_r, tiles_c, st);
     MXL_Q(MXL_FMT_E4M3, MXL_SCALE_OCP_FLOOR)
     MXL_Q(MXL_FMT_E4M3, MXL_SCALE_RCEIL)
     MXL_Q(MXL_FMT_E4M3, MXL_SCALE_EVEN)
@@ -370,8 +400,7 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
     const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
     if (gx == 0) return MXL_OK;
-    if (gx > 0x7FFFFFFF || gy > 65535) return MXL_EINVAL;
-    return dispatch_quant<false>(fmt, scale_mode, a, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream);
+    return dispatch_quant<false>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
 }
 
 extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
@@ -399,8 +428,7 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
     a.mat_rows = n;
     const int64_t gx = batch * ((n + QT - 1) / QT);
     const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
-    if (gx > 0x7FFFFFFF || gy > 65535) return MXL_EINVAL;
-    return dispatch_quant<true>(fmt, scale_mode, a, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream);
+    return dispatch_quant<true>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
 }
 
 extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,

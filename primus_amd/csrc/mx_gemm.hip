@@ -96,6 +96,14 @@ __device__ __forceinline__ void dma2(v4i rsrc, uint32_t lds_off, uint32_t voff, 
 }
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
+// Output stores are marked non-temporal: the kernel never reads its output back, and keeping it
+// out of the way leaves L2 to the operand tiles that neighbouring workgroups share.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store16_streaming(uint8_t* dst, const uint4& v) {
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (u32x4*)dst);
+}
+
 // LDS -> MFMA fragment of one 32-row tile for K step ks (0 or 1) of a slot.
 template <int FMT>
 __device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int ks, int g) {
@@ -439,14 +447,14 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
                         const uint4 v = *(const uint4*)(rd + 4 * u * SP);
-                        *(uint4*)(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off) = v;
+                        store16_streaming(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off, v);
                     }
                 } else {
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
                         const uint4 v = *(const uint4*)(rd + 4 * u * SP);
                         if (wm * 128 + i * 32 + 4 * u + rr < m_valid && cc < n_valid)
-                            *(uint4*)(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off) = v;
+                            store16_streaming(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off, v);
                     }
                 }
                 MXL_PIN;  // one 32-row block at a time: 64 accumulators live, not 256

@@ -18,6 +18,25 @@
 
 namespace mxl {
 
+// The quantisers stream: every input byte is read once and every output byte written once, by one
+// workgroup.  Non-temporal accesses keep that traffic from displacing the E8M0 scale words in L2,
+// which do have to wait there for their neighbours (see quant_tile_of_workgroup).
+typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store16_streaming(void* d, const uint4& v) {
+    const qu32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (qu32x4*)d);
+}
+__device__ __forceinline__ void store8_streaming(void* d, const uint2& v) {
+    const qu32x2 t = {v.x, v.y};
+    __builtin_nontemporal_store(t, (qu32x2*)d);
+}
+__device__ __forceinline__ void store4_streaming(void* d, uint32_t v) { __builtin_nontemporal_store(v, (uint32_t*)d); }
+__device__ __forceinline__ uint4 load16_streaming(const void* s) {
+    const qu32x4 t = __builtin_nontemporal_load((const qu32x4*)s);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+
 constexpr int QT = 128;       // tile edge
 constexpr int QTHREADS = 256;
 
@@ -119,7 +138,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     for (int it = 0; it < 8; ++it) {
         const int r = 32 * w + 8 * rg + it;
         d[it] = make_uint4(0, 0, 0, 0);
-        if (col_ok && r < rows_valid) d[it] = *(const uint4*)(a.x + (src_row0 + r) * a.cols + col);
+        if (col_ok && r < rows_valid) d[it] = load16_streaming(a.x + (src_row0 + r) * a.cols + col);
     }
 
     // ---- block maxima ----
@@ -174,7 +193,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o.x = nonfinite4_e4m3(d[it].x, d[it].y);
                     o.y = nonfinite4_e4m3(d[it].z, d[it].w);
                 }
-                if (out_ok && r < rows_valid) *(uint2*)(a.q_row + (src_row0 + r) * a.row_ld + col) = o;
+                if (out_ok && r < rows_valid) store8_streaming(a.q_row + (src_row0 + r) * a.row_ld + col, o);
             } else {
                 uint32_t o;
                 if (byte != 255u) {
@@ -185,7 +204,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o = nonfinite2_e2m1(d[it].x) | (nonfinite2_e2m1(d[it].y) << 8) | (nonfinite2_e2m1(d[it].z) << 16) |
                         (nonfinite2_e2m1(d[it].w) << 24);
                 }
-                if (out_ok && r < rows_valid) *(uint32_t*)(a.q_row + ((src_row0 + r) * a.row_ld + col) / 2) = o;
+                if (out_ok && r < rows_valid) store4_streaming(a.q_row + ((src_row0 + r) * a.row_ld + col) / 2, o);
             }
         }
     }
@@ -269,7 +288,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             const int ch = t % LPR;
             if (col0 + c < a.cols && 16 * ch < avail) {
                 const uint4 v = *(const uint4*)(t_tile + c * TPITCH + 16 * ch);
-                *(uint4*)(a.q_colT + (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch) = v;
+                store16_streaming(a.q_colT + (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch, v);
             }
         }
     }

@@ -1,0 +1,180 @@
+"""The benchmark configurations at their FULL shapes (Llama-3-8B MLP, Mixtral-8x7B,
+DeepSeek-V3 expert shard, GPT-OSS-120B with MXFP4 weights): same seeded routing and
+tensor shapes as bench.py.
+
+A full CPU oracle run at these sizes would take hours, so each case checks
+ (1) quantised bytes and scales BIT-EXACT against the oracle on sampled bands (the
+     first and last rows of experts -- where blocks restart and padding begins -- and
+     random interior rows; both the row-wise and the transposed copy),
+ (2) forward, dgrad and wgrad outputs of the differentiable op at sampled output
+     positions against the oracle's fp64 dot products of the dequantised operands
+     (tolerance 1e-2 of the largest expected magnitude, 3e-2 with FP4 operands),
+ (3) size-independent properties: an expert without tokens gets an all-zero weight
+     gradient and no output rows; outputs are finite.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import bench
+from oracle import mx_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def _u8(t):
+    return t.view(torch.uint8)
+
+
+def _deq_rows(codes_u8, scales_u8, fmt):
+    """float64 [rows, K] from uint8 numpy codes / scales (row-wise layout)."""
+    return o.dequantize_mx(codes_u8, scales_u8, fmt).astype(np.float64)
+
+
+def _bf(t):
+    return o.bf16_bits_to_f32(t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
+
+
+def _sample_rows(lens, rng, per_group=2):
+    """Row indices: first and last row of every non-empty expert plus random interior rows."""
+    rows, off = [], 0
+    for n in lens:
+        if n > 0:
+            rows += [off, off + n - 1]
+            rows += [off + int(v) for v in rng.integers(0, n, size=per_group)]
+        off += n
+    return sorted(set(rows))
+
+
+def _group_of(row, lens):
+    off = 0
+    for g, n in enumerate(lens):
+        if row < off + n:
+            return g, off
+        off += n
+    raise AssertionError
+
+
+CASES = [
+    ("llama3_8b_mlp_mxfp8", 0),
+    ("mixtral_8x7b_moe_mxfp8", 0),
+    ("deepseek_v3_shard_mxfp8", 0),
+    ("gpt_oss_120b_mxfp4", 0),
+]
+
+
+@pytest.mark.parametrize("workload,layer", [(w, l) for w, _ in CASES for l in (0, 1)])
+def test_full_size_linear(gpu, workload, layer):
+    import primus_amd.pytorch as pt
+    from primus_amd.pytorch import kernels as K
+    from primus_amd.pytorch.core import Float4QuantConfig, Float8QuantConfig, Format, ScaleDtype, ScalingGranularity
+
+    spec = bench.WORKLOADS[workload]
+    lens = bench.route(spec)
+    G, M = spec["G"], sum(lens)
+    dense = spec["routing"] == "dense"
+    k, n = ((spec["hidden"], spec["fc1_out"]), (spec["fc2_in"], spec["hidden"]))[layer]
+    fp4 = spec["fp4"]
+    a_fmt, w_fmt = o.FMT_E4M3, (o.FMT_E2M1 if fp4 else o.FMT_E4M3)
+    tol = 3e-2 if fp4 else 1e-2
+    if fp4:
+        cfg = Float4QuantConfig(activation_format=Format.E4M3)
+    else:
+        cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE,
+                                scale_dtype=ScaleDtype.E8M0, block_size=32)
+    rng = np.random.default_rng(spec["seed"] + layer)
+    gen = torch.Generator(device=gpu).manual_seed(spec["seed"] + 17 * layer)
+    x = torch.randn(M, k, generator=gen, device=gpu).bfloat16()
+    w = (torch.randn(*((n, k) if dense else (G, n, k)), generator=gen, device=gpu) * 0.02).bfloat16()
+    dy = torch.randn(M, n, generator=gen, device=gpu).bfloat16()
+    gl = None if dense else torch.tensor(lens, dtype=torch.int64, device=gpu)
+    glens = [M] if dense else lens
+
+    # ---- (1) quantised operands, bit-exact on sampled bands ----
+    xq, xs, xqT, xsT = K.quantize_mx_impl(x, a_fmt, rowwise=True, colwise=True, group_lens=gl, pad_to=K.GEMM_K_ALIGN)
+    dq, ds, dqT, dsT = K.quantize_mx_impl(dy, a_fmt, rowwise=True, colwise=True, group_lens=gl, pad_to=K.GEMM_K_ALIGN)
+    wq, ws, wqT, wsT = K.quantize_mx_weight_2d_impl(w, w_fmt, rowwise=True, colwise=True, pad_to=K.GEMM_K_ALIGN)
+    kp = k if k % 128 == 0 else (k + 127) // 128 * 128   # padded contraction width of the row-wise copies
+    rows = _sample_rows(glens, rng)
+    ridx = torch.tensor(rows, device=gpu)
+    for src, q, s, width in ((x, xq, xs, k), (dy, dq, ds, n)):
+        oq, os_ = o.quantize_mx_rowwise(src[ridx].cpu(), a_fmt)
+        assert np.array_equal(_u8(q)[ridx].cpu().numpy()[:, :width], oq)
+        assert np.array_equal(_u8(s)[ridx].cpu().numpy()[:, : width // 32], os_)
+        assert not _u8(q)[ridx][:, width:].any()          # GEMM padding: zero codes, scale byte 0
+        assert not _u8(s)[ridx][:, width // 32:].any()
+    # transposed copies: whole 128-token bands at expert starts / ends, all columns of a sampled column band
+    _, seg_off = o.segment_layout(glens)   # start of every expert's segment in the padded transposed layout
+    c0 = int(rng.integers(0, k // 32)) * 32
+    picked = [g for g, ln in enumerate(glens) if ln > 0][:3] + [g for g, ln in enumerate(glens) if ln > 0][-1:]
+    off_rows = np.concatenate([[0], np.cumsum(glens)])
+    for g in sorted(set(picked)):
+        r0, ln = int(off_rows[g]), glens[g]
+        band = x[r0 : r0 + ln, c0 : c0 + 32].cpu()
+        oqT, osT = o.quantize_mx_colwise_segmented(band, [ln], a_fmt)
+        p0 = int(seg_off[g])
+        wpad = oqT.shape[1]                                   # ln rounded up to 128
+        got_q = _u8(xqT)[c0 : c0 + 32, p0 : p0 + wpad].cpu().numpy()
+        got_s = _u8(xsT)[c0 : c0 + 32, p0 // 32 : (p0 + wpad) // 32].cpu().numpy()
+        assert np.array_equal(got_q, oqT) and np.array_equal(got_s, osT), (workload, g)
+    # weights: one 2-D tile row band of a sampled expert, both copies
+    e = int(rng.integers(0, 1 if dense else G))
+    n0 = int(rng.integers(0, n // 32)) * 32
+    wb = (w if dense else w[e])[n0 : n0 + 32].cpu()
+    oq, os_, oqT, osT = o.quantize_mx_2d(wb, w_fmt)
+    per = 2 if w_fmt == o.FMT_E2M1 else 1
+    wq_e, ws_e, wqT_e, wsT_e = ((wq, ws, wqT, wsT) if dense else (wq[e], ws[e], wqT[e], wsT[e]))
+    assert np.array_equal(_u8(wq_e)[n0 : n0 + 32].cpu().numpy()[:, : k // per], oq)
+    assert np.array_equal(_u8(ws_e)[n0 : n0 + 32].cpu().numpy()[:, : k // 32], os_)
+    assert np.array_equal(_u8(wqT_e)[:, n0 // per : (n0 + 32) // per].cpu().numpy(), oqT)
+    assert np.array_equal(_u8(wsT_e)[:, n0 // 32 : n0 // 32 + 1].cpu().numpy(), osT)
+
+    # ---- (2) the differentiable op at full size; sampled outputs against the oracle ----
+    xg, wg = x.clone().requires_grad_(), w.clone().requires_grad_()
+    if dense:
+        y = pt.ops.gemm_fp8(xg, wg, trans_a=False, trans_b=True, out_dtype=None, config=cfg)
+    elif fp4:
+        y = pt.ops.grouped_gemm_fp4(xg, wg, gl, trans_b=True, config=cfg)
+    else:
+        y = pt.ops.grouped_gemm_fp8(xg, wg, gl, trans_b=True, config=cfg)
+    y.backward(dy)
+    dx, dw = xg.grad, wg.grad
+    assert torch.isfinite(y.float()).all() and torch.isfinite(dx.float()).all() and torch.isfinite(dw.float()).all()
+
+    cols_n = np.sort(rng.choice(n, size=48, replace=False))
+    cols_k = np.sort(rng.choice(k, size=48, replace=False))
+    cn, ck = torch.tensor(cols_n, device=gpu), torch.tensor(cols_k, device=gpu)
+    a_rows = _deq_rows(_u8(xq)[ridx].cpu().numpy(), _u8(xs)[ridx].cpu().numpy(), a_fmt)        # [R, kp]
+    d_rows = _deq_rows(_u8(dq)[ridx].cpu().numpy(), _u8(ds)[ridx].cpu().numpy(), a_fmt)        # [R, np]
+    y_s, dx_s = _bf(y[ridx][:, cn]), _bf(dx[ridx][:, ck])
+    want_y, want_dx = np.zeros_like(y_s), np.zeros_like(dx_s)
+    cache = {}
+    for i, r in enumerate(rows):
+        g, _ = _group_of(r, glens)
+        if g not in cache:
+            we = (wq, ws, wqT, wsT) if dense else (wq[g], ws[g], wqT[g], wsT[g])
+            b_fwd = _deq_rows(_u8(we[0])[cn].cpu().numpy(), _u8(we[1])[cn].cpu().numpy(), w_fmt)   # [48, kp]
+            b_bwd = _deq_rows(_u8(we[2])[ck].cpu().numpy(), _u8(we[3])[ck].cpu().numpy(), w_fmt)   # [48, np]
+            cache[g] = (b_fwd, b_bwd)
+        want_y[i] = cache[g][0] @ a_rows[i]
+        want_dx[i] = cache[g][1] @ d_rows[i]
+    assert np.abs(y_s - want_y).max() <= tol * np.abs(want_y).max()
+    assert np.abs(dx_s - want_dx).max() <= tol * np.abs(want_dx).max()
+
+    # wgrad: sampled (n, k) positions of up to three experts, contraction over the expert's padded segment
+    for g in sorted(set(picked))[:3]:
+        p0, ln = int(seg_off[g]), glens[g]
+        wpad = (ln + 127) // 128 * 128
+        a_t = _deq_rows(_u8(dqT)[cn][:, p0 : p0 + wpad].cpu().numpy(), _u8(dsT)[cn][:, p0 // 32 : (p0 + wpad) // 32].cpu().numpy(), a_fmt)
+        b_t = _deq_rows(_u8(xqT)[ck][:, p0 : p0 + wpad].cpu().numpy(), _u8(xsT)[ck][:, p0 // 32 : (p0 + wpad) // 32].cpu().numpy(), a_fmt)
+        want = a_t @ b_t.T
+        got = _bf((dw if dense else dw[g])[cn][:, ck])
+        assert np.abs(got - want).max() <= tol * np.abs(want).max(), (workload, g)
+
+    # ---- (3) properties ----
+    if not dense:
+        for g, ln in enumerate(glens):
+            if ln == 0:
+                assert not dw[g].any()
+        assert y.shape == (M, n) and dx.shape == (M, k) and dw.shape == (G, n, k)

@@ -20,6 +20,7 @@ Activations and gradients use 1-D blocks of 32, weights 2-D 32x32 blocks.
 
 from __future__ import annotations
 
+import warnings
 from typing import Optional, Union
 
 import torch
@@ -102,6 +103,10 @@ def _formats(config, fp4: bool):
     if fp4:
         if not isinstance(config, Float4QuantConfig):
             raise TypeError("gemm_fp4 / grouped_gemm_fp4 expect a Float4QuantConfig")
+        if config.use_gradient_sr:
+            # stochastic rounding of gradients (primus_turbo_mxfp4_local.py:272-288) has no kernel here
+            warnings.warn("use_gradient_sr is set but gradients are rounded to nearest-even: "
+                          "stochastic rounding is not implemented", stacklevel=3)
         return fmt_code(config.activation_format), _lib.FMT_E2M1
     if not isinstance(config, Float8QuantConfig):
         raise TypeError("gemm_fp8 / grouped_gemm_fp8 expect a Float8QuantConfig")

@@ -36,7 +36,28 @@ from ..core.low_precision import (
 )
 from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
-__all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4"]
+__all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap"]
+
+# dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
+# kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
+# as dgrad's last, partial wave of tiles drains instead of leaving those CUs idle.
+_wgrad_overlap = True
+_side_streams = {}
+
+
+def set_wgrad_overlap(enabled: bool) -> None:
+    """Run wgrad on a side stream next to dgrad (default on)."""
+    global _wgrad_overlap
+    _wgrad_overlap = bool(enabled)
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    key = (device.type, device.index)
+    st = _side_streams.get(key)
+    if st is None:
+        st = torch.cuda.Stream(device=device)   # default priority
+        _side_streams[key] = st
+    return st
 
 
 class _MXLinearFunction(torch.autograd.Function):
@@ -89,13 +110,26 @@ class _MXLinearFunction(torch.autograd.Function):
             dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
         )
         grad_a = grad_b = None
+        overlap = _wgrad_overlap and need_dgrad and need_wgrad
+        if overlap:
+            main = torch.cuda.current_stream(dy.device)
+            side = _side_stream(dy.device)
+            side.wait_stream(main)   # the quantised operands are ready
         if need_dgrad:
             if grouped:
                 grad_a = K.grouped_gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, group_lens)
             else:
                 grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs)
         if need_wgrad:
-            grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
+            if overlap:
+                with torch.cuda.stream(side):
+                    grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
+                for t in (d_col, d_cs, a_col, a_cs, grad_b):
+                    t.record_stream(side)
+                grad_b.record_stream(main)
+                main.wait_stream(side)
+            else:
+                grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
         return grad_a, grad_b, None, None, None, None, None
 
 

@@ -42,6 +42,12 @@ extern "C" {
 #define MXL_SCALE_RCEIL 1
 #define MXL_SCALE_EVEN 2
 
+/* gated activations of the expert MLP and the dtype of the router probabilities */
+#define MXL_ACT_SILU 0
+#define MXL_ACT_GELU 1
+#define MXL_PROBS_F32 0
+#define MXL_PROBS_BF16 1
+
 #define MXL_BLOCK 32      /* MX block size (fp8_utils.py:48, fp4_utils.py:79) */
 #define MXL_SEG_ALIGN 128 /* padding of each expert segment in the transposed layout */
 #define MXL_MAX_GROUPS 1024
@@ -132,6 +138,22 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
                            const void* b_codes, const void* b_scales, int b_fmt, void* c_bf16,
                            const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
                            int64_t k, void* stream);
+
+/* Gated activation of the expert MLP fused with the router probability and the row mask
+ * (swiglu_with_probs / geglu_with_probs behind fused_bias_act_with_probs, primus_turbo.py:1954-1980;
+ * the unfused arithmetic is experts.py:100-118):
+ *   y[m, j] = act(x[m, j]) * x[m, F + j] * probs[m]     for bf16 x[rows, 2F], y[rows, F],
+ * computed in fp32, rounded once to bf16.  row_mask (one byte per row, may be NULL = all rows live):
+ * a row with mask 0 yields zeros (tokens_per_expert_to_mask marks the rows past the routed tokens
+ * of a worst-case sized buffer).  probs is fp32 or bf16 per probs_dtype.  Requires f % 8 == 0. */
+int mxl_glu_probs_fwd(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
+                      int64_t rows, int64_t f, int act, void* y_bf16, void* stream);
+
+/* Backward of the above: dx[rows, 2F] (bf16) and dprobs[rows] (fp32) from dy[rows, F]; masked rows
+ * get zero gradients. */
+int mxl_glu_probs_bwd(const void* dy_bf16, const void* x_bf16, const void* probs, int probs_dtype,
+                      const uint8_t* row_mask, int64_t rows, int64_t f, int act, void* dx_bf16,
+                      void* dprobs_f32, void* stream);
 
 #ifdef __cplusplus
 }

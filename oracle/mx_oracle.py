@@ -44,6 +44,14 @@ Parity status
   invariants (G=1 == dense, permutation of experts, exactly representable
   integer products) in tests/.
 
+* ``glu_with_probs_ref`` / ``glu_with_probs_bwd_ref`` (gated activation times
+  router probability with a row mask; call site primus_turbo.py:1954-1980,
+  unfused arithmetic experts.py:100-118): float64 closed forms, pinned against
+  torch's float64 ``silu`` / ``gelu`` and autograd (library routines) and by
+  the identities act(x) - act(-x) = x.  Whether the Primus-Turbo kernels round
+  once (as here, like Megatron's fused weighted SwiGLU) or after every step,
+  and which GELU flavour ``geglu_with_probs`` uses, is **parity unpinned**.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -455,3 +463,56 @@ def linear_bwd_ref(x, w, dy, fmt=FMT_E4M3, scale_mode=SCALE_OCP_FLOOR, group_len
     if dense:
         dw = dw[0]
     return dx, dw
+
+
+# --------------------------------------------------------------------------
+# gated activation x router probability (swiglu_with_probs / geglu_with_probs)
+# --------------------------------------------------------------------------
+def _erfc(x: np.ndarray) -> np.ndarray:
+    from math import erfc
+
+    return np.vectorize(erfc, otypes=[np.float64])(x)
+
+
+def _act64(g: np.ndarray, activation: str):
+    """act(g) and act'(g) in float64."""
+    if activation == "silu":
+        s = 1.0 / (1.0 + np.exp(-g))
+        return g * s, s * (1.0 + g * (1.0 - s))
+    if activation == "gelu":
+        c = 0.5 * _erfc(-g / np.sqrt(2.0))   # = Phi(g); erfc keeps the negative tail free of cancellation
+        return g * c, c + g * np.exp(-0.5 * g * g) / np.sqrt(2.0 * np.pi)
+    raise ValueError(activation)
+
+
+def glu_with_probs_ref(x, probs, row_mask=None, activation: str = "silu", out_bf16: bool = True):
+    """y[m, j] = act(x[m, j]) * x[m, F + j] * probs[m]; masked rows are zero.
+    ``x``: bf16 [M, 2F] (torch tensor, uint16 bits or floats); float64 arithmetic,
+    one rounding to bf16 (returned as bits) unless ``out_bf16`` is False."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x)).astype(np.float64)
+    f = xf.shape[1] // 2
+    p = np.asarray(probs, dtype=np.float64).reshape(-1, 1)
+    with np.errstate(over="ignore"):
+        a, _ = _act64(xf[:, :f], activation)
+    y = a * xf[:, f:] * p
+    if row_mask is not None:
+        y = np.where(np.asarray(row_mask).astype(bool).reshape(-1, 1), y, 0.0)
+    return f32_to_bf16_bits(y.astype(np.float32)) if out_bf16 else y
+
+
+def glu_with_probs_bwd_ref(dy, x, probs, row_mask=None, activation: str = "silu"):
+    """(dx [M, 2F], dprobs [M]) in float64 for bf16 ``dy`` [M, F] and ``x`` [M, 2F]."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x)).astype(np.float64)
+    d = bf16_bits_to_f32(to_bf16_bits(dy)).astype(np.float64)
+    f = xf.shape[1] // 2
+    p = np.asarray(probs, dtype=np.float64).reshape(-1, 1)
+    with np.errstate(over="ignore"):
+        a, da = _act64(xf[:, :f], activation)
+    u = xf[:, f:]
+    dx = np.concatenate([d * p * u * da, d * p * a], axis=1)
+    dp = (d * a * u).sum(axis=1)
+    if row_mask is not None:
+        m = np.asarray(row_mask).astype(bool)
+        dx = np.where(m.reshape(-1, 1), dx, 0.0)
+        dp = np.where(m, dp, 0.0)
+    return dx, dp

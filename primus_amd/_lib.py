@@ -24,6 +24,8 @@ BLOCK = 32
 SEG_ALIGN = 128
 GEMM_K_ALIGN = 128  # the GEMM kernels take the contraction dim in multiples of this
 MAX_GROUPS = 1024
+ACT_SILU, ACT_GELU = 0, 1
+PROBS_F32, PROBS_BF16 = 0, 1
 
 EXPORTS = (
     "mxl_version",
@@ -35,6 +37,8 @@ EXPORTS = (
     "mxl_gemm_nt",
     "mxl_grouped_gemm_nt",
     "mxl_grouped_gemm_wgrad",
+    "mxl_glu_probs_fwd",
+    "mxl_glu_probs_bwd",
 )
 
 
@@ -79,6 +83,10 @@ def load() -> ctypes.CDLL:
         lib.mxl_grouped_gemm_nt.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
         lib.mxl_grouped_gemm_wgrad.restype = i32
         lib.mxl_grouped_gemm_wgrad.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        lib.mxl_glu_probs_fwd.restype = i32
+        lib.mxl_glu_probs_fwd.argtypes = [vp, vp, i32, vp, i64, i64, i32, vp, vp]
+        lib.mxl_glu_probs_bwd.restype = i32
+        lib.mxl_glu_probs_bwd.argtypes = [vp, vp, vp, i32, vp, i64, i64, i32, vp, vp, vp]
         _lib = lib
     return _lib
 

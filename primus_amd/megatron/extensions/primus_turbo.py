@@ -751,6 +751,29 @@ class PrimusTurboRowParallelGroupedLinear(PrimusTurboGroupedLinear):
 
 
 # ---------------------------------------------------------------------------
+# fused activation with router probabilities (primus_turbo.py:1954-1980)
+# ---------------------------------------------------------------------------
+def fused_bias_act_with_probs(intermediate_parallel: torch.Tensor, bias_parallel: Optional[torch.Tensor],
+                              permuted_probs: torch.Tensor, tokens_per_experts: torch.Tensor,
+                              activation_func: str) -> torch.Tensor:
+    """``act(x[:, :F]) * x[:, F:] * probs`` with the rows past the routed tokens zeroed; ``x`` is
+    fc1's output ``[tokens, 2F]``, ``activation_func`` "silu" or "gelu"."""
+    assert intermediate_parallel.ndim == 2
+    assert permuted_probs.ndim == 1
+    assert tokens_per_experts.device == intermediate_parallel.device
+    if bias_parallel is not None:
+        intermediate_parallel = intermediate_parallel + bias_parallel
+    row_mask = ops.tokens_per_expert_to_mask(tokens_per_experts, intermediate_parallel.shape[0])
+    if activation_func == "silu":
+        fused = ops.swiglu_with_probs
+    elif activation_func == "gelu":
+        fused = ops.geglu_with_probs
+    else:
+        raise ValueError(f"Activation function {activation_func} is not supported.")
+    return fused(intermediate_parallel, permuted_probs, row_mask)
+
+
+# ---------------------------------------------------------------------------
 # a14  router-side padding multiple
 # ---------------------------------------------------------------------------
 def router_pad_multiple(moe_router_padding_for_quantization: bool) -> int:
@@ -779,5 +802,5 @@ __all__ = [
     "primus_turbo_fp4_autocast", "QuantizationRecipe", "QuantizationParams", "PrimusTurboLinear",
     "PrimusTurboRowParallelLinear", "PrimusTurboColumnParallelLinear", "PrimusTurboLayerNormColumnParallelLinear",
     "PrimusTurboGroupedLinear", "PrimusTurboColumnParallelGroupedLinear", "PrimusTurboRowParallelGroupedLinear",
-    "router_pad_multiple", "pad_tokens_per_expert", "QuantizedTensor", "QuantizedTensorPair",
+    "router_pad_multiple", "pad_tokens_per_expert", "fused_bias_act_with_probs", "QuantizedTensor", "QuantizedTensorPair",
 ]

@@ -113,9 +113,35 @@ class PrimusGroupedMLP(torch.nn.Module):
         return (intermediate * permuted_probs).to(dtype)
 
     def bias_act_func_with_mask(self, intermediate, bias, permuted_probs, tokens_per_experts=None):
-        if self.use_turbo_fused_act_with_probs:
-            raise NotImplementedError("the fused activation-with-probabilities kernel is not part of this package")
-        return self.bias_act_func(intermediate, bias, permuted_probs)
+        """experts.py:120-165: the fused kernel when ``use_turbo_fused_act_with_probs`` is set (gated
+        SiLU / GELU only, no clamp, no linear offset), else the unfused arithmetic."""
+        if not self.use_turbo_fused_act_with_probs:
+            return self.bias_act_func(intermediate, bias, permuted_probs)
+        from ..extensions.primus_turbo import fused_bias_act_with_probs
+
+        assert tokens_per_experts is not None, (
+            "tokens_per_experts is required when `use_turbo_fused_act_with_probs` is True."
+        )
+        assert getattr(self.config, "activation_func_clamp_value", None) is None, (
+            "`use_turbo_fused_act_with_probs` does not support activation_func_clamp_value."
+        )
+        assert getattr(self.config, "glu_linear_offset", 0.0) == 0.0, (
+            "`use_turbo_fused_act_with_probs` does not support a non-zero glu_linear_offset."
+        )
+        assert not getattr(self.config, "activation_func_fp8_input_store", False), (
+            "`use_turbo_fused_act_with_probs` does not support activation_func_fp8_input_store."
+        )
+        if self.activation_func == F.silu and self.gated:
+            activation = "silu"
+        elif self.activation_func == F.gelu and self.gated:
+            activation = "gelu"
+        else:
+            raise ValueError(
+                "Only support fusion of swiglu and gelu in PrimusGroupedMLP when `use_turbo_fused_act_with_probs` is True."
+            )
+        # forward() hands the probabilities over as [tokens, 1]; the kernel takes them 1-D
+        probs_1d = permuted_probs.squeeze(-1) if permuted_probs.dim() == 2 else permuted_probs
+        return fused_bias_act_with_probs(intermediate, bias, probs_1d, tokens_per_experts, activation)
 
     def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor,
                 permuted_probs: torch.Tensor) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:

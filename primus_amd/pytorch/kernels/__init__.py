@@ -331,6 +331,58 @@ def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total
 
 
 # --------------------------------------------------------------------------
+# gated activation with router probabilities
+# --------------------------------------------------------------------------
+_ACTS = {"silu": _lib.ACT_SILU, "gelu": _lib.ACT_GELU}
+
+
+def _glu_args(x, probs, row_mask, activation):
+    if activation not in _ACTS:
+        raise ValueError(f"Activation function {activation} is not supported.")
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % 16 != 0:
+        raise ValueError("expected a 2-D bfloat16 tensor [tokens, 2F] with F a multiple of 8")
+    if probs.dim() != 1 or probs.shape[0] != x.shape[0] or probs.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("probs must be a 1-D float32 or bfloat16 tensor with one entry per token")
+    if row_mask is not None:
+        if row_mask.dim() != 1 or row_mask.shape[0] != x.shape[0]:
+            raise ValueError("row_mask must have one entry per token")
+        if row_mask.dtype == torch.bool:
+            row_mask = row_mask.view(torch.uint8)
+        if row_mask.dtype != torch.uint8:
+            raise ValueError("row_mask must be a bool or uint8 tensor")
+    _require_cuda(x, probs, row_mask)
+    pd = _lib.PROBS_BF16 if probs.dtype == torch.bfloat16 else _lib.PROBS_F32
+    return _ACTS[activation], pd, row_mask
+
+
+def glu_with_probs_fwd_impl(x, probs, row_mask, activation: str) -> torch.Tensor:
+    """``act(x[:, :F]) * x[:, F:] * probs[:, None]`` in fp32, one rounding to bf16; masked rows give 0."""
+    act, pd, row_mask = _glu_args(x, probs, row_mask, activation)
+    rows, f = x.shape[0], x.shape[1] // 2
+    y = torch.empty((rows, f), dtype=torch.bfloat16, device=x.device)
+    with _hooked("glu_probs_fwd", rows=rows, f=f):
+        rc = _lib.load().mxl_glu_probs_fwd(_ptr(x), _ptr(probs), pd, _ptr(row_mask), rows, f, act, _ptr(y), _stream())
+    _lib.check(rc, "mxl_glu_probs_fwd")
+    return y
+
+
+def glu_with_probs_bwd_impl(dy, x, probs, row_mask, activation: str):
+    """``(dx [tokens, 2F] bf16, dprobs [tokens] fp32)``."""
+    act, pd, row_mask = _glu_args(x, probs, row_mask, activation)
+    rows, f = x.shape[0], x.shape[1] // 2
+    if dy.dtype != torch.bfloat16 or tuple(dy.shape) != (rows, f):
+        raise ValueError("dy must be bfloat16 [tokens, F]")
+    _require_cuda(dy)
+    dx = torch.empty_like(x)
+    dp = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    with _hooked("glu_probs_bwd", rows=rows, f=f):
+        rc = _lib.load().mxl_glu_probs_bwd(_ptr(dy), _ptr(x), _ptr(probs), pd, _ptr(row_mask), rows, f, act, _ptr(dx),
+                                           _ptr(dp), _stream())
+    _lib.check(rc, "mxl_glu_probs_bwd")
+    return dx, dp
+
+
+# --------------------------------------------------------------------------
 # reference-named low-level entry points (MX granularity only)
 # --------------------------------------------------------------------------
 def _require_mx(granularity) -> None:

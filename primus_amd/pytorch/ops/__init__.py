@@ -36,7 +36,8 @@ from ..core.low_precision import (
 )
 from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
-__all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap"]
+__all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
+           "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask"]
 
 # dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
 # kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
@@ -254,3 +255,48 @@ def grouped_gemm(a, b, group_lens: torch.Tensor, trans_b: bool = True,
         w = b[g].transpose(-2, -1) if trans_b else b[g]
         outs.append(torch.matmul(rows, w))
     return torch.cat(outs, dim=0)
+
+
+# ---------------------------------------------------------------------------
+# Gated activation fused with the router probability and the row mask: the three operators the
+# reference's fused_bias_act_with_probs calls (primus_turbo.py:1954-1980).
+# ---------------------------------------------------------------------------
+def tokens_per_expert_to_mask(tokens_per_expert: torch.Tensor, num_tokens: int) -> torch.Tensor:
+    """``mask[i] = i < sum(tokens_per_expert)``: the live rows of a buffer sized for the worst case.
+    Stays on the device (no host read of the counts)."""
+    total = tokens_per_expert.sum()
+    return torch.arange(num_tokens, device=tokens_per_expert.device) < total
+
+
+class _GluWithProbs(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, probs, row_mask, activation):
+        ctx.save_for_backward(x, probs, row_mask)
+        ctx.activation = activation
+        return K.glu_with_probs_fwd_impl(x, probs, row_mask, activation)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, probs, row_mask = ctx.saved_tensors
+        dy = dy.contiguous()
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        dx, dp = K.glu_with_probs_bwd_impl(dy, x, probs, row_mask, ctx.activation)
+        return dx, dp.to(probs.dtype), None, None
+
+
+def _glu_with_probs(x, probs, row_mask, activation):
+    if not x.is_contiguous():
+        x = x.contiguous()
+    return _GluWithProbs.apply(x, probs.contiguous(), row_mask, activation)
+
+
+def swiglu_with_probs(x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(x[:, :F]) * x[:, F:] * probs[:, None]`` for bf16 ``x [tokens, 2F]``; rows whose mask is
+    False give zeros.  Differentiable in ``x`` and ``probs``."""
+    return _glu_with_probs(x, probs, row_mask, "silu")
+
+
+def geglu_with_probs(x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Same with the (erf) GELU as the gate activation."""
+    return _glu_with_probs(x, probs, row_mask, "gelu")

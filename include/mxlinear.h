@@ -155,6 +155,17 @@ int mxl_glu_probs_bwd(const void* dy_bf16, const void* x_bf16, const void* probs
                       const uint8_t* row_mask, int64_t rows, int64_t f, int act, void* dx_bf16,
                       void* dprobs_f32, void* stream);
 
+/* The same activation feeding the MX quantiser directly: what mxl_quantize would produce for
+ * y = mxl_glu_probs_fwd(x, ...) (bit for bit), without y ever reaching memory.  It saves one bf16
+ * write and one bf16 read of [rows, f] between fc1 and fc2 of the expert MLP; the reference runs
+ * the activation and the quantisation inside gemm_fp8 as two kernels (experts.py:225-240,
+ * primus_turbo.py:2122-2129).  x is [rows, 2 f]; the other arguments are those of mxl_quantize with
+ * cols = f.  A row-wise copy must be requested (q_row / s_row not NULL). */
+int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
+                           int64_t rows, int64_t f, int64_t row_ld, int act, int fmt, int scale_mode,
+                           const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                           void* s_colT, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

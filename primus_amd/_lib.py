@@ -39,6 +39,7 @@ EXPORTS = (
     "mxl_grouped_gemm_wgrad",
     "mxl_glu_probs_fwd",
     "mxl_glu_probs_bwd",
+    "mxl_glu_probs_quantize",
 )
 
 
@@ -87,6 +88,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_glu_probs_fwd.argtypes = [vp, vp, i32, vp, i64, i64, i32, vp, vp]
         lib.mxl_glu_probs_bwd.restype = i32
         lib.mxl_glu_probs_bwd.argtypes = [vp, vp, vp, i32, vp, i64, i64, i32, vp, vp, vp]
+        lib.mxl_glu_probs_quantize.restype = i32
+        lib.mxl_glu_probs_quantize.argtypes = [vp, vp, i32, vp, i64, i64, i64, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp]
         _lib = lib
     return _lib
 

@@ -22,16 +22,7 @@ __device__ __forceinline__ void act_store16(void* d, const uint4& v) {
     const au32x4 t = {v.x, v.y, v.z, v.w};
     __builtin_nontemporal_store(t, (au32x4*)d);
 }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    v2bf h = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, h);
-}
-
-// act(g) and its derivative, fp32
-template <int ACT> __device__ __forceinline__ float act_fwd(float g) {
-    if (ACT == MXL_ACT_SILU) return g / (1.f + expf(-g));
-    return 0.5f * g * erfcf(-g * 0.70710678118654752f);   // erfc: no cancellation in the negative tail
-}
+// act(g) together with its derivative, fp32
 template <int ACT> __device__ __forceinline__ void act_both(float g, float& a, float& da) {
     if (ACT == MXL_ACT_SILU) {
         const float s = 1.f / (1.f + expf(-g));
@@ -42,11 +33,6 @@ template <int ACT> __device__ __forceinline__ void act_both(float g, float& a, f
         a = g * c;
         da = c + g * 0.39894228040143268f * expf(-0.5f * g * g);
     }
-}
-
-__device__ __forceinline__ float load_prob(const void* probs, int probs_bf16, int64_t row) {
-    if (probs_bf16) return __uint_as_float((uint32_t)((const uint16_t*)probs)[row] << 16);
-    return ((const float*)probs)[row];
 }
 
 template <int ACT>
@@ -60,16 +46,7 @@ __global__ __launch_bounds__(ATHREADS) void glu_probs_fwd_kernel(const uint16_t*
     for (int64_t c = (int64_t)threadIdx.x * 8; c < f; c += ATHREADS * 8) {
         uint4 o = make_uint4(0, 0, 0, 0);
         if (live) {
-            const uint4 g = act_load16(xg + c), u = act_load16(xg + f + c);
-            const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
-            uint32_t ow[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float lo = act_fwd<ACT>(bf16_lo(gw[k])) * bf16_lo(uw[k]) * p;
-                const float hi = act_fwd<ACT>(bf16_hi(gw[k])) * bf16_hi(uw[k]) * p;
-                ow[k] = pack_bf16(lo, hi);
-            }
-            o = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+            o = glu8<ACT>(act_load16(xg + c), act_load16(xg + f + c), p);
         }
         act_store16(yr + c, o);
     }

@@ -119,4 +119,31 @@ __device__ __forceinline__ uint32_t nonfinite2_e2m1(uint32_t pair) {
     return nonfinite1_e2m1(pair & 0xFFFFu) | (nonfinite1_e2m1(pair >> 16) << 4);
 }
 
+// ---- gated activation of the expert MLP (shared by the activation kernels and the fused
+// activation + quantisation path, so that both round identically) ----
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    v2bf h = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, h);
+}
+template <int ACT> __device__ __forceinline__ float act_fwd(float g) {
+    if (ACT == MXL_ACT_SILU) return g / (1.f + expf(-g));
+    return 0.5f * g * erfcf(-g * 0.70710678118654752f);   // erfc: no cancellation in the negative tail
+}
+__device__ __forceinline__ float load_prob(const void* probs, int probs_bf16, int64_t row) {
+    if (probs_bf16) return __uint_as_float((uint32_t)((const uint16_t*)probs)[row] << 16);
+    return ((const float*)probs)[row];
+}
+// 8 outputs act(g) * u * p from 8 gate and 8 linear bf16 values, rounded once to bf16
+template <int ACT> __device__ __forceinline__ uint4 glu8(const uint4& g, const uint4& u, float p) {
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float lo = act_fwd<ACT>(bf16_lo(gw[k])) * bf16_lo(uw[k]) * p;
+        const float hi = act_fwd<ACT>(bf16_hi(gw[k])) * bf16_hi(uw[k]) * p;
+        ow[k] = pack_bf16(lo, hi);
+    }
+    return make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 }  // namespace mxl

@@ -59,6 +59,11 @@ struct QuantArgs {
     int64_t row_ld;     // columns of the row-wise copy (>= cols; the excess is zero-filled padding)
     int64_t W;          // padded width of the transposed copy (elements)
     int64_t mat_rows;   // TWOD: rows per matrix (n); otherwise unused
+    // fused gated activation in front (ACT >= 0): x is fc1's output [rows, 2 * cols], the tensor that is
+    // quantised is act(x[:, :cols]) * x[:, cols:] * probs[row], masked rows are zero
+    const void* probs;
+    int probs_bf16;
+    const uint8_t* row_mask;
     int tiles_r, tiles_c;   // tile grid: row tiles (upper bound when grouped) x column tiles
     int super_c, n_super;   // 8x8-tile supertiles: count along the columns, total
 };
@@ -81,7 +86,7 @@ __device__ __forceinline__ bool quant_tile_of_workgroup(const QuantArgs& a, int&
     return pt < a.tiles_r && ct < a.tiles_c;
 }
 
-template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD>
+template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     constexpr bool FP4 = (FMT == kFmtE2M1);
     constexpr int TPITCH = FP4 ? (QT / 2 + 16) : (QT + 16);  // bytes per LDS row of the transposed tile
@@ -138,7 +143,18 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     for (int it = 0; it < 8; ++it) {
         const int r = 32 * w + 8 * rg + it;
         d[it] = make_uint4(0, 0, 0, 0);
-        if (col_ok && r < rows_valid) d[it] = load16_streaming(a.x + (src_row0 + r) * a.cols + col);
+        if (col_ok && r < rows_valid) {
+            if (ACT < 0) {
+                d[it] = load16_streaming(a.x + (src_row0 + r) * a.cols + col);
+            } else {
+                const int64_t row = src_row0 + r;
+                if (a.row_mask == nullptr || a.row_mask[row] != 0) {
+                    const uint16_t* xr = a.x + row * 2 * a.cols + col;
+                    d[it] = glu8<(ACT < 0 ? 0 : ACT)>(load16_streaming(xr), load16_streaming(xr + a.cols),
+                                                      load_prob(a.probs, a.probs_bf16, row));
+                }
+            }
+        }
     }
 
     // ---- block maxima ----
@@ -350,7 +366,7 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t* q, const
 // ---------------------------------------------------------------------------
 // host-side dispatch
 // ---------------------------------------------------------------------------
-template <int FMT, int SMODE, bool TWOD>
+template <int FMT, int SMODE, bool TWOD, int ACT = -1>
 static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
     const int64_t super_r = (tiles_r + QSUPER - 1) / QSUPER, super_c = (tiles_c + QSUPER - 1) / QSUPER;
     const int64_t n_super = super_r * super_c;
@@ -363,18 +379,20 @@ static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStrea
     const dim3 grid((unsigned)wgs);
     const bool row = a.q_row != nullptr, col = a.q_colT != nullptr;
     if (row && col)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD>), grid, dim3(QTHREADS), 0, st, a);
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD, ACT>), grid, dim3(QTHREADS), 0, st, a);
     else if (row)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD>), grid, dim3(QTHREADS), 0, st, a);
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD, ACT>), grid, dim3(QTHREADS), 0, st, a);
+    else if (ACT < 0)
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD, -1>), grid, dim3(QTHREADS), 0, st, a);
     else
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD>), grid, dim3(QTHREADS), 0, st, a);
+        return MXL_EINVAL;   // the fused activation always feeds a forward GEMM: a row-wise copy is part of it
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
-template <bool TWOD>
+template <bool TWOD, int ACT = -1>
 static int dispatch_quant(int fmt, int smode, QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
 #define MXL_Q(F, S) \
-    if (fmt == F && smode == S) return launch_quant<F, S, TWOD>(a, tiles_r, tiles_c, st);
+    if (fmt == F && smode == S) return launch_quant<F, S, TWOD, ACT>(a, tiles_r, tiles_c, st);
     MXL_Q(MXL_FMT_E4M3, MXL_SCALE_OCP_FLOOR)
     MXL_Q(MXL_FMT_E4M3, MXL_SCALE_RCEIL)
     MXL_Q(MXL_FMT_E4M3, MXL_SCALE_EVEN)
@@ -394,9 +412,9 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
     return (total_rows + (int64_t)(MXL_SEG_ALIGN - 1) * num_groups) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
 }
 
-extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
-                            const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                            void* s_colT, void* stream) {
+static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
+                       const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
+                       int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream) {
     if (row_ld == 0) row_ld = cols;
     if (row_ld < cols || row_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((!x_bf16 && rows > 0) || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
@@ -416,10 +434,33 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
     a.row_ld = row_ld;
     a.W = mxl_padded_width(rows, num_groups);
     a.mat_rows = 0;
+    a.probs = probs;
+    a.probs_bf16 = probs_dtype == MXL_PROBS_BF16;
+    a.row_mask = row_mask;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
     const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
     if (gx == 0) return MXL_OK;
+    if (act == MXL_ACT_SILU) return dispatch_quant<false, MXL_ACT_SILU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
+    if (act == MXL_ACT_GELU) return dispatch_quant<false, MXL_ACT_GELU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     return dispatch_quant<false>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
+}
+
+extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
+                            const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                            void* s_colT, void* stream) {
+    return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
+                       -1, nullptr, MXL_PROBS_F32, nullptr, stream);
+}
+
+extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
+                                      int64_t rows, int64_t f, int64_t row_ld, int act, int fmt, int scale_mode,
+                                      const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                                      void* s_colT, void* stream) {
+    if (act != MXL_ACT_SILU && act != MXL_ACT_GELU) return MXL_EINVAL;
+    if (probs_dtype != MXL_PROBS_F32 && probs_dtype != MXL_PROBS_BF16) return MXL_EINVAL;
+    if (rows > 0 && !probs) return MXL_EINVAL;
+    return quantize_1d(x_bf16, rows, f, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT, act,
+                       probs, probs_dtype, row_mask, stream);
 }
 
 extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
@@ -445,6 +486,9 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
     a.row_ld = k_ld;
     a.W = n_ld;  // transposed copy of each matrix is [k, n_ld]
     a.mat_rows = n;
+    a.probs = nullptr;
+    a.probs_bf16 = 0;
+    a.row_mask = nullptr;
     const int64_t gx = batch * ((n + QT - 1) / QT);
     const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
     return dispatch_quant<true>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);

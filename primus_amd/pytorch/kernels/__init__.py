@@ -382,6 +382,43 @@ def glu_with_probs_bwd_impl(dy, x, probs, row_mask, activation: str):
     return dx, dp
 
 
+def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *,
+                                 colwise: bool = False, group_lens: Optional[torch.Tensor] = None, pad_to: int = 1):
+    """``quantize_mx_impl(glu_with_probs_fwd_impl(x, ...))`` in one pass over ``x [tokens, 2F]``, the
+    activated tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
+    act, pd, row_mask = _glu_args(x, probs, row_mask, activation)
+    _require_cuda(group_lens)
+    rows, f = x.shape[0], x.shape[1] // 2
+    if f % BLOCK != 0:
+        raise ValueError(f"the quantised dim ({f}) must be a multiple of {BLOCK}")
+    if rows == 0:  # nothing to activate: only the padding of the transposed copy is left to write
+        return quantize_mx_impl(x[:, :f].contiguous(), fmt, scale_mode, rowwise=True, colwise=colwise,
+                                group_lens=group_lens, pad_to=pad_to)
+    G = _check_group_lens(group_lens, x.device)
+    per = _per_byte(fmt)
+    dev = x.device
+    row_ld = _round_up(f, pad_to)
+    q_row = torch.empty((rows, row_ld // per), dtype=torch.uint8, device=dev)
+    s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+    q_col = s_col = None
+    if colwise:
+        W = padded_width(rows, G)
+        q_col = torch.empty((f, W // per), dtype=torch.uint8, device=dev)
+        s_col = torch.empty((f, W // BLOCK), dtype=torch.uint8, device=dev)
+    if rows > 0 or (q_col is not None and q_col.numel() > 0):
+        row_ok = rows > 0
+        with _hooked("glu_probs_quantize", rows=rows, cols=f, fmt=fmt, rowwise=True, colwise=colwise):
+            rc = _lib.load().mxl_glu_probs_quantize(
+                _ptr(x) if row_ok else None, _ptr(probs), pd, _ptr(row_mask), rows, f, row_ld, act, fmt, scale_mode,
+                _ptr(group_lens), G, _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col),
+                _ptr(s_col), _stream(),
+            )
+        _lib.check(rc, "mxl_glu_probs_quantize")
+    cd = _code_dtype(fmt)
+    v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
+    return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0)
+
+
 # --------------------------------------------------------------------------
 # reference-named low-level entry points (MX granularity only)
 # --------------------------------------------------------------------------

@@ -48,7 +48,8 @@ class MXLinearError(RuntimeError):
 
 
 def lib_path() -> str:
-    return _build.LIB_PATH
+    """The in-tree library, or the one ``MXL_LIBRARY`` names (an alternative build of the same ABI)."""
+    return os.environ.get("MXL_LIBRARY") or _build.LIB_PATH
 
 
 def load() -> ctypes.CDLL:

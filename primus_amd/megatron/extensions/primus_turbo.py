@@ -467,12 +467,24 @@ class _LowPrecisionGemm:
         return x, pair, fuse_pattern
 
     def _gemm(self, x: torch.Tensor, weight: torch.Tensor, is_first_microbatch: bool,
-              group_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+              group_lens: Optional[torch.Tensor] = None, glu: Optional[Tuple] = None) -> torch.Tensor:
+        """``glu = (probs, row_mask, activation)``: ``x`` is the previous linear's output and the gated
+        activation is applied on the way into this GEMM (grouped only)."""
         manager = PrimusTurboLowPrecisionGlobalStateManager
         grouped = group_lens is not None
         one_microbatch = runtime.get_num_microbatches() == 1
+        assert glu is None or grouped, "the activation prologue exists for the grouped (expert) linears only"
 
         def run(op_dense, op_grouped, a, b, fuse_pattern, **kw):
+            if glu is not None:
+                probs, row_mask, activation = glu
+                if op_grouped is ops.grouped_gemm:     # outside a low-precision autocast: two plain operators
+                    act = ops.swiglu_with_probs if activation == "silu" else ops.geglu_with_probs
+                    return op_grouped(act(a, probs, row_mask), b, group_lens, trans_b=True,
+                                      fuse_bgrad_accum_pattern=fuse_pattern)
+                fused = ops.glu_grouped_gemm_fp8 if op_grouped is ops.grouped_gemm_fp8 else ops.glu_grouped_gemm_fp4
+                return fused(a, probs, b, group_lens, activation=activation, row_mask=row_mask, trans_b=True,
+                             fuse_bgrad_accum_pattern=fuse_pattern, **kw)
             if grouped:
                 return op_grouped(a, b, group_lens, trans_b=True, fuse_bgrad_accum_pattern=fuse_pattern, **kw)
             return op_dense(a, b, trans_a=False, trans_b=True, out_dtype=None,
@@ -713,19 +725,23 @@ class PrimusTurboGroupedLinear(_LowPrecisionGemm, torch.nn.Module):
         self._ensure_weight_views()
         return super()._load_from_state_dict(*args, **kwargs)
 
-    def forward(self, x: torch.Tensor, m_splits: torch.Tensor):
+    def forward(self, x: torch.Tensor, m_splits: torch.Tensor, glu: Optional[Tuple] = None):
+        """``glu = (probs [tokens], row_mask or None, "silu" | "gelu")`` makes this linear consume the
+        previous one's output ``[tokens, 2 * in_features]`` through the gated activation (no
+        counterpart in the reference, which runs the activation as its own kernel)."""
         first = self.is_first_microbatch
         with _get_fp8_autocast_for_quant_params(self.te_quant_params, self.training):
-            out = self.forward_internal(x, m_splits, first)
+            out = self.forward_internal(x, m_splits, first, glu=glu)
         self.is_first_microbatch = False
         return out
 
-    def forward_internal(self, x: torch.Tensor, m_splits: torch.Tensor, is_first_microbatch: bool = False):
+    def forward_internal(self, x: torch.Tensor, m_splits: torch.Tensor, is_first_microbatch: bool = False,
+                         glu: Optional[Tuple] = None):
         if not torch.is_tensor(m_splits):
             m_splits = torch.as_tensor(m_splits, dtype=torch.int64)
         if m_splits.device != x.device:
             m_splits = m_splits.to(x.device)  # the op consumes the lens on the device (no host read-back)
-        return self._gemm(x, self.weights, is_first_microbatch, group_lens=m_splits), None
+        return self._gemm(x, self.weights, is_first_microbatch, group_lens=m_splits, glu=glu), None
 
 
 class PrimusTurboColumnParallelGroupedLinear(PrimusTurboGroupedLinear):

@@ -18,6 +18,7 @@ import torch.nn.functional as F
 
 from .. import runtime
 from ..extensions.primus_turbo import (
+    PrimusTurboGroupedLinear,
     PrimusTurboColumnParallelGroupedLinear,
     PrimusTurboRowParallelGroupedLinear,
 )
@@ -69,6 +70,9 @@ class PrimusGroupedMLP(torch.nn.Module):
         self.use_turbo_fused_act_with_probs = bool(getattr(args, "use_turbo_fused_act_with_probs", False))
         self.moe_router_padding_for_quantization = bool(getattr(args, "moe_router_padding_for_quantization", False))
         self.turbo_grouped_gemm_without_padding = bool(getattr(args, "turbo_grouped_gemm_without_padding", False))
+        # with the fused activation, fc2 can take fc1's output directly and apply the activation inside its
+        # quantiser (same values; the activated tensor is never stored).  Not a reference flag: default on.
+        self.fuse_act_into_fc2 = bool(getattr(args, "turbo_fuse_act_into_fc2_quantize", True))
 
     # -- padding policy (experts.py:54-60) ------------------------------------
     def _use_explicit_quantization_padding(self) -> bool:
@@ -131,17 +135,30 @@ class PrimusGroupedMLP(torch.nn.Module):
         assert not getattr(self.config, "activation_func_fp8_input_store", False), (
             "`use_turbo_fused_act_with_probs` does not support activation_func_fp8_input_store."
         )
-        if self.activation_func == F.silu and self.gated:
-            activation = "silu"
-        elif self.activation_func == F.gelu and self.gated:
-            activation = "gelu"
-        else:
-            raise ValueError(
-                "Only support fusion of swiglu and gelu in PrimusGroupedMLP when `use_turbo_fused_act_with_probs` is True."
-            )
+        activation = self._fused_activation_name()
         # forward() hands the probabilities over as [tokens, 1]; the kernel takes them 1-D
         probs_1d = permuted_probs.squeeze(-1) if permuted_probs.dim() == 2 else permuted_probs
         return fused_bias_act_with_probs(intermediate, bias, probs_1d, tokens_per_experts, activation)
+
+    def _fused_activation_name(self) -> str:
+        if self.activation_func == F.silu and self.gated:
+            return "silu"
+        if self.activation_func == F.gelu and self.gated:
+            return "gelu"
+        raise ValueError(
+            "Only support fusion of swiglu and gelu in PrimusGroupedMLP when `use_turbo_fused_act_with_probs` is True."
+        )
+
+    def _can_fuse_act_into_fc2(self, bias) -> bool:
+        """fc2 applies the activation in its own quantiser: needs the fused-activation flag, no fc1
+        bias, none of the options the fused kernel rejects, and an fc2 that takes the prologue."""
+        cfg = self.config
+        return (self.use_turbo_fused_act_with_probs and self.fuse_act_into_fc2 and bias is None and self.gated
+                and self.activation_func in (F.silu, F.gelu)
+                and getattr(cfg, "activation_func_clamp_value", None) is None
+                and getattr(cfg, "glu_linear_offset", 0.0) == 0.0
+                and not getattr(cfg, "activation_func_fp8_input_store", False)
+                and isinstance(self.linear_fc2, PrimusTurboGroupedLinear))
 
     def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor,
                 permuted_probs: torch.Tensor) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
@@ -162,8 +179,15 @@ class PrimusGroupedMLP(torch.nn.Module):
             permuted_probs = torch.ones_like(permuted_probs)
 
         fc1_output, bias1 = self.linear_fc1(permuted_local_hidden_states, tokens_per_expert)
-        act = self.bias_act_func_with_mask(fc1_output, bias1, permuted_probs, tokens_per_expert)
-        output, _ = self.linear_fc2(act, tokens_per_expert)
+        if self._can_fuse_act_into_fc2(bias1):
+            from ...pytorch import ops
+
+            row_mask = ops.tokens_per_expert_to_mask(tokens_per_expert, fc1_output.shape[0])
+            output, _ = self.linear_fc2(fc1_output, tokens_per_expert,
+                                        glu=(permuted_probs.squeeze(-1), row_mask, self._fused_activation_name()))
+        else:
+            act = self.bias_act_func_with_mask(fc1_output, bias1, permuted_probs, tokens_per_expert)
+            output, _ = self.linear_fc2(act, tokens_per_expert)
         if pad:
             output = self.quantization_unpadding(output, actual)
         return output, None

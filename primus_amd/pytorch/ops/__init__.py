@@ -37,7 +37,8 @@ from ..core.low_precision import (
 from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
 __all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
-           "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask"]
+           "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask", "glu_grouped_gemm_fp8",
+           "glu_grouped_gemm_fp4"]
 
 # dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
 # kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
@@ -62,19 +63,30 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
 
 
 class _MXLinearFunction(torch.autograd.Function):
-    """Y = X . W^T on MX operands, dense (``group_lens is None``) or grouped."""
+    """Y = X . W^T on MX operands, dense (``group_lens is None``) or grouped.
+
+    With ``activation`` set, ``a`` is the previous linear's output ``[tokens, 2F]`` and
+    X = act(a[:, :F]) * a[:, F:] * probs (masked rows zero) is formed inside the quantiser: X itself
+    never reaches memory, in the forward or in the backward."""
 
     @staticmethod
-    def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode):
-        need_dgrad = a.requires_grad
+    def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode, probs=None, row_mask=None, activation=None):
+        glu = activation is not None
+        need_dgrad = a.requires_grad or (glu and probs.requires_grad)
         need_wgrad = b.requires_grad
         grouped = group_lens is not None
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
         # (row-wise copies are padded to the GEMM's K granularity, like the reference pads its
         # MXFP4 operands to 128: primus_turbo_mxfp4_local.py:119-124)
-        a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
-            a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
-        )
+        if glu:
+            a_row, a_rs, a_col, a_cs = K.glu_with_probs_quantize_impl(
+                a, probs, row_mask, activation, act_fmt, scale_mode, colwise=need_wgrad, group_lens=group_lens,
+                pad_to=K.GEMM_K_ALIGN,
+            )
+        else:
+            a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
+                a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
+            )
         if isinstance(b, QuantizedTensor):
             # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
             if b.axis != -1:
@@ -95,13 +107,17 @@ class _MXLinearFunction(torch.autograd.Function):
             y = K.grouped_gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, group_lens)
         else:
             y = K.gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs)
-        ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens)
+        if glu and need_dgrad:
+            ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens, a, probs, row_mask)
+        else:
+            ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens)
         ctx.cfg = (act_fmt, scale_mode, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape))
+        ctx.activation = activation
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        a_col, a_cs, w_col, w_cs, group_lens = ctx.saved_tensors
+        a_col, a_cs, w_col, w_cs, group_lens = ctx.saved_tensors[:5]
         act_fmt, scale_mode, total_m, need_dgrad, need_wgrad, w_shape = ctx.cfg
         grouped = group_lens is not None
         dy = dy.contiguous()
@@ -131,7 +147,13 @@ class _MXLinearFunction(torch.autograd.Function):
                 main.wait_stream(side)
             else:
                 grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
-        return grad_a, grad_b, None, None, None, None, None
+        grad_p = None
+        if ctx.activation is not None and need_dgrad:
+            # grad_a so far is dL/dX; take it through the activation to fc1's output and the probabilities
+            pre, probs, row_mask = ctx.saved_tensors[5:8]
+            grad_a, grad_p = K.glu_with_probs_bwd_impl(grad_a, pre, probs, row_mask, ctx.activation)
+            grad_p = grad_p.to(probs.dtype)
+        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None
 
 
 def _formats(config, fp4: bool):
@@ -155,7 +177,7 @@ def _formats(config, fp4: bool):
     return f, f
 
 
-def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4):
+def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4, glu=None):
     if trans_a or not trans_b:
         raise ValueError("the MX linear path is NT only: trans_a=False, trans_b=True (primus_turbo.py:1095-1103)")
     if fuse_bgrad_accum_pattern is not None:
@@ -185,11 +207,20 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
     want_dims = 2 if group_lens is None else 3
     if b.dim() != want_dims:
         raise ValueError(f"weights must have {want_dims} dims ([N, K] dense, [G, N, K] grouped)")
-    if b.shape[-1] != a.shape[-1]:
-        raise ValueError(f"contraction dims differ: activations K={a.shape[-1]}, weights K={b.shape[-1]}")
+    k_act = a.shape[-1] // 2 if glu is not None else a.shape[-1]
+    if b.shape[-1] != k_act:
+        raise ValueError(f"contraction dims differ: activations K={k_act}, weights K={b.shape[-1]}")
     if group_lens is not None and group_lens.numel() != b.shape[0]:
         raise ValueError("group_lens must have one entry per expert weight")
-    return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value)
+    if glu is None:
+        return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value)
+    probs, row_mask, activation = glu
+    if activation not in ("silu", "gelu"):
+        raise ValueError(f"activation must be 'silu' or 'gelu', got {activation!r}")
+    if probs.dim() != 1 or probs.shape[0] != a.shape[0]:
+        raise ValueError("probs must be 1-D with one entry per row of the activations")
+    return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
+                                   probs.contiguous(), row_mask, activation)
 
 
 def gemm_fp8(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
@@ -224,6 +255,27 @@ def grouped_gemm_fp8(a, b, group_lens: torch.Tensor, trans_b: bool = True,
 def grouped_gemm_fp4(a, b, group_lens: torch.Tensor, trans_b: bool = True,
                      config: Optional[Float4QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
     return _run(a, b, _lens(group_lens), False, trans_b, None, config, fuse_bgrad_accum_pattern, fp4=True)
+
+
+def glu_grouped_gemm_fp8(x, probs, b, group_lens: torch.Tensor, activation: str = "silu",
+                         row_mask: Optional[torch.Tensor] = None, trans_b: bool = True,
+                         config: Optional[Float8QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
+    """fc2 of the expert MLP with the gated activation folded into its quantiser:
+    ``grouped_gemm_fp8(swiglu_with_probs(x, probs, row_mask), b, group_lens)`` (``geglu`` for
+    ``activation="gelu"``) for ``x [tokens, 2F]`` = fc1's output, same values bit for bit, forward and
+    backward, without the activated tensor ``[tokens, F]`` being written or re-read.  Differentiable
+    in ``x``, ``probs`` and ``b``.  The reference runs the two operators separately
+    (primus/backends/megatron/core/transformer/experts.py:120-165, then :2122-2129 of
+    extensions/primus_turbo.py)."""
+    return _run(x, b, _lens(group_lens), False, trans_b, None, config, fuse_bgrad_accum_pattern, fp4=False,
+                glu=(probs, row_mask, activation))
+
+
+def glu_grouped_gemm_fp4(x, probs, b, group_lens: torch.Tensor, activation: str = "silu",
+                         row_mask: Optional[torch.Tensor] = None, trans_b: bool = True,
+                         config: Optional[Float4QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
+    return _run(x, b, _lens(group_lens), False, trans_b, None, config, fuse_bgrad_accum_pattern, fp4=True,
+                glu=(probs, row_mask, activation))
 
 
 # ---------------------------------------------------------------------------

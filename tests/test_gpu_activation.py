@@ -153,3 +153,52 @@ def test_fused_activation_quantize_equals_two_kernels(gpu, activation, fmt, lens
         yq, ys = o.quantize_mx_rowwise(y.cpu(), fmt)
         assert np.array_equal(got[0].view(torch.uint8).cpu().numpy()[:, : f // per], yq)
         assert np.array_equal(got[1].view(torch.uint8).cpu().numpy()[:, : f // 32], ys)
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu"])
+@pytest.mark.parametrize("fp4", [False, True])
+@pytest.mark.parametrize("lens,f,n", [([33, 0, 130, 1, 92], 160, 96), ([300, 212], 512, 256)])
+def test_glu_grouped_gemm_equals_activation_then_grouped_gemm(gpu, activation, fp4, lens, f, n):
+    """ops.glu_grouped_gemm_fp8 / _fp4 give exactly what the activation operator followed by the
+    grouped GEMM operator gives -- output, and the gradients of fc1's output, the probabilities and
+    the weight -- since the fused quantiser writes the same bytes and the backward runs the same kernels."""
+    import primus_amd.pytorch as pt
+    from primus_amd.pytorch.core import Float4QuantConfig, Float8QuantConfig, Format, ScaleDtype, ScalingGranularity
+
+    if fp4:
+        cfg = Float4QuantConfig(activation_format=Format.E4M3)
+        fused_op, plain_op = pt.ops.glu_grouped_gemm_fp4, pt.ops.grouped_gemm_fp4
+    else:
+        cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE,
+                                scale_dtype=ScaleDtype.E8M0, block_size=32)
+        fused_op, plain_op = pt.ops.glu_grouped_gemm_fp8, pt.ops.grouped_gemm_fp8
+    act_op = pt.ops.swiglu_with_probs if activation == "silu" else pt.ops.geglu_with_probs
+    rows, G = sum(lens), len(lens)
+    g = torch.Generator().manual_seed(rows + f + n)
+    h = (torch.randn(rows, 2 * f, generator=g) * 1.5).bfloat16().to(gpu)
+    p = torch.rand(rows, generator=g).to(gpu)
+    w = (torch.randn(G, n, f, generator=g) * 0.05).bfloat16().to(gpu)
+    dy = torch.randn(rows, n, generator=g).bfloat16().to(gpu)
+    mask = (torch.rand(rows, generator=g) > 0.1).to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+
+    outs = []
+    for fused in (True, False):
+        hh, pp, ww = h.clone().requires_grad_(), p.clone().requires_grad_(), w.clone().requires_grad_()
+        if fused:
+            y = fused_op(hh, pp, ww, gl, activation=activation, row_mask=mask, config=cfg)
+        else:
+            y = plain_op(act_op(hh, pp, mask), ww, gl, trans_b=True, config=cfg)
+        y.backward(dy)
+        outs.append((y.detach(), hh.grad, pp.grad, ww.grad))
+    for a, b in zip(*outs):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        assert torch.equal(a, b)
+    # only the probabilities need a gradient: dgrad still runs, fc1's output gets none
+    hh, pp = h.clone(), p.clone().requires_grad_()
+    fused_op(hh, pp, w, gl, activation=activation, row_mask=mask, config=cfg).backward(dy)
+    assert torch.equal(pp.grad, outs[0][2])
+    with pytest.raises(ValueError):
+        fused_op(h, p, w[:, :, : f // 2].contiguous(), gl, activation=activation, config=cfg)   # K mismatch
+    with pytest.raises(ValueError):
+        fused_op(h, p, w, gl, activation="relu", config=cfg)

@@ -198,6 +198,61 @@ def test_grouped_mlp_mxfp8_close_to_bf16(mg, gpu):
         assert _cos(a, b) >= 0.99, (name, _cos(a, b))  # the reference's bar is 0.90
 
 
+@pytest.mark.parametrize("fp4", [False, True])
+def test_grouped_mlp_fc2_takes_the_activation(mg, gpu, fp4):
+    """With the fused activation, fc2 consumes fc1's output directly (activation inside its
+    quantiser): forward and every gradient equal those of the separate activation kernel bit for
+    bit, and no activation launch is left in the forward."""
+    from contextlib import contextmanager
+
+    from primus_amd.megatron import runtime
+    from primus_amd.pytorch import kernels as K
+
+    pt = mg
+    common = dict(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                  turbo_grouped_gemm_without_padding=True, use_turbo_fused_act_with_probs=True)
+    torch.manual_seed(5)
+    runtime.set_args(**common)
+    a = _mlp(pt, gpu, 4, 256, 384)
+    runtime.set_args(turbo_fuse_act_into_fc2_quantize=False, **common)
+    b = _mlp(pt, gpu, 4, 256, 384)
+    b.load_state_dict(a.state_dict())
+    assert a.fuse_act_into_fc2 and not b.fuse_act_into_fc2
+    lens = torch.tensor([100, 0, 37, 55], device=gpu)
+    x = torch.randn(192, 256, device=gpu).bfloat16()
+    probs = torch.rand(192, device=gpu)
+    dy = torch.randn(192, 256, device=gpu).bfloat16()
+    launches = []
+
+    @contextmanager
+    def hook(name, info):
+        launches.append(name)
+        yield
+
+    res = []
+    for mod in (a, b):
+        del launches[:]
+        xx, pp = x.clone().requires_grad_(), probs.clone().requires_grad_()
+        K.set_launch_hook(hook)
+        try:
+            if fp4:
+                ctx = pt.primus_turbo_fp4_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp4(pt))
+            else:
+                ctx = pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt))
+            with ctx:
+                y, _ = mod(xx, lens, pp)
+            y.backward(dy)
+        finally:
+            K.set_launch_hook(None)
+        res.append((y.detach(), xx.grad, pp.grad, mod.linear_fc1.weights.grad, mod.linear_fc2.weights.grad,
+                    list(launches)))
+    for u, v in zip(res[0][:5], res[1][:5]):
+        assert u is not None and torch.equal(u, v)
+    assert "glu_probs_quantize" in res[0][5] and "glu_probs_fwd" not in res[0][5]
+    assert "glu_probs_fwd" in res[1][5] and "glu_probs_quantize" not in res[1][5]
+    assert len(res[0][5]) == len(res[1][5]) - 1          # one launch fewer per step
+
+
 def test_grouped_mlp_explicit_padding_gives_the_same_forward(mg, gpu):
     """Padding rows are zeros and row-wise blocks never mix rows, so the padded
     and the ragged path quantise every real row identically."""

@@ -90,6 +90,19 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
                  const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                  void* s_colT, void* stream);
 
+/* mxl_quantize with STOCHASTIC ROUNDING of the codes (fmt must be MXL_FMT_E2M1): the MXFP4 recipe's
+ * gradient quantisation, rowwise_use_sr / colwise_use_sr of quantize_mxfp4_dual
+ * (primus_turbo_mxfp4_local.py:272-288; config flag mxfp4_gradient_stochastic_rounding,
+ * primus/configs/modules/megatron/primus_turbo.yaml:21-24).  Scales are those of mxl_quantize; each
+ * element becomes one of its two neighbours on the E2M1 grid, the upper one with probability equal to
+ * its fractional position between them (so the dequantised value is unbiased), saturating at +-6.
+ * The random bits are a counter-based hash of `seed` and the element's position in the output, hence
+ * reproducible and independent of the launch geometry; the row-wise and the transposed copy draw
+ * from different streams.  All other arguments as for mxl_quantize. */
+int mxl_quantize_sr(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
+                    const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                    void* s_colT, uint64_t seed, void* stream);
+
 /* 2-D (32x32 tile) MX quantisation of `batch` independent weight matrices
  * w[batch, n, k] (weights use ScalingRecipe(use_2d_block=True):
  * primus_turbo.py:313-317; grid definition weight_deosc.py:29-33,136-174).

@@ -52,6 +52,17 @@ Parity status
   once (as here, like Megatron's fused weighted SwiGLU) or after every step,
   and which GELU flavour ``geglu_with_probs`` uses, is **parity unpinned**.
 
+* ``cast_e2m1_sr`` / ``quantize_mx_rowwise_sr`` / ``quantize_mx_colwise_segmented_sr``
+  (stochastic rounding of MXFP4 gradients, rowwise_use_sr / colwise_use_sr at
+  primus_turbo_mxfp4_local.py:272-288): written as a search in the E2M1 value
+  table; pinned by enumeration of all 2^16 random values per input (result is
+  one of the two neighbours, the upper one for exactly ceil(frac * 2^16) of
+  them, so the mean is within 2^-16 of a grid step of the input; grid points
+  never move; saturation at 6) and by uniformity checks of the counter hash.
+  Primus-Turbo's random stream cannot be reproduced (package absent, and a
+  different generator by construction): which elements round up is **parity
+  unpinned**; only the distribution is comparable.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -374,6 +385,98 @@ def quantize_mx_colwise_segmented(x, group_lens, fmt: int = FMT_E4M3, scale_mode
     for g in range(len(lens)):
         xp[poffs[g] : poffs[g] + lens[g]] = xb[offs[g] : offs[g + 1]]
     return quantize_mx_colwise(xp, fmt, scale_mode)
+
+
+# --------------------------------------------------------------------------
+# stochastic rounding to E2M1 (gradients of the MXFP4 recipe)
+# --------------------------------------------------------------------------
+_E2M1_GRID = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=np.float64)
+
+
+def _sr_mix(x: np.ndarray) -> np.ndarray:
+    """32-bit integer finaliser (xor-shift / odd-multiply rounds), a bijection on uint32."""
+    x = x.astype(np.uint64)
+    m = np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7FEB352D)) & m
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846CA68B)) & m
+    x ^= x >> np.uint64(16)
+    return x
+
+
+def sr_word(counter: np.ndarray, seed: int, stream: int) -> np.ndarray:
+    """32 random bits per 64-bit counter value: two rounds of the finaliser over the
+    counter, the 64-bit seed and the stream id.  Returned as uint32."""
+    c = np.asarray(counter, dtype=np.uint64)
+    m = np.uint64(0xFFFFFFFF)
+    seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+    h = _sr_mix((c & m) ^ np.uint64(seed & 0xFFFFFFFF))
+    t = (h + ((c >> np.uint64(32)) * np.uint64(0x9E3779B9)) + np.uint64(seed >> 32)
+         + np.uint64((int(stream) * 0x85EBCA6B) & 0xFFFFFFFF)) & m
+    return _sr_mix(t).astype(np.uint32)
+
+
+def cast_e2m1_sr(v: np.ndarray, rnd16: np.ndarray) -> np.ndarray:
+    """float32 (already divided by the block scale, finite) -> E2M1 code with stochastic rounding.
+
+    |v| lies between two neighbouring values lo <= |v| < hi of the E2M1 table.  With
+    T = floor((|v| - lo) / (hi - lo) * 2^22) the result is hi when T + 64 * rnd16 >= 2^22 and lo
+    otherwise, i.e. hi with probability ceil(T / 64) / 2^16 over a uniform 16-bit ``rnd16``;
+    values at or above 6 give 6.  The sign bit is the input's."""
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    sign = ((v.view(np.uint32) >> np.uint32(28)) & np.uint32(0x8)).astype(np.uint8)
+    w = np.abs(v).astype(np.float64)
+    idx = np.searchsorted(_E2M1_GRID, w, side="right") - 1          # largest table entry <= w
+    idx = np.clip(idx, 0, 7)
+    lo = _E2M1_GRID[idx]
+    hi = _E2M1_GRID[np.minimum(idx + 1, 7)]
+    step = np.where(idx < 7, hi - lo, 1.0)
+    frac = np.where(idx < 7, (w - lo) / step, 0.0)
+    T = np.floor(frac * float(1 << 22)).astype(np.int64)
+    up = (T + (rnd16.astype(np.int64) << 6)) >= (1 << 22)
+    code = np.minimum(idx + up.astype(np.int64), 7)
+    return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def quantize_mx_rowwise_sr(x, seed: int, scale_mode: int = SCALE_OCP_FLOOR, stream: int = 0):
+    """``quantize_mx_rowwise(x, FMT_E2M1)`` with stochastically rounded codes: same scales; the
+    random word of the element pair (row r, columns 2j and 2j+1) is
+    ``sr_word(r * K/2 + j, seed, stream)``, low half for the even column."""
+    xb = to_bf16_bits(x)
+    assert xb.ndim == 2
+    R, K = xb.shape
+    assert K % BLOCK == 0
+    blocks = xb.reshape(R, K // BLOCK, BLOCK)
+    byte = _block_scale_bytes(blocks, FMT_E2M1, scale_mode)
+    byte_el = np.broadcast_to(byte[..., None], blocks.shape).reshape(R, K)
+    xf = bf16_bits_to_f32(xb)
+    with np.errstate(invalid="ignore", over="ignore"):
+        v = (xf * inv_scale_f32(byte_el)).astype(np.float32)
+    counter = (np.arange(R, dtype=np.uint64)[:, None] * np.uint64(K // 2) + np.arange(K // 2, dtype=np.uint64)[None, :])
+    words = sr_word(counter, seed, stream)                               # [R, K/2]
+    rnd16 = np.stack([words & np.uint32(0xFFFF), words >> np.uint32(16)], axis=-1).reshape(R, K)
+    finite_block = byte_el != 255
+    code = cast_e2m1_sr(np.where(finite_block, v, np.float32(0)), rnd16)
+    # blocks holding NaN / Inf (scale byte 255) are coded as by the round-to-nearest path
+    rne = _cast_scaled(xb, byte_el, FMT_E2M1)
+    code = np.where(finite_block, code, rne).astype(np.uint8)
+    return pack_fp4(code), byte
+
+
+def quantize_mx_colwise_segmented_sr(x, group_lens, seed: int, scale_mode: int = SCALE_OCP_FLOOR):
+    """``quantize_mx_colwise_segmented(x, group_lens, FMT_E2M1)`` with stochastic rounding: the
+    row-wise routine applied to the transposed, segment-padded tensor ``[C, W]`` with stream 1."""
+    xb = to_bf16_bits(x)
+    lens = np.asarray(group_lens, dtype=np.int64)
+    total, C = xb.shape
+    assert lens.sum() == total
+    offs, poffs = segment_layout(lens)
+    W = padded_width(total, len(lens))
+    xp = np.zeros((W, C), dtype=np.uint16)
+    for g in range(len(lens)):
+        xp[poffs[g] : poffs[g] + lens[g]] = xb[offs[g] : offs[g + 1]]
+    return quantize_mx_rowwise_sr(np.ascontiguousarray(xp.T), seed, scale_mode, stream=1)
 
 
 # --------------------------------------------------------------------------

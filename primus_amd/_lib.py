@@ -32,6 +32,7 @@ EXPORTS = (
     "mxl_error_string",
     "mxl_padded_width",
     "mxl_quantize",
+    "mxl_quantize_sr",
     "mxl_quantize_weight_2d",
     "mxl_dequantize",
     "mxl_gemm_nt",
@@ -75,6 +76,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_padded_width.argtypes = [i64, i32]
         lib.mxl_quantize.restype = i32
         lib.mxl_quantize.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, vp]
+        lib.mxl_quantize_sr.restype = i32
+        lib.mxl_quantize_sr.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, ctypes.c_uint64, vp]
         lib.mxl_quantize_weight_2d.restype = i32
         lib.mxl_quantize_weight_2d.argtypes = [vp, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         lib.mxl_dequantize.restype = i32

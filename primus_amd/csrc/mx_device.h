@@ -119,6 +119,44 @@ __device__ __forceinline__ uint32_t nonfinite2_e2m1(uint32_t pair) {
     return nonfinite1_e2m1(pair & 0xFFFFu) | (nonfinite1_e2m1(pair >> 16) << 4);
 }
 
+// ---- stochastic rounding to E2M1 (gradients of the MXFP4 recipe: rowwise_use_sr / colwise_use_sr of
+// quantize_mxfp4_dual, primus/backends/megatron/core/extensions/primus_turbo_mxfp4_local.py:272-288).
+// Integer arithmetic throughout so that a CPU restatement reproduces every code:
+//   w = |x| * 2^(127 - scale byte)                         (exact: power-of-two scaling of a bf16)
+//   w >= 1: the fp32 pattern of w plus a random integer below 2^22, cut after one mantissa bit
+//           (round up with probability = the dropped fraction), saturating at 6;
+//   w <  1: floor(w * 2^23) plus the same random integer, cut at 2^22  -> 0, 0.5 or 1.
+// Random bits: a counter-based hash, 16 bits per element, two elements per 32-bit word.
+__device__ __forceinline__ uint32_t sr_mix(uint32_t x) {
+    x ^= x >> 16;
+    x *= 0x7FEB352Du;
+    x ^= x >> 15;
+    x *= 0x846CA68Bu;
+    x ^= x >> 16;
+    return x;
+}
+__device__ __forceinline__ uint32_t sr_word(uint64_t counter, uint64_t seed, uint32_t stream) {
+    const uint32_t h = sr_mix((uint32_t)counter ^ (uint32_t)seed);
+    return sr_mix(h + (uint32_t)(counter >> 32) * 0x9E3779B9u + (uint32_t)(seed >> 32) + stream * 0x85EBCA6Bu);
+}
+__device__ __forceinline__ uint32_t sr1_e2m1(float x, float inv, uint32_t rnd16) {
+    const float w = fabsf(x) * inv;
+    const uint32_t sign = (__float_as_uint(x) >> 28) & 0x8u;
+    const uint32_t add = rnd16 << 6;
+    uint32_t mag;
+    if (w < 1.f) {
+        mag = ((uint32_t)(w * 8388608.f) + add) >> 22;
+    } else {
+        mag = ((__float_as_uint(w) + add) >> 22) - 252u;
+        mag = mag > 7u ? 7u : mag;
+    }
+    return sign | mag;
+}
+// two bf16 (packed) -> two nibbles in bits 7:0, element 0 (random bits 15:0) in bits 3:0
+__device__ __forceinline__ uint32_t sr2_e2m1(uint32_t pair, float inv, uint32_t rnd) {
+    return sr1_e2m1(bf16_lo(pair), inv, rnd & 0xFFFFu) | (sr1_e2m1(bf16_hi(pair), inv, rnd >> 16) << 4);
+}
+
 // ---- gated activation of the expert MLP (shared by the activation kernels and the fused
 // activation + quantisation path, so that both round identically) ----
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {

@@ -64,6 +64,7 @@ struct QuantArgs {
     const void* probs;
     int probs_bf16;
     const uint8_t* row_mask;
+    uint64_t sr_seed;       // SR kernels: seed of the stochastic rounding
     int tiles_r, tiles_c;   // tile grid: row tiles (upper bound when grouped) x column tiles
     int super_c, n_super;   // 8x8-tile supertiles: count along the columns, total
 };
@@ -86,9 +87,14 @@ __device__ __forceinline__ bool quant_tile_of_workgroup(const QuantArgs& a, int&
     return pt < a.tiles_r && ct < a.tiles_c;
 }
 
-template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1>
+// SR (E2M1 only): codes are rounded stochastically instead of to nearest even; scales are unaffected.
+// The random word of a pair of neighbouring elements is a function of the seed and of the pair's
+// position in the OUTPUT (row-wise copy: row, column pair; transposed copy: column, position pair
+// along the padded token axis), so the result does not depend on the tiling.
+template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1, bool SR = false>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     constexpr bool FP4 = (FMT == kFmtE2M1);
+    static_assert(!SR || (FP4 && !TWOD && ACT < 0), "stochastic rounding exists for 1-D E2M1 quantisation only");
     constexpr int TPITCH = FP4 ? (QT / 2 + 16) : (QT + 16);  // bytes per LDS row of the transposed tile
     __shared__ __attribute__((aligned(16))) uint8_t t_tile[COL ? QT * TPITCH : 16];
     __shared__ uint32_t srow_tile[QT];
@@ -212,7 +218,14 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                 if (out_ok && r < rows_valid) store8_streaming(a.q_row + (src_row0 + r) * a.row_ld + col, o);
             } else {
                 uint32_t o;
-                if (byte != 255u) {
+                if (SR && byte != 255u) {
+                    const float inv = inv_scale(byte);
+                    const uint64_t key = (uint64_t)(src_row0 + r) * (uint64_t)(a.cols >> 1) + (uint64_t)(col >> 1);
+                    o = sr2_e2m1(d[it].x, inv, sr_word(key, a.sr_seed, 0)) |
+                        (sr2_e2m1(d[it].y, inv, sr_word(key + 1, a.sr_seed, 0)) << 8) |
+                        (sr2_e2m1(d[it].z, inv, sr_word(key + 2, a.sr_seed, 0)) << 16) |
+                        (sr2_e2m1(d[it].w, inv, sr_word(key + 3, a.sr_seed, 0)) << 24);
+                } else if (byte != 255u) {
                     const float sc = fwd_scale(byte);
                     o = cvt2_e2m1(d[it].x, sc) | (cvt2_e2m1(d[it].y, sc) << 8) | (cvt2_e2m1(d[it].z, sc) << 16) |
                         (cvt2_e2m1(d[it].w, sc) << 24);
@@ -254,7 +267,15 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                 *(uint2*)(t_tile + c * TPITCH + 32 * w + 8 * rg) = o;
             } else {
                 uint32_t o;
-                if (byte != 255u) {
+                if (SR && byte != 255u) {
+                    const float inv = inv_scale(byte);
+                    const uint64_t pos = (uint64_t)pt * QT + (uint64_t)(32 * w + 8 * rg);   // along the padded token axis
+                    const uint64_t key = (uint64_t)(col0 + c) * (uint64_t)(a.W >> 1) + (pos >> 1);
+                    o = sr2_e2m1(pr[0], inv, sr_word(key, a.sr_seed, 1)) |
+                        (sr2_e2m1(pr[1], inv, sr_word(key + 1, a.sr_seed, 1)) << 8) |
+                        (sr2_e2m1(pr[2], inv, sr_word(key + 2, a.sr_seed, 1)) << 16) |
+                        (sr2_e2m1(pr[3], inv, sr_word(key + 3, a.sr_seed, 1)) << 24);
+                } else if (byte != 255u) {
                     const float sc = fwd_scale(byte);
                     o = cvt2_e2m1(pr[0], sc) | (cvt2_e2m1(pr[1], sc) << 8) | (cvt2_e2m1(pr[2], sc) << 16) |
                         (cvt2_e2m1(pr[3], sc) << 24);
@@ -366,7 +387,7 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t* q, const
 // ---------------------------------------------------------------------------
 // host-side dispatch
 // ---------------------------------------------------------------------------
-template <int FMT, int SMODE, bool TWOD, int ACT = -1>
+template <int FMT, int SMODE, bool TWOD, int ACT = -1, bool SR = false>
 static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
     const int64_t super_r = (tiles_r + QSUPER - 1) / QSUPER, super_c = (tiles_c + QSUPER - 1) / QSUPER;
     const int64_t n_super = super_r * super_c;
@@ -379,11 +400,11 @@ static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStrea
     const dim3 grid((unsigned)wgs);
     const bool row = a.q_row != nullptr, col = a.q_colT != nullptr;
     if (row && col)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD, ACT>), grid, dim3(QTHREADS), 0, st, a);
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD, ACT, SR>), grid, dim3(QTHREADS), 0, st, a);
     else if (row)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD, ACT>), grid, dim3(QTHREADS), 0, st, a);
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD, ACT, SR>), grid, dim3(QTHREADS), 0, st, a);
     else if (ACT < 0)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD, -1>), grid, dim3(QTHREADS), 0, st, a);
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD, -1, SR>), grid, dim3(QTHREADS), 0, st, a);
     else
         return MXL_EINVAL;   // the fused activation always feeds a forward GEMM: a row-wise copy is part of it
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
@@ -403,6 +424,15 @@ static int dispatch_quant(int fmt, int smode, QuantArgs& a, int64_t tiles_r, int
     return MXL_EINVAL;
 }
 
+// stochastic rounding: 1-D E2M1 only
+static int dispatch_quant_sr(int smode, QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
+    if (smode == MXL_SCALE_OCP_FLOOR)
+        return launch_quant<MXL_FMT_E2M1, MXL_SCALE_OCP_FLOOR, false, -1, true>(a, tiles_r, tiles_c, st);
+    if (smode == MXL_SCALE_RCEIL) return launch_quant<MXL_FMT_E2M1, MXL_SCALE_RCEIL, false, -1, true>(a, tiles_r, tiles_c, st);
+    if (smode == MXL_SCALE_EVEN) return launch_quant<MXL_FMT_E2M1, MXL_SCALE_EVEN, false, -1, true>(a, tiles_r, tiles_c, st);
+    return MXL_EINVAL;
+}
+
 }  // namespace mxl
 
 using namespace mxl;
@@ -414,8 +444,10 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
 
 static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
-                       int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream) {
+                       int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
+                       bool sr = false, uint64_t sr_seed = 0) {
     if (row_ld == 0) row_ld = cols;
+    if (sr && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
     if (row_ld < cols || row_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((!x_bf16 && rows > 0) || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
@@ -437,9 +469,11 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.probs = probs;
     a.probs_bf16 = probs_dtype == MXL_PROBS_BF16;
     a.row_mask = row_mask;
+    a.sr_seed = sr_seed;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
     const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
     if (gx == 0) return MXL_OK;
+    if (sr) return dispatch_quant_sr(scale_mode, a, gx, gy, (hipStream_t)stream);
     if (act == MXL_ACT_SILU) return dispatch_quant<false, MXL_ACT_SILU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     if (act == MXL_ACT_GELU) return dispatch_quant<false, MXL_ACT_GELU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     return dispatch_quant<false>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
@@ -450,6 +484,13 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
                             void* s_colT, void* stream) {
     return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
                        -1, nullptr, MXL_PROBS_F32, nullptr, stream);
+}
+
+extern "C" int mxl_quantize_sr(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
+                               const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                               void* s_colT, uint64_t seed, void* stream) {
+    return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
+                       -1, nullptr, MXL_PROBS_F32, nullptr, stream, true, seed);
 }
 
 extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
@@ -489,6 +530,7 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
     a.probs = nullptr;
     a.probs_bf16 = 0;
     a.row_mask = nullptr;
+    a.sr_seed = 0;
     const int64_t gx = batch * ((n + QT - 1) / QT);
     const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
     return dispatch_quant<true>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);

@@ -11,9 +11,10 @@ copy is stored TRANSPOSED, ready to be the K-major operand of the next GEMM.
 Per-operand recipes of the reference (:234-288): activations 1-D blocks,
 weights 2-D 32x32 blocks, gradients 1-D blocks with optional stochastic
 rounding; it additionally applies a random Hadamard transform to the col-wise
-copies of activations and gradients.  The transform, stochastic rounding and
-the pre-shuffled layouts have no kernels here: the op raises for them, and the
-helpers below take ``use_rht`` (default off).  The transform is orthogonal and
+copies of activations and gradients.  The transform and the pre-shuffled
+layouts have no kernels here: the op raises for them, and the helpers below
+take ``use_rht`` (default off).  Stochastic rounding draws its seeds from
+``primus_amd.pytorch.kernels.next_sr_seed()``.  The transform is orthogonal and
 is applied to both wgrad operands, so leaving it out changes rounding noise,
 not the quantity computed.
 """
@@ -68,17 +69,26 @@ def _quantize_mxfp4_dual_op(
         raise ValueError(f"padding_align_size must be {MXFP4_PADDING_ALIGN_SIZE}")
     if rowwise_use_2d_block != colwise_use_2d_block:
         raise NotImplementedError("2-D blocks apply to both copies of a weight or to neither")
-    _unsupported(rowwise_use_sr=rowwise_use_sr, colwise_use_sr=colwise_use_sr, rowwise_use_rht=rowwise_use_rht,
-                 colwise_use_rht=colwise_use_rht, shuffle_rowwise_scale=shuffle_rowwise_scale,
+    _unsupported(rowwise_use_rht=rowwise_use_rht, colwise_use_rht=colwise_use_rht, shuffle_rowwise_scale=shuffle_rowwise_scale,
                  shuffle_rowwise=shuffle_rowwise, shuffle_colwise_scale=shuffle_colwise_scale,
                  shuffle_colwise=shuffle_colwise)
     if x.dim() != 2:
         raise ValueError("quantize_mxfp4_dual expects a 2-D tensor")
     x = x.contiguous()
     if rowwise_use_2d_block:
+        if rowwise_use_sr or colwise_use_sr:
+            raise NotImplementedError("quantize_mxfp4_dual: stochastic rounding exists for 1-D blocks only")
         return K.quantize_mx_weight_2d_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=True,
                                             pad_to=MXFP4_PADDING_ALIGN_SIZE)
-    return K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=True, pad_to=MXFP4_PADDING_ALIGN_SIZE)
+    if rowwise_use_sr == colwise_use_sr:
+        return K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=True, pad_to=MXFP4_PADDING_ALIGN_SIZE,
+                                  sr_seed=K.next_sr_seed() if rowwise_use_sr else None)
+    # only one of the copies is rounded stochastically: one launch per copy
+    q, s, _, _ = K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=False, pad_to=MXFP4_PADDING_ALIGN_SIZE,
+                                    sr_seed=K.next_sr_seed() if rowwise_use_sr else None)
+    _, _, qt, st = K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=False, colwise=True, pad_to=MXFP4_PADDING_ALIGN_SIZE,
+                                      sr_seed=K.next_sr_seed() if colwise_use_sr else None)
+    return q, s, qt, st
 
 
 @_quantize_mxfp4_dual_op.register_fake

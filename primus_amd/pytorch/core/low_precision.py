@@ -108,7 +108,7 @@ class Float4QuantConfig:
     strategy: ScalingStrategy = ScalingStrategy.DYNAMIC
     scale_dtype: ScaleDtype = ScaleDtype.E8M0
     block_size: Optional[int] = MX_BLOCK_SIZE
-    use_gradient_sr: bool = False  # stochastic rounding of gradients (not implemented)
+    use_gradient_sr: bool = False  # stochastic rounding of E2M1 gradients
     use_preshuffle: bool = False
     scale_mode: ScaleMode = ScaleMode.OCP_FLOOR
     # Element format of activations and gradients.  E2M1_X2 is plain MXFP4;

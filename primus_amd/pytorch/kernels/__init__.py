@@ -51,6 +51,29 @@ def _hooked(name: str, **info):
     return _launch_hook(name, info) if _launch_hook is not None else _NO_HOOK
 
 
+# Seeds of the stochastic-rounding quantiser.  Every call draws the next seed of a sequence that
+# depends only on the base seed (torch's global seed unless set here) and on the number of calls
+# made so far: runs repeat after ``torch.manual_seed`` + ``manual_sr_seed(None)``, and nothing is
+# read back from the device.
+_sr_base: Optional[int] = None
+_sr_calls = 0
+
+
+def manual_sr_seed(seed: Optional[int]) -> None:
+    """Restart the seed sequence of stochastic rounding from ``seed`` (``None``: from
+    ``torch.initial_seed()`` as it is at the next draw)."""
+    global _sr_base, _sr_calls
+    _sr_base = None if seed is None else int(seed)
+    _sr_calls = 0
+
+
+def next_sr_seed() -> int:
+    global _sr_calls
+    base = torch.initial_seed() if _sr_base is None else _sr_base
+    _sr_calls += 1
+    return (base * 0x9E3779B97F4A7C15 + _sr_calls * 0xD1B54A32D192ED03) & 0xFFFFFFFFFFFFFFFF
+
+
 def _round_up(x: int, m: int) -> int:
     return (x + m - 1) // m * m
 
@@ -129,8 +152,12 @@ def quantize_mx_impl(
     colwise: bool = False,
     group_lens: Optional[torch.Tensor] = None,
     pad_to: int = 1,
+    sr_seed: Optional[int] = None,
 ):
     """MX-quantise bf16 ``x[rows, cols]``.
+
+    ``sr_seed`` (an integer; E2M1 only) rounds the codes stochastically instead of to nearest even
+    (gradients of the MXFP4 recipe); the same seed reproduces the same codes.
 
     ``pad_to`` rounds the column count of the row-wise copy up to a multiple
     (zero codes, scale byte 0 in the padding) so that it can feed a GEMM,
@@ -151,6 +178,8 @@ def quantize_mx_impl(
         raise ValueError(f"the quantised dim ({cols}) must be a multiple of {BLOCK}")
     if not (rowwise or colwise):
         raise ValueError("nothing to quantise: rowwise and colwise are both False")
+    if sr_seed is not None and fmt != _lib.FMT_E2M1:
+        raise ValueError("stochastic rounding exists for the E2M1 format only")
     G = _check_group_lens(group_lens, x.device)
     per = _per_byte(fmt)
     dev = x.device
@@ -166,11 +195,13 @@ def quantize_mx_impl(
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
         row_ok = rows > 0
+        args = (_ptr(x) if row_ok else None, rows, cols, row_ld, fmt, scale_mode, _ptr(group_lens), G,
+                _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col))
         with _hooked("quantize", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
-          rc = _lib.load().mxl_quantize(
-            _ptr(x) if row_ok else None, rows, cols, row_ld, fmt, scale_mode, _ptr(group_lens), G,
-            _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col), _stream(),
-          )
+            if sr_seed is None:
+                rc = _lib.load().mxl_quantize(*args, _stream())
+            else:
+                rc = _lib.load().mxl_quantize_sr(*args, int(sr_seed) & 0xFFFFFFFFFFFFFFFF, _stream())
         _lib.check(rc, "mxl_quantize")
     cd = _code_dtype(fmt)
     v = lambda t, d: None if t is None else t.view(d)  # noqa: E731

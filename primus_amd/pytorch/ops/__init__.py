@@ -20,7 +20,6 @@ Activations and gradients use 1-D blocks of 32, weights 2-D 32x32 blocks.
 
 from __future__ import annotations
 
-import warnings
 from typing import Optional, Union
 
 import torch
@@ -38,13 +37,19 @@ from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
 __all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
            "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask", "glu_grouped_gemm_fp8",
-           "glu_grouped_gemm_fp4"]
+           "glu_grouped_gemm_fp4", "manual_sr_seed"]
 
 # dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
 # kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
 # as dgrad's last, partial wave of tiles drains instead of leaving those CUs idle.
 _wgrad_overlap = True
 _side_streams = {}
+
+
+def manual_sr_seed(seed: Optional[int]) -> None:
+    """Restart the seed sequence of stochastic gradient rounding (``Float4QuantConfig.use_gradient_sr``);
+    ``None`` ties it to ``torch.initial_seed()`` again."""
+    K.manual_sr_seed(seed)
 
 
 def set_wgrad_overlap(enabled: bool) -> None:
@@ -70,7 +75,8 @@ class _MXLinearFunction(torch.autograd.Function):
     never reaches memory, in the forward or in the backward."""
 
     @staticmethod
-    def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode, probs=None, row_mask=None, activation=None):
+    def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode, probs=None, row_mask=None, activation=None,
+                grad_sr=False):
         glu = activation is not None
         need_dgrad = a.requires_grad or (glu and probs.requires_grad)
         need_wgrad = b.requires_grad
@@ -113,6 +119,7 @@ class _MXLinearFunction(torch.autograd.Function):
             ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens)
         ctx.cfg = (act_fmt, scale_mode, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape))
         ctx.activation = activation
+        ctx.grad_sr = bool(grad_sr) and act_fmt == _lib.FMT_E2M1
         return y
 
     @staticmethod
@@ -123,8 +130,10 @@ class _MXLinearFunction(torch.autograd.Function):
         dy = dy.contiguous()
         if dy.dtype != torch.bfloat16:
             dy = dy.to(torch.bfloat16)
+        # gradients of the MXFP4 recipe may be rounded stochastically (primus_turbo_mxfp4_local.py:272-288)
         d_row, d_rs, d_col, d_cs = K.quantize_mx_impl(
-            dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
+            dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
+            sr_seed=K.next_sr_seed() if ctx.grad_sr else None,
         )
         grad_a = grad_b = None
         overlap = _wgrad_overlap and need_dgrad and need_wgrad
@@ -153,17 +162,13 @@ class _MXLinearFunction(torch.autograd.Function):
             pre, probs, row_mask = ctx.saved_tensors[5:8]
             grad_a, grad_p = K.glu_with_probs_bwd_impl(grad_a, pre, probs, row_mask, ctx.activation)
             grad_p = grad_p.to(probs.dtype)
-        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None
+        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None
 
 
 def _formats(config, fp4: bool):
     if fp4:
         if not isinstance(config, Float4QuantConfig):
             raise TypeError("gemm_fp4 / grouped_gemm_fp4 expect a Float4QuantConfig")
-        if config.use_gradient_sr:
-            # stochastic rounding of gradients (primus_turbo_mxfp4_local.py:272-288) has no kernel here
-            warnings.warn("use_gradient_sr is set but gradients are rounded to nearest-even: "
-                          "stochastic rounding is not implemented", stacklevel=3)
         return fmt_code(config.activation_format), _lib.FMT_E2M1
     if not isinstance(config, Float8QuantConfig):
         raise TypeError("gemm_fp8 / grouped_gemm_fp8 expect a Float8QuantConfig")
@@ -212,15 +217,18 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
         raise ValueError(f"contraction dims differ: activations K={k_act}, weights K={b.shape[-1]}")
     if group_lens is not None and group_lens.numel() != b.shape[0]:
         raise ValueError("group_lens must have one entry per expert weight")
+    # stochastic rounding applies to E2M1 gradients; with E4M3 activations the gradients are MXFP8
+    grad_sr = bool(fp4 and config.use_gradient_sr and act_fmt == _lib.FMT_E2M1)
     if glu is None:
-        return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value)
+        return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
+                                       None, None, None, grad_sr)
     probs, row_mask, activation = glu
     if activation not in ("silu", "gelu"):
         raise ValueError(f"activation must be 'silu' or 'gelu', got {activation!r}")
     if probs.dim() != 1 or probs.shape[0] != a.shape[0]:
         raise ValueError("probs must be 1-D with one entry per row of the activations")
     return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
-                                   probs.contiguous(), row_mask, activation)
+                                   probs.contiguous(), row_mask, activation, grad_sr)
 
 
 def gemm_fp8(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,

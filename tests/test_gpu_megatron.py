@@ -301,8 +301,11 @@ def test_mxfp4_dual_quantize_op_matches_oracle_bytes(mg, gpu):
     assert np.array_equal(wcs.view(torch.uint8).cpu().numpy()[:, :2], st)
     with pytest.raises(NotImplementedError, match="colwise_use_rht"):
         m4._quantize_input_dual(x, use_rht=True)
-    with pytest.raises(NotImplementedError, match="rowwise_use_sr"):
-        m4._quantize_grad_dual(x, use_sr=True)
+    with pytest.raises(NotImplementedError, match="shuffle_rowwise_scale"):
+        m4._quantize_grad_dual(x, preshuffle=True)
+    # stochastic rounding keeps shapes and scales (the codes are checked in test_gpu_sr.py)
+    sr = m4._quantize_grad_dual(x, use_sr=True)
+    assert torch.equal(sr[1].view(torch.uint8), row_s.view(torch.uint8)) and sr[0].shape == row.shape
 
 
 def test_mxfp4_linear_function_snr_against_bf16(mg, gpu):

@@ -90,18 +90,33 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
                  const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                  void* s_colT, void* stream);
 
-/* mxl_quantize with STOCHASTIC ROUNDING of the codes (fmt must be MXL_FMT_E2M1): the MXFP4 recipe's
- * gradient quantisation, rowwise_use_sr / colwise_use_sr of quantize_mxfp4_dual
- * (primus_turbo_mxfp4_local.py:272-288; config flag mxfp4_gradient_stochastic_rounding,
- * primus/configs/modules/megatron/primus_turbo.yaml:21-24).  Scales are those of mxl_quantize; each
- * element becomes one of its two neighbours on the E2M1 grid, the upper one with probability equal to
- * its fractional position between them (so the dequantised value is unbiased), saturating at +-6.
- * The random bits are a counter-based hash of `seed` and the element's position in the output, hence
- * reproducible and independent of the launch geometry; the row-wise and the transposed copy draw
- * from different streams.  All other arguments as for mxl_quantize. */
-int mxl_quantize_sr(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
-                    const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                    void* s_colT, uint64_t seed, void* stream);
+/* MXFP4 (E2M1) quantisation with the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
+ * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288).  Arguments as for mxl_quantize
+ * with fmt = MXL_FMT_E2M1, plus `flags`:
+ *
+ *   MXL_QF_SR      stochastic rounding of the codes of both copies (rowwise_use_sr / colwise_use_sr;
+ *                  config flag mxfp4_gradient_stochastic_rounding,
+ *                  primus/configs/modules/megatron/primus_turbo.yaml:21-24).  Scales are those of
+ *                  mxl_quantize; each element becomes one of its two neighbours on the E2M1 grid, the
+ *                  upper one with probability equal to its fractional position between them (the
+ *                  dequantised value is unbiased), saturating at +-6.  The random bits are a
+ *                  counter-based hash of `sr_seed` and the element's position in the output:
+ *                  reproducible and independent of the launch geometry; the two copies draw from
+ *                  different streams.
+ *   MXL_QF_RHT_COL randomised Hadamard transform of the transposed copy (colwise_use_rht): every 16
+ *                  consecutive token positions of an expert's segment are replaced by
+ *                  (1/4) H16 (s * x) before quantisation (H16 Sylvester-ordered, s_i = -1 where bit i
+ *                  of `rht_signs` is set; fp32 butterflies, one rounding to bf16).  Requires q_colT.
+ *                  Both operands of a wgrad GEMM must use the same `rht_signs`; the product is then
+ *                  unchanged up to rounding.  The row-wise copy is never transformed.  Groups of 16
+ *                  start at the expert's segment start, so a partially filled last group holds
+ *                  transformed data in all 16 positions (the padding rows enter as zeros) and the
+ *                  remaining padding holds +-0 codes. */
+#define MXL_QF_SR 1u
+#define MXL_QF_RHT_COL 2u
+int mxl_quantize_fp4_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int scale_mode,
+                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                        void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);
 
 /* 2-D (32x32 tile) MX quantisation of `batch` independent weight matrices
  * w[batch, n, k] (weights use ScalingRecipe(use_2d_block=True):

@@ -63,6 +63,15 @@ Parity status
   different generator by construction): which elements round up is **parity
   unpinned**; only the distribution is comparable.
 
+* ``hadamard16_rows`` (the transposed copies' random Hadamard transform,
+  colwise_use_rht at primus_turbo_mxfp4_local.py:234-250,272-288): pinned
+  against ``scipy.linalg.hadamard(16)`` in float64 (library routine; the
+  float32 butterflies agree with it to rounding and exactly on small integers),
+  by orthogonality (transforming twice with zero signs returns the input, the
+  inner product of two transformed columns equals the untransformed one) and by
+  the sign-vector definition.  The reference states neither the transform size
+  nor the sign vector (they live in Primus-Turbo's C++ op): **parity unpinned**.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -464,9 +473,8 @@ def quantize_mx_rowwise_sr(x, seed: int, scale_mode: int = SCALE_OCP_FLOOR, stre
     return pack_fp4(code), byte
 
 
-def quantize_mx_colwise_segmented_sr(x, group_lens, seed: int, scale_mode: int = SCALE_OCP_FLOOR):
-    """``quantize_mx_colwise_segmented(x, group_lens, FMT_E2M1)`` with stochastic rounding: the
-    row-wise routine applied to the transposed, segment-padded tensor ``[C, W]`` with stream 1."""
+def _segment_padded(x, group_lens):
+    """bf16 bits of x[sum(M_g), C] laid out as [W, C] with every group at its padded offset."""
     xb = to_bf16_bits(x)
     lens = np.asarray(group_lens, dtype=np.int64)
     total, C = xb.shape
@@ -476,7 +484,48 @@ def quantize_mx_colwise_segmented_sr(x, group_lens, seed: int, scale_mode: int =
     xp = np.zeros((W, C), dtype=np.uint16)
     for g in range(len(lens)):
         xp[poffs[g] : poffs[g] + lens[g]] = xb[offs[g] : offs[g + 1]]
-    return quantize_mx_rowwise_sr(np.ascontiguousarray(xp.T), seed, scale_mode, stream=1)
+    return xp
+
+
+def hadamard16_rows(xb: np.ndarray, signs: int) -> np.ndarray:
+    """Randomised Hadamard transform over groups of 16 consecutive rows of bf16 bits ``xb[W, C]``
+    (W a multiple of 16): y = (1/4) H16 (s * x) per group, H16 Sylvester-ordered, s_i = -1 where bit i
+    of ``signs`` is set.  Four float32 butterfly stages with strides 1, 2, 4, 8 (new[i] = old[i] +
+    old[i+s], new[i+s] = old[i] - old[i+s]), then * 0.25 and one rounding to bf16."""
+    W, C = xb.shape
+    assert W % 16 == 0
+    v = bf16_bits_to_f32(xb).reshape(W // 16, 16, C).astype(np.float32)
+    s = np.array([-1.0 if (signs >> i) & 1 else 1.0 for i in range(16)], dtype=np.float32)
+    v = v * s[None, :, None]
+    with np.errstate(invalid="ignore", over="ignore"):
+        for st in (1, 2, 4, 8):
+            out = np.empty_like(v)
+            for i in range(16):
+                if i & st:
+                    continue
+                out[:, i] = v[:, i] + v[:, i + st]
+                out[:, i + st] = v[:, i] - v[:, i + st]
+            v = out
+        v = v * np.float32(0.25)
+    return f32_to_bf16_bits(v.reshape(W, C))
+
+
+def quantize_mx_colwise_segmented_fp4(x, group_lens, scale_mode: int = SCALE_OCP_FLOOR, sr_seed=None, rht_signs=None):
+    """The transposed, segment-padded MXFP4 copy with the recipe's options: optional Hadamard
+    transform along the (padded) token axis first, then round-to-nearest or stochastic rounding."""
+    xp = _segment_padded(x, group_lens)
+    if rht_signs is not None:
+        xp = hadamard16_rows(xp, rht_signs)
+    xt = np.ascontiguousarray(xp.T)
+    if sr_seed is None:
+        return quantize_mx_rowwise(xt, FMT_E2M1, scale_mode)
+    return quantize_mx_rowwise_sr(xt, sr_seed, scale_mode, stream=1)
+
+
+def quantize_mx_colwise_segmented_sr(x, group_lens, seed: int, scale_mode: int = SCALE_OCP_FLOOR):
+    """``quantize_mx_colwise_segmented(x, group_lens, FMT_E2M1)`` with stochastic rounding: the
+    row-wise routine applied to the transposed, segment-padded tensor ``[C, W]`` with stream 1."""
+    return quantize_mx_colwise_segmented_fp4(x, group_lens, scale_mode, sr_seed=seed)
 
 
 # --------------------------------------------------------------------------

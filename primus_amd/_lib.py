@@ -26,13 +26,14 @@ GEMM_K_ALIGN = 128  # the GEMM kernels take the contraction dim in multiples of 
 MAX_GROUPS = 1024
 ACT_SILU, ACT_GELU = 0, 1
 PROBS_F32, PROBS_BF16 = 0, 1
+QF_SR, QF_RHT_COL = 1, 2   # flags of mxl_quantize_fp4_ex
 
 EXPORTS = (
     "mxl_version",
     "mxl_error_string",
     "mxl_padded_width",
     "mxl_quantize",
-    "mxl_quantize_sr",
+    "mxl_quantize_fp4_ex",
     "mxl_quantize_weight_2d",
     "mxl_dequantize",
     "mxl_gemm_nt",
@@ -76,8 +77,9 @@ def load() -> ctypes.CDLL:
         lib.mxl_padded_width.argtypes = [i64, i32]
         lib.mxl_quantize.restype = i32
         lib.mxl_quantize.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, vp]
-        lib.mxl_quantize_sr.restype = i32
-        lib.mxl_quantize_sr.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, ctypes.c_uint64, vp]
+        lib.mxl_quantize_fp4_ex.restype = i32
+        lib.mxl_quantize_fp4_ex.argtypes = [vp, i64, i64, i64, i32, vp, i32, vp, vp, vp, vp, ctypes.c_uint32,
+                                            ctypes.c_uint64, ctypes.c_uint32, vp]
         lib.mxl_quantize_weight_2d.restype = i32
         lib.mxl_quantize_weight_2d.argtypes = [vp, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         lib.mxl_dequantize.restype = i32

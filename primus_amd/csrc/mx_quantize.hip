@@ -65,6 +65,7 @@ struct QuantArgs {
     int probs_bf16;
     const uint8_t* row_mask;
     uint64_t sr_seed;       // SR kernels: seed of the stochastic rounding
+    uint32_t rht_signs;     // RHT kernels: sign bit i flips row i of every 16-row group before the transform
     int tiles_r, tiles_c;   // tile grid: row tiles (upper bound when grouped) x column tiles
     int super_c, n_super;   // 8x8-tile supertiles: count along the columns, total
 };
@@ -91,10 +92,19 @@ __device__ __forceinline__ bool quant_tile_of_workgroup(const QuantArgs& a, int&
 // The random word of a pair of neighbouring elements is a function of the seed and of the pair's
 // position in the OUTPUT (row-wise copy: row, column pair; transposed copy: column, position pair
 // along the padded token axis), so the result does not depend on the tiling.
-template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1, bool SR = false>
+//
+// RHT: the transposed copy is taken from a randomised Hadamard transform of the input along the token
+// axis (colwise_use_rht of quantize_mxfp4_dual, primus_turbo_mxfp4_local.py:234-250,272-288): every
+// group of 16 consecutive token positions of an expert's segment becomes (1/4) H16 (s * x), H16 the
+// Sylvester matrix and s the sign vector `rht_signs`, evaluated as four fp32 butterfly stages (strides
+// 1, 2, 4, 8) and rounded once to bf16; that tensor is then quantised like any other.  The transform is
+// orthogonal, so a wgrad GEMM whose two operands were both transformed computes the same contraction
+// while single large values are spread over 16 positions before they meet the 4-bit grid.
+template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1, bool SR = false, bool RHT = false>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     constexpr bool FP4 = (FMT == kFmtE2M1);
     static_assert(!SR || (FP4 && !TWOD && ACT < 0), "stochastic rounding exists for 1-D E2M1 quantisation only");
+    static_assert(!RHT || (COL && !TWOD && ACT < 0), "the Hadamard transform applies to the transposed 1-D copy only");
     constexpr int TPITCH = FP4 ? (QT / 2 + 16) : (QT + 16);  // bytes per LDS row of the transposed tile
     __shared__ __attribute__((aligned(16))) uint8_t t_tile[COL ? QT * TPITCH : 16];
     __shared__ uint32_t srow_tile[QT];
@@ -170,7 +180,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     for (int it = 0; it < 8; ++it) {
         const uint32_t p0 = d[it].x & 0x7FFF7FFFu, p1 = d[it].y & 0x7FFF7FFFu, p2 = d[it].z & 0x7FFF7FFFu,
                        p3 = d[it].w & 0x7FFF7FFFu;
-        if (COL && !TWOD) {
+        if (COL && !TWOD && !RHT) {
             cmax[0] = pk_max16(cmax[0], p0);
             cmax[1] = pk_max16(cmax[1], p1);
             cmax[2] = pk_max16(cmax[2], p2);
@@ -190,7 +200,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         m = max(m, (uint32_t)__shfl_xor((int)m, 16));
         m = max(m, (uint32_t)__shfl_xor((int)m, 32));
         tile_byte = scale_byte<FMT, SMODE>(m);
-    } else if (COL) {
+    } else if (COL && !RHT) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 16));
@@ -235,6 +245,55 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                 }
                 if (out_ok && r < rows_valid) store4_streaming(a.q_row + ((src_row0 + r) * a.row_ld + col) / 2, o);
             }
+        }
+    }
+
+    // ---- Hadamard transform along the rows, in place (the row-wise copy above used the plain input) ----
+    if (RHT) {
+        // a 16-row group = the 8 rows of this lane and the 8 rows of the lane 16 further (rg ^ 1)
+        const uint32_t upper = rg & 1;
+        uint32_t* tw = (uint32_t*)d;
+#pragma unroll
+        for (int j2 = 0; j2 < 4; ++j2) {
+            float lo[8], hi[8];
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                const uint32_t flip = ((a.rht_signs >> (8 * upper + it)) & 1u) ? 0x80008000u : 0u;
+                const uint32_t v = tw[it * 4 + j2] ^ flip;
+                lo[it] = bf16_lo(v);
+                hi[it] = bf16_hi(v);
+            }
+#pragma unroll
+            for (int st = 1; st < 8; st <<= 1) {
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    if (it & st) continue;
+                    const float a0 = lo[it], b0 = lo[it + st], a1 = hi[it], b1 = hi[it + st];
+                    lo[it] = a0 + b0;
+                    lo[it + st] = a0 - b0;
+                    hi[it] = a1 + b1;
+                    hi[it + st] = a1 - b1;
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                const float o0 = __shfl_xor(lo[it], 16), o1 = __shfl_xor(hi[it], 16);
+                const float r0 = upper ? (o0 - lo[it]) : (lo[it] + o0);
+                const float r1 = upper ? (o1 - hi[it]) : (hi[it] + o1);
+                tw[it * 4 + j2] = pack_bf16(r0 * 0.25f, r1 * 0.25f);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            cmax[0] = pk_max16(cmax[0], d[it].x & 0x7FFF7FFFu);
+            cmax[1] = pk_max16(cmax[1], d[it].y & 0x7FFF7FFFu);
+            cmax[2] = pk_max16(cmax[2], d[it].z & 0x7FFF7FFFu);
+            cmax[3] = pk_max16(cmax[3], d[it].w & 0x7FFF7FFFu);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 16));
+            cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 32));
         }
     }
 
@@ -387,7 +446,7 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t* q, const
 // ---------------------------------------------------------------------------
 // host-side dispatch
 // ---------------------------------------------------------------------------
-template <int FMT, int SMODE, bool TWOD, int ACT = -1, bool SR = false>
+template <int FMT, int SMODE, bool TWOD, int ACT = -1, bool SR = false, bool RHT = false>
 static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
     const int64_t super_r = (tiles_r + QSUPER - 1) / QSUPER, super_c = (tiles_c + QSUPER - 1) / QSUPER;
     const int64_t n_super = super_r * super_c;
@@ -400,11 +459,12 @@ static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStrea
     const dim3 grid((unsigned)wgs);
     const bool row = a.q_row != nullptr, col = a.q_colT != nullptr;
     if (row && col)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD, ACT, SR>), grid, dim3(QTHREADS), 0, st, a);
-    else if (row)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD, ACT, SR>), grid, dim3(QTHREADS), 0, st, a);
-    else if (ACT < 0)
-        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD, -1, SR>), grid, dim3(QTHREADS), 0, st, a);
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, true, TWOD, ACT, SR, RHT>), grid, dim3(QTHREADS), 0, st, a);
+    else if (row && !RHT)
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, true, false, TWOD, ACT, SR, false>), grid, dim3(QTHREADS), 0, st,
+                           a);
+    else if (ACT < 0 && col)
+        hipLaunchKernelGGL((mx_quant_kernel<FMT, SMODE, false, true, TWOD, -1, SR, RHT>), grid, dim3(QTHREADS), 0, st, a);
     else
         return MXL_EINVAL;   // the fused activation always feeds a forward GEMM: a row-wise copy is part of it
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
@@ -424,12 +484,13 @@ static int dispatch_quant(int fmt, int smode, QuantArgs& a, int64_t tiles_r, int
     return MXL_EINVAL;
 }
 
-// stochastic rounding: 1-D E2M1 only
-static int dispatch_quant_sr(int smode, QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
+// the MXFP4 recipe's options (1-D E2M1 only): stochastic rounding, Hadamard transform of the transposed copy
+template <bool SR, bool RHT>
+static int dispatch_quant_fp4(int smode, QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
     if (smode == MXL_SCALE_OCP_FLOOR)
-        return launch_quant<MXL_FMT_E2M1, MXL_SCALE_OCP_FLOOR, false, -1, true>(a, tiles_r, tiles_c, st);
-    if (smode == MXL_SCALE_RCEIL) return launch_quant<MXL_FMT_E2M1, MXL_SCALE_RCEIL, false, -1, true>(a, tiles_r, tiles_c, st);
-    if (smode == MXL_SCALE_EVEN) return launch_quant<MXL_FMT_E2M1, MXL_SCALE_EVEN, false, -1, true>(a, tiles_r, tiles_c, st);
+        return launch_quant<MXL_FMT_E2M1, MXL_SCALE_OCP_FLOOR, false, -1, SR, RHT>(a, tiles_r, tiles_c, st);
+    if (smode == MXL_SCALE_RCEIL) return launch_quant<MXL_FMT_E2M1, MXL_SCALE_RCEIL, false, -1, SR, RHT>(a, tiles_r, tiles_c, st);
+    if (smode == MXL_SCALE_EVEN) return launch_quant<MXL_FMT_E2M1, MXL_SCALE_EVEN, false, -1, SR, RHT>(a, tiles_r, tiles_c, st);
     return MXL_EINVAL;
 }
 
@@ -445,9 +506,10 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
 static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
                        int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
-                       bool sr = false, uint64_t sr_seed = 0) {
+                       bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0) {
     if (row_ld == 0) row_ld = cols;
-    if (sr && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
+    if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
+    if (rht && !q_colT) return MXL_EINVAL;   // the transform belongs to the transposed copy
     if (row_ld < cols || row_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((!x_bf16 && rows > 0) || rows < 0 || cols <= 0 || cols % MXL_BLOCK != 0) return MXL_EINVAL;
     if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
@@ -470,10 +532,13 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.probs_bf16 = probs_dtype == MXL_PROBS_BF16;
     a.row_mask = row_mask;
     a.sr_seed = sr_seed;
+    a.rht_signs = rht_signs & 0xFFFFu;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
     const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
     if (gx == 0) return MXL_OK;
-    if (sr) return dispatch_quant_sr(scale_mode, a, gx, gy, (hipStream_t)stream);
+    if (sr && rht) return dispatch_quant_fp4<true, true>(scale_mode, a, gx, gy, (hipStream_t)stream);
+    if (sr) return dispatch_quant_fp4<true, false>(scale_mode, a, gx, gy, (hipStream_t)stream);
+    if (rht) return dispatch_quant_fp4<false, true>(scale_mode, a, gx, gy, (hipStream_t)stream);
     if (act == MXL_ACT_SILU) return dispatch_quant<false, MXL_ACT_SILU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     if (act == MXL_ACT_GELU) return dispatch_quant<false, MXL_ACT_GELU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     return dispatch_quant<false>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
@@ -486,11 +551,13 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
                        -1, nullptr, MXL_PROBS_F32, nullptr, stream);
 }
 
-extern "C" int mxl_quantize_sr(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
-                               const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                               void* s_colT, uint64_t seed, void* stream) {
-    return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
-                       -1, nullptr, MXL_PROBS_F32, nullptr, stream, true, seed);
+extern "C" int mxl_quantize_fp4_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int scale_mode,
+                                   const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                                   void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream) {
+    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL)) return MXL_EINVAL;
+    return quantize_1d(x_bf16, rows, cols, row_ld, MXL_FMT_E2M1, scale_mode, group_lens, num_groups, q_row, s_row, q_colT,
+                       s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, (flags & MXL_QF_SR) != 0, sr_seed,
+                       (flags & MXL_QF_RHT_COL) != 0, rht_signs);
 }
 
 extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
@@ -531,6 +598,7 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
     a.probs_bf16 = 0;
     a.row_mask = nullptr;
     a.sr_seed = 0;
+    a.rht_signs = 0;
     const int64_t gx = batch * ((n + QT - 1) / QT);
     const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
     return dispatch_quant<true>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);

@@ -10,13 +10,12 @@ copy is stored TRANSPOSED, ready to be the K-major operand of the next GEMM.
 
 Per-operand recipes of the reference (:234-288): activations 1-D blocks,
 weights 2-D 32x32 blocks, gradients 1-D blocks with optional stochastic
-rounding; it additionally applies a random Hadamard transform to the col-wise
-copies of activations and gradients.  The transform and the pre-shuffled
-layouts have no kernels here: the op raises for them, and the helpers below
-take ``use_rht`` (default off).  Stochastic rounding draws its seeds from
-``primus_amd.pytorch.kernels.next_sr_seed()``.  The transform is orthogonal and
-is applied to both wgrad operands, so leaving it out changes rounding noise,
-not the quantity computed.
+rounding; the col-wise copies of activations and gradients -- the two wgrad
+operands -- go through a random Hadamard transform (16 tokens, the fixed sign
+vector ``RHT_SIGNS``; orthogonal, so the contraction is unchanged).  The
+pre-shuffled layouts and a transform of the row-wise copy have no kernels
+here: the op raises for them.  Stochastic rounding draws its seeds from
+``primus_amd.pytorch.kernels.next_sr_seed()``.
 """
 
 from __future__ import annotations
@@ -31,6 +30,7 @@ from ...pytorch.core.low_precision import ScalingGranularity, float4_e2m1fn_x2, 
 
 MXFP4_BLOCK_SIZE = 32
 MXFP4_PADDING_ALIGN_SIZE = 128
+RHT_SIGNS = 0xA6C9   # sign vector of the Hadamard transform; any value works if both wgrad operands share it
 
 _FP4_DTYPE = float4_e2m1fn_x2
 _GRAN_VALUE = ScalingGranularity.MX_BLOCKWISE.value
@@ -69,25 +69,27 @@ def _quantize_mxfp4_dual_op(
         raise ValueError(f"padding_align_size must be {MXFP4_PADDING_ALIGN_SIZE}")
     if rowwise_use_2d_block != colwise_use_2d_block:
         raise NotImplementedError("2-D blocks apply to both copies of a weight or to neither")
-    _unsupported(rowwise_use_rht=rowwise_use_rht, colwise_use_rht=colwise_use_rht, shuffle_rowwise_scale=shuffle_rowwise_scale,
+    _unsupported(rowwise_use_rht=rowwise_use_rht, shuffle_rowwise_scale=shuffle_rowwise_scale,
                  shuffle_rowwise=shuffle_rowwise, shuffle_colwise_scale=shuffle_colwise_scale,
                  shuffle_colwise=shuffle_colwise)
     if x.dim() != 2:
         raise ValueError("quantize_mxfp4_dual expects a 2-D tensor")
     x = x.contiguous()
+    rht = RHT_SIGNS if colwise_use_rht else None
     if rowwise_use_2d_block:
-        if rowwise_use_sr or colwise_use_sr:
-            raise NotImplementedError("quantize_mxfp4_dual: stochastic rounding exists for 1-D blocks only")
+        if rowwise_use_sr or colwise_use_sr or colwise_use_rht:
+            raise NotImplementedError("quantize_mxfp4_dual: stochastic rounding and the Hadamard transform "
+                                      "exist for 1-D blocks only")
         return K.quantize_mx_weight_2d_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=True,
                                             pad_to=MXFP4_PADDING_ALIGN_SIZE)
     if rowwise_use_sr == colwise_use_sr:
         return K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=True, pad_to=MXFP4_PADDING_ALIGN_SIZE,
-                                  sr_seed=K.next_sr_seed() if rowwise_use_sr else None)
+                                  sr_seed=K.next_sr_seed() if rowwise_use_sr else None, rht_signs=rht)
     # only one of the copies is rounded stochastically: one launch per copy
     q, s, _, _ = K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=True, colwise=False, pad_to=MXFP4_PADDING_ALIGN_SIZE,
                                     sr_seed=K.next_sr_seed() if rowwise_use_sr else None)
     _, _, qt, st = K.quantize_mx_impl(x, _lib.FMT_E2M1, rowwise=False, colwise=True, pad_to=MXFP4_PADDING_ALIGN_SIZE,
-                                      sr_seed=K.next_sr_seed() if colwise_use_sr else None)
+                                      sr_seed=K.next_sr_seed() if colwise_use_sr else None, rht_signs=rht)
     return q, s, qt, st
 
 
@@ -130,7 +132,7 @@ def _dual(x, two_d, sr, rht, shuffle):
     )
 
 
-def _quantize_input_dual(input_2d, preshuffle: bool = False, use_rht: bool = False):
+def _quantize_input_dual(input_2d, preshuffle: bool = False, use_rht: bool = True):
     """Activations: 1-D blocks (:234-250)."""
     return _dual(input_2d, False, False, use_rht, (preshuffle, False, preshuffle, preshuffle))
 
@@ -140,7 +142,7 @@ def _quantize_weight_dual(weight, preshuffle: bool = False):
     return _dual(weight, True, False, False, (preshuffle,) * 4)
 
 
-def _quantize_grad_dual(grad_2d, preshuffle: bool = False, use_sr: bool = False, use_rht: bool = False):
+def _quantize_grad_dual(grad_2d, preshuffle: bool = False, use_sr: bool = False, use_rht: bool = True):
     """Gradients: the activation recipe plus optional stochastic rounding (:272-288)."""
     return _dual(grad_2d, False, use_sr, use_rht, (preshuffle, False, preshuffle, False))
 

@@ -114,6 +114,9 @@ class Float4QuantConfig:
     # Element format of activations and gradients.  E2M1_X2 is plain MXFP4;
     # E4M3 gives MXFP4 weights with MXFP8 activations (GPT-OSS style).
     activation_format: Format = Format.E2M1_X2
+    # Randomised Hadamard transform (16 tokens) of the transposed copies of activations and gradients,
+    # i.e. of both wgrad operands: None = off, else the 16 sign bits.  E2M1 activations only.
+    colwise_rht_signs: Optional[int] = None
 
     def __post_init__(self):
         if self.format != Format.E2M1_X2:

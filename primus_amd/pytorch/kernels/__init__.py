@@ -153,11 +153,14 @@ def quantize_mx_impl(
     group_lens: Optional[torch.Tensor] = None,
     pad_to: int = 1,
     sr_seed: Optional[int] = None,
+    rht_signs: Optional[int] = None,
 ):
     """MX-quantise bf16 ``x[rows, cols]``.
 
     ``sr_seed`` (an integer; E2M1 only) rounds the codes stochastically instead of to nearest even
-    (gradients of the MXFP4 recipe); the same seed reproduces the same codes.
+    (gradients of the MXFP4 recipe); the same seed reproduces the same codes.  ``rht_signs`` (16 sign
+    bits; E2M1 only, needs ``colwise``) takes the transposed copy from the randomised Hadamard
+    transform of ``x`` over groups of 16 tokens; both operands of a wgrad GEMM must use the same signs.
 
     ``pad_to`` rounds the column count of the row-wise copy up to a multiple
     (zero codes, scale byte 0 in the padding) so that it can feed a GEMM,
@@ -178,8 +181,10 @@ def quantize_mx_impl(
         raise ValueError(f"the quantised dim ({cols}) must be a multiple of {BLOCK}")
     if not (rowwise or colwise):
         raise ValueError("nothing to quantise: rowwise and colwise are both False")
-    if sr_seed is not None and fmt != _lib.FMT_E2M1:
-        raise ValueError("stochastic rounding exists for the E2M1 format only")
+    if (sr_seed is not None or rht_signs is not None) and fmt != _lib.FMT_E2M1:
+        raise ValueError("stochastic rounding and the Hadamard transform exist for the E2M1 format only")
+    if rht_signs is not None and not colwise:
+        raise ValueError("the Hadamard transform applies to the transposed (colwise) copy")
     G = _check_group_lens(group_lens, x.device)
     per = _per_byte(fmt)
     dev = x.device
@@ -198,10 +203,13 @@ def quantize_mx_impl(
         args = (_ptr(x) if row_ok else None, rows, cols, row_ld, fmt, scale_mode, _ptr(group_lens), G,
                 _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col))
         with _hooked("quantize", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
-            if sr_seed is None:
+            if sr_seed is None and rht_signs is None:
                 rc = _lib.load().mxl_quantize(*args, _stream())
             else:
-                rc = _lib.load().mxl_quantize_sr(*args, int(sr_seed) & 0xFFFFFFFFFFFFFFFF, _stream())
+                flags = (_lib.QF_SR if sr_seed is not None else 0) | (_lib.QF_RHT_COL if rht_signs is not None else 0)
+                rc = _lib.load().mxl_quantize_fp4_ex(
+                    *args[:4], *args[5:], flags, int(sr_seed or 0) & 0xFFFFFFFFFFFFFFFF, int(rht_signs or 0) & 0xFFFF,
+                    _stream())
         _lib.check(rc, "mxl_quantize")
     cd = _code_dtype(fmt)
     v = lambda t, d: None if t is None else t.view(d)  # noqa: E731

@@ -76,7 +76,7 @@ class _MXLinearFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode, probs=None, row_mask=None, activation=None,
-                grad_sr=False):
+                grad_sr=False, rht_signs=None):
         glu = activation is not None
         need_dgrad = a.requires_grad or (glu and probs.requires_grad)
         need_wgrad = b.requires_grad
@@ -91,7 +91,8 @@ class _MXLinearFunction(torch.autograd.Function):
             )
         else:
             a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
-                a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN
+                a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
+                rht_signs=rht_signs if need_wgrad else None,
             )
         if isinstance(b, QuantizedTensor):
             # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
@@ -120,6 +121,7 @@ class _MXLinearFunction(torch.autograd.Function):
         ctx.cfg = (act_fmt, scale_mode, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape))
         ctx.activation = activation
         ctx.grad_sr = bool(grad_sr) and act_fmt == _lib.FMT_E2M1
+        ctx.rht_signs = rht_signs
         return y
 
     @staticmethod
@@ -134,6 +136,7 @@ class _MXLinearFunction(torch.autograd.Function):
         d_row, d_rs, d_col, d_cs = K.quantize_mx_impl(
             dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
             sr_seed=K.next_sr_seed() if ctx.grad_sr else None,
+            rht_signs=ctx.rht_signs if need_wgrad else None,   # same signs as the saved activation copy
         )
         grad_a = grad_b = None
         overlap = _wgrad_overlap and need_dgrad and need_wgrad
@@ -162,7 +165,7 @@ class _MXLinearFunction(torch.autograd.Function):
             pre, probs, row_mask = ctx.saved_tensors[5:8]
             grad_a, grad_p = K.glu_with_probs_bwd_impl(grad_a, pre, probs, row_mask, ctx.activation)
             grad_p = grad_p.to(probs.dtype)
-        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None
+        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None, None
 
 
 def _formats(config, fp4: bool):
@@ -219,9 +222,12 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
         raise ValueError("group_lens must have one entry per expert weight")
     # stochastic rounding applies to E2M1 gradients; with E4M3 activations the gradients are MXFP8
     grad_sr = bool(fp4 and config.use_gradient_sr and act_fmt == _lib.FMT_E2M1)
+    rht = getattr(config, "colwise_rht_signs", None) if fp4 and act_fmt == _lib.FMT_E2M1 else None
     if glu is None:
         return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
-                                       None, None, None, grad_sr)
+                                       None, None, None, grad_sr, rht)
+    if rht is not None:
+        raise NotImplementedError("the activation prologue and the Hadamard transform cannot be combined")
     probs, row_mask, activation = glu
     if activation not in ("silu", "gelu"):
         raise ValueError(f"activation must be 'silu' or 'gelu', got {activation!r}")

@@ -47,7 +47,7 @@ def test_host_only_entry_points(lib):
 
 def test_constants_match_the_header():
     text = open(HEADER).read()
-    defs = dict(re.findall(r"#define\s+(MXL_\w+)\s+\(?(-?\d+)\)?", text))
+    defs = dict(re.findall(r"#define\s+(MXL_\w+)\s+\(?(-?\d+)u?\)?", text))
     assert int(defs["MXL_BLOCK"]) == _lib.BLOCK == o.BLOCK
     assert int(defs["MXL_SEG_ALIGN"]) == _lib.SEG_ALIGN == o.SEG_ALIGN
     assert int(defs["MXL_MAX_GROUPS"]) == _lib.MAX_GROUPS
@@ -55,6 +55,7 @@ def test_constants_match_the_header():
     assert (int(defs["MXL_SCALE_OCP_FLOOR"]), int(defs["MXL_SCALE_RCEIL"]), int(defs["MXL_SCALE_EVEN"])) == (
         o.SCALE_OCP_FLOOR, o.SCALE_RCEIL, o.SCALE_EVEN)
     assert (int(defs["MXL_ACT_SILU"]), int(defs["MXL_ACT_GELU"])) == (_lib.ACT_SILU, _lib.ACT_GELU)
+    assert (int(defs["MXL_QF_SR"]), int(defs["MXL_QF_RHT_COL"])) == (_lib.QF_SR, _lib.QF_RHT_COL)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -288,9 +288,14 @@ def test_mxfp4_dual_quantize_op_matches_oracle_bytes(mg, gpu):
     assert np.array_equal(row.view(torch.uint8).cpu().numpy()[:, :48], q)
     assert np.array_equal(row_s.view(torch.uint8).cpu().numpy()[:, :3], s)
     assert not row.view(torch.uint8)[:, 48:].any() and not row_s.view(torch.uint8)[:, 3:].any()
-    qT, sT = o.quantize_mx_colwise_segmented(x.cpu(), [100], o.FMT_E2M1)
+    # the col-wise copy of an activation goes through the Hadamard transform, like the reference's
+    qT, sT = o.quantize_mx_colwise_segmented_fp4(x.cpu(), [100], rht_signs=m4.RHT_SIGNS)
     assert np.array_equal(col.view(torch.uint8).cpu().numpy(), qT)
     assert np.array_equal(col_s.view(torch.uint8).cpu().numpy(), sT)
+    _, _, col0, col0_s = m4._quantize_input_dual(x, use_rht=False)
+    qT, sT = o.quantize_mx_colwise_segmented(x.cpu(), [100], o.FMT_E2M1)
+    assert np.array_equal(col0.view(torch.uint8).cpu().numpy(), qT)
+    assert np.array_equal(col0_s.view(torch.uint8).cpu().numpy(), sT)
 
     w = (torch.randn(64, 96, device=gpu) * 0.05).bfloat16()  # weight recipe: 2-D blocks
     wr, wrs, wc, wcs = m4._quantize_weight_dual(w)
@@ -299,11 +304,11 @@ def test_mxfp4_dual_quantize_op_matches_oracle_bytes(mg, gpu):
     assert np.array_equal(wrs.view(torch.uint8).cpu().numpy()[:, :3], s)
     assert np.array_equal(wc.view(torch.uint8).cpu().numpy()[:, :32], qt)
     assert np.array_equal(wcs.view(torch.uint8).cpu().numpy()[:, :2], st)
-    with pytest.raises(NotImplementedError, match="colwise_use_rht"):
-        m4._quantize_input_dual(x, use_rht=True)
+    with pytest.raises(NotImplementedError, match="rowwise_use_rht"):
+        m4._quantize_mxfp4_dual_op(x, m4._FP4_DTYPE, 128, False, False, True, False, False, True, False, False, False, False)
     with pytest.raises(NotImplementedError, match="shuffle_rowwise_scale"):
         m4._quantize_grad_dual(x, preshuffle=True)
-    # stochastic rounding keeps shapes and scales (the codes are checked in test_gpu_sr.py)
+    # stochastic rounding keeps shapes and scales (the codes are checked in test_gpu_fp4_options.py)
     sr = m4._quantize_grad_dual(x, use_sr=True)
     assert torch.equal(sr[1].view(torch.uint8), row_s.view(torch.uint8)) and sr[0].shape == row.shape
 

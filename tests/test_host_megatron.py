@@ -706,9 +706,10 @@ def test_dual_quantize_recipes_per_operand(monkeypatch):
     mxfp4_local._quantize_input_dual(x, preshuffle=True, use_rht=True)
     fp4, pad = torch.float4_e2m1fn_x2, 128
     #            dtype pad  r2d   rsr    rrht   c2d   csr    crht   shuffles
-    assert calls[0] == (fp4, pad, False, False, False, False, False, False, False, False, False, False)
+    # activations and gradients: transform on the col-wise copy (the reference's recipes, :234-250, :272-288)
+    assert calls[0] == (fp4, pad, False, False, False, False, False, True, False, False, False, False)
     assert calls[1] == (fp4, pad, True, False, False, True, False, False, False, False, False, False)
-    assert calls[2] == (fp4, pad, False, True, False, False, True, False, False, False, False, False)
+    assert calls[2] == (fp4, pad, False, True, False, False, True, True, False, False, False, False)
     # the reference's activation recipe: transform on the col-wise copy only; shuffled scales, shuffled col data
     assert calls[3] == (fp4, pad, False, False, False, False, False, True, True, False, True, True)
 

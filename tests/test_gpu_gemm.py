@@ -125,6 +125,77 @@ def test_exact_integer_products_bit_exact(gpu):
     assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want)
 
 
+def _exact_operands(rng, rows, k, fmt):
+    """Codes whose values are small multiples of 1/2 and scales within 2^-2..2^2: all products and all
+    partial sums of a row of a few hundred of them are exact in fp32."""
+    if fmt == o.FMT_E4M3:
+        q, s = _int_operands(rng, rows, k)
+        return q, s
+    nib = rng.integers(0, 16, size=(rows, k)).astype(np.uint8)          # every E2M1 value is a multiple of 1/2
+    return o.pack_fp4(nib), rng.integers(125, 130, size=(rows, k // 32)).astype(np.uint8)
+
+
+@pytest.mark.parametrize("afmt,bfmt", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("lens,n,k", [([300, 0, 77, 135], 288, 384), ([513], 256, 128), ([1, 0, 255, 257, 31], 96, 512),
+                                      ([40] * 12, 544, 256)])
+def test_exact_products_bit_exact_all_formats(gpu, afmt, bfmt, lens, n, k):
+    """Forward / dgrad kernel, every operand-format pair: bit-equal to the oracle on operands whose
+    arithmetic is exact, i.e. independent of accumulation order -- every output element, not a norm."""
+    from primus_amd.pytorch import kernels as K
+
+    rng = np.random.default_rng(afmt * 7 + bfmt * 3 + n + k)
+    m, G = sum(lens), len(lens)
+    aq, as_ = _exact_operands(rng, m, k, afmt)
+    bq, bs = _exact_operands(rng, G * n, k, bfmt)
+    bq, bs = bq.reshape(G, n, -1), bs.reshape(G, n, k // 32)
+    want = o.grouped_gemm_nt_ref(aq, as_, bq, bs, lens, afmt, bfmt)
+    A, SA = _dev(aq, gpu, _dt(afmt)), _dev(as_, gpu, torch.float8_e8m0fnu)
+    B, SB = _dev(bq, gpu, _dt(bfmt)), _dev(bs, gpu, torch.float8_e8m0fnu)
+    if G == 1:
+        got = K.gemm_mx_nt_impl(A, SA, B[0], SB[0])
+    else:
+        got = K.grouped_gemm_mx_nt_impl(A, SA, B, SB, torch.tensor(lens, dtype=torch.int64, device=gpu))
+    assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want)
+
+
+@pytest.mark.parametrize("afmt,bfmt", [(0, 0), (1, 1), (0, 1)])
+@pytest.mark.parametrize("lens,n,k", [([300, 0, 77, 135], 288, 160), ([513], 256, 128), ([1, 0, 255, 257, 31], 96, 320)])
+def test_wgrad_exact_products_bit_exact(gpu, afmt, bfmt, lens, n, k):
+    """Variable-K wgrad kernel on exact operands in the segment-padded transposed layout (zero codes in
+    the padding): bit-equal to the oracle, empty experts exactly zero."""
+    from primus_amd.pytorch import kernels as K
+
+    rng = np.random.default_rng(afmt * 5 + bfmt + n + k)
+    m, G = sum(lens), len(lens)
+    W = o.padded_width(m, G)
+    _, poffs = o.segment_layout(lens)
+    live = np.zeros(W, dtype=bool)
+    for g, ln in enumerate(lens):
+        live[poffs[g] : poffs[g] + ln] = True
+
+    def operand(rows, fmt):
+        q, s = _exact_operands(rng, rows, W, fmt)
+        if fmt == o.FMT_E2M1:
+            nib = o.unpack_fp4(q)
+            nib[:, ~live] = 0
+            q = o.pack_fp4(nib)
+        else:
+            q[:, ~live] = 0
+        return q, s
+
+    aq, as_ = operand(n, afmt)
+    bq, bs = operand(k, bfmt)
+    want = o.grouped_gemm_wgrad_ref(aq, as_, bq, bs, lens, afmt, bfmt)
+    got = K.grouped_gemm_mx_wgrad_impl(_dev(aq, gpu, _dt(afmt)), _dev(as_, gpu, torch.float8_e8m0fnu),
+                                       _dev(bq, gpu, _dt(bfmt)), _dev(bs, gpu, torch.float8_e8m0fnu),
+                                       torch.tensor(lens, dtype=torch.int64, device=gpu), m)
+    got = got.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    for g, ln in enumerate(lens):
+        if ln == 0:
+            assert not got[g].any()
+
+
 @pytest.mark.parametrize(
     "lens,n,k",
     [([300, 0, 5, 695], 320, 288), ([128], 256, 256), ([0, 33, 1, 64], 96, 160), ([0, 0], 64, 32), ([200, 200, 200], 512, 96)],

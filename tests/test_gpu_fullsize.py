@@ -178,3 +178,68 @@ def test_full_size_linear(gpu, workload, layer):
             if ln == 0:
                 assert not dw[g].any()
         assert y.shape == (M, n) and dx.shape == (M, k) and dw.shape == (G, n, k)
+
+
+def _exact_codes(gen, rows, k, dev):
+    """E4M3 codes of small integers (0, +-1, +-2, +-3, 4) and scales 2^-1..2^1: every product and every
+    partial sum over a few thousand of them is exact in fp32, whatever the accumulation order."""
+    vals = torch.tensor([0x00, 0x38, 0x40, 0x44, 0x48, 0xB8, 0xC0, 0xC4], dtype=torch.uint8, device=dev)
+    q = vals[torch.randint(0, 8, (rows, k), generator=gen, device=dev)]
+    s = torch.randint(126, 129, (rows, k // 32), generator=gen, device=dev, dtype=torch.uint8)
+    return q.view(torch.float8_e4m3fn), s.view(torch.float8_e8m0fnu)
+
+
+def test_full_size_mixtral_every_output_bit_exact(gpu):
+    """Mixtral fc1 at full size (32 768 routed rows, ragged over 8 experts, [8, 28672, 4096] weights) on
+    exactly representable operands: EVERY element of the forward output and of the weight gradient
+    equals the fp32 matrix product of the dequantised operands bit for bit (the exact result does not
+    depend on summation order, so the fp32 library GEMM is a valid reference at this size, where the
+    CPU oracle would need hours; the dequantiser used to build it is itself tested against the oracle)."""
+    from primus_amd.pytorch import kernels as K
+
+    spec = bench.WORKLOADS["mixtral_8x7b_moe_mxfp8"]
+    lens = bench.route(spec)
+    G, M, k, n = spec["G"], sum(lens), spec["hidden"], spec["fc1_out"]
+    gen = torch.Generator(device=gpu).manual_seed(77)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+
+    # forward: Y = X . W_g^T per expert
+    xq, xs = _exact_codes(gen, M, k, gpu)
+    wq, ws = _exact_codes(gen, G * n, k, gpu)
+    y = K.grouped_gemm_mx_nt_impl(xq, xs, wq.view(G, n, k), ws.view(G, n, k // 32), gl)
+    xf = K.dequantize_mx_impl(xq, xs).float()
+    wf = K.dequantize_mx_impl(wq, ws).float().view(G, n, k)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        want = (xf[a:b] @ wf[g].T).bfloat16()
+        assert torch.equal(y[a:b], want), g
+    del y, wq, ws, wf
+
+    # wgrad: dW_g = dY_g^T . X_g on the segment-padded transposed layout (zero codes in the padding).  Row-wise
+    # scales do not transpose into per-32-token blocks, so the transposed operands reuse the CODES with scale 1.
+    W = K.padded_width(M, G)
+    _, poffs = o.segment_layout(lens)
+    nd = 512                                                      # a 512-column slice of dY keeps the test short
+    dq, _ = _exact_codes(gen, M, nd, gpu)
+
+    def unit_scales(rows, cols):
+        return torch.full((rows, cols // 32), 127, dtype=torch.uint8, device=gpu).view(torch.float8_e8m0fnu)
+
+    def transposed(codes_rows):
+        cols = codes_rows.shape[1]
+        qT = torch.zeros(cols, W, dtype=torch.uint8, device=gpu)
+        for g in range(G):
+            a, b, p = int(offs[g]), int(offs[g + 1]), int(poffs[g])
+            qT[:, p : p + (b - a)] = codes_rows.view(torch.uint8)[a:b].T
+        return qT.view(torch.float8_e4m3fn), unit_scales(cols, W)
+
+    dyf = K.dequantize_mx_impl(dq, unit_scales(M, nd)).float()
+    xf1 = K.dequantize_mx_impl(xq, unit_scales(M, k)).float()
+    dqT, dsT = transposed(dq)
+    xqT, xsT = transposed(xq)
+    dw = K.grouped_gemm_mx_wgrad_impl(dqT, dsT, xqT, xsT, gl, M)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        want = (dyf[a:b].T @ xf1[a:b]).bfloat16()
+        assert torch.equal(dw[g], want), g

@@ -513,14 +513,19 @@ static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tile
 
 using namespace mxl;
 
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t words) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < words) dst[i] = 0u;
+}
+
 extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                                    const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                                    int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
-    if (!a_codes || !a_scales || !b_codes || !b_scales || !c_bf16) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if (num_groups > 1 && !group_lens) return MXL_EINVAL;
-    if (total_m == 0) return MXL_OK;
+    if (total_m == 0) return MXL_OK;   // no rows: nothing to read or write (the row operands may be null)
+    if (!a_codes || !a_scales || !b_codes || !b_scales || !c_bf16) return MXL_EINVAL;
     GemmArgs a;
     a.a = (const uint8_t*)a_codes;
     a.sa = (const uint8_t*)a_scales;
@@ -547,11 +552,26 @@ extern "C" int mxl_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt,
 extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                                       const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                                       int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
-    if (!a_codes || !a_scales || !b_codes || !b_scales || !c_bf16) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
     if (num_groups < 0 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if ((num_groups > 0) != (group_lens != nullptr)) return MXL_EINVAL;
     const int G = num_groups > 0 ? num_groups : 1;
+    if (!c_bf16) return MXL_EINVAL;
+    // a padded width of 0 (no tokens, one group) leaves nothing to read: the operands may be null and the
+    // kernel only writes the zero gradient
+    const bool nothing_to_read = mxl_padded_width(total_m, G) == 0;
+    if (nothing_to_read) {
+        // The GEMM kernel requests the first K slot of every tile unconditionally, so it is never launched on
+        // operands that do not exist; a fill kernel (not a memset, which callers could not capture in a graph)
+        // writes the zero gradient.
+        const int64_t words = (int64_t)G * n * k / 2;   // n and k are multiples of 32
+        const int64_t grid = (words + 255) / 256;
+        if (grid > 0x7FFFFFFF) return MXL_EINVAL;
+        hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (uint32_t*)c_bf16,
+                           words);
+        return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+    }
+    if (!a_codes || !a_scales || !b_codes || !b_scales) return MXL_EINVAL;
     GemmArgs a;
     a.a = (const uint8_t*)a_codes;
     a.sa = (const uint8_t*)a_scales;
@@ -564,7 +584,6 @@ extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales,
     a.m = n;  // rows of the output per group
     a.n = k;  // columns of the output
     a.k = mxl_padded_width(total_m, G);
-    if (a.k == 0) a.k = MXL_SEG_ALIGN;  // keeps pitches non-zero; no tile reads it
     const int64_t max_tiles = (int64_t)G * ((n + BM - 1) / BM) * ((k + BN - 1) / BN);
     return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (hipStream_t)stream);
 }

@@ -157,7 +157,7 @@ def test_fused_activation_quantize_equals_two_kernels(gpu, activation, fmt, lens
 
 @pytest.mark.parametrize("activation", ["silu", "gelu"])
 @pytest.mark.parametrize("fp4", [False, True])
-@pytest.mark.parametrize("lens,f,n", [([33, 0, 130, 1, 92], 160, 96), ([300, 212], 512, 256)])
+@pytest.mark.parametrize("lens,f,n", [([33, 0, 130, 1, 92], 160, 96), ([300, 212], 512, 256), ([0, 0], 64, 32)])
 def test_glu_grouped_gemm_equals_activation_then_grouped_gemm(gpu, activation, fp4, lens, f, n):
     """ops.glu_grouped_gemm_fp8 / _fp4 give exactly what the activation operator followed by the
     grouped GEMM operator gives -- output, and the gradients of fc1's output, the probabilities and

@@ -72,6 +72,30 @@ def test_grouped_gemm_fp8_fwd_bwd(gpu, lens):
     assert torch.equal(y2, y.detach())
 
 
+@pytest.mark.parametrize("fp4", [False, True])
+def test_no_tokens_at_all(gpu, fp4):
+    """A step in which no token reaches this rank's experts (and a dense linear on an empty batch):
+    empty output, empty input gradient, all-zero weight gradient, no error."""
+    import primus_amd.pytorch as pt
+    from primus_amd.pytorch.core import Float4QuantConfig
+
+    cfg = Float4QuantConfig() if fp4 else _cfg8()
+    grouped = pt.ops.grouped_gemm_fp4 if fp4 else pt.ops.grouped_gemm_fp8
+    dense = pt.ops.gemm_fp4 if fp4 else pt.ops.gemm_fp8
+    x = torch.empty(0, 160, device=gpu, dtype=torch.bfloat16, requires_grad=True)
+    w = (torch.randn(3, 96, 160, device=gpu) * 0.05).bfloat16().requires_grad_()
+    gl = torch.zeros(3, dtype=torch.int64, device=gpu)
+    y = grouped(x, w, gl, trans_b=True, config=cfg)
+    assert y.shape == (0, 96)
+    y.backward(torch.empty(0, 96, device=gpu, dtype=torch.bfloat16))
+    assert x.grad.shape == (0, 160) and w.grad.shape == w.shape and not w.grad.any()
+    w2 = w.detach()[0].clone().requires_grad_()
+    x2 = torch.empty(0, 160, device=gpu, dtype=torch.bfloat16, requires_grad=True)
+    y2 = dense(x2, w2, trans_a=False, trans_b=True, out_dtype=None, config=cfg)
+    y2.backward(torch.empty(0, 96, device=gpu, dtype=torch.bfloat16))
+    assert y2.shape == (0, 96) and not w2.grad.any()
+
+
 def test_cached_weight_pair_matches_bf16_weight_path(gpu):
     """QuantizedTensorPair path (primus_turbo.py:1105-1134): same bytes as
     quantising inside the op, gradient flows to pair.data."""

@@ -294,3 +294,36 @@ def test_bad_arguments_return_errors(gpu):
     lens = torch.tensor([4], dtype=torch.int32, device=gpu)
     with pytest.raises(ValueError):
         K.grouped_gemm_mx_nt_impl(a, s, b[None, :, :64].contiguous(), sb[None, :, :2].contiguous(), lens)  # int32 lens
+
+
+def test_one_thousand_experts(gpu):
+    """The largest expert count the device-side tile tables hold (1024), most experts with 0-3 rows:
+    forward and wgrad against the oracle; one more expert is refused with an error, not a fault."""
+    from primus_amd import _lib
+    from primus_amd.pytorch import kernels as K
+
+    rng = np.random.default_rng(1024)
+    G, n, k = _lib.MAX_GROUPS, 64, 128
+    lens = rng.integers(0, 4, size=G).tolist()
+    lens[17] = 300
+    m = sum(lens)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(G, n, k, generator=g) * 0.05).bfloat16()
+    got, want = _run_fwd(gpu, x, w, lens, o.FMT_E4M3, o.FMT_E4M3)
+    _check(got, want)
+    dy = torch.randn(m, n, generator=g).bfloat16()
+    dyT, dysT = o.quantize_mx_colwise_segmented(dy, lens, o.FMT_E4M3)
+    xT, xsT = o.quantize_mx_colwise_segmented(x, lens, o.FMT_E4M3)
+    want = o.grouped_gemm_wgrad_ref(dyT, dysT, xT, xsT, lens, out_bf16=False)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    dw = _bf16_np(K.grouped_gemm_mx_wgrad_impl(
+        _dev(dyT, gpu, torch.float8_e4m3fn), _dev(dysT, gpu, torch.float8_e8m0fnu), _dev(xT, gpu, torch.float8_e4m3fn),
+        _dev(xsT, gpu, torch.float8_e8m0fnu), gl, m))
+    _check(dw, want)
+    # the quantiser writes the same transposed layout for that many groups
+    q = K.quantize_mx_impl(x.to(gpu), o.FMT_E4M3, rowwise=False, colwise=True, group_lens=gl)
+    assert np.array_equal(q[2].view(torch.uint8).cpu().numpy(), xT) and np.array_equal(q[3].view(torch.uint8).cpu().numpy(), xsT)
+    too_many = torch.zeros(G + 1, dtype=torch.int64, device=gpu)
+    with pytest.raises(Exception):
+        K.quantize_mx_impl(x.to(gpu), o.FMT_E4M3, rowwise=False, colwise=True, group_lens=too_many)

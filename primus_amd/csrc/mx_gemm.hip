@@ -160,18 +160,28 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     const uint32_t smem_base = (uint32_t)(uintptr_t)smem;  // LDS byte address of the ring
 
     // ---- per-workgroup group tables (device-side, no host sync) ----
+    // The lens are fetched by all threads at once and summed by one.  They are clamped to what the
+    // operands hold (no negative length; the running sum never passes total_m, resp. the padded width),
+    // so that lens which do not match the buffers cannot send a tile outside them.
+    for (int i = t; i < G; i += GTHREADS) pre_rows[i + 1] = p.group_lens ? p.group_lens[i] : p.total_m;
+    __syncthreads();
     if (t == 0) {
         int tiles = 0;
         int64_t rows = 0;
+        const int64_t cap = (MODE == MODE_FWD) ? p.total_m : p.k;
         pre_tiles[0] = 0;
         pre_rows[0] = 0;
         for (int i = 0; i < G; ++i) {
-            const int64_t len = p.group_lens ? p.group_lens[i] : p.total_m;
+            int64_t len = pre_rows[i + 1];
+            len = len < 0 ? 0 : len;
             if (MODE == MODE_FWD) {
+                len = len > cap - rows ? cap - rows : len;
                 tiles += (int)((len + BM - 1) / BM);
                 rows += len;
             } else {
-                rows += (len + MXL_SEG_ALIGN - 1) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
+                int64_t seg = (len + MXL_SEG_ALIGN - 1) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
+                seg = seg > cap - rows ? cap - rows : seg;
+                rows += seg;
             }
             pre_tiles[i + 1] = tiles;
             pre_rows[i + 1] = rows;

@@ -136,7 +136,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         int64_t off = 0;
         int pto = 0;
         for (int g = 0; g < a.num_groups; ++g) {
-            const int64_t len = a.group_lens[g];
+            // clamped to the rows that exist, so that lens which do not match the buffer cannot read outside it
+            int64_t len = a.group_lens[g];
+            len = len < 0 ? 0 : (len > a.rows - off ? a.rows - off : len);
             const int nt = (int)((len + QT - 1) / QT);
             if (pt < pto + nt) {
                 const int64_t r = (int64_t)(pt - pto) * QT;

@@ -327,3 +327,32 @@ def test_one_thousand_experts(gpu):
     too_many = torch.zeros(G + 1, dtype=torch.int64, device=gpu)
     with pytest.raises(Exception):
         K.quantize_mx_impl(x.to(gpu), o.FMT_E4M3, rowwise=False, colwise=True, group_lens=too_many)
+
+
+@pytest.mark.parametrize("bad,clamped", [([200, 300], [200, 56]), ([-5, 256, 9], [0, 256, 0]), ([1000, 1000], [256, 0])])
+def test_group_lens_that_do_not_match_the_buffers_are_clamped(gpu, bad, clamped):
+    """Token counts live on the device, so no host check can catch counts that disagree with the
+    buffers (stale or corrupted counts).  The kernels clamp them -- negative to 0, the running sum to
+    the rows that exist -- and so behave exactly as for the clamped counts instead of leaving the
+    buffers."""
+    from primus_amd.pytorch import kernels as K
+
+    rows, k, n = 256, 128, 64
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(rows, k, generator=g).bfloat16().to(gpu)
+    w = (torch.randn(len(bad), n, k, generator=g) * 0.05).bfloat16().to(gpu)
+    dy = torch.randn(rows, n, generator=g).bfloat16().to(gpu)
+    outs = []
+    for lens in (bad, clamped):
+        gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+        xq, xs, xqT, xsT = K.quantize_mx_impl(x, o.FMT_E4M3, rowwise=True, colwise=True, group_lens=gl, pad_to=128)
+        _, _, dqT, dsT = K.quantize_mx_impl(dy, o.FMT_E4M3, rowwise=False, colwise=True, group_lens=gl)
+        wq, ws, _, _ = K.quantize_mx_weight_2d_impl(w, o.FMT_E4M3, rowwise=True, colwise=False, pad_to=128)
+        y = K.grouped_gemm_mx_nt_impl(xq, xs, wq, ws, gl)
+        dw = K.grouped_gemm_mx_wgrad_impl(dqT, dsT, xqT, xsT, gl, rows)
+        covered = sum(clamped)
+        outs.append((xq.view(torch.uint8)[:covered], xs.view(torch.uint8)[:covered], xqT.view(torch.uint8),
+                     xsT.view(torch.uint8), y[:covered], dw))
+    torch.cuda.synchronize()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)

@@ -220,6 +220,14 @@ def main():
         dy = torch.randn(M, n, generator=gen, device=dev).bfloat16()
         layers.append((x, w, dy, k, n))
     gl = torch.tensor(lens, dtype=torch.int64, device=dev)
+    if not spec.get("wgrad", True):
+        # Without a weight gradient the weights cannot change between steps: they are quantised once, before
+        # the timed region, and the steps run on the cached copies (the reference's multi-microbatch path,
+        # primus/backends/megatron/core/extensions/primus_turbo.py:1105-1115).
+        from primus_amd.pytorch.core import QuantizedTensorPair, create_quantized_weight, float4_e2m1fn_x2, float8_e4m3
+
+        dest = float4_e2m1fn_x2 if spec["fp4"] else float8_e4m3
+        layers = [(x, QuantizedTensorPair(*create_quantized_weight(w, dest, cfg)), dy, k, n) for (x, w, dy, k, n) in layers]
     # forward + dgrad (+ wgrad unless the workload is defined without it): 2 M N K flops each
     passes = 3.0 if spec.get("wgrad", True) else 2.0
     flops_step = sum(2.0 * passes * M * n * k for (_, _, _, k, n) in layers)
@@ -232,7 +240,8 @@ def main():
                 y = pt.ops.gemm_fp8(x, w, trans_a=False, trans_b=True, out_dtype=None, config=cfg)
             y.backward(dy)
             x.grad = None
-            w.grad = None
+            if torch.is_tensor(w):
+                w.grad = None
 
     if args.calibrate_traffic:
         src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)   # 1 GiB

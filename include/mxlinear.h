@@ -141,7 +141,9 @@ int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t 
  * primus_turbo_float8_local.py:239-250, primus_turbo_mxfp4_local.py:319-331):
  *   c[m, n] (bf16) = dq(a)[m, k] . dq(b)[n, k]^T, fp32 accumulation.
  * Requires k % 128 == 0 (scale rows must be dword aligned; callers get there
- * with the row_ld / k_ld padding of the quantisers) and n % 32 == 0. */
+ * with the row_ld / k_ld padding of the quantisers) and n % 32 == 0.  The contraction length (k here, the
+ * padded token width in mxl_grouped_gemm_wgrad) may not exceed 2^23.  group_lens of the grouped entry points
+ * are clamped on the device to what the buffers hold (negative counts to 0, the running sum to total_m). */
 int mxl_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                 const void* b_scales, int b_fmt, void* c_bf16, int64_t m, int64_t n, int64_t k,
                 void* stream);

@@ -523,6 +523,9 @@ static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tile
 
 using namespace mxl;
 
+// Offsets inside a tile's operand rows (up to 256 rows of the contraction length) are 32-bit.
+constexpr int64_t MAX_CONTRACTION = (int64_t)1 << 23;
+
 __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t words) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < words) dst[i] = 0u;
@@ -532,6 +535,7 @@ extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, in
                                    const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                                    int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
+    if (k > MAX_CONTRACTION) return MXL_EINVAL;   // tile-relative byte offsets are 32-bit
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if (num_groups > 1 && !group_lens) return MXL_EINVAL;
     if (total_m == 0) return MXL_OK;   // no rows: nothing to read or write (the row operands may be null)
@@ -569,6 +573,7 @@ extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales,
     if (!c_bf16) return MXL_EINVAL;
     // a padded width of 0 (no tokens, one group) leaves nothing to read: the operands may be null and the
     // kernel only writes the zero gradient
+    if (mxl_padded_width(total_m, G) > MAX_CONTRACTION) return MXL_EINVAL;
     const bool nothing_to_read = mxl_padded_width(total_m, G) == 0;
     if (nothing_to_read) {
         // The GEMM kernel requests the first K slot of every tile unconditionally, so it is never launched on

@@ -9,11 +9,13 @@
 // derived on the device from group_lens, so nothing is read back to the host
 // and empty experts cost nothing.  A workgroup (4 waves, 2x2) owns a 256x256
 // output tile; each wave a 128x128 sub-tile = 4x4 MFMA tiles of 32x32 with
-// fp32 accumulators (256 accumulator registers per lane).  K advances 64
-// elements (2 MX blocks, one MFMA K step) per stage through a 4-stage LDS ring
-// that is filled by asynchronous global->LDS loads (buffer_load ... lds), three
-// stages ahead; fragments of stage s+1 are read from LDS while the MFMAs of
-// stage s run, so there is one barrier per stage and no register staging.
+// fp32 accumulators (256 accumulator registers per lane).  K advances in slots of 128
+// elements -- one full 128-byte line per FP8 row, two MFMA K steps of 64 (two MX blocks
+// each) -- through a 2-slot LDS ring (2 x 64 KiB) that is filled by asynchronous
+// global->LDS loads (buffer_load ... lds).  The requests for the next slots are spread
+// between the MFMAs of the current one, and the fragments of K step s+1 are read from LDS
+// while the MFMAs of step s run: one barrier per K step, no register staging.  E8M0 scales
+// travel in double-buffered "panels" (16 bytes per row = the scales of 8 K slots).
 // 16-byte chunks are XOR-swizzled so the fragment reads are bank-conflict free.
 //
 // MFMA operand layout (measured on gfx950): lane l holds row l%32; its 32
@@ -83,13 +85,6 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, int64_t bytes) {
 }
 __device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds_off), "v"(voff), "s"(rsrc), "s"(soff)
-                 : "memory");
-}
-// two scale bytes of one row, zero-extended into that lane's LDS dword
-__device__ __forceinline__ void dma2(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, %3 offen lds"
                  :
                  : "s"(lds_off), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory");

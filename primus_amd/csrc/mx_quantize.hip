@@ -151,6 +151,19 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         }
     }
 
+    // fused activation: the tile's 128 probabilities (and row-mask bits) are fetched once by 128 lanes and
+    // handed round through LDS; fetched per lane and row they would double the number of load instructions
+    __shared__ float prob_tile[ACT >= 0 ? QT : 1];
+    __shared__ uint8_t live_tile[ACT >= 0 ? QT : 1];
+    if (ACT >= 0) {
+        if (t < QT) {
+            const bool live = t < rows_valid && (a.row_mask == nullptr || a.row_mask[src_row0 + t] != 0);
+            live_tile[t] = live ? 1 : 0;
+            prob_tile[t] = live ? load_prob(a.probs, a.probs_bf16, src_row0 + t) : 0.f;
+        }
+        __syncthreads();
+    }
+
     const int64_t col = col0 + 8 * c16;
     const bool col_ok = col < a.cols;      // source column exists
     const bool out_ok = col < a.row_ld;    // row-wise output column exists (padding is written as zeros)
@@ -165,11 +178,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             if (ACT < 0) {
                 d[it] = load16_streaming(a.x + (src_row0 + r) * a.cols + col);
             } else {
-                const int64_t row = src_row0 + r;
-                if (a.row_mask == nullptr || a.row_mask[row] != 0) {
-                    const uint16_t* xr = a.x + row * 2 * a.cols + col;
-                    d[it] = glu8<(ACT < 0 ? 0 : ACT)>(load16_streaming(xr), load16_streaming(xr + a.cols),
-                                                      load_prob(a.probs, a.probs_bf16, row));
+                if (live_tile[r]) {
+                    const uint16_t* xr = a.x + (src_row0 + r) * 2 * a.cols + col;
+                    d[it] = glu8<(ACT < 0 ? 0 : ACT)>(load16_streaming(xr), load16_streaming(xr + a.cols), prob_tile[r]);
                 }
             }
         }

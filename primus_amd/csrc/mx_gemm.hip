@@ -428,7 +428,12 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         // requests above do not touch), so that the global stores are 16 bytes per lane and each
         // store instruction covers 4 rows x 256 contiguous bytes ----
         {
-            constexpr int SP = 272;  // bytes per staged row (256 + 16: spreads the rows over the banks)
+            // bytes per staged row: 256 + 16 spreads the rows over the banks; with two FP4 operands ring slot 1
+            // is only 32 KiB, which the four 32-row patches fill exactly without the padding -- a padded patch
+            // would reach into the scale panels behind the ring, which the next tile's first requests are
+            // already writing
+            constexpr int SP = (4 * 32 * 272 <= STAGE) ? 272 : 256;
+            static_assert(4 * 32 * SP <= STAGE, "the epilogue patches must stay inside ring slot 1");
             uint8_t* stg = smem + STAGE + w * (32 * SP);
             uint8_t* wr = stg + lr * SP + 8 * g;                   // this lane's row while writing
             const uint8_t* rd = stg + (l >> 4) * SP + (l & 15) * 16;  // this lane's 16 bytes while reading

@@ -115,6 +115,7 @@ extern "C" int mxl_glu_probs_fwd(const void* x_bf16, const void* probs, int prob
                                  int64_t rows, int64_t f, int act, void* y_bf16, void* stream) {
     if (!act_args_ok(x_bf16, y_bf16, probs, probs_dtype, rows, f, act)) return MXL_EINVAL;
     if (rows == 0) return MXL_OK;
+    if (!device_is_gfx950()) return MXL_ENODEV;
     const dim3 grid((unsigned)rows), block(ATHREADS);
     hipStream_t st = (hipStream_t)stream;
     if (act == MXL_ACT_SILU)
@@ -132,6 +133,7 @@ extern "C" int mxl_glu_probs_bwd(const void* dy_bf16, const void* x_bf16, const 
     if (!act_args_ok(x_bf16, dx_bf16, probs, probs_dtype, rows, f, act)) return MXL_EINVAL;
     if (rows == 0) return MXL_OK;
     if (!dy_bf16 || !dprobs_f32) return MXL_EINVAL;
+    if (!device_is_gfx950()) return MXL_ENODEV;
     const dim3 grid((unsigned)rows), block(ATHREADS);
     hipStream_t st = (hipStream_t)stream;
     if (act == MXL_ACT_SILU)

@@ -5,7 +5,28 @@
 
 #include "../../include/mxlinear.h"
 
+#include <string.h>
+
+#include <atomic>
+
 namespace mxl {
+
+// Host side: is the current device a gfx950?  The kernels exist for that target only; every entry point
+// asks before its first launch on a device (answer cached per device index) and returns MXL_ENODEV otherwise.
+inline bool device_is_gfx950() {
+    static std::atomic<int> known[64];   // 0 unknown, 1 yes, 2 no
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    const int slot = dev & 63;
+    int v = known[slot].load(std::memory_order_relaxed);
+    if (v == 0) {
+        hipDeviceProp_t pr;
+        if (hipGetDeviceProperties(&pr, dev) != hipSuccess) return false;
+        v = strncmp(pr.gcnArchName, "gfx950", 6) == 0 ? 1 : 2;
+        known[slot].store(v, std::memory_order_relaxed);
+    }
+    return v == 1;
+}
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));

@@ -25,7 +25,6 @@
 // four registers (low nibble first).  The kernel feeds the N-side operand as
 // MFMA source 0 so a lane ends up with 4 consecutive output columns (one
 // 8-byte bf16 store).
-#include <atomic>
 #include <type_traits>
 
 #include "mx_device.h"
@@ -496,6 +495,7 @@ static int num_cus() {
 template <int AFMT, int BFMT, int MODE>
 static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = gemm_lds_bytes(AFMT, BFMT);
+    if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set{false};
     auto kern = mx_gemm_kernel<AFMT, BFMT, MODE>;
     if (!attr_set.load(std::memory_order_acquire)) {
@@ -582,6 +582,7 @@ extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales,
         const int64_t words = (int64_t)G * n * k / 2;   // n and k are multiples of 32
         const int64_t grid = (words + 255) / 256;
         if (grid > 0x7FFFFFFF) return MXL_EINVAL;
+        if (!device_is_gfx950()) return MXL_ENODEV;
         hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (uint32_t*)c_bf16,
                            words);
         return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;

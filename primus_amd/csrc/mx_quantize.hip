@@ -465,6 +465,7 @@ static int launch_quant(QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStrea
     const int64_t n_super = super_r * super_c;
     const int64_t wgs = (n_super + 7) / 8 * 8 * QSUPER * QSUPER;
     if (tiles_r > 0x7FFFFFFF || tiles_c > 0x7FFFFFFF || wgs > 0x7FFFFFFF) return MXL_EINVAL;
+    if (!device_is_gfx950()) return MXL_ENODEV;
     a.tiles_r = (int)tiles_r;
     a.tiles_c = (int)tiles_c;
     a.super_c = (int)super_c;
@@ -625,6 +626,8 @@ extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t row
     const int64_t threads = nblocks * 4;
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7FFFFFFF) return MXL_EINVAL;
+    if (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E2M1) return MXL_EINVAL;
+    if (!device_is_gfx950()) return MXL_ENODEV;
     if (fmt == MXL_FMT_E4M3)
         hipLaunchKernelGGL((mx_dequant_kernel<MXL_FMT_E4M3>), dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
                            (const uint8_t*)codes, (const uint8_t*)scales, (uint16_t*)out_bf16, nblocks);

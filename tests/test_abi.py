@@ -63,3 +63,20 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "lib_path", lambda: str(tmp_path / "nope.so"))
     with pytest.raises(_lib.MXLinearError, match="no fallback"):
         _lib.load()
+
+
+def test_without_a_gfx950_device_the_entry_points_refuse(lib):
+    """On a machine without a GPU a well-formed call returns MXL_ENODEV before anything is launched
+    (bad arguments are still reported as such first)."""
+    import torch
+
+    if torch.cuda.device_count() > 0:
+        pytest.skip("a GPU is present: this call would be a real launch")
+    buf = ctypes.create_string_buffer(128 * 128 * 2)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.mxl_quantize(p, 128, 128, 128, _lib.FMT_E4M3, 0, None, 0, p, p, None, None, None) == -3
+    assert lib.mxl_quantize(p, 128, 100, 128, _lib.FMT_E4M3, 0, None, 0, p, p, None, None, None) == -1   # cols % 32
+    assert lib.mxl_gemm_nt(p, p, 0, p, p, 0, p, 128, 128, 128, None) == -3
+    assert lib.mxl_gemm_nt(p, p, 0, p, p, 0, p, 128, 128, 100, None) == -1                                 # k % 128
+    assert lib.mxl_glu_probs_fwd(p, p, 0, None, 4, 32, 0, p, None) == -3
+    assert lib.mxl_error_string(-3).decode().startswith("device")

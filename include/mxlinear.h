@@ -90,9 +90,20 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
                  const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                  void* s_colT, void* stream);
 
-/* MXFP4 (E2M1) quantisation with the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
- * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288).  Arguments as for mxl_quantize
- * with fmt = MXL_FMT_E2M1, plus `flags`:
+/* mxl_quantize with options (`flags`):
+ *
+ *   MXL_QF_KCHUNK  K-chunk-major code layout for both copies: instead of codes[rows, ld] the codes are stored
+ *                  as [ld / 128][rows][128 elements] (128 or 64 bytes), i.e. the 128 elements of a row that
+ *                  one GEMM K slot consumes stay together and consecutive rows follow each other.  A GEMM
+ *                  tile's K slot is then one contiguous block (256 rows x 128 bytes) wherever a ragged
+ *                  expert starts, and the quantiser writes 16 KiB pieces instead of 128-byte ones.  Needs
+ *                  row_ld % 128 == 0.  The transposed copy becomes [W / 128][cols][128].  Scales keep their
+ *                  row-major layout.  The GEMM entry points take such operands with MXL_GF_KCHUNK.  This is
+ *                  the role the reference's pre-shuffled layouts play for its kernels (use_preshuffle,
+ *                  primus_turbo_mxfp4_local.py:184-198); the arrangement itself is this library's own.
+ *
+ * and, for fmt = MXL_FMT_E2M1 only, the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
+ * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288):
  *
  *   MXL_QF_SR      stochastic rounding of the codes of both copies (rowwise_use_sr / colwise_use_sr;
  *                  config flag mxfp4_gradient_stochastic_rounding,
@@ -114,9 +125,10 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
  *                  remaining padding holds +-0 codes. */
 #define MXL_QF_SR 1u
 #define MXL_QF_RHT_COL 2u
-int mxl_quantize_fp4_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int scale_mode,
-                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                        void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);
+#define MXL_QF_KCHUNK 4u
+int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
+                    const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                    void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);
 
 /* 2-D (32x32 tile) MX quantisation of `batch` independent weight matrices
  * w[batch, n, k] (weights use ScalingRecipe(use_2d_block=True):
@@ -131,6 +143,11 @@ int mxl_quantize_fp4_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t 
 int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
                            int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
                            void* stream);
+/* The same with `flags` (MXL_QF_KCHUNK: both copies K-chunk-major over the flattened batch, i.e.
+ * [k_ld / 128][batch * n][128] and [n_ld / 128][batch * k][128]; needs k_ld % 128 == 0 resp. n_ld % 128 == 0). */
+int mxl_quantize_weight_2d_ex(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
+                              int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
+                              void* s_colT, uint32_t flags, void* stream);
 
 /* Row-wise dequantise to bf16 (QuantizedTensor.dequantize(),
  * weight_deosc.py:155-168): out[rows, k] = decode(codes) * 2^(scale-127). */
@@ -169,6 +186,18 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
                            const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
                            int64_t k, void* stream);
 
+/* The three GEMMs with `flags`.  MXL_GF_KCHUNK: both operands' CODES are K-chunk-major, as written by the
+ * quantisers with MXL_QF_KCHUNK -- [k / 128][rows][128 elements] over all rows of the operand (total_m rows
+ * of a and num_groups * n rows of b in the forward / dgrad GEMM; n rows of a and k rows of b over the padded
+ * token width in wgrad).  Scales stay row-major.  Same results bit for bit; an operand must stay below 4 GiB. */
+#define MXL_GF_KCHUNK 1u
+int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                           const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                           int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);
+int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                              const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                              int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);
+
 /* Gated activation of the expert MLP fused with the router probability and the row mask
  * (swiglu_with_probs / geglu_with_probs behind fused_bias_act_with_probs, primus_turbo.py:1954-1980;
  * the unfused arithmetic is experts.py:100-118):
@@ -190,11 +219,11 @@ int mxl_glu_probs_bwd(const void* dy_bf16, const void* x_bf16, const void* probs
  * write and one bf16 read of [rows, f] between fc1 and fc2 of the expert MLP; the reference runs
  * the activation and the quantisation inside gemm_fp8 as two kernels (experts.py:225-240,
  * primus_turbo.py:2122-2129).  x is [rows, 2 f]; the other arguments are those of mxl_quantize with
- * cols = f.  A row-wise copy must be requested (q_row / s_row not NULL). */
+ * cols = f.  A row-wise copy must be requested (q_row / s_row not NULL).  flags: 0 or MXL_QF_KCHUNK. */
 int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
                            int64_t rows, int64_t f, int64_t row_ld, int act, int fmt, int scale_mode,
                            const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                           void* s_colT, void* stream);
+                           void* s_colT, uint32_t flags, void* stream);
 
 #ifdef __cplusplus
 }

@@ -26,19 +26,23 @@ GEMM_K_ALIGN = 128  # the GEMM kernels take the contraction dim in multiples of 
 MAX_GROUPS = 1024
 ACT_SILU, ACT_GELU = 0, 1
 PROBS_F32, PROBS_BF16 = 0, 1
-QF_SR, QF_RHT_COL = 1, 2   # flags of mxl_quantize_fp4_ex
+QF_SR, QF_RHT_COL, QF_KCHUNK = 1, 2, 4   # flags of mxl_quantize_ex
+GF_KCHUNK = 1                            # flag of the GEMM _ex entry points: operands are K-chunk-major
 
 EXPORTS = (
     "mxl_version",
     "mxl_error_string",
     "mxl_padded_width",
     "mxl_quantize",
-    "mxl_quantize_fp4_ex",
+    "mxl_quantize_ex",
+    "mxl_quantize_weight_2d_ex",
     "mxl_quantize_weight_2d",
     "mxl_dequantize",
     "mxl_gemm_nt",
     "mxl_grouped_gemm_nt",
     "mxl_grouped_gemm_wgrad",
+    "mxl_grouped_gemm_nt_ex",
+    "mxl_grouped_gemm_wgrad_ex",
     "mxl_glu_probs_fwd",
     "mxl_glu_probs_bwd",
     "mxl_glu_probs_quantize",
@@ -77,15 +81,21 @@ def load() -> ctypes.CDLL:
         lib.mxl_padded_width.argtypes = [i64, i32]
         lib.mxl_quantize.restype = i32
         lib.mxl_quantize.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, vp]
-        lib.mxl_quantize_fp4_ex.restype = i32
-        lib.mxl_quantize_fp4_ex.argtypes = [vp, i64, i64, i64, i32, vp, i32, vp, vp, vp, vp, ctypes.c_uint32,
-                                            ctypes.c_uint64, ctypes.c_uint32, vp]
+        u32 = ctypes.c_uint32
+        lib.mxl_quantize_ex.restype = i32
+        lib.mxl_quantize_ex.argtypes = [vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, u32, ctypes.c_uint64, u32, vp]
+        lib.mxl_quantize_weight_2d_ex.restype = i32
+        lib.mxl_quantize_weight_2d_ex.argtypes = [vp, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, u32, vp]
         lib.mxl_quantize_weight_2d.restype = i32
         lib.mxl_quantize_weight_2d.argtypes = [vp, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         lib.mxl_dequantize.restype = i32
         lib.mxl_dequantize.argtypes = [vp, vp, i64, i64, i32, vp, vp]
         lib.mxl_gemm_nt.restype = i32
         lib.mxl_gemm_nt.argtypes = [vp, vp, i32, vp, vp, i32, vp, i64, i64, i64, vp]
+        lib.mxl_grouped_gemm_nt_ex.restype = i32
+        lib.mxl_grouped_gemm_nt_ex.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, ctypes.c_uint32, vp]
+        lib.mxl_grouped_gemm_wgrad_ex.restype = i32
+        lib.mxl_grouped_gemm_wgrad_ex.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, ctypes.c_uint32, vp]
         lib.mxl_grouped_gemm_nt.restype = i32
         lib.mxl_grouped_gemm_nt.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
         lib.mxl_grouped_gemm_wgrad.restype = i32
@@ -95,7 +105,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_glu_probs_bwd.restype = i32
         lib.mxl_glu_probs_bwd.argtypes = [vp, vp, vp, i32, vp, i64, i64, i32, vp, vp, vp]
         lib.mxl_glu_probs_quantize.restype = i32
-        lib.mxl_glu_probs_quantize.argtypes = [vp, vp, i32, vp, i64, i64, i64, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp]
+        lib.mxl_glu_probs_quantize.argtypes = [vp, vp, i32, vp, i64, i64, i64, i32, i32, i32, vp, i32, vp, vp, vp, vp,
+                                               ctypes.c_uint32, vp]
         _lib = lib
     return _lib
 

@@ -130,7 +130,10 @@ struct Frags {
     int sa[4], sb[4];
 };
 
-template <int AFMT, int BFMT, int MODE>
+// LAYOUT 0: operand codes row-major [rows, K].  LAYOUT 1: K-chunk-major [K / 128][rows][128 elements] (what the
+// quantisers write with MXL_QF_KCHUNK): the rows of a tile's K slot are one contiguous block, so a load round
+// fetches 4 KiB in a row instead of 16..64 row pieces; scales are row-major in both.
+template <int AFMT, int BFMT, int MODE, int LAYOUT>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     constexpr int A_BYTES = Op<AFMT>::tile_bytes, B_BYTES = Op<BFMT>::tile_bytes;
     constexpr int STAGE = A_BYTES + B_BYTES;            // one slot: K = 128 of both operands
@@ -207,8 +210,11 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 
     // per-thread constants of the global -> LDS mapping
     const int a_row = t / Op<AFMT>::cpr, b_row = t / Op<BFMT>::cpr;
-    const uint32_t a_voff = (uint32_t)(a_row * (int)lda + 16 * ((t % Op<AFMT>::cpr) ^ Op<AFMT>::swz(a_row)));
-    const uint32_t b_voff = (uint32_t)(b_row * (int)ldb + 16 * ((t % Op<BFMT>::cpr) ^ Op<BFMT>::swz(b_row)));
+    const uint32_t a_voff = (uint32_t)(a_row * (LAYOUT ? Op<AFMT>::kb : (int)lda) + 16 * ((t % Op<AFMT>::cpr) ^ Op<AFMT>::swz(a_row)));
+    const uint32_t b_voff = (uint32_t)(b_row * (LAYOUT ? Op<BFMT>::kb : (int)ldb) + 16 * ((t % Op<BFMT>::cpr) ^ Op<BFMT>::swz(b_row)));
+    // LAYOUT 1: bytes from one K chunk of an operand to the next (the host has checked that an operand stays below 4 GiB)
+    const uint32_t a_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * Op<AFMT>::kb));
+    const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * Op<BFMT>::kb));
     const uint32_t s_voff = (uint32_t)(t * (int)ld_s);
 
     // Everything a tile needs, decoded from its index on the device.
@@ -266,12 +272,19 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         d.np = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BKP));
         // Rows past the end of the operand read as zero; rows of a neighbouring group are read
         // but never stored.
-        d.ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
-        d.rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
+        if (LAYOUT) {
+            // anchored at the tile's first row inside chunk 0; everything up to the end of the operand is readable
+            d.ra = make_rsrc(p.a + a_row0 * Op<AFMT>::kb, a_rows_total * lda - a_row0 * Op<AFMT>::kb);
+            d.rb = make_rsrc(p.b + b_row0 * Op<BFMT>::kb, b_rows_total * ldb - b_row0 * Op<BFMT>::kb);
+        } else {
+            d.ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
+            d.rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
+        }
         d.rsa = make_rsrc(p.sa + a_row0 * ld_s, (a_rows_total - a_row0) * ld_s);
         d.rsb = make_rsrc(p.sb + b_row0 * ld_s, (b_rows_total - b_row0) * ld_s);
-        d.ka0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<AFMT>::fp4 ? k0 / 2 : k0));
-        d.kb0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(Op<BFMT>::fp4 ? k0 / 2 : k0));
+        // first byte of the contraction range inside a row (LAYOUT 0) or its first K chunk (LAYOUT 1)
+        d.ka0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(LAYOUT ? k0 / BKP : (Op<AFMT>::fp4 ? k0 / 2 : k0)));
+        d.kb0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(LAYOUT ? k0 / BKP : (Op<BFMT>::fp4 ? k0 / 2 : k0)));
         d.ks0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(k0 / 32));
         return d;
     };
@@ -280,12 +293,14 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // the N-side operand for LPA <= r < LPT; a round past the end is a no-op.
     auto issue_1 = [&](const Tile& d, int kp, int slot, int r) __attribute__((always_inline)) {
         if (r < LPA) {
-            dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff,
-                  d.ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda);
+            const uint32_t soff = LAYOUT ? (d.ka0 + (uint32_t)kp) * a_cstride + (uint32_t)(r * Op<AFMT>::rows_per_ld * Op<AFMT>::kb)
+                                         : d.ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda;
+            dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff, soff);
         } else if (r < LPT) {
             const int i = r - LPA;
-            dma16(d.rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff,
-                  d.kb0 + kp * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb);
+            const uint32_t soff = LAYOUT ? (d.kb0 + (uint32_t)kp) * b_cstride + (uint32_t)(i * Op<BFMT>::rows_per_ld * Op<BFMT>::kb)
+                                         : d.kb0 + kp * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb;
+            dma16(d.rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff, soff);
         }
     };
     // scale panel pn (K slots 4pn .. 4pn+3) into panel buffer pn & 1
@@ -492,12 +507,12 @@ static int num_cus() {
     return pr.multiProcessorCount;
 }
 
-template <int AFMT, int BFMT, int MODE>
+template <int AFMT, int BFMT, int MODE, int LAYOUT>
 static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = gemm_lds_bytes(AFMT, BFMT);
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set{false};
-    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE>;
+    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT>;
     if (!attr_set.load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
@@ -510,13 +525,23 @@ static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
-template <int MODE>
-static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
-    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE>(a, max_tiles, st);
-    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E2M1) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E2M1, MODE>(a, max_tiles, st);
-    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E4M3, MODE>(a, max_tiles, st);
-    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E2M1) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E2M1, MODE>(a, max_tiles, st);
+template <int MODE, int LAYOUT>
+static int dispatch_gemm_l(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, LAYOUT>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E2M1) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E2M1, MODE, LAYOUT>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E4M3, MODE, LAYOUT>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E2M1) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E2M1, MODE, LAYOUT>(a, max_tiles, st);
     return MXL_EINVAL;
+}
+
+// a_rows / b_rows: rows of the whole operands (for the 4 GiB bound of the chunk-major layout)
+template <int MODE>
+static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, bool kchunk, int64_t a_rows, int64_t b_rows,
+                         hipStream_t st) {
+    if (!kchunk) return dispatch_gemm_l<MODE, 0>(afmt, bfmt, a, max_tiles, st);
+    // chunk offsets inside an operand are 32-bit
+    if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
+    return dispatch_gemm_l<MODE, 1>(afmt, bfmt, a, max_tiles, st);
 }
 
 }  // namespace mxl
@@ -531,9 +556,10 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t w
     if (i < words) dst[i] = 0u;
 }
 
-extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
-                                   const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
-                                   int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
+extern "C" int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                      const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                      int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream) {
+    if (flags & ~(uint32_t)MXL_GF_KCHUNK) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
     if (k > MAX_CONTRACTION) return MXL_EINVAL;   // tile-relative byte offsets are 32-bit
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
@@ -553,19 +579,28 @@ extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, in
     a.n = n;
     a.k = k;
     const int64_t max_tiles = (total_m / BM + num_groups) * ((n + BN - 1) / BN);
-    return dispatch_gemm<MODE_FWD>(a_fmt, b_fmt, a, max_tiles, (hipStream_t)stream);
+    return dispatch_gemm<MODE_FWD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, total_m,
+                                   (int64_t)num_groups * n, (hipStream_t)stream);
+}
+
+extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                   const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                   int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
+    return mxl_grouped_gemm_nt_ex(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, group_lens, num_groups, total_m,
+                                  n, k, 0, stream);
 }
 
 extern "C" int mxl_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                            const void* b_scales, int b_fmt, void* c_bf16, int64_t m, int64_t n, int64_t k,
                            void* stream) {
-    return mxl_grouped_gemm_nt(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, nullptr, 1, m, n, k,
-                               stream);
+    return mxl_grouped_gemm_nt_ex(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, nullptr, 1, m, n, k, 0, stream);
 }
 
-extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
-                                      const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
-                                      int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
+extern "C" int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                         const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                         int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags,
+                                         void* stream) {
+    if (flags & ~(uint32_t)MXL_GF_KCHUNK) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
     if (num_groups < 0 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if ((num_groups > 0) != (group_lens != nullptr)) return MXL_EINVAL;
@@ -601,7 +636,14 @@ extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales,
     a.n = k;  // columns of the output
     a.k = mxl_padded_width(total_m, G);
     const int64_t max_tiles = (int64_t)G * ((n + BM - 1) / BM) * ((k + BN - 1) / BN);
-    return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (hipStream_t)stream);
+    return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, n, k, (hipStream_t)stream);
+}
+
+extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                      const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                      int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
+    return mxl_grouped_gemm_wgrad_ex(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, group_lens, num_groups,
+                                     total_m, n, k, 0, stream);
 }
 
 extern "C" int mxl_version(void) { return 1; }

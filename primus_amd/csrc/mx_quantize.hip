@@ -64,6 +64,12 @@ struct QuantArgs {
     const void* probs;
     int probs_bf16;
     const uint8_t* row_mask;
+    // Code layout of both copies.  0: row-major [rows, ld].  1: K-chunk-major [ld / 128][rows][128 elements]:
+    // the 128 elements of a row that one GEMM K slot consumes stay together and consecutive rows follow
+    // each other, so a GEMM tile's slot is one contiguous block and this kernel writes 128 x 128-element
+    // pieces contiguously.  chunk_rows_row / chunk_rows_col: rows of the whole row-wise / transposed operand.
+    int kchunk;
+    int64_t chunk_rows_row, chunk_rows_col;
     uint64_t sr_seed;       // SR kernels: seed of the stochastic rounding
     uint32_t rht_signs;     // RHT kernels: sign bit i flips row i of every 16-row group before the transform
     int tiles_r, tiles_c;   // tile grid: row tiles (upper bound when grouped) x column tiles
@@ -238,7 +244,11 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o.x = nonfinite4_e4m3(d[it].x, d[it].y);
                     o.y = nonfinite4_e4m3(d[it].z, d[it].w);
                 }
-                if (out_ok && r < rows_valid) store8_streaming(a.q_row + (src_row0 + r) * a.row_ld + col, o);
+                if (out_ok && r < rows_valid) {
+                    const int64_t at = a.kchunk ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
+                                                : (src_row0 + r) * a.row_ld + col;
+                    store8_streaming(a.q_row + at, o);
+                }
             } else {
                 uint32_t o;
                 if (SR && byte != 255u) {
@@ -256,7 +266,11 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o = nonfinite2_e2m1(d[it].x) | (nonfinite2_e2m1(d[it].y) << 8) | (nonfinite2_e2m1(d[it].z) << 16) |
                         (nonfinite2_e2m1(d[it].w) << 24);
                 }
-                if (out_ok && r < rows_valid) store4_streaming(a.q_row + ((src_row0 + r) * a.row_ld + col) / 2, o);
+                if (out_ok && r < rows_valid) {
+                    const int64_t at = a.kchunk ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
+                                                : (src_row0 + r) * a.row_ld + col;
+                    store4_streaming(a.q_row + at / 2, o);
+                }
             }
         }
     }
@@ -397,7 +411,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             const int ch = t % LPR;
             if (col0 + c < a.cols && 16 * ch < avail) {
                 const uint4 v = *(const uint4*)(t_tile + c * TPITCH + 16 * ch);
-                store16_streaming(a.q_colT + (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch, v);
+                const int64_t at = a.kchunk ? ((m0 / QT) * a.chunk_rows_col + out_rows_base + col0 + c) * ROWB + 16 * ch
+                                            : (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch;
+                store16_streaming(a.q_colT + at, v);
             }
         }
     }
@@ -520,8 +536,10 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
 static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
                        int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
-                       bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0) {
+                       bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0,
+                       bool kchunk = false) {
     if (row_ld == 0) row_ld = cols;
+    if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
     if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
     if (rht && !q_colT) return MXL_EINVAL;   // the transform belongs to the transposed copy
     if (row_ld < cols || row_ld % MXL_BLOCK != 0) return MXL_EINVAL;
@@ -547,6 +565,9 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.row_mask = row_mask;
     a.sr_seed = sr_seed;
     a.rht_signs = rht_signs & 0xFFFFu;
+    a.kchunk = kchunk ? 1 : 0;
+    a.chunk_rows_row = rows;
+    a.chunk_rows_col = cols;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
     const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
     if (gx == 0) return MXL_OK;
@@ -565,31 +586,33 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
                        -1, nullptr, MXL_PROBS_F32, nullptr, stream);
 }
 
-extern "C" int mxl_quantize_fp4_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int scale_mode,
-                                   const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                                   void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream) {
-    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL)) return MXL_EINVAL;
-    return quantize_1d(x_bf16, rows, cols, row_ld, MXL_FMT_E2M1, scale_mode, group_lens, num_groups, q_row, s_row, q_colT,
+extern "C" int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
+                               const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
+                               void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream) {
+    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK)) return MXL_EINVAL;
+    return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT,
                        s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, (flags & MXL_QF_SR) != 0, sr_seed,
-                       (flags & MXL_QF_RHT_COL) != 0, rht_signs);
+                       (flags & MXL_QF_RHT_COL) != 0, rht_signs, (flags & MXL_QF_KCHUNK) != 0);
 }
 
 extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
                                       int64_t rows, int64_t f, int64_t row_ld, int act, int fmt, int scale_mode,
                                       const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
-                                      void* s_colT, void* stream) {
+                                      void* s_colT, uint32_t flags, void* stream) {
     if (act != MXL_ACT_SILU && act != MXL_ACT_GELU) return MXL_EINVAL;
     if (probs_dtype != MXL_PROBS_F32 && probs_dtype != MXL_PROBS_BF16) return MXL_EINVAL;
     if (rows > 0 && !probs) return MXL_EINVAL;
+    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, f, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT, act,
-                       probs, probs_dtype, row_mask, stream);
+                       probs, probs_dtype, row_mask, stream, false, 0, false, 0, (flags & MXL_QF_KCHUNK) != 0);
 }
 
-extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
-                                      int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
-                                      void* s_colT, void* stream) {
+static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld, int64_t n_ld, int fmt,
+                              int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT, bool kchunk,
+                              void* stream) {
     if (k_ld == 0) k_ld = k;
     if (n_ld == 0) n_ld = n;
+    if (kchunk && ((q_row && k_ld % QT != 0) || (q_colT && n_ld % QT != 0))) return MXL_EINVAL;   // whole chunks
     if (k_ld < k || n_ld < n || k_ld % MXL_BLOCK != 0 || n_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if (n_ld > (n + QT - 1) / QT * QT) return MXL_EINVAL;  // padding of the transposed copy stays inside the last tile
     if (!w_bf16 || batch <= 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
@@ -613,9 +636,26 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
     a.row_mask = nullptr;
     a.sr_seed = 0;
     a.rht_signs = 0;
+    a.kchunk = kchunk ? 1 : 0;
+    a.chunk_rows_row = batch * n;   // the batch is one operand of batch * n rows (resp. batch * k for the transposed copy)
+    a.chunk_rows_col = batch * k;
     const int64_t gx = batch * ((n + QT - 1) / QT);
     const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
     return dispatch_quant<true>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
+}
+
+extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
+                                      int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
+                                      void* s_colT, void* stream) {
+    return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, scale_mode, q_row, s_row, q_colT, s_colT, false, stream);
+}
+
+extern "C" int mxl_quantize_weight_2d_ex(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
+                                         int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
+                                         void* s_colT, uint32_t flags, void* stream) {
+    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, scale_mode, q_row, s_row, q_colT, s_colT,
+                              (flags & MXL_QF_KCHUNK) != 0, stream);
 }
 
 extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,

@@ -78,6 +78,20 @@ def _round_up(x: int, m: int) -> int:
     return (x + m - 1) // m * m
 
 
+KCHUNK = 128   # elements of a row that stay together in the K-chunk-major code layout (one GEMM K slot)
+
+
+def _code_shape(rows: int, ld: int, per: int, kchunk: bool):
+    return (ld // KCHUNK, rows, KCHUNK // per) if kchunk else (rows, ld // per)
+
+
+def unchunk(codes: torch.Tensor) -> torch.Tensor:
+    """K-chunk-major codes ``[ld / 128, rows, 128]`` as a row-major ``[rows, ld]`` tensor (a copy)."""
+    if codes.dim() != 3:
+        raise ValueError("expected 3-D K-chunk-major codes")
+    return codes.permute(1, 0, 2).reshape(codes.shape[1], codes.shape[0] * codes.shape[2])
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None or t.numel() == 0 else t.data_ptr()
 
@@ -154,8 +168,13 @@ def quantize_mx_impl(
     pad_to: int = 1,
     sr_seed: Optional[int] = None,
     rht_signs: Optional[int] = None,
+    kchunk: bool = False,
 ):
     """MX-quantise bf16 ``x[rows, cols]``.
+
+    ``kchunk`` stores the codes K-chunk-major, the layout the GEMMs load fastest: the code tensors come
+    back 3-D, ``[ld / 128, rows, 128]`` (``64`` bytes in the last dim for FP4) instead of ``[rows, ld]``
+    (``unchunk`` turns them back); the column count is padded to a multiple of 128; scales are unchanged.
 
     ``sr_seed`` (an integer; E2M1 only) rounds the codes stochastically instead of to nearest even
     (gradients of the MXFP4 recipe); the same seed reproduces the same codes.  ``rht_signs`` (16 sign
@@ -189,13 +208,13 @@ def quantize_mx_impl(
     per = _per_byte(fmt)
     dev = x.device
     q_row = s_row = q_col = s_col = None
-    row_ld = _round_up(cols, pad_to)
+    row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
-        q_row = torch.empty((rows, row_ld // per), dtype=torch.uint8, device=dev)
+        q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
         s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        q_col = torch.empty((cols, W // per), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
         s_col = torch.empty((cols, W // BLOCK), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
@@ -203,13 +222,13 @@ def quantize_mx_impl(
         args = (_ptr(x) if row_ok else None, rows, cols, row_ld, fmt, scale_mode, _ptr(group_lens), G,
                 _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col), _ptr(s_col))
         with _hooked("quantize", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
-            if sr_seed is None and rht_signs is None:
+            if sr_seed is None and rht_signs is None and not kchunk:
                 rc = _lib.load().mxl_quantize(*args, _stream())
             else:
-                flags = (_lib.QF_SR if sr_seed is not None else 0) | (_lib.QF_RHT_COL if rht_signs is not None else 0)
-                rc = _lib.load().mxl_quantize_fp4_ex(
-                    *args[:4], *args[5:], flags, int(sr_seed or 0) & 0xFFFFFFFFFFFFFFFF, int(rht_signs or 0) & 0xFFFF,
-                    _stream())
+                flags = ((_lib.QF_SR if sr_seed is not None else 0) | (_lib.QF_RHT_COL if rht_signs is not None else 0)
+                         | (_lib.QF_KCHUNK if kchunk else 0))
+                rc = _lib.load().mxl_quantize_ex(
+                    *args, flags, int(sr_seed or 0) & 0xFFFFFFFFFFFFFFFF, int(rht_signs or 0) & 0xFFFF, _stream())
         _lib.check(rc, "mxl_quantize")
     cd = _code_dtype(fmt)
     v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
@@ -224,11 +243,13 @@ def quantize_mx_weight_2d_impl(
     rowwise: bool = True,
     colwise: bool = True,
     pad_to: int = 1,
+    kchunk: bool = False,
 ):
     """2-D (32x32 tile) MX quantisation of ``w[n, k]`` or ``w[G, n, k]``;
     returns ``(q_row [.., n, k], s_row [.., n, k/32], q_colT [.., k, n],
     s_colT [.., k, n/32])`` with ``None`` for a copy that was not requested.
-    ``pad_to`` rounds the last dim of both copies up (zero padding)."""
+    ``pad_to`` rounds the last dim of both copies up (zero padding).  With ``kchunk`` the codes come back
+    K-chunk-major over the flattened batch: ``[k_ld / 128, G * n, 128]`` and ``[n_ld / 128, G * k, 128]``."""
     if w.dtype != torch.bfloat16 or w.dim() not in (2, 3):
         raise ValueError("weight quantisation expects a 2-D or 3-D bfloat16 tensor")
     _require_cuda(w)
@@ -242,16 +263,19 @@ def quantize_mx_weight_2d_impl(
     per = _per_byte(fmt)
     dev = w.device
     q_row = s_row = q_col = s_col = None
-    k_ld, n_ld = _round_up(k, pad_to), _round_up(n, pad_to)
+    k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     if rowwise:
-        q_row = torch.empty(lead + (n, k_ld // per), dtype=torch.uint8, device=dev)
+        shape = _code_shape(batch * n, k_ld, per, True) if kchunk else lead + (n, k_ld // per)
+        q_row = torch.empty(shape, dtype=torch.uint8, device=dev)
         s_row = torch.empty(lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
-        q_col = torch.empty(lead + (k, n_ld // per), dtype=torch.uint8, device=dev)
+        shape = _code_shape(batch * k, n_ld, per, True) if kchunk else lead + (k, n_ld // per)
+        q_col = torch.empty(shape, dtype=torch.uint8, device=dev)
         s_col = torch.empty(lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
-        rc = _lib.load().mxl_quantize_weight_2d(
-            _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col), _stream()
+        rc = _lib.load().mxl_quantize_weight_2d_ex(
+            _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
+            _lib.QF_KCHUNK if kchunk else 0, _stream()
         )
     _lib.check(rc, "mxl_quantize_weight_2d")
     cd = _code_dtype(fmt)
@@ -298,11 +322,20 @@ def _check_out_dtype(out_dtype) -> None:
         raise ValueError("the MX GEMMs produce bfloat16 output")
 
 
-def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16) -> torch.Tensor:
-    """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T."""
+def _chunked_dims(codes: torch.Tensor, fmt: int):
+    """(rows, k) of K-chunk-major codes [k / 128, rows, 128]."""
+    if codes.dim() != 3 or codes.shape[2] * _per_byte(fmt) != KCHUNK or not codes.is_contiguous():
+        raise ValueError("K-chunk-major codes must be a contiguous [k / 128, rows, 128-element] tensor")
+    return codes.shape[1], codes.shape[0] * KCHUNK
+
+
+def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk: bool = False) -> torch.Tensor:
+    """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T.  ``kchunk``: both code tensors are K-chunk-major."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if kchunk:
+        return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale.unsqueeze(0), None, kchunk=True)
     m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
     n, kb = b.shape[0], b.shape[1] * _per_byte(b_fmt)
     if k != kb:
@@ -318,13 +351,31 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16) -> torch.T
     return c
 
 
-def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16) -> torch.Tensor:
+def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16, kchunk: bool = False) -> torch.Tensor:
     """Forward / dgrad grouped GEMM: rows of ``a[total_m, k]`` split by
-    ``group_lens``; ``b`` is ``[G, n, k]``."""
+    ``group_lens``; ``b`` is ``[G, n, k]``.  ``kchunk``: both code tensors are K-chunk-major,
+    ``a [k / 128, total_m, 128]`` and ``b [k / 128, G * n, 128]``; ``b_scale`` is ``[G, n, k / 32]`` as always."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale, group_lens)
     G = _check_group_lens(group_lens, a.device)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if kchunk:
+        total_m, k = _chunked_dims(a, a_fmt)
+        b_rows, kb = _chunked_dims(b, b_fmt)
+        groups = max(G, 1)
+        if b_scale.dim() != 3 or b_scale.shape[0] != groups or b_scale.shape[0] * b_scale.shape[1] != b_rows:
+            raise ValueError("b_scale must be [num_groups, n, k/32] and match the rows of b")
+        n = b_scale.shape[1]
+        if k != kb or tuple(a_scale.shape) != (total_m, k // BLOCK) or b_scale.shape[2] != k // BLOCK:
+            raise ValueError("contraction dims / scale shapes do not match")
+        c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+        with _hooked("grouped_gemm_nt" if G else "gemm_nt", m=total_m, n=n, k=k):
+            rc = _lib.load().mxl_grouped_gemm_nt_ex(
+                _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), groups, total_m, n, k,
+                _lib.GF_KCHUNK, _stream()
+            )
+        _lib.check(rc, "mxl_grouped_gemm_nt_ex")
+        return c
     if b.dim() != 3 or b.shape[0] != G:
         raise ValueError("grouped GEMM expects weights of shape [num_groups, n, k]")
     total_m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
@@ -344,7 +395,8 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
     return c
 
 
-def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total_m, out_dtype=torch.bfloat16) -> torch.Tensor:
+def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total_m, out_dtype=torch.bfloat16,
+                               kchunk: bool = False) -> torch.Tensor:
     """Variable-K (wgrad) grouped GEMM on segment-padded transposed operands:
     ``a_t`` = dY^T codes ``[n, W]``, ``b_t`` = X^T codes ``[k, W]``; returns
     ``[G, n, k]`` (``[n, k]`` when ``group_lens`` is None).  An expert with no
@@ -354,16 +406,22 @@ def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total
     G = _check_group_lens(group_lens, a_t.device)
     a_fmt, b_fmt = fmt_of(a_t), fmt_of(b_t)
     W = padded_width(total_m, G)
-    n, k = a_t.shape[0], b_t.shape[0]
-    if a_t.shape[1] * _per_byte(a_fmt) != W or b_t.shape[1] * _per_byte(b_fmt) != W:
-        raise ValueError(f"transposed operands must have padded width {W}")
+    if kchunk:
+        (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt), _chunked_dims(b_t, b_fmt)
+        if wa != W or wb != W:
+            raise ValueError(f"transposed operands must have padded width {W}")
+    else:
+        n, k = a_t.shape[0], b_t.shape[0]
+        if a_t.shape[1] * _per_byte(a_fmt) != W or b_t.shape[1] * _per_byte(b_fmt) != W:
+            raise ValueError(f"transposed operands must have padded width {W}")
     if tuple(a_t_scale.shape) != (n, W // BLOCK) or tuple(b_t_scale.shape) != (k, W // BLOCK):
         raise ValueError("scale shapes must be [rows, W/32]")
     shape = (n, k) if group_lens is None else (G, n, k)
     c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
     with _hooked("grouped_gemm_wgrad", m=total_m, n=n, k=k):
-        rc = _lib.load().mxl_grouped_gemm_wgrad(
-            _ptr(a_t), _ptr(a_t_scale), a_fmt, _ptr(b_t), _ptr(b_t_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()
+        rc = _lib.load().mxl_grouped_gemm_wgrad_ex(
+            _ptr(a_t), _ptr(a_t_scale), a_fmt, _ptr(b_t), _ptr(b_t_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k,
+            _lib.GF_KCHUNK if kchunk else 0, _stream()
         )
     _lib.check(rc, "mxl_grouped_gemm_wgrad")
     return c
@@ -422,7 +480,8 @@ def glu_with_probs_bwd_impl(dy, x, probs, row_mask, activation: str):
 
 
 def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *,
-                                 colwise: bool = False, group_lens: Optional[torch.Tensor] = None, pad_to: int = 1):
+                                 colwise: bool = False, group_lens: Optional[torch.Tensor] = None, pad_to: int = 1,
+                                 kchunk: bool = False):
     """``quantize_mx_impl(glu_with_probs_fwd_impl(x, ...))`` in one pass over ``x [tokens, 2F]``, the
     activated tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
     act, pd, row_mask = _glu_args(x, probs, row_mask, activation)
@@ -432,17 +491,17 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
         raise ValueError(f"the quantised dim ({f}) must be a multiple of {BLOCK}")
     if rows == 0:  # nothing to activate: only the padding of the transposed copy is left to write
         return quantize_mx_impl(x[:, :f].contiguous(), fmt, scale_mode, rowwise=True, colwise=colwise,
-                                group_lens=group_lens, pad_to=pad_to)
+                                group_lens=group_lens, pad_to=pad_to, kchunk=kchunk)
     G = _check_group_lens(group_lens, x.device)
     per = _per_byte(fmt)
     dev = x.device
-    row_ld = _round_up(f, pad_to)
-    q_row = torch.empty((rows, row_ld // per), dtype=torch.uint8, device=dev)
+    row_ld = _round_up(f, KCHUNK if kchunk else pad_to)
+    q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
     s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, G)
-        q_col = torch.empty((f, W // per), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
         s_col = torch.empty((f, W // BLOCK), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         row_ok = rows > 0
@@ -450,7 +509,7 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
             rc = _lib.load().mxl_glu_probs_quantize(
                 _ptr(x) if row_ok else None, _ptr(probs), pd, _ptr(row_mask), rows, f, row_ld, act, fmt, scale_mode,
                 _ptr(group_lens), G, _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col),
-                _ptr(s_col), _stream(),
+                _ptr(s_col), _lib.QF_KCHUNK if kchunk else 0, _stream(),
             )
         _lib.check(rc, "mxl_glu_probs_quantize")
     cd = _code_dtype(fmt)

@@ -55,7 +55,8 @@ def test_constants_match_the_header():
     assert (int(defs["MXL_SCALE_OCP_FLOOR"]), int(defs["MXL_SCALE_RCEIL"]), int(defs["MXL_SCALE_EVEN"])) == (
         o.SCALE_OCP_FLOOR, o.SCALE_RCEIL, o.SCALE_EVEN)
     assert (int(defs["MXL_ACT_SILU"]), int(defs["MXL_ACT_GELU"])) == (_lib.ACT_SILU, _lib.ACT_GELU)
-    assert (int(defs["MXL_QF_SR"]), int(defs["MXL_QF_RHT_COL"])) == (_lib.QF_SR, _lib.QF_RHT_COL)
+    assert (int(defs["MXL_QF_SR"]), int(defs["MXL_QF_RHT_COL"]), int(defs["MXL_QF_KCHUNK"])) == (
+        _lib.QF_SR, _lib.QF_RHT_COL, _lib.QF_KCHUNK)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -68,8 +68,10 @@ def test_sr_with_non_finite_blocks_and_bad_arguments(gpu):
     lib = _lib.load()
     xd = x.to(gpu)
     buf = torch.empty(64 * 64, dtype=torch.uint8, device=gpu)
-    assert lib.mxl_quantize_fp4_ex(xd.data_ptr(), 64, 64, 48, 0, None, 0, buf.data_ptr(), buf.data_ptr(),
-                                   None, None, _lib.QF_SR, 1, 0, None) == -1       # row_ld below cols
+    assert lib.mxl_quantize_ex(xd.data_ptr(), 64, 64, 48, _lib.FMT_E2M1, 0, None, 0, buf.data_ptr(), buf.data_ptr(),
+                               None, None, _lib.QF_SR, 1, 0, None) == -1           # row_ld below cols
+    assert lib.mxl_quantize_ex(xd.data_ptr(), 64, 64, 64, _lib.FMT_E4M3, 0, None, 0, buf.data_ptr(), buf.data_ptr(),
+                               None, None, _lib.QF_SR, 1, 0, None) == -1           # stochastic rounding is E2M1 only
 
 
 def test_gemm_fp4_gradient_sr_is_reproducible_and_unbiased(gpu):
@@ -199,10 +201,12 @@ def test_hadamard_bad_arguments(gpu):
         K.quantize_mx_impl(x, o.FMT_E4M3, rowwise=True, colwise=True, rht_signs=1)
     buf = torch.empty(64 * 64, dtype=torch.uint8, device=gpu)
     lib = _lib.load()
-    assert lib.mxl_quantize_fp4_ex(x.data_ptr(), 64, 64, 64, 0, None, 0, buf.data_ptr(), buf.data_ptr(), None, None,
-                                   _lib.QF_RHT_COL, 0, 1, None) == -1          # transform without a transposed copy
-    assert lib.mxl_quantize_fp4_ex(x.data_ptr(), 64, 64, 64, 0, None, 0, buf.data_ptr(), buf.data_ptr(), None, None,
-                                   8, 0, 0, None) == -1                         # unknown flag
+    assert lib.mxl_quantize_ex(x.data_ptr(), 64, 64, 64, _lib.FMT_E2M1, 0, None, 0, buf.data_ptr(), buf.data_ptr(), None, None,
+                               _lib.QF_RHT_COL, 0, 1, None) == -1              # transform without a transposed copy
+    assert lib.mxl_quantize_ex(x.data_ptr(), 64, 64, 64, _lib.FMT_E2M1, 0, None, 0, buf.data_ptr(), buf.data_ptr(), None, None,
+                               64, 0, 0, None) == -1                            # unknown flag
+    assert lib.mxl_quantize_ex(x.data_ptr(), 64, 64, 64, _lib.FMT_E2M1, 0, None, 0, buf.data_ptr(), buf.data_ptr(), None, None,
+                               _lib.QF_KCHUNK, 0, 0, None) == -1                # chunk-major needs row_ld % 128 == 0
 
 
 def test_grouped_gemm_fp4_with_hadamard_config(gpu):

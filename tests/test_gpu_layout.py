@@ -1,0 +1,115 @@
+"""The K-chunk-major code layout ([ld / 128, rows, 128] instead of [rows, ld]): the quantisers write the
+same codes, only arranged differently, and the GEMMs give the same results bit for bit on either layout."""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _same(a, b):
+    return a.dtype == b.dtype and torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("lens,cols", [([33, 0, 130, 1, 92], 160), ([300], 2048), (None, 64), ([0, 0], 96), ([257, 255], 384)])
+def test_quantiser_kchunk_is_a_rearrangement(gpu, fmt, lens, cols):
+    from primus_amd.pytorch import kernels as K
+
+    rows = 257 if lens is None else sum(lens)
+    g = torch.Generator().manual_seed(rows + cols)
+    x = (torch.randn(rows, cols, generator=g) * torch.logspace(-2, 2, cols)[None, :]).bfloat16().to(gpu)
+    gl = None if lens is None else torch.tensor(lens, dtype=torch.int64, device=gpu)
+    a = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128)
+    b = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=True, group_lens=gl, kchunk=True)
+    assert b[0].dim() == 3 and b[0].shape[1] == rows and b[2].dim() == 3 and b[2].shape[1] == cols
+    assert _same(K.unchunk(b[0]), a[0]) and _same(b[1], a[1])
+    assert _same(K.unchunk(b[2]), a[2]) and _same(b[3], a[3])
+    if rows:
+        r = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=False, kchunk=True)
+        assert _same(r[0], b[0])
+    c = K.quantize_mx_impl(x, fmt, rowwise=False, colwise=True, group_lens=gl, kchunk=True)
+    assert _same(c[2], b[2])
+    if fmt == 1:
+        e = K.quantize_mx_impl(x, 1, rowwise=True, colwise=True, group_lens=gl, pad_to=128, sr_seed=5, rht_signs=0x1234)
+        f = K.quantize_mx_impl(x, 1, rowwise=True, colwise=True, group_lens=gl, kchunk=True, sr_seed=5, rht_signs=0x1234)
+        assert _same(K.unchunk(f[0]), e[0]) and _same(K.unchunk(f[2]), e[2])
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("shape", [(96, 160), (3, 256, 128), (2, 416, 288), (1, 32, 32)])
+def test_weight_quantiser_kchunk_is_a_rearrangement(gpu, fmt, shape):
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator().manual_seed(sum(shape))
+    w = (torch.randn(*shape, generator=g) * 0.05).bfloat16().to(gpu)
+    n, k = shape[-2], shape[-1]
+    a = K.quantize_mx_weight_2d_impl(w, fmt, rowwise=True, colwise=True, pad_to=128)
+    b = K.quantize_mx_weight_2d_impl(w, fmt, rowwise=True, colwise=True, kchunk=True)
+    assert _same(K.unchunk(b[0]), a[0].reshape(-1, a[0].shape[-1])) and _same(b[1], a[1])
+    assert _same(K.unchunk(b[2]), a[2].reshape(-1, a[2].shape[-1])) and _same(b[3], a[3])
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu"])
+def test_fused_activation_quantiser_kchunk(gpu, activation):
+    from primus_amd.pytorch import kernels as K
+
+    lens, f = [33, 0, 130, 1, 92], 160
+    rows = sum(lens)
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(rows, 2 * f, generator=g) * 2).bfloat16().to(gpu)
+    p = torch.rand(rows, generator=g).to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    a = K.glu_with_probs_quantize_impl(x, p, None, activation, 0, colwise=True, group_lens=gl, pad_to=128)
+    b = K.glu_with_probs_quantize_impl(x, p, None, activation, 0, colwise=True, group_lens=gl, kchunk=True)
+    assert _same(K.unchunk(b[0]), a[0]) and _same(K.unchunk(b[2]), a[2]) and _same(b[1], a[1]) and _same(b[3], a[3])
+
+
+@pytest.mark.parametrize("afmt,wfmt", [(0, 0), (0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("lens,n,k", [([33, 0, 130, 1, 92], 96, 160), ([300, 212], 544, 512), (None, 320, 384),
+                                      ([1500, 0, 700, 2048, 300, 1024], 2048, 1024)])
+def test_gemms_give_identical_results_on_either_layout(gpu, afmt, wfmt, lens, n, k):
+    """Forward, dgrad and wgrad from K-chunk-major operands equal those from row-major operands bit for bit
+    (same codes, same scales, same MFMA sequence; only the addresses of the operand loads differ)."""
+    from primus_amd.pytorch import kernels as K
+
+    m = 257 if lens is None else sum(lens)
+    G = 1 if lens is None else len(lens)
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16().to(gpu)
+    dy = torch.randn(m, n, generator=g).bfloat16().to(gpu)
+    w = (torch.randn(G, n, k, generator=g) * 0.05).bfloat16().to(gpu)
+    gl = None if lens is None else torch.tensor(lens, dtype=torch.int64, device=gpu)
+    res = []
+    for kc in (False, True):
+        xq = K.quantize_mx_impl(x, afmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kc)
+        dq = K.quantize_mx_impl(dy, afmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kc)
+        wq = K.quantize_mx_weight_2d_impl(w, wfmt, rowwise=True, colwise=True, pad_to=128, kchunk=kc)
+        if lens is None:
+            ws_row, ws_col = wq[1][0], wq[3][0]
+            w_row = wq[0] if kc else wq[0][0]
+            w_col = wq[2] if kc else wq[2][0]
+            y = K.gemm_mx_nt_impl(xq[0], xq[1], w_row, ws_row, kchunk=kc)
+            dx = K.gemm_mx_nt_impl(dq[0], dq[1], w_col, ws_col, kchunk=kc)
+        else:
+            y = K.grouped_gemm_mx_nt_impl(xq[0], xq[1], wq[0], wq[1], gl, kchunk=kc)
+            dx = K.grouped_gemm_mx_nt_impl(dq[0], dq[1], wq[2], wq[3], gl, kchunk=kc)
+        dw = K.grouped_gemm_mx_wgrad_impl(dq[2], dq[3], xq[2], xq[3], gl, m, kchunk=kc)
+        res.append((y, dx[:, :k], dw))
+    for a, b in zip(*res):
+        assert a.shape == b.shape and torch.equal(a, b)
+
+
+def test_kchunk_argument_checks(gpu):
+    from primus_amd.pytorch import kernels as K
+
+    x = torch.randn(64, 128, device=gpu).bfloat16()
+    q = K.quantize_mx_impl(x, 0, rowwise=True, colwise=False, kchunk=True)
+    w = K.quantize_mx_weight_2d_impl(x[:32].contiguous(), 0, rowwise=True, colwise=False, kchunk=True)
+    with pytest.raises(ValueError):
+        K.gemm_mx_nt_impl(K.unchunk(q[0]), q[1], w[0], w[1], kchunk=True)          # row-major codes passed as chunk-major
+    with pytest.raises(ValueError):
+        K.unchunk(K.unchunk(q[0]))
+    y = K.gemm_mx_nt_impl(q[0], q[1], w[0], w[1], kchunk=True)
+    assert y.shape == (64, 32)

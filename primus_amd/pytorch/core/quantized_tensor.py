@@ -49,18 +49,21 @@ class QuantizedTensor(torch.Tensor):
     payload (and therefore the logical shape) TRANSPOSED
     (primus_turbo.py:346-354).  ``segment_lens`` marks a transposed activation
     copy whose blocks restart at expert boundaries and whose token dim is
-    padded per expert.
+    padded per expert.  ``kchunk`` marks a payload stored K-chunk-major
+    (``codes[ld/128, rows, 128 elements]``, the layout the GEMMs load fastest);
+    the scales have the same shape in both layouts.
     """
 
     @staticmethod
     def __new__(cls, codes, scales, *, logical_shape, orig_dtype=torch.bfloat16, axis=-1, use_2d_block=False,
-                scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False):
+                scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False, kchunk=False):
         return torch.Tensor._make_wrapper_subclass(
             cls, tuple(logical_shape), dtype=orig_dtype, device=codes.device, requires_grad=requires_grad
         )
 
     def __init__(self, codes, scales, *, logical_shape, orig_dtype=torch.bfloat16, axis=-1, use_2d_block=False,
-                 scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False):
+                 scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False, kchunk=False):
+        self._kchunk = bool(kchunk)
         self._codes = codes
         self._scales = scales
         self._axis = axis
@@ -87,6 +90,17 @@ class QuantizedTensor(torch.Tensor):
         return self._use_2d_block
 
     @property
+    def kchunk(self) -> bool:
+        return self._kchunk
+
+    def rowmajor_codes(self) -> torch.Tensor:
+        """The payload as ``[..., rows, ld]`` whatever layout it is stored in (a copy if K-chunk-major)."""
+        if not self._kchunk:
+            return self._codes
+        flat = K.unchunk(self._codes)
+        return flat.view(tuple(self.shape[:-1]) + (flat.shape[-1],))
+
+    @property
     def fmt(self) -> int:
         return dtype_to_fmt_code(self._codes.dtype)
 
@@ -94,7 +108,7 @@ class QuantizedTensor(torch.Tensor):
         return QuantizedTensor(
             self._codes, self._scales, logical_shape=self.shape, orig_dtype=self.dtype, axis=self._axis,
             use_2d_block=self._use_2d_block, scale_mode=self._scale_mode, segment_lens=self._segment_lens,
-            total_rows=self._total_rows,
+            total_rows=self._total_rows, kchunk=self._kchunk,
         )
 
     def __repr__(self):  # noqa: D105
@@ -167,7 +181,7 @@ class QuantizedTensor(torch.Tensor):
     def dequantize(self) -> torch.Tensor:
         """Back to the original dtype in the payload's orientation.  For a
         transposed copy of ``rows`` tokens the padding columns are dropped."""
-        out = K.dequantize_mx_impl(self._codes, self._scales, self.dtype)
+        out = K.dequantize_mx_impl(self.rowmajor_codes(), self._scales, self.dtype)
         if self._axis == -2 and not self._use_2d_block and self._segment_lens is not None:
             raise NotImplementedError("dequantize of a segment-padded activation copy")
         # drop the padding of the contraction dim (GEMM granularity / token padding)
@@ -198,11 +212,13 @@ def create_quantized_weight(
     dest_dtype: torch.dtype,
     quant_config: Union[Float8QuantConfig, Float4QuantConfig],
     need_weight_transpose_cache: bool = True,
+    kchunk: Optional[bool] = None,
 ) -> Tuple[QuantizedTensor, Optional[QuantizedTensor]]:
     """``(rowwise, colwise_or_None)`` for a weight ``[n, k]`` or ``[G, n, k]``
     (primus_turbo.py:295-301).  Weights use 2-D 32x32 blocks
     (primus_turbo.py:313-317), so both copies come out of one pass over the
-    weight and hold the same codes."""
+    weight and hold the same codes.  ``kchunk`` picks the storage layout of the
+    codes (default: K-chunk-major whenever the GEMMs accept it for this size)."""
     if quant_config.granularity != ScalingGranularity.MX_BLOCKWISE:
         raise NotImplementedError("only ScalingGranularity.MX_BLOCKWISE has kernels in this build")
     fmt = dtype_to_fmt_code(dest_dtype)
@@ -210,14 +226,18 @@ def create_quantized_weight(
     if w.dtype != torch.bfloat16:
         raise ValueError("create_quantized_weight expects a bfloat16 weight")
     mode = quant_config.scale_mode
+    if kchunk is None:
+        kchunk = K.kchunk_default() and K.kchunk_fits(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1,
+                                                      w.shape[-2], w.shape[-1])
     q_row, s_row, q_col, s_col = K.quantize_mx_weight_2d_impl(
-        w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN
+        w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN,
+        kchunk=kchunk,
     )
     row = QuantizedTensor(q_row, s_row, logical_shape=w.shape, orig_dtype=w.dtype, axis=-1, use_2d_block=True,
-                          scale_mode=mode)
+                          scale_mode=mode, kchunk=kchunk)
     col = None
     if need_weight_transpose_cache:
         shape = tuple(w.shape[:-2]) + (w.shape[-1], w.shape[-2])
         col = QuantizedTensor(q_col, s_col, logical_shape=shape, orig_dtype=w.dtype, axis=-2, use_2d_block=True,
-                              scale_mode=mode)
+                              scale_mode=mode, kchunk=kchunk)
     return row, col

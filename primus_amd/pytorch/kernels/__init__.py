@@ -85,6 +85,31 @@ def _code_shape(rows: int, ld: int, per: int, kchunk: bool):
     return (ld // KCHUNK, rows, KCHUNK // per) if kchunk else (rows, ld // per)
 
 
+_kchunk_default = True
+
+
+def set_kchunk_default(enabled: bool) -> None:
+    """Whether the differentiable operators and ``create_quantized_weight`` store codes K-chunk-major
+    (default) or row-major.  Results are identical; the GEMMs load the chunked layout faster."""
+    global _kchunk_default
+    _kchunk_default = bool(enabled)
+
+
+def kchunk_default() -> bool:
+    return _kchunk_default
+
+
+def kchunk_fits(groups: int, n: int, k: int, rows: int = 0) -> bool:
+    """The GEMMs address a K-chunk-major operand with 32-bit offsets from its base, so every operand of a
+    linear with weights ``[groups, n, k]`` and ``rows`` tokens has to stay under 4 GiB."""
+    np_, kp = _round_up(n, KCHUNK), _round_up(k, KCHUNK)
+    limit = 1 << 32
+    if groups * np_ * kp >= limit:
+        return False
+    w = padded_width(rows, groups) if rows else 0
+    return w * max(np_, kp) < limit
+
+
 def unchunk(codes: torch.Tensor) -> torch.Tensor:
     """K-chunk-major codes ``[ld / 128, rows, 128]`` as a row-major ``[rows, ld]`` tensor (a copy)."""
     if codes.dim() != 3:

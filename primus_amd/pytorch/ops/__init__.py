@@ -37,7 +37,7 @@ from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
 __all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
            "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask", "glu_grouped_gemm_fp8",
-           "glu_grouped_gemm_fp4", "manual_sr_seed"]
+           "glu_grouped_gemm_fp4", "manual_sr_seed", "set_kchunk_layout"]
 
 # dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
 # kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
@@ -50,6 +50,12 @@ def manual_sr_seed(seed: Optional[int]) -> None:
     """Restart the seed sequence of stochastic gradient rounding (``Float4QuantConfig.use_gradient_sr``);
     ``None`` ties it to ``torch.initial_seed()`` again."""
     K.manual_sr_seed(seed)
+
+
+def set_kchunk_layout(enabled: bool) -> None:
+    """Store quantised operands K-chunk-major between the quantisers and the GEMMs (default on; the
+    row-major layout gives the same results bit for bit and is what operands of 4 GiB or more use)."""
+    K.set_kchunk_default(enabled)
 
 
 def set_wgrad_overlap(enabled: bool) -> None:
@@ -67,6 +73,12 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
     return st
 
 
+def _cached_codes(q: QuantizedTensor, kchunk: bool) -> torch.Tensor:
+    """Codes of a cached weight copy in the layout this call's GEMMs use.  A K-chunk-major cache is
+    rearranged (one pass over the weight) only when this call cannot use that layout."""
+    return q.codes if q.kchunk == kchunk else q.rowmajor_codes()
+
+
 class _MXLinearFunction(torch.autograd.Function):
     """Y = X . W^T on MX operands, dense (``group_lens is None``) or grouped.
 
@@ -81,39 +93,45 @@ class _MXLinearFunction(torch.autograd.Function):
         need_dgrad = a.requires_grad or (glu and probs.requires_grad)
         need_wgrad = b.requires_grad
         grouped = group_lens is not None
+        # Every operand of the three GEMMs is stored in one layout, K-chunk-major unless an operand is
+        # too large for it (or the layout is switched off): same codes, same results, faster loads.
+        groups = b.shape[0] if grouped else 1
+        kc = K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])
+        if isinstance(b, QuantizedTensor):   # cached copies decide: row-major caches are used as they are
+            kc = kc and b.kchunk and (b_t is None or b_t.kchunk)
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
         # (row-wise copies are padded to the GEMM's K granularity, like the reference pads its
         # MXFP4 operands to 128: primus_turbo_mxfp4_local.py:119-124)
         if glu:
             a_row, a_rs, a_col, a_cs = K.glu_with_probs_quantize_impl(
                 a, probs, row_mask, activation, act_fmt, scale_mode, colwise=need_wgrad, group_lens=group_lens,
-                pad_to=K.GEMM_K_ALIGN,
+                pad_to=K.GEMM_K_ALIGN, kchunk=kc,
             )
         else:
             a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
                 a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
-                rht_signs=rht_signs if need_wgrad else None,
+                rht_signs=rht_signs if need_wgrad else None, kchunk=kc,
             )
         if isinstance(b, QuantizedTensor):
             # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
             if b.axis != -1:
                 raise ValueError("the forward weight copy must be quantised along axis=-1")
-            w_row, w_rs = b.codes, b.scales
+            w_row, w_rs = _cached_codes(b, kc), b.scales
             w_col = w_cs = None
             if need_dgrad:
                 if b_t is None:
                     raise ValueError("dgrad needs the transposed weight copy (QuantizedTensorPair.data_t)")
                 if b_t.axis != -2:
                     raise ValueError("QuantizedTensorPair.data_t must be quantised along axis=-2")
-                w_col, w_cs = b_t.codes, b_t.scales
+                w_col, w_cs = _cached_codes(b_t, kc), b_t.scales
         else:
             w_row, w_rs, w_col, w_cs = K.quantize_mx_weight_2d_impl(
-                b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN
+                b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
             )
         if grouped:
-            y = K.grouped_gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, group_lens)
+            y = K.grouped_gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, group_lens, kchunk=kc)
         else:
-            y = K.gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs)
+            y = K.gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, kchunk=kc)
         if glu and need_dgrad:
             ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens, a, probs, row_mask)
         else:
@@ -122,6 +140,7 @@ class _MXLinearFunction(torch.autograd.Function):
         ctx.activation = activation
         ctx.grad_sr = bool(grad_sr) and act_fmt == _lib.FMT_E2M1
         ctx.rht_signs = rht_signs
+        ctx.kchunk = kc
         return y
 
     @staticmethod
@@ -137,7 +156,9 @@ class _MXLinearFunction(torch.autograd.Function):
             dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
             sr_seed=K.next_sr_seed() if ctx.grad_sr else None,
             rht_signs=ctx.rht_signs if need_wgrad else None,   # same signs as the saved activation copy
+            kchunk=ctx.kchunk,
         )
+        kc = ctx.kchunk
         grad_a = grad_b = None
         overlap = _wgrad_overlap and need_dgrad and need_wgrad
         if overlap:
@@ -146,19 +167,19 @@ class _MXLinearFunction(torch.autograd.Function):
             side.wait_stream(main)   # the quantised operands are ready
         if need_dgrad:
             if grouped:
-                grad_a = K.grouped_gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, group_lens)
+                grad_a = K.grouped_gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, group_lens, kchunk=kc)
             else:
-                grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs)
+                grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc)
         if need_wgrad:
             if overlap:
                 with torch.cuda.stream(side):
-                    grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
+                    grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc).view(w_shape)
                 for t in (d_col, d_cs, a_col, a_cs, grad_b):
                     t.record_stream(side)
                 grad_b.record_stream(main)
                 main.wait_stream(side)
             else:
-                grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m).view(w_shape)
+                grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc).view(w_shape)
         grad_p = None
         if ctx.activation is not None and need_dgrad:
             # grad_a so far is dL/dX; take it through the activation to fc1's output and the probabilities

@@ -113,3 +113,96 @@ def test_kchunk_argument_checks(gpu):
         K.unchunk(K.unchunk(q[0]))
     y = K.gemm_mx_nt_impl(q[0], q[1], w[0], w[1], kchunk=True)
     assert y.shape == (64, 32)
+
+
+def _op_run(gpu, fp4, lens, n, k, cached, glu):
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import (Float4QuantConfig, Float8QuantConfig, Format, QuantizedTensorPair, ScaleDtype,
+                                         ScalingGranularity, create_quantized_weight, float4_e2m1fn_x2, float8_e4m3)
+
+    if fp4:
+        cfg = Float4QuantConfig(format=Format.E2M1_X2, granularity=ScalingGranularity.MX_BLOCKWISE,
+                                scale_dtype=ScaleDtype.E8M0, block_size=32)
+        dest = float4_e2m1fn_x2
+    else:
+        cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE,
+                                scale_dtype=ScaleDtype.E8M0, block_size=32)
+        dest = float8_e4m3
+    rows = 200 if lens is None else sum(lens)
+    g = torch.Generator().manual_seed(rows + n + k)
+    x = torch.randn(rows, 2 * k if glu else k, generator=g).bfloat16().to(gpu).requires_grad_()
+    wshape = (n, k) if lens is None else (len(lens), n, k)
+    w = (torch.randn(*wshape, generator=g) * 0.05).bfloat16().to(gpu).requires_grad_()
+    dy = torch.randn(rows, n, generator=g).bfloat16().to(gpu)
+    b = QuantizedTensorPair(*create_quantized_weight(w, dest, cfg)) if cached else w
+    if lens is None:
+        y = (turbo.ops.gemm_fp4 if fp4 else turbo.ops.gemm_fp8)(x, b, config=cfg)
+        probs = None
+    else:
+        gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+        if glu:
+            probs = torch.rand(rows, generator=g).to(gpu).requires_grad_()
+            y = (turbo.ops.glu_grouped_gemm_fp4 if fp4 else turbo.ops.glu_grouped_gemm_fp8)(x, probs, b, gl, config=cfg)
+        else:
+            probs = None
+            y = (turbo.ops.grouped_gemm_fp4 if fp4 else turbo.ops.grouped_gemm_fp8)(x, b, gl, config=cfg)
+    outs = [y]
+    if cached:
+        outs += list(torch.autograd.grad(y, [x] + ([probs] if glu else []), dy))
+        outs.append(b.data.dequantize())
+        outs.append(b.data_t.dequantize())
+    else:
+        outs += list(torch.autograd.grad(y, [x, w] + ([probs] if glu else []), dy))
+    torch.cuda.synchronize()
+    return outs
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+@pytest.mark.parametrize("lens,n,k,glu", [(None, 96, 160, False), ([33, 0, 130, 1, 92], 160, 96, False),
+                                          ([257, 255], 384, 256, False), ([33, 0, 130, 1, 92], 96, 160, True),
+                                          ([0, 0], 64, 64, False)])
+@pytest.mark.parametrize("cached", [False, True])
+def test_operators_same_on_both_layouts(gpu, fp4, lens, n, k, glu, cached):
+    """The differentiable operators keep their operands K-chunk-major by default; forward, dgrad, wgrad,
+    probability gradients and the dequantised weight caches equal the row-major run bit for bit."""
+    import primus_amd.pytorch as turbo
+
+    try:
+        turbo.ops.set_kchunk_layout(False)
+        ref = _op_run(gpu, fp4, lens, n, k, cached, glu)
+        turbo.ops.set_kchunk_layout(True)
+        out = _op_run(gpu, fp4, lens, n, k, cached, glu)
+    finally:
+        turbo.ops.set_kchunk_layout(True)
+    assert len(ref) == len(out)
+    for r, o in zip(ref, out):
+        assert r.shape == o.shape and _same(r, o)
+
+
+def test_cache_layout_decides(gpu):
+    """A row-major weight cache is used as it is; a chunked cache still serves a row-major call."""
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import (Float8QuantConfig, Format, QuantizedTensorPair, ScaleDtype, ScalingGranularity,
+                                         create_quantized_weight, float8_e4m3)
+
+    cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0,
+                            block_size=32)
+    g = torch.Generator().manual_seed(3)
+    lens = [70, 0, 58]
+    x = torch.randn(sum(lens), 160, generator=g).bfloat16().to(gpu).requires_grad_()
+    w = (torch.randn(3, 96, 160, generator=g) * 0.05).bfloat16().to(gpu)
+    dy = torch.randn(sum(lens), 96, generator=g).bfloat16().to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    res = []
+    for cache_kc, call_kc in [(False, False), (False, True), (True, False), (True, True)]:
+        pair = QuantizedTensorPair(*create_quantized_weight(w, float8_e4m3, cfg, kchunk=cache_kc))
+        assert pair.data.kchunk == cache_kc and pair.data.codes.dim() == 3
+        try:
+            turbo.ops.set_kchunk_layout(call_kc)
+            y = turbo.ops.grouped_gemm_fp8(x, pair, gl, config=cfg)
+            (dx,) = torch.autograd.grad(y, [x], dy)
+        finally:
+            turbo.ops.set_kchunk_layout(True)
+        res.append((y, dx))
+    for y, dx in res[1:]:
+        assert _same(y, res[0][0]) and _same(dx, res[0][1])

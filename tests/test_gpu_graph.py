@@ -1,0 +1,115 @@
+"""The operators under HIP graph capture: tokens-per-expert stays on the device and no entry point
+allocates, synchronises or reads device memory from the host, so a captured forward + backward can be
+replayed on new inputs AND new routing.  Every replay is checked against the eager result."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg(fp4):
+    from primus_amd.pytorch.core import Float4QuantConfig, Float8QuantConfig, Format, ScaleDtype, ScalingGranularity
+
+    if fp4:
+        return Float4QuantConfig(format=Format.E2M1_X2, granularity=ScalingGranularity.MX_BLOCKWISE,
+                                 scale_dtype=ScaleDtype.E8M0, block_size=32)
+    return Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0,
+                             block_size=32)
+
+
+def _same(a, b):
+    return torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+@pytest.mark.parametrize("overlap", [True, False])
+def test_grouped_linear_replays_with_new_routing(gpu, fp4, overlap):
+    import primus_amd.pytorch as turbo
+
+    op = turbo.ops.grouped_gemm_fp4 if fp4 else turbo.ops.grouped_gemm_fp8
+    cfg = _cfg(fp4)
+    G, n, k, rows = 4, 384, 256, 700
+    gen = torch.Generator().manual_seed(11)
+    x = torch.randn(rows, k, generator=gen).bfloat16().to(gpu).requires_grad_()
+    w = (torch.randn(G, n, k, generator=gen) * 0.05).bfloat16().to(gpu).requires_grad_()
+    dy = torch.randn(rows, n, generator=gen).bfloat16().to(gpu)
+    lens = torch.tensor([100, 0, 343, 257], dtype=torch.int64, device=gpu)
+
+    def step():
+        y = op(x, w, lens, config=cfg)
+        dx, dw = torch.autograd.grad(y, [x, w], dy)
+        return y, dx, dw
+
+    turbo.ops.set_wgrad_overlap(overlap)
+    try:
+        # warm-up on a side stream, as torch asks for before a capture
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            step()
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = step()
+        cases = [([100, 0, 343, 257], 1), ([0, 0, 0, 700], 2), ([175, 175, 175, 175], 3), ([699, 1, 0, 0], 4),
+                 ([100, 0, 343, 257], 5)]
+        for new_lens, seed in cases:
+            g2 = torch.Generator().manual_seed(seed)
+            with torch.no_grad():
+                x.copy_(torch.randn(rows, k, generator=g2).bfloat16())
+                w.copy_((torch.randn(G, n, k, generator=g2) * 0.05).bfloat16())
+                dy.copy_(torch.randn(rows, n, generator=g2).bfloat16())
+                lens.copy_(torch.tensor(new_lens, dtype=torch.int64))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [t.clone() for t in outs]
+            want = step()          # eager work and a synchronisation between the replays
+            torch.cuda.synchronize()
+            for a, b in zip(got, want):
+                assert _same(a, b), (new_lens, seed)
+    finally:
+        turbo.ops.set_wgrad_overlap(True)
+
+
+def test_dense_and_fused_activation_replay(gpu):
+    import primus_amd.pytorch as turbo
+
+    cfg = _cfg(False)
+    rows, f, n, G = 512, 256, 128, 2
+    gen = torch.Generator().manual_seed(5)
+    h = torch.randn(rows, 2 * f, generator=gen).bfloat16().to(gpu).requires_grad_()
+    probs = torch.rand(rows, generator=gen).to(gpu).requires_grad_()
+    w2 = (torch.randn(G, n, f, generator=gen) * 0.05).bfloat16().to(gpu).requires_grad_()
+    wd = (torch.randn(2 * f, n, generator=gen) * 0.05).bfloat16().to(gpu).requires_grad_()
+    dy = torch.randn(rows, 2 * f, generator=gen).bfloat16().to(gpu)
+    lens = torch.tensor([200, 312], dtype=torch.int64, device=gpu)
+
+    def step():
+        y = turbo.ops.glu_grouped_gemm_fp8(h, probs, w2, lens, config=cfg)      # [rows, n]
+        z = turbo.ops.gemm_fp8(y, wd, config=cfg)                                # [rows, 2f]
+        return (z,) + torch.autograd.grad(z, [h, probs, w2, wd], dy)
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for new_lens, seed in [([200, 312], 1), ([512, 0], 2), ([1, 511], 3)]:
+        g2 = torch.Generator().manual_seed(seed)
+        with torch.no_grad():
+            h.copy_(torch.randn(rows, 2 * f, generator=g2).bfloat16())
+            probs.copy_(torch.rand(rows, generator=g2))
+            lens.copy_(torch.tensor(new_lens, dtype=torch.int64))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert _same(a, b), (new_lens, seed)

@@ -496,14 +496,21 @@ constexpr int gemm_lds_bytes(int afmt, int bfmt) {
            (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
 }
 
-static int num_cus() {
-    static std::atomic<int> cached{0};
-    int v = cached.load(std::memory_order_relaxed);
+// Per-device caches are indexed by the device ordinal (64 slots; a process with more devices shares slots,
+// which only costs a repeated query).
+static int current_device_slot() {
+    int dev = 0;
+    return hipGetDevice(&dev) == hipSuccess ? (dev & 63) : 0;
+}
+
+static int num_cus(int slot) {
+    static std::atomic<int> cached[64];
+    int v = cached[slot].load(std::memory_order_relaxed);
     if (v) return v;
     int dev = 0;
     hipDeviceProp_t pr;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&pr, dev) != hipSuccess) return 256;
-    cached.store(pr.multiProcessorCount, std::memory_order_relaxed);
+    cached[slot].store(pr.multiProcessorCount, std::memory_order_relaxed);
     return pr.multiProcessorCount;
 }
 
@@ -511,14 +518,15 @@ template <int AFMT, int BFMT, int MODE, int LAYOUT>
 static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = gemm_lds_bytes(AFMT, BFMT);
     if (!device_is_gfx950()) return MXL_ENODEV;
-    static std::atomic<bool> attr_set{false};
+    static std::atomic<bool> attr_set[64];   // the attribute belongs to the (kernel, device) pair
+    const int slot = current_device_slot();
     auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT>;
-    if (!attr_set.load(std::memory_order_acquire)) {
+    if (!attr_set[slot].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
-        attr_set.store(true, std::memory_order_release);
+        attr_set[slot].store(true, std::memory_order_release);
     }
-    int64_t grid = num_cus();
+    int64_t grid = num_cus(slot);
     if (max_tiles < grid) grid = max_tiles;
     if (grid <= 0) return MXL_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(GTHREADS), lds, st, a);

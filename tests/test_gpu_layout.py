@@ -206,3 +206,33 @@ def test_cache_layout_decides(gpu):
         res.append((y, dx))
     for y, dx in res[1:]:
         assert _same(y, res[0][0]) and _same(dx, res[0][1])
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_operators_same_on_both_layouts_random_shapes(gpu, seed):
+    """Seeded sweep of the comparison above: dense and grouped, FP8 / FP4 / mixed, fused activation, cached
+    weights, contraction and output dims that need padding, empty and one-row experts."""
+    rng = np.random.default_rng(seed)
+    import primus_amd.pytorch as turbo
+
+    done = 0
+    while done < 40:
+        dense = rng.random() < 0.25
+        lens = None if dense else [int(v) for v in rng.choice([0, 1, 33, 128, 257, 300], size=int(rng.choice([1, 2, 5, 33])))]
+        if lens is not None and sum(lens) == 0:
+            continue
+        n = int(rng.choice([32, 96, 160, 256, 544]))
+        k = int(rng.choice([32, 64, 160, 352, 1024]))
+        fp4 = bool(rng.random() < 0.5)
+        glu = (not dense) and rng.random() < 0.3
+        cached = bool(rng.random() < 0.3)
+        try:
+            turbo.ops.set_kchunk_layout(False)
+            ref = _op_run(gpu, fp4, lens, n, k, cached, glu)
+            turbo.ops.set_kchunk_layout(True)
+            out = _op_run(gpu, fp4, lens, n, k, cached, glu)
+        finally:
+            turbo.ops.set_kchunk_layout(True)
+        for i, (r, o) in enumerate(zip(ref, out)):
+            assert r.shape == o.shape and _same(r, o), (i, fp4, lens, n, k, cached, glu)
+        done += 1

@@ -225,6 +225,33 @@ int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtyp
                            const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                            void* s_colT, uint32_t flags, void* stream);
 
+/* RMSNorm in front of the column-parallel linear (rmsnorm(x, layer_norm_weight, eps) in
+ * PrimusTurboLayerNormColumnParallelLinear.forward_internal, primus_turbo.py:1689-1700):
+ *   rstd[m] = 1 / sqrt(mean_j x[m, j]^2 + eps),   y[m, j] = (x[m, j] * rstd[m]) * w[j]
+ * for bf16 x[rows, k], w[k]; fp32 arithmetic, y rounded once to bf16, rstd[rows] fp32 (kept for the backward).
+ * y_bf16 may be NULL: then only rstd is written (what mxl_rmsnorm_quantize needs).  Requires k % 8 == 0 and
+ * k <= 16384.  The sum of squares is taken in a fixed order, so results do not depend on the launch. */
+int mxl_rmsnorm_fwd(const void* x_bf16, const void* w_bf16, float eps, int64_t rows, int64_t k, void* y_bf16,
+                    void* rstd_f32, void* stream);
+
+/* Backward of the above: dx[rows, k] (bf16) and dw[k] (bf16; zeros for rows == 0) from dy[rows, k].  The column
+ * sums of dw go through `workspace`, at least mxl_rmsnorm_bwd_workspace_bytes(rows, k) bytes of device
+ * memory, 16-byte aligned, owned by the caller (the library allocates nothing); its contents need no
+ * initialisation and are dead after the call's kernels have run. */
+int64_t mxl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t k);
+int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows,
+                    int64_t k, void* dx_bf16, void* dw_bf16, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* The normalisation feeding the MX quantiser directly: what mxl_quantize would produce for
+ * y = mxl_rmsnorm_fwd(x, w, ...) (bit for bit) from x, w and rstd (mxl_rmsnorm_fwd with y_bf16 = NULL), without
+ * y reaching memory: the quantised copies are all the following GEMMs read.  The reference runs rmsnorm and the
+ * quantisation inside gemm_fp8 / gemm_fp4 as separate kernels (primus_turbo.py:1689-1741).  The other arguments
+ * are those of mxl_quantize with cols = k (k % 32 == 0); a row-wise copy must be requested.  flags: 0 or
+ * MXL_QF_KCHUNK. */
+int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows, int64_t k,
+                         int64_t row_ld, int fmt, int scale_mode, const int64_t* group_lens, int num_groups,
+                         void* q_row, void* s_row, void* q_colT, void* s_colT, uint32_t flags, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -72,6 +72,16 @@ Parity status
   the sign-vector definition.  The reference states neither the transform size
   nor the sign vector (they live in Primus-Turbo's C++ op): **parity unpinned**.
 
+* ``rmsnorm_rstd`` / ``rmsnorm_ref`` / ``rmsnorm_bwd_ref`` (RMSNorm in front of the
+  column-parallel linear, ``rmsnorm(x, layer_norm_weight, eps)`` at
+  primus_turbo.py:1689-1700): y = (x * rstd) * w in float32 with one rounding, the
+  sum of squares in the fixed order the HIP kernel documents (so rstd and y are
+  reproduced bit for bit); pinned against float64 closed forms, against torch's
+  ``rms_norm`` (library routine, to one bf16 ulp) and its autograd, and by the
+  invariants rms(y / w) = 1 and scale invariance of y in x.  Whether Primus-Turbo's
+  kernel rounds once or after the normalisation and again after the weight
+  (as torch's composite does) is **parity unpinned** (package absent).
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -668,3 +678,56 @@ def glu_with_probs_bwd_ref(dy, x, probs, row_mask=None, activation: str = "silu"
         dx = np.where(m.reshape(-1, 1), dx, 0.0)
         dp = np.where(m, dp, 0.0)
     return dx, dp
+
+
+# --------------------------------------------------------------------------
+# RMSNorm in front of the column-parallel linear (primus_turbo.py:1689-1700)
+# --------------------------------------------------------------------------
+_NORM_THREADS = 256
+
+
+def rmsnorm_rstd(x, eps: float) -> np.ndarray:
+    """rstd[m] = 1 / sqrt(mean_j x[m, j]^2 + eps) in float32, summed in the order of the HIP kernel:
+    lane t of 256 adds the squares of its 8-element chunks (columns 8t + 2048 i ...) one element at a
+    time, the 64 lanes of a wave are combined by an xor butterfly from distance 32 down to 1, the four
+    waves are added in order.  (Squares of bf16 values are exact in float32.)"""
+    xf = bf16_bits_to_f32(to_bf16_bits(x))
+    rows, k = xf.shape
+    assert k % 8 == 0
+    chunks = -(-k // (_NORM_THREADS * 8))
+    pad = np.zeros((rows, chunks * _NORM_THREADS * 8), dtype=np.float32)
+    pad[:, :k] = xf
+    sq = (pad * pad).reshape(rows, chunks, _NORM_THREADS, 8)
+    lane = np.zeros((rows, _NORM_THREADS), dtype=np.float32)
+    for c in range(chunks):
+        for e in range(8):
+            lane = lane + sq[:, c, :, e]
+    v = lane.reshape(rows, 4, 64)
+    for s_ in (32, 16, 8, 4, 2, 1):
+        v = v + v[:, :, np.arange(64) ^ s_]
+    part = v[:, :, 0]
+    total = ((part[:, 0] + part[:, 1]) + part[:, 2]) + part[:, 3]
+    mean = total / np.float32(k)
+    return (np.float32(1.0) / np.sqrt(mean + np.float32(eps), dtype=np.float32)).astype(np.float32)
+
+
+def rmsnorm_ref(x, w, eps: float):
+    """(y bits [rows, k], rstd [rows]): y = (x * rstd) * w, float32 products in that order, one rounding."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x))
+    wf = bf16_bits_to_f32(to_bf16_bits(w)).reshape(1, -1)
+    rstd = rmsnorm_rstd(x, eps)
+    y = (xf * rstd.reshape(-1, 1)) * wf
+    return f32_to_bf16_bits(y.astype(np.float32)), rstd
+
+
+def rmsnorm_bwd_ref(dy, x, w, eps: float):
+    """(dx [rows, k], dw [k]) in float64 from the closed form: with g = dy * w, xh = x * rstd,
+    dx = (g - xh * mean_j(g * xh)) * rstd and dw = sum_m dy * xh."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x)).astype(np.float64)
+    d = bf16_bits_to_f32(to_bf16_bits(dy)).astype(np.float64)
+    wf = bf16_bits_to_f32(to_bf16_bits(w)).astype(np.float64).reshape(1, -1)
+    rstd = 1.0 / np.sqrt((xf * xf).mean(axis=1, keepdims=True) + eps)
+    xh = xf * rstd
+    g = d * wf
+    dx = (g - xh * (g * xh).mean(axis=1, keepdims=True)) * rstd
+    return dx, (d * xh).sum(axis=0)

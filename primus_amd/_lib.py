@@ -46,6 +46,10 @@ EXPORTS = (
     "mxl_glu_probs_fwd",
     "mxl_glu_probs_bwd",
     "mxl_glu_probs_quantize",
+    "mxl_rmsnorm_fwd",
+    "mxl_rmsnorm_bwd",
+    "mxl_rmsnorm_bwd_workspace_bytes",
+    "mxl_rmsnorm_quantize",
 )
 
 
@@ -107,6 +111,14 @@ def load() -> ctypes.CDLL:
         lib.mxl_glu_probs_quantize.restype = i32
         lib.mxl_glu_probs_quantize.argtypes = [vp, vp, i32, vp, i64, i64, i64, i32, i32, i32, vp, i32, vp, vp, vp, vp,
                                                ctypes.c_uint32, vp]
+        lib.mxl_rmsnorm_fwd.restype = i32
+        lib.mxl_rmsnorm_fwd.argtypes = [vp, vp, ctypes.c_float, i64, i64, vp, vp, vp]
+        lib.mxl_rmsnorm_bwd_workspace_bytes.restype = i64
+        lib.mxl_rmsnorm_bwd_workspace_bytes.argtypes = [i64, i64]
+        lib.mxl_rmsnorm_bwd.restype = i32
+        lib.mxl_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i64, vp]
+        lib.mxl_rmsnorm_quantize.restype = i32
+        lib.mxl_rmsnorm_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, u32, vp]
         _lib = lib
     return _lib
 

@@ -205,4 +205,15 @@ template <int ACT> __device__ __forceinline__ uint4 glu8(const uint4& g, const u
     return make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
+// ---- RMSNorm (shared by the normalisation kernels and the fused normalisation + quantisation path) ----
+// 8 outputs (x * rstd) * w from 8 input and 8 weight bf16 values, fp32 products in that order, rounded once
+__device__ __forceinline__ uint4 norm8(const uint4& x, const uint4& wv, float rstd) {
+    const uint32_t xw[4] = {x.x, x.y, x.z, x.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        ow[k] = pack_bf16(bf16_lo(xw[k]) * rstd * bf16_lo(ww[k]), bf16_hi(xw[k]) * rstd * bf16_hi(ww[k]));
+    return make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 }  // namespace mxl

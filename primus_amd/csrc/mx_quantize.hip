@@ -64,6 +64,9 @@ struct QuantArgs {
     const void* probs;
     int probs_bf16;
     const uint8_t* row_mask;
+    // fused RMSNorm in front (ACT == PRO_RMSNORM): the tensor that is quantised is (x * rstd[row]) * norm_w[col];
+    // rstd travels in `probs` (fp32)
+    const uint16_t* norm_w;
     // Code layout of both copies.  0: row-major [rows, ld].  1: K-chunk-major [ld / 128][rows][128 elements]:
     // the 128 elements of a row that one GEMM K slot consumes stay together and consecutive rows follow
     // each other, so a GEMM tile's slot is one contiguous block and this kernel writes 128 x 128-element
@@ -106,6 +109,8 @@ __device__ __forceinline__ bool quant_tile_of_workgroup(const QuantArgs& a, int&
 // 1, 2, 4, 8) and rounded once to bf16; that tensor is then quantised like any other.  The transform is
 // orthogonal, so a wgrad GEMM whose two operands were both transformed computes the same contraction
 // while single large values are spread over 16 positions before they meet the 4-bit grid.
+constexpr int PRO_RMSNORM = 2;   // value of ACT next to MXL_ACT_SILU (0) and MXL_ACT_GELU (1)
+
 template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1, bool SR = false, bool RHT = false>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     constexpr bool FP4 = (FMT == kFmtE2M1);
@@ -161,7 +166,11 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     // handed round through LDS; fetched per lane and row they would double the number of load instructions
     __shared__ float prob_tile[ACT >= 0 ? QT : 1];
     __shared__ uint8_t live_tile[ACT >= 0 ? QT : 1];
-    if (ACT >= 0) {
+    float my_rstd = 0.f;
+    if (ACT == PRO_RMSNORM) {
+        // only requested here; it is handed round after the tile's own loads have gone out
+        if (t < QT && t < rows_valid) my_rstd = ((const float*)a.probs)[src_row0 + t];
+    } else if (ACT >= 0) {
         if (t < QT) {
             const bool live = t < rows_valid && (a.row_mask == nullptr || a.row_mask[src_row0 + t] != 0);
             live_tile[t] = live ? 1 : 0;
@@ -176,6 +185,8 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 
     // ---- load 8 rows x 8 columns per lane ----
     uint4 d[8];
+    uint4 norm_wv = make_uint4(0, 0, 0, 0);
+    if (ACT == PRO_RMSNORM && col_ok) norm_wv = *(const uint4*)(a.norm_w + col);
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
         const int r = 32 * w + 8 * rg + it;
@@ -183,12 +194,26 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         if (col_ok && r < rows_valid) {
             if (ACT < 0) {
                 d[it] = load16_streaming(a.x + (src_row0 + r) * a.cols + col);
+            } else if (ACT == PRO_RMSNORM) {
+                d[it] = load16_streaming(a.x + (src_row0 + r) * a.cols + col);
             } else {
                 if (live_tile[r]) {
                     const uint16_t* xr = a.x + (src_row0 + r) * 2 * a.cols + col;
-                    d[it] = glu8<(ACT < 0 ? 0 : ACT)>(load16_streaming(xr), load16_streaming(xr + a.cols), prob_tile[r]);
+                    d[it] = glu8<(ACT == MXL_ACT_GELU ? MXL_ACT_GELU : MXL_ACT_SILU)>(load16_streaming(xr),
+                                                                                      load16_streaming(xr + a.cols),
+                                                                                      prob_tile[r]);
                 }
             }
+        }
+    }
+
+    if (ACT == PRO_RMSNORM) {
+        if (t < QT) prob_tile[t] = my_rstd;
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = 32 * w + 8 * rg + it;
+            if (col_ok && r < rows_valid) d[it] = norm8(d[it], norm_wv, prob_tile[r]);
         }
     }
 
@@ -537,7 +562,7 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
                        int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
                        bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0,
-                       bool kchunk = false) {
+                       bool kchunk = false, const void* norm_w = nullptr) {
     if (row_ld == 0) row_ld = cols;
     if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
     if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
@@ -563,6 +588,7 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.probs = probs;
     a.probs_bf16 = probs_dtype == MXL_PROBS_BF16;
     a.row_mask = row_mask;
+    a.norm_w = (const uint16_t*)norm_w;
     a.sr_seed = sr_seed;
     a.rht_signs = rht_signs & 0xFFFFu;
     a.kchunk = kchunk ? 1 : 0;
@@ -576,6 +602,7 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     if (rht) return dispatch_quant_fp4<false, true>(scale_mode, a, gx, gy, (hipStream_t)stream);
     if (act == MXL_ACT_SILU) return dispatch_quant<false, MXL_ACT_SILU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     if (act == MXL_ACT_GELU) return dispatch_quant<false, MXL_ACT_GELU>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
+    if (act == PRO_RMSNORM) return dispatch_quant<false, PRO_RMSNORM>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
     return dispatch_quant<false>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
 }
 
@@ -607,6 +634,16 @@ extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int
                        probs, probs_dtype, row_mask, stream, false, 0, false, 0, (flags & MXL_QF_KCHUNK) != 0);
 }
 
+extern "C" int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows, int64_t k,
+                                    int64_t row_ld, int fmt, int scale_mode, const int64_t* group_lens, int num_groups,
+                                    void* q_row, void* s_row, void* q_colT, void* s_colT, uint32_t flags, void* stream) {
+    if (!w_bf16 || (rows > 0 && !rstd_f32)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    return quantize_1d(x_bf16, rows, k, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
+                       PRO_RMSNORM, rstd_f32, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
+                       (flags & MXL_QF_KCHUNK) != 0, w_bf16);
+}
+
 static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld, int64_t n_ld, int fmt,
                               int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT, bool kchunk,
                               void* stream) {
@@ -634,6 +671,7 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
     a.probs = nullptr;
     a.probs_bf16 = 0;
     a.row_mask = nullptr;
+    a.norm_w = nullptr;
     a.sr_seed = 0;
     a.rht_signs = 0;
     a.kchunk = kchunk ? 1 : 0;

@@ -467,15 +467,26 @@ class _LowPrecisionGemm:
         return x, pair, fuse_pattern
 
     def _gemm(self, x: torch.Tensor, weight: torch.Tensor, is_first_microbatch: bool,
-              group_lens: Optional[torch.Tensor] = None, glu: Optional[Tuple] = None) -> torch.Tensor:
+              group_lens: Optional[torch.Tensor] = None, glu: Optional[Tuple] = None,
+              norm: Optional[Tuple] = None) -> torch.Tensor:
         """``glu = (probs, row_mask, activation)``: ``x`` is the previous linear's output and the gated
-        activation is applied on the way into this GEMM (grouped only)."""
+        activation is applied on the way into this GEMM (grouped only).  ``norm = (weight, eps)``: ``x`` is
+        the input of an RMSNorm that is applied on the way into this GEMM (dense only)."""
         manager = PrimusTurboLowPrecisionGlobalStateManager
         grouped = group_lens is not None
         one_microbatch = runtime.get_num_microbatches() == 1
         assert glu is None or grouped, "the activation prologue exists for the grouped (expert) linears only"
+        assert norm is None or not grouped, "the normalisation prologue exists for the dense linears only"
 
         def run(op_dense, op_grouped, a, b, fuse_pattern, **kw):
+            if norm is not None:
+                norm_weight, eps = norm
+                if op_dense is ops.gemm:               # outside a low-precision autocast: two plain operators
+                    return op_dense(ops.rmsnorm(a, norm_weight, eps), b, trans_a=False, trans_b=True, out_dtype=None,
+                                    fuse_bgrad_accum_pattern=fuse_pattern)
+                fused = ops.rmsnorm_gemm_fp8 if op_dense is ops.gemm_fp8 else ops.rmsnorm_gemm_fp4
+                return fused(a, norm_weight, eps, b, trans_a=False, trans_b=True, out_dtype=None,
+                             fuse_bgrad_accum_pattern=fuse_pattern, **kw)
             if glu is not None:
                 probs, row_mask, activation = glu
                 if op_grouped is ops.grouped_gemm:     # outside a low-precision autocast: two plain operators
@@ -585,8 +596,14 @@ class PrimusTurboLinear(_LowPrecisionGemm, torch.nn.Module):
     def _prologue(self, x: torch.Tensor) -> torch.Tensor:
         return x
 
+    def _norm_for_gemm(self, x: torch.Tensor) -> Optional[Tuple]:
+        """``(weight, eps)`` if a normalisation in front of this linear is to be folded into the GEMM's
+        quantiser; the plain linears have none."""
+        return None
+
     def forward_internal(self, x: torch.Tensor, is_first_microbatch: bool = False):
-        inp = self._prologue(x)
+        norm = self._norm_for_gemm(x)
+        inp = x if norm is not None else self._prologue(x)
         weight = self._parameters["weight"]
         bias_tensor = torch.cat([getattr(self, n) for n in self.bias_names]) if self.use_bias else None
         shape = x.size()
@@ -595,7 +612,7 @@ class PrimusTurboLinear(_LowPrecisionGemm, torch.nn.Module):
         inp = inp.view(-1, shape[-1])
         if _use_split_wgrad_op():
             raise NotImplementedError("the split-wgrad (zero-bubble) GEMM is a bf16 path outside this package")
-        out = self._gemm(inp, weight, is_first_microbatch)
+        out = self._gemm(inp, weight, is_first_microbatch, norm=norm)
         out = out.view(shape[0], shape[1], -1)
         if bias_tensor is not None:
             out = out + bias_tensor
@@ -647,6 +664,9 @@ class PrimusTurboLayerNormColumnParallelLinear(PrimusTurboColumnParallelLinear):
                          tp_comm_buffer_name=tp_comm_buffer_name, tp_group=tp_group)
         self.normalization = getattr(config, "normalization", "LayerNorm")
         self.eps = float(getattr(config, "layernorm_epsilon", 1e-5))
+        # fold the RMSNorm into the quantiser of the GEMM's input (same values bit for bit, the normalised
+        # tensor is never written); off = the reference's kernel sequence
+        self.fuse_norm_into_quantize = bool(getattr(runtime.get_args(), "turbo_fuse_norm_into_quantize", True))
         dtype, device = self.weight.dtype, self.weight.device
         self.layer_norm_weight = torch.nn.Parameter(torch.ones(self.in_features, dtype=dtype, device=device))
         if self.normalization == "LayerNorm":
@@ -654,10 +674,24 @@ class PrimusTurboLayerNormColumnParallelLinear(PrimusTurboColumnParallelLinear):
         else:
             self.register_parameter("layer_norm_bias", None)
 
+    def _native_rmsnorm_ok(self, x: torch.Tensor) -> bool:
+        """The RMSNorm kernels take bf16 CUDA tensors with a last dim that is a multiple of 8 up to 16384."""
+        k = x.size(-1)
+        return (self.normalization == "RMSNorm" and x.is_cuda and x.dtype == torch.bfloat16
+                and self.layer_norm_weight.dtype == torch.bfloat16 and k % 8 == 0 and k <= 16384)
+
+    def _norm_for_gemm(self, x: torch.Tensor) -> Optional[Tuple]:
+        if not (self.fuse_norm_into_quantize and self._native_rmsnorm_ok(x) and x.size(-1) % 32 == 0):
+            return None
+        return self.layer_norm_weight, self.eps
+
     def _prologue(self, x: torch.Tensor) -> torch.Tensor:
         if self.normalization == "LayerNorm":
             return torch.nn.functional.layer_norm(x, [x.size(-1)], self.layer_norm_weight, self.layer_norm_bias, self.eps)
         if self.normalization == "RMSNorm":
+            if self._native_rmsnorm_ok(x):
+                return ops.rmsnorm(x, self.layer_norm_weight, self.eps)     # primus_turbo.py:1696-1698
+            # other dtypes / devices: the library routine (the reference's operator is GPU-only as well)
             return torch.nn.functional.rms_norm(x, [x.size(-1)], self.layer_norm_weight, self.eps)
         raise AssertionError("Not support normalization type.")
 

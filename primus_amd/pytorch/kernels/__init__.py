@@ -543,6 +543,91 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
 
 
 # --------------------------------------------------------------------------
+# RMSNorm in front of the column-parallel linear (rmsnorm(x, weight, eps),
+# primus_turbo.py:1689-1700)
+# --------------------------------------------------------------------------
+RMSNORM_MAX_K = 16384
+
+
+def _norm_args(x, weight):
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("expected a contiguous 2-D bfloat16 tensor [tokens, K]")
+    k = x.shape[1]
+    if k % 8 != 0 or k > RMSNORM_MAX_K:
+        raise ValueError(f"the normalised dim ({k}) must be a multiple of 8 and at most {RMSNORM_MAX_K}")
+    if weight.dtype != torch.bfloat16 or tuple(weight.shape) != (k,) or not weight.is_contiguous():
+        raise ValueError("the norm weight must be a contiguous bfloat16 vector [K]")
+    _require_cuda(x, weight)
+
+
+def rmsnorm_fwd_impl(x, weight, eps: float, want_y: bool = True):
+    """``(y, rstd)``: ``y = (x * rstd) * weight`` in fp32 rounded once to bf16 (``None`` if not wanted),
+    ``rstd = 1 / sqrt(mean(x^2) + eps)`` per row in fp32."""
+    _norm_args(x, weight)
+    rows, k = x.shape
+    y = torch.empty_like(x) if want_y else None
+    rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    with _hooked("rmsnorm_fwd", rows=rows, k=k):
+        rc = _lib.load().mxl_rmsnorm_fwd(_ptr(x), _ptr(weight), float(eps), rows, k, _ptr(y), _ptr(rstd), _stream())
+    _lib.check(rc, "mxl_rmsnorm_fwd")
+    return y, rstd
+
+
+def rmsnorm_bwd_impl(dy, x, weight, rstd):
+    """``(dx [tokens, K] bf16, dweight [K] bf16)``."""
+    _norm_args(x, weight)
+    rows, k = x.shape
+    if dy.dtype != torch.bfloat16 or tuple(dy.shape) != (rows, k) or not dy.is_contiguous():
+        raise ValueError("dy must be a contiguous bfloat16 tensor of the shape of x")
+    if rstd.dtype != torch.float32 or tuple(rstd.shape) != (rows,):
+        raise ValueError("rstd must be float32 [tokens]")
+    _require_cuda(dy, rstd)
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    dw = torch.empty_like(weight)
+    ws = torch.empty((max(int(lib.mxl_rmsnorm_bwd_workspace_bytes(rows, k)), 16) // 4,), dtype=torch.float32, device=x.device)
+    with _hooked("rmsnorm_bwd", rows=rows, k=k):
+        rc = lib.mxl_rmsnorm_bwd(_ptr(dy), _ptr(x), _ptr(weight), _ptr(rstd), rows, k, _ptr(dx), _ptr(dw), _ptr(ws),
+                                 ws.numel() * 4, _stream())
+    _lib.check(rc, "mxl_rmsnorm_bwd")
+    return dx, dw
+
+
+def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *, colwise: bool = False,
+                          pad_to: int = 1, kchunk: bool = False):
+    """``quantize_mx_impl(rmsnorm_fwd_impl(x, weight, eps)[0])`` in one pass over ``x`` given ``rstd``, the
+    normalised tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
+    _norm_args(x, weight)
+    rows, k = x.shape
+    if k % BLOCK != 0:
+        raise ValueError(f"the quantised dim ({k}) must be a multiple of {BLOCK}")
+    if rstd.dtype != torch.float32 or tuple(rstd.shape) != (rows,):
+        raise ValueError("rstd must be float32 [tokens]")
+    _require_cuda(rstd)
+    if rows == 0:
+        return quantize_mx_impl(x, fmt, scale_mode, rowwise=True, colwise=colwise, pad_to=pad_to, kchunk=kchunk)
+    per = _per_byte(fmt)
+    dev = x.device
+    row_ld = _round_up(k, KCHUNK if kchunk else pad_to)
+    q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+    s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+    q_col = s_col = None
+    if colwise:
+        W = padded_width(rows, 0)
+        q_col = torch.empty(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = torch.empty((k, W // BLOCK), dtype=torch.uint8, device=dev)
+    with _hooked("rmsnorm_quantize", rows=rows, cols=k, fmt=fmt, rowwise=True, colwise=colwise):
+        rc = _lib.load().mxl_rmsnorm_quantize(
+            _ptr(x), _ptr(weight), _ptr(rstd), rows, k, row_ld, fmt, scale_mode, None, 0, _ptr(q_row), _ptr(s_row),
+            _ptr(q_col), _ptr(s_col), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+        )
+    _lib.check(rc, "mxl_rmsnorm_quantize")
+    cd = _code_dtype(fmt)
+    v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
+    return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0)
+
+
+# --------------------------------------------------------------------------
 # reference-named low-level entry points (MX granularity only)
 # --------------------------------------------------------------------------
 def _require_mx(granularity) -> None:

@@ -37,7 +37,7 @@ from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
 __all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
            "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask", "glu_grouped_gemm_fp8",
-           "glu_grouped_gemm_fp4", "manual_sr_seed", "set_kchunk_layout"]
+           "glu_grouped_gemm_fp4", "manual_sr_seed", "set_kchunk_layout", "rmsnorm", "rmsnorm_gemm_fp8", "rmsnorm_gemm_fp4"]
 
 # dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
 # kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
@@ -88,9 +88,10 @@ class _MXLinearFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode, probs=None, row_mask=None, activation=None,
-                grad_sr=False, rht_signs=None):
+                grad_sr=False, rht_signs=None, norm_weight=None, norm_eps=0.0):
         glu = activation is not None
-        need_dgrad = a.requires_grad or (glu and probs.requires_grad)
+        norm = norm_weight is not None
+        need_dgrad = a.requires_grad or (glu and probs.requires_grad) or (norm and norm_weight.requires_grad)
         need_wgrad = b.requires_grad
         grouped = group_lens is not None
         # Every operand of the three GEMMs is stored in one layout, K-chunk-major unless an operand is
@@ -106,6 +107,12 @@ class _MXLinearFunction(torch.autograd.Function):
             a_row, a_rs, a_col, a_cs = K.glu_with_probs_quantize_impl(
                 a, probs, row_mask, activation, act_fmt, scale_mode, colwise=need_wgrad, group_lens=group_lens,
                 pad_to=K.GEMM_K_ALIGN, kchunk=kc,
+            )
+        elif norm:
+            # X = rmsnorm(a) is formed inside the quantiser from a, the norm weight and the row statistics
+            _, rstd = K.rmsnorm_fwd_impl(a, norm_weight.detach(), norm_eps, want_y=False)
+            a_row, a_rs, a_col, a_cs = K.rmsnorm_quantize_impl(
+                a, norm_weight.detach(), rstd, act_fmt, scale_mode, colwise=need_wgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
             )
         else:
             a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
@@ -134,6 +141,8 @@ class _MXLinearFunction(torch.autograd.Function):
             y = K.gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, kchunk=kc)
         if glu and need_dgrad:
             ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens, a, probs, row_mask)
+        elif norm and need_dgrad:
+            ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens, a, norm_weight.detach(), rstd)
         else:
             ctx.save_for_backward(a_col, a_cs, w_col, w_cs, group_lens)
         ctx.cfg = (act_fmt, scale_mode, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape))
@@ -141,6 +150,7 @@ class _MXLinearFunction(torch.autograd.Function):
         ctx.grad_sr = bool(grad_sr) and act_fmt == _lib.FMT_E2M1
         ctx.rht_signs = rht_signs
         ctx.kchunk = kc
+        ctx.norm = norm
         return y
 
     @staticmethod
@@ -186,7 +196,12 @@ class _MXLinearFunction(torch.autograd.Function):
             pre, probs, row_mask = ctx.saved_tensors[5:8]
             grad_a, grad_p = K.glu_with_probs_bwd_impl(grad_a, pre, probs, row_mask, ctx.activation)
             grad_p = grad_p.to(probs.dtype)
-        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None, None
+        grad_nw = None
+        if ctx.norm and need_dgrad:
+            # grad_a so far is dL/dX for X = rmsnorm(a); take it through the normalisation
+            pre, nw, rstd = ctx.saved_tensors[5:8]
+            grad_a, grad_nw = K.rmsnorm_bwd_impl(grad_a, pre, nw, rstd)
+        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None, None, grad_nw, None
 
 
 def _formats(config, fp4: bool):
@@ -206,7 +221,7 @@ def _formats(config, fp4: bool):
     return f, f
 
 
-def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4, glu=None):
+def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4, glu=None, norm=None):
     if trans_a or not trans_b:
         raise ValueError("the MX linear path is NT only: trans_a=False, trans_b=True (primus_turbo.py:1095-1103)")
     if fuse_bgrad_accum_pattern is not None:
@@ -244,6 +259,14 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
     # stochastic rounding applies to E2M1 gradients; with E4M3 activations the gradients are MXFP8
     grad_sr = bool(fp4 and config.use_gradient_sr and act_fmt == _lib.FMT_E2M1)
     rht = getattr(config, "colwise_rht_signs", None) if fp4 and act_fmt == _lib.FMT_E2M1 else None
+    if norm is not None:
+        if rht is not None or group_lens is not None:
+            raise NotImplementedError("the normalisation prologue exists for the dense linear without the Hadamard transform")
+        norm_weight, eps = norm
+        if norm_weight.dtype != torch.bfloat16 or tuple(norm_weight.shape) != (a.shape[-1],):
+            raise ValueError("the norm weight must be a bfloat16 vector of the contraction length")
+        return _MXLinearFunction.apply(a, b, b_t, None, act_fmt, w_fmt, config.scale_mode.value,
+                                       None, None, None, grad_sr, None, norm_weight.contiguous(), float(eps))
     if glu is None:
         return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
                                        None, None, None, grad_sr, rht)
@@ -269,6 +292,56 @@ def gemm_fp4(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optio
              config: Optional[Float4QuantConfig] = None, fuse_bgrad_accum_pattern: Optional[str] = None):
     """Same with MXFP4 weights (activations per ``config.activation_format``)."""
     return _run(a, b, None, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4=True)
+
+
+class _RMSNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        w = weight.detach().contiguous()
+        y, rstd = K.rmsnorm_fwd_impl(x2, w, eps)
+        ctx.save_for_backward(x2, w, rstd)
+        ctx.shape = shape
+        return y.view(shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, w, rstd = ctx.saved_tensors
+        dy2 = dy.reshape(x2.shape)
+        if dy2.dtype != torch.bfloat16:
+            dy2 = dy2.to(torch.bfloat16)
+        dx, dw = K.rmsnorm_bwd_impl(dy2.contiguous(), x2, w, rstd)
+        return dx.view(ctx.shape), dw, None
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """``(x / sqrt(mean(x^2, -1) + eps)) * weight`` over the last dim, bf16 in and out, fp32 arithmetic with one
+    rounding; differentiable in ``x`` and ``weight``.  Call site of the reference: ``rmsnorm(x,
+    self.layer_norm_weight, self.eps)`` in front of the column-parallel linear (primus_turbo.py:1689-1700)."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("rmsnorm expects bfloat16 input and weight")
+    return _RMSNormFunction.apply(x, weight, float(eps))
+
+
+def rmsnorm_gemm_fp8(x, norm_weight, eps: float, b, trans_a: bool = False, trans_b: bool = True,
+                     out_dtype: Optional[torch.dtype] = None, config: Optional[Float8QuantConfig] = None,
+                     fuse_bgrad_accum_pattern: Optional[str] = None):
+    """``gemm_fp8(rmsnorm(x, norm_weight, eps), b)`` for 2-D ``x`` with the normalisation folded into the
+    quantiser of the GEMM's input: same values bit for bit, forward and backward, without the normalised
+    tensor being written or re-read.  Differentiable in ``x``, ``norm_weight`` and ``b``.  The reference runs
+    the two operators one after the other (primus_turbo.py:1689-1741)."""
+    return _run(x, b, None, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4=False,
+                norm=(norm_weight, eps))
+
+
+def rmsnorm_gemm_fp4(x, norm_weight, eps: float, b, trans_a: bool = False, trans_b: bool = True,
+                     out_dtype: Optional[torch.dtype] = None, config: Optional[Float4QuantConfig] = None,
+                     fuse_bgrad_accum_pattern: Optional[str] = None):
+    return _run(x, b, None, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4=True,
+                norm=(norm_weight, eps))
 
 
 def _lens(group_lens: torch.Tensor) -> torch.Tensor:

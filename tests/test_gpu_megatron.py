@@ -351,3 +351,58 @@ def test_qdq_mxfp4_is_the_forward_weight_grid(mg, gpu):
     shard = w.reshape(-1)[start:end].float()
     local = qdq_mxfp4_local_shard(shard, tuple(w.shape), start, end, torch.bfloat16)
     assert torch.equal(local, got.reshape(-1)[start:end])
+
+
+@pytest.mark.parametrize("fp4", [False, True])
+@pytest.mark.parametrize("microbatches", [1, 2])
+def test_layernorm_linear_folds_the_rmsnorm_into_the_quantiser(mg, gpu, fp4, microbatches):
+    """RMSNorm + column-parallel linear: with the normalisation folded into the GEMM's quantiser the module
+    returns the same output and gradients, bit for bit, as with the two operators run one after the other
+    (the reference's sequence, primus_turbo.py:1689-1741), and both stay close to the bf16 module."""
+    pt = mg
+    from primus_amd.megatron import runtime
+
+    runtime.set_num_microbatches(microbatches)
+    res = {}
+    for fuse in (True, False):
+        runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                         turbo_grouped_gemm_without_padding=True, turbo_fuse_norm_into_quantize=fuse)
+        torch.manual_seed(9)
+        ln = pt.PrimusTurboLayerNormColumnParallelLinear(256, 160, config=_cfg(), bias=True)
+        assert ln.fuse_norm_into_quantize is fuse
+        with torch.no_grad():
+            ln.layer_norm_weight.copy_(1 + 0.1 * torch.randn(256))
+        ln.weight.main_grad = torch.zeros_like(ln.weight, dtype=torch.float32)
+        ln.weight.grad_added_to_main_grad = False
+        x = torch.randn(12, 8, 256, device=gpu).bfloat16().requires_grad_()
+        dy = torch.randn(12, 8, 160, device=gpu).bfloat16()
+        calls = []
+        from primus_amd.pytorch import kernels as K
+        import contextlib
+
+        def hook(name, info):
+            calls.append(name)
+            return contextlib.nullcontext()
+
+        K.set_launch_hook(hook)
+        try:
+            if fp4:
+                ctx = pt.primus_turbo_fp4_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp4(pt))
+            else:
+                ctx = pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=_mxfp8(pt))
+            with ctx:
+                y, _ = ln(x)
+            y.backward(dy)
+        finally:
+            K.set_launch_hook(None)
+        assert ("rmsnorm_quantize" in calls) is fuse
+        wgrad = ln.weight.main_grad.clone() if microbatches > 1 else ln.weight.grad.float()
+        res[fuse] = (y.detach(), x.grad, ln.layer_norm_weight.grad, wgrad, ln.bias.grad)
+        if fuse:
+            y_bf16, _ = ln(x.detach())
+            want = torch.nn.functional.linear(
+                torch.nn.functional.rms_norm(x.detach(), [256], ln.layer_norm_weight, 1e-5), ln.weight, ln.bias)
+            assert _cos(y_bf16, want) > 0.9999
+            assert _cos(y, want) > (0.97 if fp4 else 0.999)
+    for a, b in zip(res[True], res[False]):
+        assert a.shape == b.shape and torch.equal(a, b)

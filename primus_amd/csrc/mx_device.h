@@ -185,8 +185,27 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, h);
 }
 template <int ACT> __device__ __forceinline__ float act_fwd(float g) {
-    if (ACT == MXL_ACT_SILU) return g / (1.f + expf(-g));
-    return 0.5f * g * erfcf(-g * 0.70710678118654752f);   // erfc: no cancellation in the negative tail
+    // hardware exp2 and reciprocal (about 1 ulp each in fp32, far inside the bf16 rounding of the result); the
+    // IEEE division and the range handling of expf would make the fused quantiser ALU-bound
+    if (ACT == MXL_ACT_SILU) return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+    // 0.5 g erfc(-g / sqrt 2); erfc (not 1 + erf): no cancellation in the negative tail.  erfc(z), z >= 0, from
+    // the rational-exponential fit t exp(-z^2 + P(t)), t = 1 / (1 + z / 2) (fractional error below 1.2e-7
+    // everywhere, Numerical Recipes 6.2), with the hardware reciprocal and exp2: the library erfcf would make
+    // the fused quantiser ALU-bound.
+    const float x = g * -0.70710678118654752f, z = fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(1.f + 0.5f * z);
+    float p = 0.17087277f;
+    p = p * t - 0.82215223f;
+    p = p * t + 1.48851587f;
+    p = p * t - 1.13520398f;
+    p = p * t + 0.27886807f;
+    p = p * t - 0.18628806f;
+    p = p * t + 0.09678418f;
+    p = p * t + 0.37409196f;
+    p = p * t + 1.00002368f;
+    p = p * t - 1.26551223f;
+    const float e = t * __builtin_amdgcn_exp2f((p - z * z) * 1.4426950408889634f);
+    return 0.5f * g * (x >= 0.f ? e : 2.f - e);
 }
 __device__ __forceinline__ float load_prob(const void* probs, int probs_bf16, int64_t row) {
     if (probs_bf16) return __uint_as_float((uint32_t)((const uint16_t*)probs)[row] << 16);

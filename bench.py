@@ -42,6 +42,8 @@ WORKLOADS = {
     "deepseek_v3_shard_mxfp8": dict(G=32, topk=8, tokens=8192, hidden=7168, fc1_out=4096, fc2_in=2048, routing="zipf", seed=1004, fp4=False),
     "gpt_oss_120b_mxfp4": dict(G=128, topk=4, tokens=16384, hidden=2880, fc1_out=5760, fc2_in=2880, routing="uniform", seed=1005, fp4=True, wgrad=False),
     "llama3_8b_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False),
+    # the same MLP with the RMSNorm that precedes fc1 in the layer (LayerNormColumnParallelLinear), folded into fc1's quantiser
+    "llama3_8b_norm_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, norm=True),
 }
 
 
@@ -104,6 +106,14 @@ class _Bracket:
             self.e1.record(torch.cuda.current_stream())
             self.o.records.append((self.name, self.info, self.e0, self.e1))
         return False
+
+
+def norm_bytes(name, info):
+    """Algorithmic bytes of one RMSNorm launch: bf16 read (+ bf16 write); backward reads x, dy and writes dx."""
+    el = info["rows"] * info["k"]
+    if name == "rmsnorm_bwd":
+        return el * 6.0
+    return el * (4.0 if info.get("want_y", True) else 2.0)
 
 
 def quant_bytes(info):
@@ -220,6 +230,7 @@ def main():
         dy = torch.randn(M, n, generator=gen, device=dev).bfloat16()
         layers.append((x, w, dy, k, n))
     gl = torch.tensor(lens, dtype=torch.int64, device=dev)
+    norm_w = torch.ones(spec["hidden"], device=dev).bfloat16().requires_grad_() if spec.get("norm") else None
     if not spec.get("wgrad", True):
         # Without a weight gradient the weights cannot change between steps: they are quantised once, before
         # the timed region, and the steps run on the cached copies (the reference's multi-microbatch path,
@@ -233,15 +244,19 @@ def main():
     flops_step = sum(2.0 * passes * M * n * k for (_, _, _, k, n) in layers)
 
     def step():
-        for (x, w, dy, k, n) in layers:
+        for i, (x, w, dy, k, n) in enumerate(layers):
             if grouped:
                 y = op(x, w, gl, trans_b=True, config=cfg)
+            elif norm_w is not None and i == 0:
+                y = pt.ops.rmsnorm_gemm_fp8(x, norm_w, 1e-5, w, config=cfg)
             else:
                 y = pt.ops.gemm_fp8(x, w, trans_a=False, trans_b=True, out_dtype=None, config=cfg)
             y.backward(dy)
             x.grad = None
             if torch.is_tensor(w):
                 w.grad = None
+            if norm_w is not None:
+                norm_w.grad = None
 
     if args.calibrate_traffic:
         src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)   # 1 GiB
@@ -285,6 +300,8 @@ def main():
         a["n"] += 1
         if "gemm" in name:
             a["flops"] += 2.0 * info["m"] * info["n"] * info["k"]
+        elif name in ("rmsnorm_fwd", "rmsnorm_bwd"):
+            a["bytes"] += norm_bytes(name, info)
         else:
             a["bytes"] += quant_bytes(info)
     fwd_name = "grouped_gemm_nt" if grouped else "gemm_nt"

@@ -567,7 +567,7 @@ def rmsnorm_fwd_impl(x, weight, eps: float, want_y: bool = True):
     rows, k = x.shape
     y = torch.empty_like(x) if want_y else None
     rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
-    with _hooked("rmsnorm_fwd", rows=rows, k=k):
+    with _hooked("rmsnorm_fwd", rows=rows, k=k, want_y=want_y):
         rc = _lib.load().mxl_rmsnorm_fwd(_ptr(x), _ptr(weight), float(eps), rows, k, _ptr(y), _ptr(rstd), _stream())
     _lib.check(rc, "mxl_rmsnorm_fwd")
     return y, rstd

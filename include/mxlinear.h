@@ -35,6 +35,7 @@ extern "C" {
 
 #define MXL_FMT_E4M3 0
 #define MXL_FMT_E2M1 1
+#define MXL_FMT_E5M2 2   /* tensor-wise scaled entry points only */
 
 /* E8M0 scale rule (explicit because the reference's kernel library is not in
  * its tree): OCP MX v1.0 floor rule, round-up rule, AITER/Quark "even" rule. */
@@ -224,6 +225,44 @@ int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtyp
                            int64_t rows, int64_t f, int64_t row_ld, int act, int fmt, int scale_mode,
                            const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                            void* s_colT, uint32_t flags, void* stream);
+
+/* ---- tensor-wise ("current") FP8 scaling: the non-MX recipe that the same operators serve -------------------
+ * One fp32 scale per tensor (the arithmetic the reference restates in _quantize_fp8_tensorwise,
+ * primus_turbo_float8_local.py:194-207, and hands to gemm_fp8_impl at :239-250):
+ *   amax = max |x|,  scale = fp8_max / max(amax, 1e-12),  q = cast_fp8(clamp(x * scale, +-fp8_max)),
+ *   scale_inv = 1 / scale,      fp8_max = 448 (E4M3), 57344 (E5M2: gradients of the HYBRID format),
+ * all in fp32 (bf16 -> fp32 is exact), round to nearest even.  A NaN or Inf anywhere in the tensor makes every
+ * code NaN. */
+
+/* amax_f32[0] = max |x[i]| over n bf16 values (0 for n == 0); x 16-byte aligned. */
+int mxl_amax(const void* x_bf16, int64_t n, void* amax_f32, void* stream);
+
+/* mxl_quantize with the tensor's scale instead of block scales: codes in the same layouts (row-wise copy,
+ * transposed segment-padded copy, row-major or K-chunk-major), fmt = MXL_FMT_E4M3 or MXL_FMT_E5M2, the scale
+ * taken from amax_f32 (device, written by mxl_amax on the same stream).  s_row / s_colT receive the E8M0
+ * byte 127 (2^0) for every block, so that the codes can be handed to the GEMMs below unchanged, and
+ * scale_inv_f32[0] (device, may be NULL) receives 1 / scale. */
+int mxl_quantize_tensorwise(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt,
+                            const void* amax_f32, const int64_t* group_lens, int num_groups, void* q_row, void* s_row,
+                            void* q_colT, void* s_colT, void* scale_inv_f32, uint32_t flags, void* stream);
+
+/* The same for weights [batch, n, k] (both copies, layouts of mxl_quantize_weight_2d); one scale for the whole
+ * tensor, amax_f32 taken over all of it. */
+int mxl_quantize_weight_tensorwise(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld, int64_t n_ld,
+                                   int fmt, const void* amax_f32, void* q_row, void* s_row, void* q_colT, void* s_colT,
+                                   void* scale_inv_f32, uint32_t flags, void* stream);
+
+/* The GEMMs with a per-tensor factor: c = (dq(a) . dq(b)^T) * alpha_a[0] * alpha_b[0], the factors read on the
+ * device (the scale_inv outputs above), applied in fp32 before the rounding to bf16.  Operand formats:
+ * E4M3 x E4M3 and E5M2 (a) x E4M3 (b). */
+int mxl_grouped_gemm_nt_scaled(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                               const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                               int num_groups, int64_t total_m, int64_t n, int64_t k, const float* alpha_a,
+                               const float* alpha_b, uint32_t flags, void* stream);
+int mxl_grouped_gemm_wgrad_scaled(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                  const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                  int num_groups, int64_t total_m, int64_t n, int64_t k, const float* alpha_a,
+                                  const float* alpha_b, uint32_t flags, void* stream);
 
 /* RMSNorm in front of the column-parallel linear (rmsnorm(x, layer_norm_weight, eps) in
  * PrimusTurboLayerNormColumnParallelLinear.forward_internal, primus_turbo.py:1689-1700):

@@ -82,6 +82,16 @@ Parity status
   kernel rounds once or after the normalisation and again after the weight
   (as torch's composite does) is **parity unpinned** (package absent).
 
+* ``cast_e5m2`` / ``quantize_tensorwise`` / ``tensorwise_gemm_nt_ref`` (tensor-wise "current" FP8
+  scaling, the non-MX recipe behind the same operators; restated in the reference itself at
+  primus_turbo_float8_local.py:194-207 and :215-306): scale = fp8_max / max(amax, 1e-12) and
+  scale_inv = 1 / scale in float32, q = cast(clamp(x * scale)).  ``cast_e5m2`` is pinned against
+  ``torch.float8_e5m2`` (library routine) over every bf16 value and over float32 samples next to the
+  rounding boundaries; the quantiser against the reference's formula evaluated with torch ops.  The
+  reference's experimental "decomposed" variant multiplies in bf16 and its shipping variant calls a
+  Primus-Turbo C++ op whose source is absent: the float32 product used here is **parity unpinned**
+  against that op.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -95,6 +105,7 @@ BLOCK = 32
 # element formats
 FMT_E4M3 = 0
 FMT_E2M1 = 1
+FMT_E5M2 = 2  # tensor-wise scaled operands only
 
 # E8M0 scale rules
 SCALE_OCP_FLOOR = 0  # OCP MX v1.0: floor(log2 amax) - emax_elem
@@ -731,3 +742,74 @@ def rmsnorm_bwd_ref(dy, x, w, eps: float):
     g = d * wf
     dx = (g - xh * (g * xh).mean(axis=1, keepdims=True)) * rstd
     return dx, (d * xh).sum(axis=0)
+
+
+# --------------------------------------------------------------------------
+# Tensor-wise ("current") FP8 scaling (primus_turbo_float8_local.py:194-207, :215-306)
+# --------------------------------------------------------------------------
+_FP8_MAX = {FMT_E4M3: 448.0, FMT_E5M2: 57344.0}
+
+
+def cast_e5m2(v: np.ndarray) -> np.ndarray:
+    """float32 -> FP8 E5M2 code, RNE, saturating at +-57344, sign kept on zero results, NaN -> sign|0x7F."""
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    u = v.view(np.uint32)
+    sign = ((u >> np.uint32(24)) & np.uint32(0x80)).astype(np.uint8)
+    a_bits = u & np.uint32(0x7FFFFFFF)
+    nan = a_bits > np.uint32(0x7F800000)
+    a = np.minimum(a_bits.view(np.float32), np.float32(57344.0))
+    a = np.where(nan, np.float32(0.0), a).astype(np.float32)
+    ab = a.view(np.uint32).astype(np.int64)
+    # normal range of e5m2: >= 2^-14; two mantissa bits are kept
+    rounded = (ab + 0xFFFFF + ((ab >> 21) & 1)) >> 21  # (exp32 << 2) | m2 after carry
+    code_n = rounded - ((127 - 15) << 2)
+    # subnormal range: multiples of 2^-16
+    code_s = np.rint(a.astype(np.float64) * 65536.0).astype(np.int64)
+    code = np.where(a >= np.float32(2.0**-14), code_n, code_s)
+    code = np.minimum(code, 0x7B)
+    code = np.where(nan, 0x7F, code)
+    return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def decode_e5m2(code: np.ndarray) -> np.ndarray:
+    c = code.astype(np.int64)
+    s = np.where(c & 0x80, -1.0, 1.0)
+    e = (c >> 2) & 0x1F
+    m = c & 0x3
+    val = np.where(e == 0, m * 2.0**-16, (4 + m) * np.exp2(e.astype(np.float64) - 17.0))
+    val = np.where(e == 31, np.where(m == 0, np.inf, np.nan), val)
+    return (s * val).astype(np.float32)
+
+
+def tensor_amax(x) -> np.float32:
+    xf = bf16_bits_to_f32(to_bf16_bits(x))
+    return np.float32(np.abs(xf).max()) if xf.size else np.float32(0.0)
+
+
+def quantize_tensorwise(x, fmt: int = FMT_E4M3):
+    """(codes uint8 of the shape of x, scale_inv float32): one scale for the whole tensor,
+    scale = fp8_max / max(amax, 1e-12), codes = cast(clamp(x * scale, +-fp8_max)), scale_inv = 1 / scale,
+    float32 arithmetic.  A NaN or Inf in the tensor turns every code into NaN (0x7F)."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x))
+    amax = tensor_amax(x)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        scale = np.float32(_FP8_MAX[fmt]) / np.maximum(amax, np.float32(1e-12))
+        scale_inv = np.float32(1.0) / scale
+    if not np.isfinite(amax):
+        return np.full(xf.shape, 0x7F, dtype=np.uint8), np.float32(scale_inv)
+    y = (xf * scale).astype(np.float32)
+    codes = cast_e5m2(y) if fmt == FMT_E5M2 else cast_e4m3(y)
+    return codes, np.float32(scale_inv)
+
+
+def decode_fp8(codes: np.ndarray, fmt: int) -> np.ndarray:
+    return decode_e5m2(codes) if fmt == FMT_E5M2 else decode_e4m3(codes)
+
+
+def tensorwise_gemm_nt_ref(a_codes, a_scale_inv, b_codes, b_scale_inv, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, out_bf16=True):
+    """c = (decode(a) . decode(b)^T) * a_scale_inv * b_scale_inv: float32 accumulation, the two factors applied
+    to the sum, one rounding to bf16 (gemm_fp8_impl with tensor-wise granularity,
+    primus_turbo_float8_local.py:239-250)."""
+    acc = _matmul_nt_f32(decode_fp8(a_codes, a_fmt), decode_fp8(b_codes, b_fmt))
+    c = (acc * (np.float32(a_scale_inv) * np.float32(b_scale_inv))).astype(np.float32)
+    return f32_to_bf16_bits(c) if out_bf16 else c

@@ -17,6 +17,7 @@ _lib = None
 
 FMT_E4M3 = 0
 FMT_E2M1 = 1
+FMT_E5M2 = 2   # tensor-wise scaled operands only
 SCALE_OCP_FLOOR = 0
 SCALE_RCEIL = 1
 SCALE_EVEN = 2
@@ -50,6 +51,11 @@ EXPORTS = (
     "mxl_rmsnorm_bwd",
     "mxl_rmsnorm_bwd_workspace_bytes",
     "mxl_rmsnorm_quantize",
+    "mxl_amax",
+    "mxl_quantize_tensorwise",
+    "mxl_quantize_weight_tensorwise",
+    "mxl_grouped_gemm_nt_scaled",
+    "mxl_grouped_gemm_wgrad_scaled",
 )
 
 
@@ -119,6 +125,16 @@ def load() -> ctypes.CDLL:
         lib.mxl_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i64, vp]
         lib.mxl_rmsnorm_quantize.restype = i32
         lib.mxl_rmsnorm_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, u32, vp]
+        lib.mxl_amax.restype = i32
+        lib.mxl_amax.argtypes = [vp, i64, vp, vp]
+        lib.mxl_quantize_tensorwise.restype = i32
+        lib.mxl_quantize_tensorwise.argtypes = [vp, i64, i64, i64, i32, vp, vp, i32, vp, vp, vp, vp, vp, u32, vp]
+        lib.mxl_quantize_weight_tensorwise.restype = i32
+        lib.mxl_quantize_weight_tensorwise.argtypes = [vp, i64, i64, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, u32, vp]
+        lib.mxl_grouped_gemm_nt_scaled.restype = i32
+        lib.mxl_grouped_gemm_nt_scaled.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp, vp, u32, vp]
+        lib.mxl_grouped_gemm_wgrad_scaled.restype = i32
+        lib.mxl_grouped_gemm_wgrad_scaled.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp, vp, u32, vp]
         _lib = lib
     return _lib
 

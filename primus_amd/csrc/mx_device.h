@@ -38,6 +38,7 @@ typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 
 constexpr int kFmtE4M3 = MXL_FMT_E4M3;
 constexpr int kFmtE2M1 = MXL_FMT_E2M1;
+constexpr int kFmtE5M2 = MXL_FMT_E5M2;   // tensor-wise scaled operands only (gradients of the HYBRID format)
 
 // Exponent of the largest normal, its fp32 mantissa field, explicit mantissa bits.
 template <int FMT> struct Elem;
@@ -113,6 +114,19 @@ __device__ __forceinline__ uint32_t cvt4_e4m3(uint32_t p0, uint32_t p1, float in
     int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
     r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
     return (uint32_t)r;
+}
+// The same for E5M2 (tensor-wise scaled gradients): multiply, clamp at +-57344, round to nearest even.
+__device__ __forceinline__ uint32_t cvt4_e5m2(uint32_t p0, uint32_t p1, float inv) {
+    float a = __builtin_amdgcn_fmed3f(bf16_lo(p0) * inv, -57344.f, 57344.f);
+    float b = __builtin_amdgcn_fmed3f(bf16_hi(p0) * inv, -57344.f, 57344.f);
+    float c = __builtin_amdgcn_fmed3f(bf16_lo(p1) * inv, -57344.f, 57344.f);
+    float d = __builtin_amdgcn_fmed3f(bf16_hi(p1) * inv, -57344.f, 57344.f);
+    int r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+    return (uint32_t)r;
+}
+template <int FMT> __device__ __forceinline__ uint32_t cvt4_fp8(uint32_t p0, uint32_t p1, float inv) {
+    return FMT == kFmtE5M2 ? cvt4_e5m2(p0, p1, inv) : cvt4_e4m3(p0, p1, inv);
 }
 // Slow path for a block that holds a NaN/Inf: finite lanes -> signed zero,
 // non-finite lanes -> NaN code with the input's sign.

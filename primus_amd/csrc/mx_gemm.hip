@@ -52,6 +52,8 @@ struct GemmArgs {
     int64_t m;          // WGRAD: rows of a (fixed)   | FWD: unused
     int64_t n;          // columns of c / rows of b (per group in FWD)
     int64_t k;          // FWD: contraction length; WGRAD: padded width W
+    const float* alpha_a;   // ALPHA kernels: the output is multiplied by *alpha_a * *alpha_b (per-tensor
+    const float* alpha_b;   // scales of tensor-wise quantised operands) before it is rounded
 };
 
 template <int FMT> struct Op {
@@ -103,7 +105,7 @@ template <int FMT>
 __device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int ks, int g) {
     v8i f;
     const int s = Op<FMT>::swz(row);
-    if (FMT == kFmtE4M3) {
+    if (FMT != kFmtE2M1) {
         const uint4 lo = *(const uint4*)(lds + row * 128 + 16 * ((4 * ks + g) ^ s));
         const uint4 hi = *(const uint4*)(lds + row * 128 + 16 * ((4 * ks + 2 + g) ^ s));
         f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
@@ -133,7 +135,7 @@ struct Frags {
 // LAYOUT 0: operand codes row-major [rows, K].  LAYOUT 1: K-chunk-major [K / 128][rows][128 elements] (what the
 // quantisers write with MXL_QF_KCHUNK): the rows of a tile's K slot are one contiguous block, so a load round
 // fetches 4 KiB in a row instead of 16..64 row pieces; scales are row-major in both.
-template <int AFMT, int BFMT, int MODE, int LAYOUT>
+template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     constexpr int A_BYTES = Op<AFMT>::tile_bytes, B_BYTES = Op<BFMT>::tile_bytes;
     constexpr int STAGE = A_BYTES + B_BYTES;            // one slot: K = 128 of both operands
@@ -143,7 +145,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // (K = 512), one 16-byte request per row per operand, double-buffered.
     constexpr int PANEL = 256 * 16;           // one operand
     constexpr int PANELS = 2 * 2 * PANEL;     // 2 buffers x 2 operands
-    constexpr int CB = BFMT == kFmtE2M1 ? 4 : 0, BL = AFMT == kFmtE2M1 ? 4 : 0;
+    // operand format codes of the MFMA: 0 = E4M3, 1 = E5M2, 4 = E2M1
+    constexpr int CB = BFMT == kFmtE2M1 ? 4 : BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE2M1 ? 4 : AFMT == kFmtE5M2 ? 1 : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* panels = smem + NSLOT * STAGE;
     int* pre_tiles = (int*)(panels + PANELS);                        // [G+1] prefix of row tiles (FWD)
@@ -454,6 +457,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             const int rr = l >> 4, cc = wn * 128 + (l & 15) * 8;
             const uint32_t lane_off = (uint32_t)((rr * (int)p.n + (l & 15) * 8) * 2);
             const bool full = (m_valid == BM) && (n_valid == BN);
+            float alpha = 1.f;
+            if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 // lane (lr, g) holds row lr of this 32-row block: columns j*32 + 8q + 4g .. +3
@@ -461,6 +466,10 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
+                        if (ALPHA) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] *= alpha;
+                        }
                         v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
                                   (__bf16)acc[i][j][4 * q + 3]};
                         *(v4bf*)(wr + (j * 32 + 8 * q) * 2) = o;
@@ -514,13 +523,13 @@ static int num_cus(int slot) {
     return pr.multiProcessorCount;
 }
 
-template <int AFMT, int BFMT, int MODE, int LAYOUT>
+template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false>
 static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = gemm_lds_bytes(AFMT, BFMT);
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set[64];   // the attribute belongs to the (kernel, device) pair
     const int slot = current_device_slot();
-    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT>;
+    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT, ALPHA>;
     if (!attr_set[slot].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
@@ -542,14 +551,28 @@ static int dispatch_gemm_l(int afmt, int bfmt, const GemmArgs& a, int64_t max_ti
     return MXL_EINVAL;
 }
 
+// tensor-wise scaled operands: E4M3 x E4M3 (forward, or every GEMM of the E4M3 format) and E5M2 x E4M3
+// (gradient times weight / activation of the HYBRID format), output times *alpha_a * *alpha_b
+template <int MODE, int LAYOUT>
+static int dispatch_gemm_alpha_l(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3)
+        return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, LAYOUT, true>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E4M3)
+        return launch_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE, LAYOUT, true>(a, max_tiles, st);
+    return MXL_EINVAL;
+}
+
 // a_rows / b_rows: rows of the whole operands (for the 4 GiB bound of the chunk-major layout)
 template <int MODE>
 static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, bool kchunk, int64_t a_rows, int64_t b_rows,
                          hipStream_t st) {
-    if (!kchunk) return dispatch_gemm_l<MODE, 0>(afmt, bfmt, a, max_tiles, st);
+    const bool alpha = a.alpha_a != nullptr;
+    if (!kchunk) return alpha ? dispatch_gemm_alpha_l<MODE, 0>(afmt, bfmt, a, max_tiles, st)
+                              : dispatch_gemm_l<MODE, 0>(afmt, bfmt, a, max_tiles, st);
     // chunk offsets inside an operand are 32-bit
     if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
-    return dispatch_gemm_l<MODE, 1>(afmt, bfmt, a, max_tiles, st);
+    return alpha ? dispatch_gemm_alpha_l<MODE, 1>(afmt, bfmt, a, max_tiles, st)
+                 : dispatch_gemm_l<MODE, 1>(afmt, bfmt, a, max_tiles, st);
 }
 
 }  // namespace mxl
@@ -564,10 +587,11 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t w
     if (i < words) dst[i] = 0u;
 }
 
-extern "C" int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
-                                      const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
-                                      int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream) {
+static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes, const void* b_scales,
+                           int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
+                           int64_t k, const float* alpha_a, const float* alpha_b, uint32_t flags, void* stream) {
     if (flags & ~(uint32_t)MXL_GF_KCHUNK) return MXL_EINVAL;
+    if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
     if (k > MAX_CONTRACTION) return MXL_EINVAL;   // tile-relative byte offsets are 32-bit
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
@@ -586,9 +610,27 @@ extern "C" int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales,
     a.m = 0;
     a.n = n;
     a.k = k;
+    a.alpha_a = alpha_a;
+    a.alpha_b = alpha_b;
     const int64_t max_tiles = (total_m / BM + num_groups) * ((n + BN - 1) / BN);
     return dispatch_gemm<MODE_FWD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, total_m,
                                    (int64_t)num_groups * n, (hipStream_t)stream);
+}
+
+extern "C" int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                      const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                      int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream) {
+    return grouped_gemm_nt(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, group_lens, num_groups, total_m, n, k,
+                           nullptr, nullptr, flags, stream);
+}
+
+extern "C" int mxl_grouped_gemm_nt_scaled(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                          const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                          int num_groups, int64_t total_m, int64_t n, int64_t k, const float* alpha_a,
+                                          const float* alpha_b, uint32_t flags, void* stream) {
+    if (!alpha_a || !alpha_b) return MXL_EINVAL;
+    return grouped_gemm_nt(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, group_lens, num_groups, total_m, n, k,
+                           alpha_a, alpha_b, flags, stream);
 }
 
 extern "C" int mxl_grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
@@ -604,11 +646,12 @@ extern "C" int mxl_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt,
     return mxl_grouped_gemm_nt_ex(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, nullptr, 1, m, n, k, 0, stream);
 }
 
-extern "C" int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
-                                         const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
-                                         int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags,
-                                         void* stream) {
+static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                              const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups,
+                              int64_t total_m, int64_t n, int64_t k, const float* alpha_a, const float* alpha_b,
+                              uint32_t flags, void* stream) {
     if (flags & ~(uint32_t)MXL_GF_KCHUNK) return MXL_EINVAL;
+    if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
     if (num_groups < 0 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if ((num_groups > 0) != (group_lens != nullptr)) return MXL_EINVAL;
@@ -643,8 +686,27 @@ extern "C" int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scal
     a.m = n;  // rows of the output per group
     a.n = k;  // columns of the output
     a.k = mxl_padded_width(total_m, G);
+    a.alpha_a = alpha_a;
+    a.alpha_b = alpha_b;
     const int64_t max_tiles = (int64_t)G * ((n + BM - 1) / BM) * ((k + BN - 1) / BN);
     return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, n, k, (hipStream_t)stream);
+}
+
+extern "C" int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                         const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                         int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags,
+                                         void* stream) {
+    return grouped_gemm_wgrad(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, group_lens, num_groups, total_m, n,
+                              k, nullptr, nullptr, flags, stream);
+}
+
+extern "C" int mxl_grouped_gemm_wgrad_scaled(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
+                                             const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                             int num_groups, int64_t total_m, int64_t n, int64_t k, const float* alpha_a,
+                                             const float* alpha_b, uint32_t flags, void* stream) {
+    if (!alpha_a || !alpha_b) return MXL_EINVAL;
+    return grouped_gemm_wgrad(a_codes, a_scales, a_fmt, b_codes, b_scales, b_fmt, c_bf16, group_lens, num_groups, total_m, n,
+                              k, alpha_a, alpha_b, flags, stream);
 }
 
 extern "C" int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,

@@ -67,6 +67,11 @@ struct QuantArgs {
     // fused RMSNorm in front (ACT == PRO_RMSNORM): the tensor that is quantised is (x * rstd[row]) * norm_w[col];
     // rstd travels in `probs` (fp32)
     const uint16_t* norm_w;
+    // tensor-wise scaling (SMODE == SCALE_TENSOR): one fp32 scale for the whole tensor, fp8_max / max(amax, 1e-12),
+    // from the tensor's abs-max on the device; its reciprocal is written to scale_inv_out (may be null).  The
+    // block-scale arrays are filled with 127 (2^0), so the scaled GEMM reads the codes unchanged.
+    const float* tensor_amax;
+    float* scale_inv_out;
     // Code layout of both copies.  0: row-major [rows, ld].  1: K-chunk-major [ld / 128][rows][128 elements]:
     // the 128 elements of a row that one GEMM K slot consumes stay together and consecutive rows follow
     // each other, so a GEMM tile's slot is one contiguous block and this kernel writes 128 x 128-element
@@ -110,10 +115,22 @@ __device__ __forceinline__ bool quant_tile_of_workgroup(const QuantArgs& a, int&
 // orthogonal, so a wgrad GEMM whose two operands were both transformed computes the same contraction
 // while single large values are spread over 16 positions before they meet the 4-bit grid.
 constexpr int PRO_RMSNORM = 2;   // value of ACT next to MXL_ACT_SILU (0) and MXL_ACT_GELU (1)
+constexpr int SCALE_TENSOR = 3;  // value of SMODE next to the three E8M0 rules: per-tensor fp32 scale
+
+template <int FMT, int SMODE> __device__ __forceinline__ uint32_t block_byte(uint32_t amax16) {
+    if constexpr (SMODE == SCALE_TENSOR) {
+        return 127u;
+    } else {
+        return scale_byte<FMT, SMODE>(amax16);
+    }
+}
 
 template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1, bool SR = false, bool RHT = false>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     constexpr bool FP4 = (FMT == kFmtE2M1);
+    constexpr bool TENSOR = (SMODE == SCALE_TENSOR);
+    static_assert(TENSOR || FMT != kFmtE5M2, "E5M2 exists for tensor-wise scaling only");
+    static_assert(!TENSOR || (!FP4 && !SR && !RHT && ACT < 0), "tensor-wise scaling: FP8 codes, plain input");
     static_assert(!SR || (FP4 && !TWOD && ACT < 0), "stochastic rounding exists for 1-D E2M1 quantisation only");
     static_assert(!RHT || (COL && !TWOD && ACT < 0), "the Hadamard transform applies to the transposed 1-D copy only");
     constexpr int TPITCH = FP4 ? (QT / 2 + 16) : (QT + 16);  // bytes per LDS row of the transposed tile
@@ -123,6 +140,14 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 
     const int t = threadIdx.x;
     const int w = t >> 6, l = t & 63, c16 = l & 15, rg = l >> 4;
+    float tscale = 1.f;
+    bool tensor_bad = false;   // abs-max is NaN or Inf: every code becomes NaN
+    if (TENSOR) {
+        const float amax = *a.tensor_amax;
+        tensor_bad = !(amax < __uint_as_float(0x7F800000u));
+        tscale = (FMT == kFmtE5M2 ? 57344.f : 448.f) / fmaxf(amax, 1e-12f);
+        if (blockIdx.x == 0 && t == 0 && a.scale_inv_out) *a.scale_inv_out = 1.0f / tscale;
+    }
     int pt, ct;
     if (!quant_tile_of_workgroup(a, pt, ct)) return;   // uniform over the workgroup
     const int64_t col0 = (int64_t)ct * QT;
@@ -243,7 +268,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         for (int it = 1; it < 8; ++it) m = max(m, rmax[it]);
         m = max(m, (uint32_t)__shfl_xor((int)m, 16));
         m = max(m, (uint32_t)__shfl_xor((int)m, 32));
-        tile_byte = scale_byte<FMT, SMODE>(m);
+        tile_byte = block_byte<FMT, SMODE>(m);
     } else if (COL && !RHT) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -257,11 +282,14 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
             const int r = 32 * w + 8 * rg + it;
-            const uint32_t byte = TWOD ? tile_byte : scale_byte<FMT, SMODE>(rmax[it]);
+            const uint32_t byte = TWOD ? tile_byte : block_byte<FMT, SMODE>(rmax[it]);
             if ((c16 & 3) == 0) ((uint8_t*)srow_tile)[r * 4 + (c16 >> 2)] = (uint8_t)byte;
             if (!FP4) {
                 uint2 o;
-                if (byte != 255u) {
+                if (TENSOR) {
+                    o.x = tensor_bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(d[it].x, d[it].y, tscale);
+                    o.y = tensor_bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(d[it].z, d[it].w, tscale);
+                } else if (byte != 255u) {
                     const float inv = inv_scale(byte);
                     o.x = cvt4_e4m3(d[it].x, d[it].y, inv);
                     o.y = cvt4_e4m3(d[it].z, d[it].w, inv);
@@ -355,7 +383,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const uint32_t amax = (j & 1) ? (cmax[j >> 1] >> 16) : (cmax[j >> 1] & 0xFFFFu);
-            const uint32_t byte = TWOD ? tile_byte : scale_byte<FMT, SMODE>(amax);
+            const uint32_t byte = TWOD ? tile_byte : block_byte<FMT, SMODE>(amax);
             const int c = 8 * c16 + j;
             if (rg == 0) ((uint8_t*)scol_tile)[c * 4 + w] = (uint8_t)byte;
             // the lane's 8 rows of column j, as 4 packed (row 2i, row 2i+1) pairs
@@ -367,7 +395,10 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             }
             if (!FP4) {
                 uint2 o;
-                if (byte != 255u) {
+                if (TENSOR) {
+                    o.x = tensor_bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(pr[0], pr[1], tscale);
+                    o.y = tensor_bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(pr[2], pr[3], tscale);
+                } else if (byte != 255u) {
                     const float inv = inv_scale(byte);
                     o.x = cvt4_e4m3(pr[0], pr[1], inv);
                     o.y = cvt4_e4m3(pr[2], pr[3], inv);
@@ -549,9 +580,57 @@ static int dispatch_quant_fp4(int smode, QuantArgs& a, int64_t tiles_r, int64_t 
     return MXL_EINVAL;
 }
 
+// tensor-wise scaling: E4M3 or E5M2 codes, 1-D (activations, gradients) or batched-matrix (weights) tiling
+template <bool TWOD>
+static int dispatch_quant_tensor(int fmt, QuantArgs& a, int64_t tiles_r, int64_t tiles_c, hipStream_t st) {
+    if (fmt == MXL_FMT_E4M3) return launch_quant<MXL_FMT_E4M3, SCALE_TENSOR, TWOD>(a, tiles_r, tiles_c, st);
+    if (fmt == MXL_FMT_E5M2) return launch_quant<MXL_FMT_E5M2, SCALE_TENSOR, TWOD>(a, tiles_r, tiles_c, st);
+    return MXL_EINVAL;
+}
+
+// abs-max of a bf16 tensor: non-negative floats order like their bit patterns, so an integer atomic max on the
+// fp32 pattern does it (a NaN pattern is larger than every number and wins).  One atomic per workgroup.
+__global__ __launch_bounds__(256) void amax_kernel(const uint16_t* x, int64_t n8, int64_t n, uint32_t* out) {
+    __shared__ uint32_t part[4];
+    uint32_t m = 0;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
+        const uint4 v = load16_streaming(x + i * 8);
+        m = pk_max16(m, pk_max16(pk_max16(v.x & 0x7FFF7FFFu, v.y & 0x7FFF7FFFu), pk_max16(v.z & 0x7FFF7FFFu, v.w & 0x7FFF7FFFu)));
+    }
+    m = hmax16(m);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        for (int64_t i = n8 * 8; i < n; ++i) m = max(m, (uint32_t)(x[i] & 0x7FFFu));   // tail of fewer than 8 elements
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, s));
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = max(max(part[0], part[1]), max(part[2], part[3]));
+        atomicMax(out, m << 16);   // bf16 pattern -> fp32 pattern
+    }
+}
+
+__global__ void amax_init_kernel(uint32_t* out) { *out = 0u; }
+
 }  // namespace mxl
 
 using namespace mxl;
+
+extern "C" int mxl_amax(const void* x_bf16, int64_t n, void* amax_f32, void* stream) {
+    if (n < 0 || !amax_f32 || (n > 0 && !x_bf16) || ((uintptr_t)x_bf16 & 15) != 0) return MXL_EINVAL;
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    hipStream_t st = (hipStream_t)stream;
+    // a fill kernel, not a memset: callers may be capturing the stream into a graph
+    hipLaunchKernelGGL(amax_init_kernel, dim3(1), dim3(1), 0, st, (uint32_t*)amax_f32);
+    if (hipGetLastError() != hipSuccess) return MXL_ELAUNCH;
+    if (n == 0) return MXL_OK;
+    const int64_t n8 = n / 8;
+    int64_t grid = (n8 + 256 * 8 - 1) / (256 * 8);   // about 8 loads per lane
+    grid = grid < 1 ? 1 : grid > 4096 ? 4096 : grid;
+    hipLaunchKernelGGL(amax_kernel, dim3((unsigned)grid), dim3(256), 0, st, (const uint16_t*)x_bf16, n8, n, (uint32_t*)amax_f32);
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
 
 extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
     if (num_groups < 1) num_groups = 1;
@@ -562,7 +641,8 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
                        int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
                        bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0,
-                       bool kchunk = false, const void* norm_w = nullptr) {
+                       bool kchunk = false, const void* norm_w = nullptr, const void* tensor_amax = nullptr,
+                       void* scale_inv_out = nullptr) {
     if (row_ld == 0) row_ld = cols;
     if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
     if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
@@ -589,6 +669,8 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.probs_bf16 = probs_dtype == MXL_PROBS_BF16;
     a.row_mask = row_mask;
     a.norm_w = (const uint16_t*)norm_w;
+    a.tensor_amax = (const float*)tensor_amax;
+    a.scale_inv_out = (float*)scale_inv_out;
     a.sr_seed = sr_seed;
     a.rht_signs = rht_signs & 0xFFFFu;
     a.kchunk = kchunk ? 1 : 0;
@@ -596,6 +678,11 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.chunk_rows_col = cols;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
     const int64_t gy = ((q_row ? row_ld : cols) + QT - 1) / QT;
+    if (tensor_amax) {
+        if (sr || rht || act >= 0) return MXL_EINVAL;
+        if (gx == 0) return MXL_OK;   // nothing to quantise (scale_inv_out is then left unwritten)
+        return dispatch_quant_tensor<false>(fmt, a, gx, gy, (hipStream_t)stream);
+    }
     if (gx == 0) return MXL_OK;
     if (sr && rht) return dispatch_quant_fp4<true, true>(scale_mode, a, gx, gy, (hipStream_t)stream);
     if (sr) return dispatch_quant_fp4<true, false>(scale_mode, a, gx, gy, (hipStream_t)stream);
@@ -646,7 +733,7 @@ extern "C" int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, cons
 
 static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld, int64_t n_ld, int fmt,
                               int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT, bool kchunk,
-                              void* stream) {
+                              void* stream, const void* tensor_amax = nullptr, void* scale_inv_out = nullptr) {
     if (k_ld == 0) k_ld = k;
     if (n_ld == 0) n_ld = n;
     if (kchunk && ((q_row && k_ld % QT != 0) || (q_colT && n_ld % QT != 0))) return MXL_EINVAL;   // whole chunks
@@ -672,6 +759,8 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
     a.probs_bf16 = 0;
     a.row_mask = nullptr;
     a.norm_w = nullptr;
+    a.tensor_amax = (const float*)tensor_amax;
+    a.scale_inv_out = (float*)scale_inv_out;
     a.sr_seed = 0;
     a.rht_signs = 0;
     a.kchunk = kchunk ? 1 : 0;
@@ -679,6 +768,7 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
     a.chunk_rows_col = batch * k;
     const int64_t gx = batch * ((n + QT - 1) / QT);
     const int64_t gy = ((q_row ? k_ld : k) + QT - 1) / QT;
+    if (tensor_amax) return dispatch_quant_tensor<true>(fmt, a, gx, gy, (hipStream_t)stream);
     return dispatch_quant<true>(fmt, scale_mode, a, gx, gy, (hipStream_t)stream);
 }
 
@@ -694,6 +784,27 @@ extern "C" int mxl_quantize_weight_2d_ex(const void* w_bf16, int64_t batch, int6
     if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
     return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, scale_mode, q_row, s_row, q_colT, s_colT,
                               (flags & MXL_QF_KCHUNK) != 0, stream);
+}
+
+extern "C" int mxl_quantize_tensorwise(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt,
+                                       const void* amax_f32, const int64_t* group_lens, int num_groups, void* q_row,
+                                       void* s_row, void* q_colT, void* s_colT, void* scale_inv_f32, uint32_t flags,
+                                       void* stream) {
+    if (!amax_f32 || (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    return quantize_1d(x_bf16, rows, cols, row_ld, fmt, MXL_SCALE_OCP_FLOOR, group_lens, num_groups, q_row, s_row, q_colT,
+                       s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
+                       (flags & MXL_QF_KCHUNK) != 0, nullptr, amax_f32, scale_inv_f32);
+}
+
+extern "C" int mxl_quantize_weight_tensorwise(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
+                                              int64_t n_ld, int fmt, const void* amax_f32, void* q_row, void* s_row,
+                                              void* q_colT, void* s_colT, void* scale_inv_f32, uint32_t flags,
+                                              void* stream) {
+    if (!amax_f32 || (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, MXL_SCALE_OCP_FLOOR, q_row, s_row, q_colT, s_colT,
+                              (flags & MXL_QF_KCHUNK) != 0, stream, amax_f32, scale_inv_f32);
 }
 
 extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,

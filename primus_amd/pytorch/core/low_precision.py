@@ -174,8 +174,10 @@ def dtype_to_fmt_code(dtype: torch.dtype) -> int:
         return _lib.FMT_E4M3
     if dtype == float4_e2m1fn_x2:
         return _lib.FMT_E2M1
+    if dtype == float8_e5m2:
+        return _lib.FMT_E5M2
     raise ValueError(f"no MX kernel for dest_dtype {dtype}")
 
 
 def fmt_code_to_dtype(code: int) -> torch.dtype:
-    return float8_e4m3 if code == _lib.FMT_E4M3 else float4_e2m1fn_x2
+    return {_lib.FMT_E4M3: float8_e4m3, _lib.FMT_E2M1: float4_e2m1fn_x2, _lib.FMT_E5M2: float8_e5m2}[code]

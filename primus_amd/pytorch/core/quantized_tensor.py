@@ -56,13 +56,18 @@ class QuantizedTensor(torch.Tensor):
 
     @staticmethod
     def __new__(cls, codes, scales, *, logical_shape, orig_dtype=torch.bfloat16, axis=-1, use_2d_block=False,
-                scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False, kchunk=False):
+                scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False, kchunk=False,
+                tensor_scale_inv=None):
         return torch.Tensor._make_wrapper_subclass(
             cls, tuple(logical_shape), dtype=orig_dtype, device=codes.device, requires_grad=requires_grad
         )
 
     def __init__(self, codes, scales, *, logical_shape, orig_dtype=torch.bfloat16, axis=-1, use_2d_block=False,
-                 scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False, kchunk=False):
+                 scale_mode=ScaleMode.OCP_FLOOR, segment_lens=None, total_rows=None, requires_grad=False, kchunk=False,
+                 tensor_scale_inv=None):
+        # tensor-wise scaled payload: float32 reciprocal scale of the whole tensor (one element, on the device);
+        # ``scales`` then holds unit E8M0 bytes, which only make the codes acceptable to the GEMM kernels
+        self._tensor_scale_inv = tensor_scale_inv
         self._kchunk = bool(kchunk)
         self._codes = codes
         self._scales = scales
@@ -93,6 +98,10 @@ class QuantizedTensor(torch.Tensor):
     def kchunk(self) -> bool:
         return self._kchunk
 
+    @property
+    def tensor_scale_inv(self) -> Optional[torch.Tensor]:
+        return self._tensor_scale_inv
+
     def rowmajor_codes(self) -> torch.Tensor:
         """The payload as ``[..., rows, ld]`` whatever layout it is stored in (a copy if K-chunk-major)."""
         if not self._kchunk:
@@ -108,7 +117,7 @@ class QuantizedTensor(torch.Tensor):
         return QuantizedTensor(
             self._codes, self._scales, logical_shape=self.shape, orig_dtype=self.dtype, axis=self._axis,
             use_2d_block=self._use_2d_block, scale_mode=self._scale_mode, segment_lens=self._segment_lens,
-            total_rows=self._total_rows, kchunk=self._kchunk,
+            total_rows=self._total_rows, kchunk=self._kchunk, tensor_scale_inv=self._tensor_scale_inv,
         )
 
     def __repr__(self):  # noqa: D105
@@ -138,12 +147,29 @@ class QuantizedTensor(torch.Tensor):
         axis: int = -1,
     ) -> "QuantizedTensor":
         """Signature of the reference's call sites (primus_turbo.py:321-354)."""
-        if granularity != ScalingGranularity.MX_BLOCKWISE:
-            raise NotImplementedError("only ScalingGranularity.MX_BLOCKWISE has kernels in this build")
-        if block_size not in (None, _lib.BLOCK):
-            raise ValueError(f"MX block size must be {_lib.BLOCK}")
+        if granularity not in (ScalingGranularity.MX_BLOCKWISE, ScalingGranularity.TENSORWISE):
+            raise NotImplementedError("only MX_BLOCKWISE and TENSORWISE scaling have kernels in this build")
         if axis not in (-1, -2):
             raise ValueError("axis must be -1 (row-wise) or -2 (column-wise, transposed result)")
+        if granularity == ScalingGranularity.TENSORWISE:
+            # one scale for the whole tensor; axis=-2 gives the transposed payload like the MX copies do
+            fmt = dtype_to_fmt_code(dest_dtype)
+            x = x.detach()
+            if x.dtype != torch.bfloat16 or x.dim() not in (2, 3):
+                raise ValueError("quantize expects a 2-D or 3-D bfloat16 tensor")
+            if x.dim() == 3:
+                q_row, s_row, q_col, s_col, si = K.quantize_weight_tensorwise_impl(
+                    x.contiguous(), fmt, rowwise=(axis == -1), colwise=(axis == -2))
+            else:
+                q_row, s_row, q_col, s_col, si = K.quantize_tensorwise_impl(
+                    x.contiguous(), fmt, rowwise=(axis == -1), colwise=(axis == -2))
+            if axis == -1:
+                return cls(q_row, s_row, logical_shape=x.shape, orig_dtype=x.dtype, axis=-1, tensor_scale_inv=si)
+            shape = tuple(x.shape[:-2]) + (x.shape[-1], x.shape[-2])
+            return cls(q_col, s_col, logical_shape=shape, orig_dtype=x.dtype, axis=-2, tensor_scale_inv=si,
+                       total_rows=x.shape[-2])
+        if block_size not in (None, _lib.BLOCK):
+            raise ValueError(f"MX block size must be {_lib.BLOCK}")
         recipe = scaling_recipe or MXScalingRecipe()
         fmt = dtype_to_fmt_code(dest_dtype)
         x = x.detach()
@@ -182,6 +208,8 @@ class QuantizedTensor(torch.Tensor):
         """Back to the original dtype in the payload's orientation.  For a
         transposed copy of ``rows`` tokens the padding columns are dropped."""
         out = K.dequantize_mx_impl(self.rowmajor_codes(), self._scales, self.dtype)
+        if self._tensor_scale_inv is not None:
+            out = (out.float() * self._tensor_scale_inv).to(self.dtype)   # FP8 values are exact in bf16: one rounding
         if self._axis == -2 and not self._use_2d_block and self._segment_lens is not None:
             raise NotImplementedError("dequantize of a segment-padded activation copy")
         # drop the padding of the contraction dim (GEMM granularity / token padding)
@@ -219,13 +247,26 @@ def create_quantized_weight(
     (primus_turbo.py:313-317), so both copies come out of one pass over the
     weight and hold the same codes.  ``kchunk`` picks the storage layout of the
     codes (default: K-chunk-major whenever the GEMMs accept it for this size)."""
-    if quant_config.granularity != ScalingGranularity.MX_BLOCKWISE:
-        raise NotImplementedError("only ScalingGranularity.MX_BLOCKWISE has kernels in this build")
+    if quant_config.granularity not in (ScalingGranularity.MX_BLOCKWISE, ScalingGranularity.TENSORWISE):
+        raise NotImplementedError("only MX_BLOCKWISE and TENSORWISE scaling have kernels in this build")
     fmt = dtype_to_fmt_code(dest_dtype)
     w = weight.detach()
     if w.dtype != torch.bfloat16:
         raise ValueError("create_quantized_weight expects a bfloat16 weight")
     mode = quant_config.scale_mode
+    if quant_config.granularity == ScalingGranularity.TENSORWISE:
+        if kchunk is None:
+            kchunk = K.kchunk_default() and K.kchunk_fits(w.numel() // (w.shape[-1] * w.shape[-2]), w.shape[-2], w.shape[-1])
+        q_row, s_row, q_col, s_col, si = K.quantize_weight_tensorwise_impl(
+            w.contiguous(), fmt, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN, kchunk=kchunk)
+        row = QuantizedTensor(q_row, s_row, logical_shape=w.shape, orig_dtype=w.dtype, axis=-1, kchunk=kchunk,
+                              tensor_scale_inv=si)
+        col = None
+        if need_weight_transpose_cache:
+            shape = tuple(w.shape[:-2]) + (w.shape[-1], w.shape[-2])
+            col = QuantizedTensor(q_col, s_col, logical_shape=shape, orig_dtype=w.dtype, axis=-2, kchunk=kchunk,
+                                  tensor_scale_inv=si)
+        return row, col
     if kchunk is None:
         kchunk = K.kchunk_default() and K.kchunk_fits(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1,
                                                       w.shape[-2], w.shape[-1])

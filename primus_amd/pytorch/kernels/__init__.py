@@ -20,6 +20,7 @@ from ..core.low_precision import (
     dtype_to_fmt_code,
     float4_e2m1fn_x2,
     float8_e4m3,
+    float8_e5m2,
     float8_e8m0,
 )
 
@@ -144,7 +145,7 @@ def _per_byte(fmt: int) -> int:
 
 
 def _code_dtype(fmt: int) -> torch.dtype:
-    return float4_e2m1fn_x2 if fmt == _lib.FMT_E2M1 else float8_e4m3
+    return {_lib.FMT_E4M3: float8_e4m3, _lib.FMT_E2M1: float4_e2m1fn_x2, _lib.FMT_E5M2: float8_e5m2}[fmt]
 
 
 def fmt_of(codes: torch.Tensor) -> int:
@@ -540,6 +541,172 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
     cd = _code_dtype(fmt)
     v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
     return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0)
+
+
+# --------------------------------------------------------------------------
+# Tensor-wise ("current") FP8 scaling: one fp32 scale per tensor
+# (primus_turbo_float8_local.py:194-207 restates the arithmetic, :215-306 the operand flow)
+# --------------------------------------------------------------------------
+_TW_FMTS = (_lib.FMT_E4M3, _lib.FMT_E5M2)
+
+
+def amax_impl(x: torch.Tensor) -> torch.Tensor:
+    """``max |x|`` of a contiguous bfloat16 tensor as a float32 tensor of one element, on the device."""
+    if x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("expected a contiguous bfloat16 tensor")
+    _require_cuda(x)
+    out = torch.empty((1,), dtype=torch.float32, device=x.device)
+    with _hooked("amax", n=x.numel()):
+        rc = _lib.load().mxl_amax(_ptr(x) if x.numel() else None, x.numel(), _ptr(out), _stream())
+    _lib.check(rc, "mxl_amax")
+    return out
+
+
+def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool = False,
+                             group_lens: Optional[torch.Tensor] = None, pad_to: int = 1, kchunk: bool = False,
+                             amax: Optional[torch.Tensor] = None):
+    """``(q_row, s_row, q_colT, s_colT, scale_inv)`` for a 2-D bfloat16 ``x``: codes in the layouts of
+    ``quantize_mx_impl`` but scaled by ``fp8_max / max(amax, 1e-12)`` for the whole tensor; the ``s_*`` arrays
+    hold the unit E8M0 byte (they only make the codes acceptable to the GEMMs), ``scale_inv`` is the float32
+    reciprocal scale (one element, on the device).  ``fmt``: E4M3 or E5M2."""
+    if fmt not in _TW_FMTS:
+        raise ValueError("tensor-wise scaling produces E4M3 or E5M2 codes")
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("expected a contiguous 2-D bfloat16 tensor")
+    if not (rowwise or colwise):
+        raise ValueError("nothing to do: rowwise and colwise are both False")
+    _require_cuda(x, group_lens, amax)
+    rows, cols = x.shape
+    if cols % BLOCK != 0:
+        raise ValueError(f"the last dim ({cols}) must be a multiple of {BLOCK}")
+    G = _check_group_lens(group_lens, x.device) if colwise else 0
+    dev = x.device
+    if amax is None:
+        amax = amax_impl(x)
+    scale_inv = torch.empty((1,), dtype=torch.float32, device=dev)
+    q_row = s_row = q_col = s_col = None
+    row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
+    if rowwise:
+        q_row = torch.empty(_code_shape(rows, row_ld, 1, kchunk), dtype=torch.uint8, device=dev)
+        s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+    if colwise:
+        W = padded_width(rows, G)
+        q_col = torch.empty(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
+        s_col = torch.empty((cols, W // BLOCK), dtype=torch.uint8, device=dev)
+    if rows == 0 and not (colwise and q_col.numel()):
+        scale_inv.fill_(1e-12 / (448.0 if fmt == _lib.FMT_E4M3 else 57344.0))
+    else:
+        with _hooked("quantize_tensorwise", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
+            rc = _lib.load().mxl_quantize_tensorwise(
+                _ptr(x) if rows else None, rows, cols, row_ld if rowwise else 0, fmt, _ptr(amax),
+                _ptr(group_lens) if colwise else None, G, _ptr(q_row) if rows else None, _ptr(s_row) if rows else None,
+                _ptr(q_col), _ptr(s_col), _ptr(scale_inv), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+            )
+        _lib.check(rc, "mxl_quantize_tensorwise")
+    cd = _code_dtype(fmt)
+    v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
+    return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0), scale_inv
+
+
+def quantize_weight_tensorwise_impl(w, fmt: int, *, rowwise: bool = True, colwise: bool = False, pad_to: int = 1,
+                                    kchunk: bool = False):
+    """Weights ``[n, k]`` or ``[G, n, k]`` with one scale for the whole tensor: the row-wise copy and the
+    transposed copy per matrix in the layouts of ``quantize_mx_weight_2d_impl``, plus ``scale_inv``."""
+    if fmt not in _TW_FMTS:
+        raise ValueError("tensor-wise scaling produces E4M3 or E5M2 codes")
+    if w.dim() not in (2, 3) or w.dtype != torch.bfloat16 or not w.is_contiguous():
+        raise ValueError("expected a contiguous bfloat16 weight [n, k] or [G, n, k]")
+    _require_cuda(w)
+    lead = tuple(w.shape[:-2])
+    batch = 1 if not lead else lead[0]
+    n, k = w.shape[-2], w.shape[-1]
+    if n % BLOCK or k % BLOCK:
+        raise ValueError(f"weight dims must be multiples of {BLOCK}")
+    dev = w.device
+    amax = amax_impl(w)
+    scale_inv = torch.empty((1,), dtype=torch.float32, device=dev)
+    k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
+    q_row = s_row = q_col = s_col = None
+    if rowwise:
+        q_row = torch.empty(_code_shape(batch * n, k_ld, 1, True) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
+    if colwise:
+        q_col = torch.empty(_code_shape(batch * k, n_ld, 1, True) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
+    with _hooked("quantize_weight_tensorwise", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
+        rc = _lib.load().mxl_quantize_weight_tensorwise(
+            _ptr(w), batch, n, k, k_ld, n_ld, fmt, _ptr(amax), _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
+            _ptr(scale_inv), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+        )
+    _lib.check(rc, "mxl_quantize_weight_tensorwise")
+    cd = _code_dtype(fmt)
+    v = lambda t, d: None if t is None else t.view(d)  # noqa: E731
+    return v(q_row, cd), v(s_row, float8_e8m0), v(q_col, cd), v(s_col, float8_e8m0), scale_inv
+
+
+def _alpha_ok(*alphas):
+    for t in alphas:
+        if t.dtype != torch.float32 or t.numel() != 1:
+            raise ValueError("per-tensor factors must be float32 tensors of one element")
+    _require_cuda(*alphas)
+
+
+def gemm_tw_nt_impl(a, a_unit, a_scale_inv, b, b_unit, b_scale_inv, group_lens=None, kchunk: bool = False) -> torch.Tensor:
+    """``c = (a . b^T) * a_scale_inv * b_scale_inv`` on tensor-wise scaled codes, dense (``group_lens`` None,
+    ``b [n, k]``) or grouped (``b [G, n, k]``); layouts and the unit block scales as the quantisers above
+    return them (``b_unit`` is ``[n, k/32]`` or ``[G, n, k/32]``).  The contraction dim must be padded to 128."""
+    _require_cuda(a, a_unit, b, b_unit, group_lens)
+    _alpha_ok(a_scale_inv, b_scale_inv)
+    G = _check_group_lens(group_lens, a.device)
+    groups = max(G, 1)
+    a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if kchunk:
+        total_m, k = _chunked_dims(a, a_fmt)
+        b_rows, kb = _chunked_dims(b, b_fmt)
+    else:
+        total_m, k = a.shape
+        b_rows, kb = b.numel() // b.shape[-1], b.shape[-1]
+    n = b_unit.shape[-2]
+    if k != kb or k % _lib.GEMM_K_ALIGN or b_rows != groups * n or b_unit.numel() != b_rows * (k // BLOCK):
+        raise ValueError("operand shapes do not match (the contraction dim must be padded to 128)")
+    if tuple(a_unit.shape) != (total_m, k // BLOCK):
+        raise ValueError("scale shapes must be [rows, k/32]")
+    c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+    with _hooked("grouped_gemm_nt" if G else "gemm_nt", m=total_m, n=n, k=k):
+        rc = _lib.load().mxl_grouped_gemm_nt_scaled(
+            _ptr(a), _ptr(a_unit), a_fmt, _ptr(b), _ptr(b_unit), b_fmt, _ptr(c), _ptr(group_lens), groups, total_m, n, k,
+            _ptr(a_scale_inv), _ptr(b_scale_inv), _lib.GF_KCHUNK if kchunk else 0, _stream(),
+        )
+    _lib.check(rc, "mxl_grouped_gemm_nt_scaled")
+    return c
+
+
+def gemm_tw_wgrad_impl(a_t, a_t_unit, a_scale_inv, b_t, b_t_unit, b_scale_inv, group_lens, total_m,
+                       kchunk: bool = False) -> torch.Tensor:
+    """Variable-K (wgrad) GEMM on tensor-wise scaled transposed operands, times the two factors; shapes as
+    ``grouped_gemm_mx_wgrad_impl``."""
+    _require_cuda(a_t, a_t_unit, b_t, b_t_unit, group_lens)
+    _alpha_ok(a_scale_inv, b_scale_inv)
+    G = _check_group_lens(group_lens, a_t.device)
+    a_fmt, b_fmt = fmt_of(a_t), fmt_of(b_t)
+    W = padded_width(total_m, G)
+    if kchunk:
+        (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt), _chunked_dims(b_t, b_fmt)
+    else:
+        (n, wa), (k, wb) = a_t.shape, b_t.shape
+    if wa != W or wb != W:
+        raise ValueError(f"transposed operands must have padded width {W}")
+    if tuple(a_t_unit.shape) != (n, W // BLOCK) or tuple(b_t_unit.shape) != (k, W // BLOCK):
+        raise ValueError("scale shapes must be [rows, W/32]")
+    shape = (n, k) if group_lens is None else (G, n, k)
+    c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
+    with _hooked("grouped_gemm_wgrad", m=total_m, n=n, k=k):
+        rc = _lib.load().mxl_grouped_gemm_wgrad_scaled(
+            _ptr(a_t), _ptr(a_t_unit), a_fmt, _ptr(b_t), _ptr(b_t_unit), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k,
+            _ptr(a_scale_inv), _ptr(b_scale_inv), _lib.GF_KCHUNK if kchunk else 0, _stream(),
+        )
+    _lib.check(rc, "mxl_grouped_gemm_wgrad_scaled")
+    return c
 
 
 # --------------------------------------------------------------------------

@@ -204,6 +204,100 @@ class _MXLinearFunction(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None, None, grad_nw, None
 
 
+def _transposed_cache(q: QuantizedTensor, kchunk: bool):
+    """Transposed copy (codes, unit scales) of a tensor-wise scaled weight cache that holds the row-wise copy
+    only (the reference keeps no transposed cache under current scaling, primus_turbo.py:1105-1115: its
+    dgrad GEMM reads the same codes in NN layout).  The scale belongs to the whole tensor, so transposing
+    the codes is all there is to do: one pass over the weight's bytes per call."""
+    codes = q.rowmajor_codes()
+    k = q.shape[-1]
+    t = codes[..., :k].transpose(-1, -2)                       # [..., k, n]
+    n = t.shape[-1]
+    n_ld = (n + K.GEMM_K_ALIGN - 1) // K.GEMM_K_ALIGN * K.GEMM_K_ALIGN
+    out = torch.zeros(tuple(t.shape[:-1]) + (n_ld,), dtype=torch.uint8, device=codes.device)
+    out[..., :n] = t.view(torch.uint8)
+    unit = torch.full(tuple(t.shape[:-1]) + (n_ld // _lib.BLOCK,), 127, dtype=torch.uint8, device=codes.device)
+    if kchunk:
+        out = out.reshape(-1, n_ld // K.KCHUNK, K.KCHUNK).permute(1, 0, 2).contiguous()
+    return out.view(codes.dtype), unit.view(q.scales.dtype)
+
+
+class _TWLinearFunction(torch.autograd.Function):
+    """Y = X . W^T on tensor-wise scaled FP8 operands (one float32 scale per tensor, computed from the
+    tensor's abs-max at every call: "current" scaling), dense or grouped.  Operand flow of the reference's
+    tensor-wise linear (primus_turbo_float8_local.py:215-306): X and W in the forward format, dY in the
+    backward format (E5M2 for Format.HYBRID); here every GEMM is NT, so the quantisers also write the
+    transposed copies that dgrad and wgrad read."""
+
+    @staticmethod
+    def forward(ctx, a, b, b_t, group_lens, fwd_fmt, bwd_fmt):
+        need_dgrad = a.requires_grad
+        need_wgrad = b.requires_grad
+        grouped = group_lens is not None
+        groups = b.shape[0] if grouped else 1
+        kc = K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])
+        if isinstance(b, QuantizedTensor):
+            kc = kc and b.kchunk and (b_t is None or b_t.kchunk)
+        a_row, a_ru, a_col, a_cu, a_si = K.quantize_tensorwise_impl(
+            a, fwd_fmt, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
+        if isinstance(b, QuantizedTensor):
+            if b.axis != -1 or b.tensor_scale_inv is None:
+                raise ValueError("the forward weight copy must be a tensor-wise scaled copy quantised along axis=-1")
+            w_row, w_ru, w_si = _cached_codes(b, kc), b.scales, b.tensor_scale_inv
+            w_col = w_cu = None
+            if need_dgrad:
+                if b_t is not None:
+                    w_col, w_cu = _cached_codes(b_t, kc), b_t.scales
+                else:
+                    w_col, w_cu = _transposed_cache(b, kc)
+        else:
+            w_row, w_ru, w_col, w_cu, w_si = K.quantize_weight_tensorwise_impl(
+                b.detach(), fwd_fmt, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
+        y = K.gemm_tw_nt_impl(a_row, a_ru, a_si, w_row, w_ru, w_si, group_lens, kchunk=kc)
+        ctx.save_for_backward(a_col, a_cu, a_si, w_col, w_cu, w_si, group_lens)
+        ctx.cfg = (bwd_fmt, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape), kc)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        a_col, a_cu, a_si, w_col, w_cu, w_si, group_lens = ctx.saved_tensors
+        bwd_fmt, total_m, need_dgrad, need_wgrad, w_shape, kc = ctx.cfg
+        dy = dy.contiguous()
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        d_row, d_ru, d_col, d_cu, d_si = K.quantize_tensorwise_impl(
+            dy, bwd_fmt, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
+        grad_a = grad_b = None
+        overlap = _wgrad_overlap and need_dgrad and need_wgrad
+        if overlap:
+            main = torch.cuda.current_stream(dy.device)
+            side = _side_stream(dy.device)
+            side.wait_stream(main)
+        if need_dgrad:
+            grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc)
+        if need_wgrad:
+            if overlap:
+                with torch.cuda.stream(side):
+                    grad_b = K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc).view(w_shape)
+                for t in (d_col, d_cu, d_si, a_col, a_cu, a_si, grad_b):
+                    t.record_stream(side)
+                grad_b.record_stream(main)
+                main.wait_stream(side)
+            else:
+                grad_b = K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc).view(w_shape)
+        return grad_a, grad_b, None, None, None, None
+
+
+def _tensorwise_formats(config):
+    """(forward, backward) code formats of the tensor-wise recipe (_get_fp8_dtype,
+    primus_turbo_float8_local.py:146-154)."""
+    if config.format == Format.E4M3:
+        return _lib.FMT_E4M3, _lib.FMT_E4M3
+    if config.format == Format.HYBRID:
+        return _lib.FMT_E4M3, _lib.FMT_E5M2
+    raise NotImplementedError(f"tensor-wise scaling is defined for Format.E4M3 and Format.HYBRID (got {config.format})")
+
+
 def _formats(config, fp4: bool):
     if fp4:
         if not isinstance(config, Float4QuantConfig):
@@ -231,7 +325,12 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
         raise ValueError("the MX GEMMs produce bfloat16 output")
     if config is None:
         raise ValueError("config (Float8QuantConfig / Float4QuantConfig) is required")
-    act_fmt, w_fmt = _formats(config, fp4)
+    tensorwise = (not fp4) and isinstance(config, Float8QuantConfig) and config.granularity == ScalingGranularity.TENSORWISE
+    if tensorwise:
+        fwd_fmt, bwd_fmt = _tensorwise_formats(config)
+        act_fmt = w_fmt = fwd_fmt
+    else:
+        act_fmt, w_fmt = _formats(config, fp4)
     if a.dim() != 2 or a.dtype != torch.bfloat16:
         raise ValueError("activations must be a 2-D bfloat16 tensor (callers flatten to [tokens, K])")
     if not a.is_contiguous():
@@ -256,6 +355,10 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
         raise ValueError(f"contraction dims differ: activations K={k_act}, weights K={b.shape[-1]}")
     if group_lens is not None and group_lens.numel() != b.shape[0]:
         raise ValueError("group_lens must have one entry per expert weight")
+    if tensorwise:
+        if glu is not None or norm is not None:
+            raise NotImplementedError("the activation / normalisation prologues exist for the MX recipes only")
+        return _TWLinearFunction.apply(a, b, b_t, group_lens, fwd_fmt, bwd_fmt)
     # stochastic rounding applies to E2M1 gradients; with E4M3 activations the gradients are MXFP8
     grad_sr = bool(fp4 and config.use_gradient_sr and act_fmt == _lib.FMT_E2M1)
     rht = getattr(config, "colwise_rht_signs", None) if fp4 and act_fmt == _lib.FMT_E2M1 else None

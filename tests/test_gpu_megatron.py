@@ -406,3 +406,50 @@ def test_layernorm_linear_folds_the_rmsnorm_into_the_quantiser(mg, gpu, fp4, mic
             assert _cos(y, want) > (0.97 if fp4 else 0.999)
     for a, b in zip(res[True], res[False]):
         assert a.shape == b.shape and torch.equal(a, b)
+
+
+@pytest.mark.parametrize("hybrid", [False, True])
+@pytest.mark.parametrize("microbatches", [1, 2])
+def test_linear_and_grouped_linear_under_the_tensorwise_recipe(mg, gpu, hybrid, microbatches):
+    """The non-MX "current scaling" recipe through the same modules (quant_config.current_scaling(),
+    primus_turbo.py:1087-1135): close to the bf16 module, and with several microbatches the cached row-wise
+    weight copy (no transposed cache under current scaling, :1105-1115) gives the same gradients."""
+    pt = mg
+    from primus_amd.megatron import runtime
+    from primus_amd.pytorch.core import Format, ScalingGranularity
+
+    runtime.set_num_microbatches(microbatches)
+    qc = pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.TENSORWISE, format=Format.HYBRID if hybrid else Format.E4M3)
+    assert qc.current_scaling() and not qc.mxfp8_scaling()
+    torch.manual_seed(21)
+    lin = pt.PrimusTurboLinear(256, 160, parallel_mode=None, config=_cfg(), bias=False, skip_bias_add=False)
+    lin.weight.main_grad = torch.zeros_like(lin.weight, dtype=torch.float32)
+    lin.weight.grad_added_to_main_grad = False
+    x = torch.randn(16, 8, 256, device=gpu).bfloat16().requires_grad_()
+    dy = torch.randn(16, 8, 160, device=gpu).bfloat16()
+    with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc):
+        y, _ = lin(x)
+    y.backward(dy)
+    if microbatches > 1:
+        assert lin.quantized_weight_buffer.tensor_scale_inv is not None and lin.quantized_weight_t_buffer is None
+    xr = x.detach().clone().requires_grad_()
+    wr = lin.weight.detach().clone().requires_grad_()
+    yr = torch.nn.functional.linear(xr, wr)
+    yr.backward(dy)
+    wgrad = lin.weight.main_grad if microbatches > 1 else lin.weight.grad
+    assert _cos(y, yr) > 0.998 and _cos(x.grad, xr.grad) > (0.99 if hybrid else 0.998)
+    assert _cos(wgrad, wr.grad) > (0.99 if hybrid else 0.998)
+
+    lens = [33, 0, 130, 1, 92]
+    gl = pt.PrimusTurboColumnParallelGroupedLinear(5, 128, 96, config=_cfg())
+    gl.weights.main_grad = torch.zeros_like(gl.weights, dtype=torch.float32)
+    gl.weights.grad_added_to_main_grad = False
+    xg = torch.randn(sum(lens), 128, device=gpu).bfloat16().requires_grad_()
+    dyg = torch.randn(sum(lens), 96, device=gpu).bfloat16()
+    with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc):
+        yg, _ = gl(xg, torch.tensor(lens))
+    yg.backward(dyg)
+    want = torch.cat([xs @ gl.weights[e].detach().t() for e, xs in enumerate(torch.split(xg.detach(), lens))])
+    assert _cos(yg, want) > 0.998
+    wg = gl.weights.main_grad if microbatches > 1 else gl.weights.grad
+    assert not wg[1].any() and wg[0].abs().sum() > 0

@@ -171,5 +171,12 @@ def test_quantized_tensor_quantize_axes(gpu):
     assert np.array_equal(r2.codes.view(torch.uint8).cpu().numpy(), q2) and np.array_equal(c2.codes.view(torch.uint8).cpu().numpy(), q2t)
     with pytest.raises(NotImplementedError):
         r.transpose(-2, -1)
+    tw = QuantizedTensor.quantize(wd, dest_dtype=float8_e4m3, granularity=ScalingGranularity.TENSORWISE)
+    want, want_si = o.quantize_tensorwise(w, o.FMT_E4M3)
+    assert np.array_equal(tw.codes.view(torch.uint8).cpu().numpy(), want) and tw.tensor_scale_inv.item() == float(want_si)
+    twt = QuantizedTensor.quantize(wd, dest_dtype=float8_e4m3, granularity=ScalingGranularity.TENSORWISE, axis=-2)
+    assert tuple(twt.shape) == (160, 96) and np.array_equal(twt.codes.view(torch.uint8).cpu().numpy()[:, :96], want.T)
+    deq = tw.dequantize().float().cpu().numpy()
+    assert np.abs(deq - w.float().numpy()).max() <= 0.07 * np.abs(w.float().numpy()).max()   # E4M3: 2^-4 relative steps
     with pytest.raises(NotImplementedError):
-        QuantizedTensor.quantize(wd, dest_dtype=float8_e4m3, granularity=ScalingGranularity.TENSORWISE)
+        QuantizedTensor.quantize(wd, dest_dtype=float8_e4m3, granularity=ScalingGranularity.BLOCKWISE)

@@ -42,6 +42,8 @@ WORKLOADS = {
     "deepseek_v3_shard_mxfp8": dict(G=32, topk=8, tokens=8192, hidden=7168, fc1_out=4096, fc2_in=2048, routing="zipf", seed=1004, fp4=False),
     "gpt_oss_120b_mxfp4": dict(G=128, topk=4, tokens=16384, hidden=2880, fc1_out=5760, fc2_in=2880, routing="uniform", seed=1005, fp4=True, wgrad=False),
     "llama3_8b_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False),
+    # the non-MX "current scaling" recipe on the headline shapes (HYBRID: E4M3 forward, E5M2 gradients)
+    "mixtral_8x7b_moe_fp8_tensorwise": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, tensorwise=True),
     # the same MLP with the RMSNorm that precedes fc1 in the layer (LayerNormColumnParallelLinear), folded into fc1's quantiser
     "llama3_8b_norm_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, norm=True),
 }
@@ -216,6 +218,9 @@ def main():
     if spec["fp4"]:
         cfg = Float4QuantConfig(activation_format=Format.E4M3)
         op = pt.ops.grouped_gemm_fp4
+    elif spec.get("tensorwise"):
+        cfg = Float8QuantConfig(format=Format.HYBRID, granularity=ScalingGranularity.TENSORWISE)
+        op = pt.ops.grouped_gemm_fp8 if grouped else None
     else:
         cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0, block_size=32)
         op = pt.ops.grouped_gemm_fp8 if grouped else None
@@ -302,13 +307,16 @@ def main():
             a["flops"] += 2.0 * info["m"] * info["n"] * info["k"]
         elif name in ("rmsnorm_fwd", "rmsnorm_bwd"):
             a["bytes"] += norm_bytes(name, info)
+        elif name == "amax":
+            a["bytes"] += 2.0 * info["n"]
         else:
             a["bytes"] += quant_bytes(info)
     fwd_name = "grouped_gemm_nt" if grouped else "gemm_nt"
     gk = acc[fwd_name]
     gemm_tflops = gk["flops"] / gk["sec"] / 1e12
     roofline = {
-        "kernel": "mx_gemm_kernel<e4m3,%s,fwd/dgrad> (%s)" % ("e2m1" if spec["fp4"] else "e4m3", fwd_name),
+        "kernel": "mx_gemm_kernel<%s,%s,fwd/dgrad%s> (%s)" % ("e4m3|e5m2" if spec.get("tensorwise") else "e4m3", "e2m1" if spec["fp4"] else "e4m3",
+                                                               ",alpha" if spec.get("tensorwise") else "", fwd_name),
         "bound": "mfma",
         "achieved": round(gemm_tflops, 2),
         "peak": FP8_PEAK_TFLOPS,
@@ -332,8 +340,8 @@ def main():
     gemm_flops = sum(a["flops"] for nme, a in acc.items() if "gemm" in nme)
 
     out = {
-        "metric": "MXFP8 grouped-GEMM TFLOPS (%s, quantisers inside the timed step)"
-                  % ("fwd+dgrad+wgrad" if spec.get("wgrad", True) else "fwd+dgrad"),
+        "metric": "%s grouped-GEMM TFLOPS (%s, quantisers inside the timed step)"
+                  % ("FP8 tensor-wise" if spec.get("tensorwise") else "MXFP8", "fwd+dgrad+wgrad" if spec.get("wgrad", True) else "fwd+dgrad"),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -343,7 +351,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"] else "mxfp8_e4m3 (E8M0 block scales), fp32 accumulate",
+        "dtype": "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"]
+                 else "fp8 e4m3 forward / e5m2 gradients, one fp32 scale per tensor, fp32 accumulate" if spec.get("tensorwise")
+                 else "mxfp8_e4m3 (E8M0 block scales), fp32 accumulate",
         "data": "synthetic (seeded, generated on the GPU; random-init weights N(0,0.02))",
         "config": {
             "workload": args.workload,

@@ -192,6 +192,11 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * of a and num_groups * n rows of b in the forward / dgrad GEMM; n rows of a and k rows of b over the padded
  * token width in wgrad).  Scales stay row-major.  Same results bit for bit; an operand must stay below 4 GiB. */
 #define MXL_GF_KCHUNK 1u
+/* mxl_grouped_gemm_wgrad_ex / _scaled only, together with MXL_GF_KCHUNK: c_bf16 points to FLOAT32 [g, n, k] and the
+ * result is ADDED to it in fp32 (no rounding to bf16).  This is the gradient-accumulation fusion of the reference
+ * (fuse_bgrad_accum_pattern = "megatron": the GEMM's beta = 1 epilogue adds into weight.main_grad,
+ * primus_turbo.py:166-240, 243-275) -- available here for the MX recipes too.  With no tokens nothing is added. */
+#define MXL_GF_ACCUM_F32 2u
 int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                            const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                            int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);

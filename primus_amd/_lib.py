@@ -28,7 +28,8 @@ MAX_GROUPS = 1024
 ACT_SILU, ACT_GELU = 0, 1
 PROBS_F32, PROBS_BF16 = 0, 1
 QF_SR, QF_RHT_COL, QF_KCHUNK = 1, 2, 4   # flags of mxl_quantize_ex
-GF_KCHUNK = 1                            # flag of the GEMM _ex entry points: operands are K-chunk-major
+GF_KCHUNK = 1                               # flag of the GEMM _ex entry points: operands are K-chunk-major
+GF_ACCUM_F32 = 2                            # wgrad: the output is float32 and the result is added to it
 
 EXPORTS = (
     "mxl_version",

@@ -135,7 +135,11 @@ struct Frags {
 // LAYOUT 0: operand codes row-major [rows, K].  LAYOUT 1: K-chunk-major [K / 128][rows][128 elements] (what the
 // quantisers write with MXL_QF_KCHUNK): the rows of a tile's K slot are one contiguous block, so a load round
 // fetches 4 KiB in a row instead of 16..64 row pieces; scales are row-major in both.
-template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false>
+// ACCUM: the output is float32 and the result is ADDED to what it holds (the weight gradient going straight
+// into the fp32 main_grad buffer that the reference's bridge otherwise adds it to in a separate pass,
+// primus/backends/megatron/core/extensions/primus_turbo.py:166-240); every output tile belongs to one
+// workgroup, so the read-modify-write needs no atomics.
+template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false, bool ACCUM = false>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     constexpr int A_BYTES = Op<AFMT>::tile_bytes, B_BYTES = Op<BFMT>::tile_bytes;
     constexpr int STAGE = A_BYTES + B_BYTES;            // one slot: K = 128 of both operands
@@ -459,6 +463,38 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             const bool full = (m_valid == BM) && (n_valid == BN);
             float alpha = 1.f;
             if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
+            if (ACCUM) {
+                // float32 read-modify-write, 64 columns (256 bytes per row) of a 32-row block at a time through
+                // the same patch: a store instruction covers 4 rows x 256 contiguous bytes
+                float* ctile32 = (float*)p.c + (ctile - p.c);
+                uint8_t* wr32 = stg + lr * SP + 16 * g;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                        for (int jl = 0; jl < 2; ++jl)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                const int j = 2 * jj + jl;
+                                v4f o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                                if (ALPHA) o *= alpha;
+                                *(v4f*)(wr32 + (jl * 32 + 8 * q) * 4) = o;
+                            }
+                        const int col = wn * 128 + jj * 64 + (l & 15) * 4;
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            const v4f v = *(const v4f*)(rd + 4 * u * SP);
+                            const int row = wm * 128 + i * 32 + 4 * u + rr;
+                            if (full || (row < m_valid && col < n_valid)) {
+                                v4f* dst = (v4f*)(ctile32 + (int64_t)row * p.n + col);
+                                *dst = *dst + v;
+                            }
+                        }
+                    }
+                    MXL_PIN;
+                }
+            } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 // lane (lr, g) holds row lr of this 32-row block: columns j*32 + 8q + 4g .. +3
@@ -492,6 +528,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
                 }
                 MXL_PIN;  // one 32-row block at a time: 64 accumulators live, not 256
             }
+            }
         }
     }
 #undef MXL_MFMA
@@ -523,13 +560,13 @@ static int num_cus(int slot) {
     return pr.multiProcessorCount;
 }
 
-template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false>
+template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false, bool ACCUM = false>
 static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = gemm_lds_bytes(AFMT, BFMT);
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set[64];   // the attribute belongs to the (kernel, device) pair
     const int slot = current_device_slot();
-    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT, ALPHA>;
+    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT, ALPHA, ACCUM>;
     if (!attr_set[slot].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
@@ -562,10 +599,30 @@ static int dispatch_gemm_alpha_l(int afmt, int bfmt, const GemmArgs& a, int64_t 
     return MXL_EINVAL;
 }
 
+// wgrad accumulated into a float32 buffer: K-chunk-major operands only
+static int dispatch_wgrad_accum(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    constexpr int W = MODE_WGRAD;
+    if (a.alpha_a != nullptr) {
+        if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, W, 1, true, true>(a, max_tiles, st);
+        if (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, W, 1, true, true>(a, max_tiles, st);
+        return MXL_EINVAL;
+    }
+    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, W, 1, false, true>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E2M1) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E2M1, W, 1, false, true>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E4M3, W, 1, false, true>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E2M1) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E2M1, W, 1, false, true>(a, max_tiles, st);
+    return MXL_EINVAL;
+}
+
 // a_rows / b_rows: rows of the whole operands (for the 4 GiB bound of the chunk-major layout)
 template <int MODE>
 static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, bool kchunk, int64_t a_rows, int64_t b_rows,
-                         hipStream_t st) {
+                         hipStream_t st, bool accum = false) {
+    if (accum) {
+        if (MODE != MODE_WGRAD || !kchunk) return MXL_EINVAL;
+        if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
+        return dispatch_wgrad_accum(afmt, bfmt, a, max_tiles, st);
+    }
     const bool alpha = a.alpha_a != nullptr;
     if (!kchunk) return alpha ? dispatch_gemm_alpha_l<MODE, 0>(afmt, bfmt, a, max_tiles, st)
                               : dispatch_gemm_l<MODE, 0>(afmt, bfmt, a, max_tiles, st);
@@ -650,7 +707,9 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
                               const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups,
                               int64_t total_m, int64_t n, int64_t k, const float* alpha_a, const float* alpha_b,
                               uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)MXL_GF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_ACCUM_F32)) return MXL_EINVAL;
+    const bool accum = (flags & MXL_GF_ACCUM_F32) != 0;
+    if (accum && !(flags & MXL_GF_KCHUNK)) return MXL_EINVAL;
     if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
     if (num_groups < 0 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
@@ -661,6 +720,7 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
     // kernel only writes the zero gradient
     if (mxl_padded_width(total_m, G) > MAX_CONTRACTION) return MXL_EINVAL;
     const bool nothing_to_read = mxl_padded_width(total_m, G) == 0;
+    if (nothing_to_read && accum) return MXL_OK;   // nothing to add
     if (nothing_to_read) {
         // The GEMM kernel requests the first K slot of every tile unconditionally, so it is never launched on
         // operands that do not exist; a fill kernel (not a memset, which callers could not capture in a graph)
@@ -689,7 +749,7 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
     a.alpha_a = alpha_a;
     a.alpha_b = alpha_b;
     const int64_t max_tiles = (int64_t)G * ((n + BM - 1) / BM) * ((k + BN - 1) / BN);
-    return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, n, k, (hipStream_t)stream);
+    return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, n, k, (hipStream_t)stream, accum);
 }
 
 extern "C" int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,

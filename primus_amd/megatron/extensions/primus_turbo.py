@@ -418,11 +418,17 @@ def _fuse_wgrad_accum_pattern(config, weight: torch.Tensor) -> Optional[str]:
     if not getattr(config, "gradient_accumulation_fusion", False):
         return None
     manager = PrimusTurboLowPrecisionGlobalStateManager
+    # the wgrad kernel of this package adds into a float32 buffer for every recipe; the reference's kernels do
+    # so for bf16 and tensor-wise FP8 only, which stays the default (switch: turbo_fuse_wgrad_accum_mx, ours)
+    mx_too = bool(getattr(runtime.get_args(), "turbo_fuse_wgrad_accum_mx", False))
     if manager.is_turbo_fp4_enabled():
-        return None
-    if manager.is_turbo_fp8_enabled():
+        if not mx_too:
+            return None
+    elif manager.is_turbo_fp8_enabled():
         quant_config = manager.get_turbo_quant_config()
-        if quant_config is None or not quant_config.current_scaling():
+        if quant_config is None:
+            return None
+        if not quant_config.current_scaling() and not (mx_too and quant_config.mxfp8_scaling()):
             return None
     elif weight.dtype not in (torch.bfloat16, torch.float16):
         return None

@@ -421,8 +421,18 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
     return c
 
 
+def _accum_target(accum_into, shape, kchunk, device):
+    """Checks the float32 buffer a wgrad GEMM is to add its result to."""
+    if not kchunk:
+        raise ValueError("accumulating wgrad needs K-chunk-major operands")
+    if (accum_into.dtype != torch.float32 or tuple(accum_into.shape) != tuple(shape) or not accum_into.is_contiguous()
+            or accum_into.device != device):
+        raise ValueError(f"accum_into must be a contiguous float32 tensor of shape {tuple(shape)} on the operands' device")
+    return accum_into
+
+
 def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total_m, out_dtype=torch.bfloat16,
-                               kchunk: bool = False) -> torch.Tensor:
+                               kchunk: bool = False, accum_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Variable-K (wgrad) grouped GEMM on segment-padded transposed operands:
     ``a_t`` = dY^T codes ``[n, W]``, ``b_t`` = X^T codes ``[k, W]``; returns
     ``[G, n, k]`` (``[n, k]`` when ``group_lens`` is None).  An expert with no
@@ -443,11 +453,17 @@ def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total
     if tuple(a_t_scale.shape) != (n, W // BLOCK) or tuple(b_t_scale.shape) != (k, W // BLOCK):
         raise ValueError("scale shapes must be [rows, W/32]")
     shape = (n, k) if group_lens is None else (G, n, k)
-    c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
+    flags = _lib.GF_KCHUNK if kchunk else 0
+    if accum_into is not None:
+        # the result is added, in float32, to accum_into (which is returned)
+        c = _accum_target(accum_into, shape, kchunk, a_t.device)
+        flags |= _lib.GF_ACCUM_F32
+    else:
+        c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
     with _hooked("grouped_gemm_wgrad", m=total_m, n=n, k=k):
         rc = _lib.load().mxl_grouped_gemm_wgrad_ex(
             _ptr(a_t), _ptr(a_t_scale), a_fmt, _ptr(b_t), _ptr(b_t_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k,
-            _lib.GF_KCHUNK if kchunk else 0, _stream()
+            flags, _stream()
         )
     _lib.check(rc, "mxl_grouped_gemm_wgrad")
     return c
@@ -682,9 +698,9 @@ def gemm_tw_nt_impl(a, a_unit, a_scale_inv, b, b_unit, b_scale_inv, group_lens=N
 
 
 def gemm_tw_wgrad_impl(a_t, a_t_unit, a_scale_inv, b_t, b_t_unit, b_scale_inv, group_lens, total_m,
-                       kchunk: bool = False) -> torch.Tensor:
+                       kchunk: bool = False, accum_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Variable-K (wgrad) GEMM on tensor-wise scaled transposed operands, times the two factors; shapes as
-    ``grouped_gemm_mx_wgrad_impl``."""
+    ``grouped_gemm_mx_wgrad_impl`` (also ``accum_into``)."""
     _require_cuda(a_t, a_t_unit, b_t, b_t_unit, group_lens)
     _alpha_ok(a_scale_inv, b_scale_inv)
     G = _check_group_lens(group_lens, a_t.device)
@@ -699,11 +715,16 @@ def gemm_tw_wgrad_impl(a_t, a_t_unit, a_scale_inv, b_t, b_t_unit, b_scale_inv, g
     if tuple(a_t_unit.shape) != (n, W // BLOCK) or tuple(b_t_unit.shape) != (k, W // BLOCK):
         raise ValueError("scale shapes must be [rows, W/32]")
     shape = (n, k) if group_lens is None else (G, n, k)
-    c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
+    flags = _lib.GF_KCHUNK if kchunk else 0
+    if accum_into is not None:
+        c = _accum_target(accum_into, shape, kchunk, a_t.device)
+        flags |= _lib.GF_ACCUM_F32
+    else:
+        c = torch.empty(shape, dtype=torch.bfloat16, device=a_t.device)
     with _hooked("grouped_gemm_wgrad", m=total_m, n=n, k=k):
         rc = _lib.load().mxl_grouped_gemm_wgrad_scaled(
             _ptr(a_t), _ptr(a_t_unit), a_fmt, _ptr(b_t), _ptr(b_t_unit), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k,
-            _ptr(a_scale_inv), _ptr(b_scale_inv), _lib.GF_KCHUNK if kchunk else 0, _stream(),
+            _ptr(a_scale_inv), _ptr(b_scale_inv), flags, _stream(),
         )
     _lib.check(rc, "mxl_grouped_gemm_wgrad_scaled")
     return c

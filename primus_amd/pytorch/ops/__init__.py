@@ -73,6 +73,43 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
     return st
 
 
+_dummy_wgrads = {}
+
+
+def _finish_wgrad(grad_b, accum, fused: bool, w_shape):
+    """Gradient-accumulation fusion (``fuse_bgrad_accum_pattern="megatron"``): the weight gradient belongs in
+    the float32 ``main_grad`` of the operand.  ``fused``: the GEMM has added it already; otherwise it is added
+    here.  Either way the operand's ``grad_added_to_main_grad`` is set and autograd gets a placeholder of the
+    weight's shape, whose only purpose is to make the parameter's gradient hooks fire
+    (primus/backends/megatron/core/extensions/primus_turbo.py:141-163, 166-240)."""
+    if accum is None:
+        return grad_b.view(w_shape)
+    target, owner = accum
+    if not fused:
+        target.add_(grad_b.view(w_shape))
+    owner.grad_added_to_main_grad = True
+    key = (tuple(w_shape), target.device)
+    dummy = _dummy_wgrads.get(key)
+    if dummy is None:
+        dummy = torch.empty(tuple(w_shape), dtype=torch.bfloat16, device=target.device)
+        _dummy_wgrads[key] = dummy
+    return dummy
+
+
+def _accum_from(b, pattern):
+    """``(main_grad, operand)`` for ``fuse_bgrad_accum_pattern="megatron"``, else None."""
+    if pattern is None:
+        return None
+    if pattern != "megatron":
+        raise ValueError(f"unknown fuse_bgrad_accum_pattern {pattern!r} (the reference passes 'megatron' or None)")
+    main_grad = getattr(b, "main_grad", None)
+    if main_grad is None or not hasattr(b, "grad_added_to_main_grad"):
+        raise ValueError("fuse_bgrad_accum_pattern='megatron' needs main_grad and grad_added_to_main_grad on the weight operand")
+    if main_grad.dtype != torch.float32 or tuple(main_grad.shape) != tuple(b.shape) or not main_grad.is_contiguous():
+        raise ValueError("main_grad must be a contiguous float32 tensor of the weight's shape")
+    return main_grad, b
+
+
 def _cached_codes(q: QuantizedTensor, kchunk: bool) -> torch.Tensor:
     """Codes of a cached weight copy in the layout this call's GEMMs use.  A K-chunk-major cache is
     rearranged (one pass over the weight) only when this call cannot use that layout."""
@@ -88,7 +125,7 @@ class _MXLinearFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, b, b_t, group_lens, act_fmt, w_fmt, scale_mode, probs=None, row_mask=None, activation=None,
-                grad_sr=False, rht_signs=None, norm_weight=None, norm_eps=0.0):
+                grad_sr=False, rht_signs=None, norm_weight=None, norm_eps=0.0, accum=None):
         glu = activation is not None
         norm = norm_weight is not None
         need_dgrad = a.requires_grad or (glu and probs.requires_grad) or (norm and norm_weight.requires_grad)
@@ -123,6 +160,8 @@ class _MXLinearFunction(torch.autograd.Function):
             # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
             if b.axis != -1:
                 raise ValueError("the forward weight copy must be quantised along axis=-1")
+            if b.tensor_scale_inv is not None:
+                raise ValueError("the cached weight copy is tensor-wise scaled, the operator's config is an MX recipe")
             w_row, w_rs = _cached_codes(b, kc), b.scales
             w_col = w_cs = None
             if need_dgrad:
@@ -151,6 +190,7 @@ class _MXLinearFunction(torch.autograd.Function):
         ctx.rht_signs = rht_signs
         ctx.kchunk = kc
         ctx.norm = norm
+        ctx.accum = accum      # (float32 buffer the weight gradient is added to, object that gets the flag) or None
         return y
 
     @staticmethod
@@ -181,15 +221,23 @@ class _MXLinearFunction(torch.autograd.Function):
             else:
                 grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc)
         if need_wgrad:
+            target = ctx.accum[0] if ctx.accum is not None else None
+            fused = target is not None and kc          # the GEMM's epilogue adds into the float32 buffer
+
+            def wgrad():
+                return K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc,
+                                                    accum_into=target if fused else None)
+
             if overlap:
                 with torch.cuda.stream(side):
-                    grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc).view(w_shape)
+                    grad_b = wgrad()
                 for t in (d_col, d_cs, a_col, a_cs, grad_b):
                     t.record_stream(side)
                 grad_b.record_stream(main)
                 main.wait_stream(side)
             else:
-                grad_b = K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc).view(w_shape)
+                grad_b = wgrad()
+            grad_b = _finish_wgrad(grad_b, ctx.accum, fused, w_shape)
         grad_p = None
         if ctx.activation is not None and need_dgrad:
             # grad_a so far is dL/dX; take it through the activation to fc1's output and the probabilities
@@ -201,7 +249,7 @@ class _MXLinearFunction(torch.autograd.Function):
             # grad_a so far is dL/dX for X = rmsnorm(a); take it through the normalisation
             pre, nw, rstd = ctx.saved_tensors[5:8]
             grad_a, grad_nw = K.rmsnorm_bwd_impl(grad_a, pre, nw, rstd)
-        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None, None, grad_nw, None
+        return grad_a, grad_b, None, None, None, None, None, grad_p, None, None, None, None, grad_nw, None, None
 
 
 def _transposed_cache(q: QuantizedTensor, kchunk: bool):
@@ -230,7 +278,7 @@ class _TWLinearFunction(torch.autograd.Function):
     transposed copies that dgrad and wgrad read."""
 
     @staticmethod
-    def forward(ctx, a, b, b_t, group_lens, fwd_fmt, bwd_fmt):
+    def forward(ctx, a, b, b_t, group_lens, fwd_fmt, bwd_fmt, accum=None):
         need_dgrad = a.requires_grad
         need_wgrad = b.requires_grad
         grouped = group_lens is not None
@@ -256,6 +304,7 @@ class _TWLinearFunction(torch.autograd.Function):
         y = K.gemm_tw_nt_impl(a_row, a_ru, a_si, w_row, w_ru, w_si, group_lens, kchunk=kc)
         ctx.save_for_backward(a_col, a_cu, a_si, w_col, w_cu, w_si, group_lens)
         ctx.cfg = (bwd_fmt, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape), kc)
+        ctx.accum = accum
         return y
 
     @staticmethod
@@ -276,16 +325,24 @@ class _TWLinearFunction(torch.autograd.Function):
         if need_dgrad:
             grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc)
         if need_wgrad:
+            target = ctx.accum[0] if ctx.accum is not None else None
+            fused = target is not None and kc
+
+            def wgrad():
+                return K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc,
+                                            accum_into=target if fused else None)
+
             if overlap:
                 with torch.cuda.stream(side):
-                    grad_b = K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc).view(w_shape)
+                    grad_b = wgrad()
                 for t in (d_col, d_cu, d_si, a_col, a_cu, a_si, grad_b):
                     t.record_stream(side)
                 grad_b.record_stream(main)
                 main.wait_stream(side)
             else:
-                grad_b = K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc).view(w_shape)
-        return grad_a, grad_b, None, None, None, None
+                grad_b = wgrad()
+            grad_b = _finish_wgrad(grad_b, ctx.accum, fused, w_shape)
+        return grad_a, grad_b, None, None, None, None, None
 
 
 def _tensorwise_formats(config):
@@ -318,9 +375,6 @@ def _formats(config, fp4: bool):
 def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern, fp4, glu=None, norm=None):
     if trans_a or not trans_b:
         raise ValueError("the MX linear path is NT only: trans_a=False, trans_b=True (primus_turbo.py:1095-1103)")
-    if fuse_bgrad_accum_pattern is not None:
-        # never set for MX / FP4 by the reference (primus_turbo.py:247-249,259-264)
-        raise NotImplementedError("fused wgrad accumulation is not available for MX recipes")
     if out_dtype not in (None, torch.bfloat16):
         raise ValueError("the MX GEMMs produce bfloat16 output")
     if config is None:
@@ -355,10 +409,13 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
         raise ValueError(f"contraction dims differ: activations K={k_act}, weights K={b.shape[-1]}")
     if group_lens is not None and group_lens.numel() != b.shape[0]:
         raise ValueError("group_lens must have one entry per expert weight")
+    # the reference sets the pattern for tensor-wise FP8 only (primus_turbo.py:243-275); the wgrad kernel here
+    # accumulates for every recipe
+    accum = _accum_from(b, fuse_bgrad_accum_pattern)
     if tensorwise:
         if glu is not None or norm is not None:
             raise NotImplementedError("the activation / normalisation prologues exist for the MX recipes only")
-        return _TWLinearFunction.apply(a, b, b_t, group_lens, fwd_fmt, bwd_fmt)
+        return _TWLinearFunction.apply(a, b, b_t, group_lens, fwd_fmt, bwd_fmt, accum)
     # stochastic rounding applies to E2M1 gradients; with E4M3 activations the gradients are MXFP8
     grad_sr = bool(fp4 and config.use_gradient_sr and act_fmt == _lib.FMT_E2M1)
     rht = getattr(config, "colwise_rht_signs", None) if fp4 and act_fmt == _lib.FMT_E2M1 else None
@@ -369,10 +426,10 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
         if norm_weight.dtype != torch.bfloat16 or tuple(norm_weight.shape) != (a.shape[-1],):
             raise ValueError("the norm weight must be a bfloat16 vector of the contraction length")
         return _MXLinearFunction.apply(a, b, b_t, None, act_fmt, w_fmt, config.scale_mode.value,
-                                       None, None, None, grad_sr, None, norm_weight.contiguous(), float(eps))
+                                       None, None, None, grad_sr, None, norm_weight.contiguous(), float(eps), accum)
     if glu is None:
         return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
-                                       None, None, None, grad_sr, rht)
+                                       None, None, None, grad_sr, rht, None, 0.0, accum)
     if rht is not None:
         raise NotImplementedError("the activation prologue and the Hadamard transform cannot be combined")
     probs, row_mask, activation = glu
@@ -381,7 +438,7 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
     if probs.dim() != 1 or probs.shape[0] != a.shape[0]:
         raise ValueError("probs must be 1-D with one entry per row of the activations")
     return _MXLinearFunction.apply(a, b, b_t, group_lens, act_fmt, w_fmt, config.scale_mode.value,
-                                   probs.contiguous(), row_mask, activation, grad_sr)
+                                   probs.contiguous(), row_mask, activation, grad_sr, None, None, 0.0, accum)
 
 
 def gemm_fp8(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
@@ -496,10 +553,41 @@ def glu_grouped_gemm_fp4(x, probs, b, group_lens: torch.Tensor, activation: str 
 # the library GEMM behind ``torch.matmul``, the grouped one a loop of those
 # (which reads ``group_lens`` back to the host).
 # ---------------------------------------------------------------------------
+class _PlainLinearAccum(torch.autograd.Function):
+    """Unquantised ``a . b^T`` (dense or per expert) whose weight gradient is added to ``b.main_grad``."""
+
+    @staticmethod
+    def forward(ctx, a, b, lens, accum):
+        ctx.save_for_backward(a, b)
+        ctx.lens, ctx.accum = lens, accum
+        if lens is None:
+            return torch.matmul(a, b.transpose(-2, -1))
+        return torch.cat([torch.matmul(rows, b[g].transpose(-2, -1)) for g, rows in enumerate(torch.split(a, lens, dim=0))], dim=0)
+
+    @staticmethod
+    def backward(ctx, dy):
+        a, b = ctx.saved_tensors
+        target, _ = ctx.accum
+        if ctx.lens is None:
+            grad_a = torch.matmul(dy, b)
+            target.add_(torch.matmul(dy.transpose(-2, -1), a))
+        else:
+            parts = []
+            for g, (d, rows) in enumerate(zip(torch.split(dy, ctx.lens, dim=0), torch.split(a, ctx.lens, dim=0))):
+                parts.append(torch.matmul(d, b[g]))
+                target[g].add_(torch.matmul(d.transpose(-2, -1), rows))
+            grad_a = torch.cat(parts, dim=0)
+        return grad_a, _finish_wgrad(None, ctx.accum, True, tuple(b.shape)), None, None
+
+
 def gemm(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
          fuse_bgrad_accum_pattern: Optional[str] = None):
-    if fuse_bgrad_accum_pattern is not None:
-        raise NotImplementedError("fused wgrad accumulation is not implemented")
+    accum = _accum_from(b, fuse_bgrad_accum_pattern)
+    if accum is not None:
+        if trans_a or not trans_b or a.dim() != 2:
+            raise ValueError("fuse_bgrad_accum_pattern is defined for the NT linear on 2-D activations")
+        out = _PlainLinearAccum.apply(a, b, None, accum)
+        return out if out_dtype is None else out.to(out_dtype)
     a2 = a.transpose(-2, -1) if trans_a else a
     b2 = b.transpose(-2, -1) if trans_b else b
     out = torch.matmul(a2, b2)
@@ -508,11 +596,14 @@ def gemm(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[
 
 def grouped_gemm(a, b, group_lens: torch.Tensor, trans_b: bool = True,
                  fuse_bgrad_accum_pattern: Optional[str] = None):
-    if fuse_bgrad_accum_pattern is not None:
-        raise NotImplementedError("fused wgrad accumulation is not implemented")
     lens = [int(v) for v in _lens(group_lens).tolist()]
     if sum(lens) != a.shape[0]:
         raise ValueError("group_lens must sum to the number of rows of a")
+    accum = _accum_from(b, fuse_bgrad_accum_pattern)
+    if accum is not None:
+        if not trans_b:
+            raise ValueError("fuse_bgrad_accum_pattern is defined for the NT linear")
+        return _PlainLinearAccum.apply(a, b, lens, accum)
     outs = []
     for g, rows in enumerate(torch.split(a, lens, dim=0)):
         w = b[g].transpose(-2, -1) if trans_b else b[g]

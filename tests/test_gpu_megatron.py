@@ -453,3 +453,63 @@ def test_linear_and_grouped_linear_under_the_tensorwise_recipe(mg, gpu, hybrid, 
     assert _cos(yg, want) > 0.998
     wg = gl.weights.main_grad if microbatches > 1 else gl.weights.grad
     assert not wg[1].any() and wg[0].abs().sum() > 0
+
+
+@pytest.mark.parametrize("recipe", ["bf16", "tensorwise", "mxfp8"])
+def test_gradient_accumulation_fusion_adds_into_main_grad(mg, gpu, recipe):
+    """config.gradient_accumulation_fusion: the wgrad GEMM adds into weight.main_grad itself
+    (_fuse_wgrad_accum_pattern, primus_turbo.py:243-275: bf16 and tensor-wise FP8 in the reference; the MX
+    recipes with the switch turbo_fuse_wgrad_accum_mx).  Two microbatches; the sum equals the unfused run's."""
+    pt = mg
+    from primus_amd.megatron import runtime
+    from primus_amd.pytorch.core import Format, ScalingGranularity
+
+    runtime.set_num_microbatches(2)
+    qc = None
+    if recipe == "tensorwise":
+        qc = pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.TENSORWISE, format=Format.HYBRID)
+    elif recipe == "mxfp8":
+        qc = _mxfp8(pt)
+    res = {}
+    for fuse in (False, True):
+        runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                         turbo_grouped_gemm_without_padding=True, turbo_fuse_wgrad_accum_mx=True)
+        torch.manual_seed(31)
+        lin = pt.PrimusTurboLinear(256, 160, parallel_mode=None, config=_cfg(gradient_accumulation_fusion=fuse), bias=False,
+                                   skip_bias_add=False)
+        gl = pt.PrimusTurboColumnParallelGroupedLinear(3, 128, 96, config=_cfg(gradient_accumulation_fusion=fuse))
+        for p_ in (lin.weight, gl.weights):
+            p_.main_grad = torch.zeros_like(p_, dtype=torch.float32)
+        outs = []
+        calls = []
+        for mb in range(2):
+            for p_ in (lin.weight, gl.weights):
+                p_.grad_added_to_main_grad = False
+            x = torch.randn(16, 8, 256, device=gpu).bfloat16().requires_grad_()
+            dy = torch.randn(16, 8, 160, device=gpu).bfloat16()
+            xg = torch.randn(200, 128, device=gpu).bfloat16().requires_grad_()
+            dyg = torch.randn(200, 96, device=gpu).bfloat16()
+            if qc is not None:
+                ctx = pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc)
+            else:
+                import contextlib
+                ctx = contextlib.nullcontext()
+            with ctx:
+                assert (pt._fuse_wgrad_accum_pattern(lin.config, lin.weight) == "megatron") is fuse
+                y, _ = lin(x)
+                yg, _ = gl(xg, torch.tensor([70, 0, 130]))
+            y.backward(dy)
+            yg.backward(dyg)
+            assert lin.weight.grad_added_to_main_grad is (fuse or qc is not None)
+            outs += [y.detach(), x.grad, yg.detach(), xg.grad]
+        res[fuse] = (outs, lin.weight.main_grad.clone(), gl.weights.main_grad.clone(), lin.weight.grad, gl.weights.grad)
+    for a, b in zip(res[False][0], res[True][0]):
+        assert torch.equal(a, b)
+    if recipe == "bf16":     # outside an autocast the unfused run leaves the gradient in .grad (summed by autograd)
+        assert not res[False][1].any() and not res[False][2].any()
+        ref_lin, ref_gl = res[False][3].float(), res[False][4].float()
+    else:
+        ref_lin, ref_gl = res[False][1], res[False][2]
+    for ref, got in ((ref_lin, res[True][1]), (ref_gl, res[True][2])):
+        assert ref.abs().sum() > 0 and (ref - got).abs().max() <= 2.0 ** -6 * ref.abs().max()
+    assert not res[True][2][1].any()

@@ -439,6 +439,23 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         __syncthreads();
         const int m_valid = d.m_valid, n_valid = d.n_valid;
         uint16_t* ctile = p.c + d.c_off;
+        // ACCUM: the old float32 values of the first 32-row block are requested before the next tile's operand
+        // requests go out (memory returns in order per wave: behind them they would wait for 64 KiB of loads)
+        float* ctile32 = (float*)p.c + d.c_off;
+        const bool full_tile = (m_valid == BM) && (n_valid == BN);
+        v4f old[ACCUM ? 2 : 1][ACCUM ? 16 : 1];
+        auto fetch_old = [&](int i, v4f* dst) {
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int row = wm * 128 + i * 32 + 4 * u + (l >> 4), col = wn * 128 + (l & 15) * 4 + jj * 64;
+                    dst[jj * 8 + u] = v4f{0.f, 0.f, 0.f, 0.f};
+                    if (full_tile || (row < m_valid && col < n_valid))
+                        dst[jj * 8 + u] = *(const v4f*)(ctile32 + (int64_t)row * p.n + col);
+                }
+        };
+        if (ACCUM) fetch_old(0, old[0]);
         tile += nwg;
         // (past the last tile the requests are still sent, for the last tile again: nobody reads them)
         d = decode(tile < total_tiles ? tile : total_tiles - 1);
@@ -465,11 +482,14 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
             if (ACCUM) {
                 // float32 read-modify-write, 64 columns (256 bytes per row) of a 32-row block at a time through
-                // the same patch: a store instruction covers 4 rows x 256 contiguous bytes
-                float* ctile32 = (float*)p.c + (ctile - p.c);
+                // the same patch: a memory instruction covers 4 rows x 256 contiguous bytes.  The old values of
+                // a 32-row block (16 x 16 bytes per lane) are requested one block ahead, so their latency is
+                // covered by the staging and the stores of the block before.
                 uint8_t* wr32 = stg + lr * SP + 16 * g;
+                const int colq = wn * 128 + (l & 15) * 4;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    if (i + 1 < 4) fetch_old(i + 1, old[(i + 1) & 1]);
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
@@ -481,15 +501,12 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
                                 if (ALPHA) o *= alpha;
                                 *(v4f*)(wr32 + (jl * 32 + 8 * q) * 4) = o;
                             }
-                        const int col = wn * 128 + jj * 64 + (l & 15) * 4;
 #pragma unroll
                         for (int u = 0; u < 8; ++u) {
                             const v4f v = *(const v4f*)(rd + 4 * u * SP);
-                            const int row = wm * 128 + i * 32 + 4 * u + rr;
-                            if (full || (row < m_valid && col < n_valid)) {
-                                v4f* dst = (v4f*)(ctile32 + (int64_t)row * p.n + col);
-                                *dst = *dst + v;
-                            }
+                            const int row = wm * 128 + i * 32 + 4 * u + rr, col = colq + jj * 64;
+                            if (full || (row < m_valid && col < n_valid))
+                                *(v4f*)(ctile32 + (int64_t)row * p.n + col) = old[i & 1][jj * 8 + u] + v;
                         }
                     }
                     MXL_PIN;

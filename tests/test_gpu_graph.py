@@ -113,3 +113,59 @@ def test_dense_and_fused_activation_replay(gpu):
         torch.cuda.synchronize()
         for a, b in zip(got, want):
             assert _same(a, b), (new_lens, seed)
+
+
+@pytest.mark.parametrize("recipe", ["tensorwise", "mxfp8"])
+def test_tensorwise_norm_and_fused_accumulation_replay(gpu, recipe):
+    """The later additions under capture: the tensor-wise recipe (abs-max by atomics into a kernel-initialised
+    word), the RMSNorm folded into the quantiser and the wgrad that adds into a float32 main_grad."""
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import Float8QuantConfig, Format, ScalingGranularity
+
+    cfg = (Float8QuantConfig(format=Format.HYBRID, granularity=ScalingGranularity.TENSORWISE) if recipe == "tensorwise"
+           else _cfg(False))
+    G, n, k, rows = 3, 256, 256, 600
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(rows, k, generator=gen).bfloat16().to(gpu).requires_grad_()
+    nw = (1 + 0.1 * torch.randn(k, generator=gen)).bfloat16().to(gpu).requires_grad_()
+    w1 = (torch.randn(k, k, generator=gen) * 0.05).bfloat16().to(gpu).requires_grad_()
+    w2 = (torch.randn(G, n, k, generator=gen) * 0.05).bfloat16().to(gpu).requires_grad_()
+    dy = torch.randn(rows, n, generator=gen).bfloat16().to(gpu)
+    lens = torch.tensor([100, 0, 500], dtype=torch.int64, device=gpu)
+    w2.main_grad = torch.zeros(G, n, k, device=gpu)
+    w2.grad_added_to_main_grad = False
+
+    def step():
+        if recipe == "tensorwise":
+            h = turbo.ops.gemm_fp8(turbo.ops.rmsnorm(x, nw, 1e-5), w1, config=cfg)
+        else:
+            h = turbo.ops.rmsnorm_gemm_fp8(x, nw, 1e-5, w1, config=cfg)
+        y = turbo.ops.grouped_gemm_fp8(h, w2, lens, config=cfg, fuse_bgrad_accum_pattern="megatron")
+        return (y,) + torch.autograd.grad(y, [x, nw, w1, w2], dy)[:3]
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for new_lens, seed in [([100, 0, 500], 1), ([600, 0, 0], 2), ([1, 299, 300], 3)]:
+        g2 = torch.Generator().manual_seed(seed)
+        with torch.no_grad():
+            x.copy_(torch.randn(rows, k, generator=g2).bfloat16() * (seed * 3.0))     # the abs-max changes too
+            dy.copy_(torch.randn(rows, n, generator=g2).bfloat16())
+            lens.copy_(torch.tensor(new_lens, dtype=torch.int64))
+            w2.main_grad.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs] + [w2.main_grad.clone()]
+        with torch.no_grad():
+            w2.main_grad.zero_()
+        want = list(step()) + [w2.main_grad.clone()]
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert _same(a, b), (new_lens, seed)
+        assert got[-1].abs().sum() > 0

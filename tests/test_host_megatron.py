@@ -320,6 +320,15 @@ def test_fused_wgrad_accumulation_is_off_for_mx_and_fp4():
         assert pt._fuse_wgrad_accum_pattern(cfg, w) is None
     with pt.primus_turbo_fp8_autocast(enabled_turbo=True, turbo_quant_config=pt.PrimusTurboQuantConfig()):
         assert pt._fuse_wgrad_accum_pattern(cfg, w) == "megatron"  # tensorwise has the epilogue
+    # this package's wgrad kernel accumulates for the MX recipes too: opt-in switch
+    runtime.set_args(turbo_fuse_wgrad_accum_mx=True)
+    try:
+        with pt.primus_turbo_fp8_autocast(enabled_turbo=True, turbo_quant_config=_mxfp8()):
+            assert pt._fuse_wgrad_accum_pattern(cfg, w) == "megatron"
+        with pt.primus_turbo_fp4_autocast(enabled_turbo=True, turbo_quant_config=_mxfp4()):
+            assert pt._fuse_wgrad_accum_pattern(cfg, w) == "megatron"
+    finally:
+        runtime.set_args()
     bare = torch.nn.Parameter(torch.zeros(32, 32, dtype=torch.bfloat16))
     with pytest.raises(AssertionError):
         pt._fuse_wgrad_accum_pattern(cfg, bare)

@@ -54,7 +54,7 @@ WORKLOADS = {
 # step, each scaled by what the same counter reads for a 1 GiB -> 1 GiB elementwise kernel: 2.000 and
 # 1.000).  The counter summary is committed as profiles/bench_mixtral_mxfp8_hbm_traffic.txt.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "mixtral_8x7b_moe_mxfp8": (2835681.1 * 2.000 + 836700.1 * 1.000) * 1024,
+    "mixtral_8x7b_moe_mxfp8": (2802905.4 * 2.000 + 836113.3 * 1.000) * 1024,
 }
 
 

@@ -88,10 +88,11 @@ def _finish_wgrad(grad_b, accum, fused: bool, w_shape):
     if not fused:
         target.add_(grad_b.view(w_shape))
     owner.grad_added_to_main_grad = True
-    key = (tuple(w_shape), target.device)
+    dtype = getattr(owner, "dtype", torch.bfloat16)
+    key = (tuple(w_shape), dtype, target.device)
     dummy = _dummy_wgrads.get(key)
     if dummy is None:
-        dummy = torch.empty(tuple(w_shape), dtype=torch.bfloat16, device=target.device)
+        dummy = torch.empty(tuple(w_shape), dtype=dtype, device=target.device)
         _dummy_wgrads[key] = dummy
     return dummy
 

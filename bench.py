@@ -18,7 +18,7 @@ Prints ONE JSON line:  metric = grouped-GEMM algorithmic TFLOP/s of the whole
 step (2*M*N*K per GEMM over all six GEMMs, divided by the wall time of the
 step including every quantiser), plus a roofline object for the dominant
 kernel and a CPU baseline (the C restatement of the oracle, timed on the host
-cores on a 1/32 row sample).
+cores on a 1/16 row sample).
 """
 
 from __future__ import annotations
@@ -126,7 +126,7 @@ def quant_bytes(info):
     return el * (2.0 + copies * (code + 1.0 / 32.0))
 
 
-def cpu_baseline(spec, lens, sample_div=32):
+def cpu_baseline(spec, lens, sample_div=16):
     """The oracle's C restatement on the host cores, on 1/sample_div of the rows
     (same experts and weights shapes): quantise -> dequantise -> fp32 matmul
     (torch CPU) -> bf16, forward + dgrad + wgrad of both linears."""

@@ -81,3 +81,44 @@ def test_without_a_gfx950_device_the_entry_points_refuse(lib):
     assert lib.mxl_gemm_nt(p, p, 0, p, p, 0, p, 128, 128, 100, None) == -1                                 # k % 128
     assert lib.mxl_glu_probs_fwd(p, p, 0, None, 4, 32, 0, p, None) == -3
     assert lib.mxl_error_string(-3).decode().startswith("device")
+
+
+def test_newer_entry_points_validate_before_they_touch_the_device(lib):
+    """RMSNorm, tensor-wise scaling and the accumulating wgrad: malformed calls are MXL_EINVAL (-1), well-formed ones
+    MXL_ENODEV (-3) on a machine without a GPU."""
+    import torch
+
+    if torch.cuda.device_count() > 0:
+        pytest.skip("a GPU is present: the well-formed calls would be real launches")
+    buf = ctypes.create_string_buffer(256 * 256 * 4)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    f32 = ctypes.c_float
+    # RMSNorm
+    assert lib.mxl_rmsnorm_fwd(p, p, f32(1e-5), 4, 256, p, p, None) == -3
+    assert lib.mxl_rmsnorm_fwd(p, p, f32(1e-5), 4, 100, p, p, None) == -1            # k % 8
+    assert lib.mxl_rmsnorm_fwd(p, p, f32(1e-5), 4, 32768, p, p, None) == -1          # k > 16384
+    assert lib.mxl_rmsnorm_fwd(p, p, f32(-1.0), 4, 256, p, p, None) == -1            # eps < 0
+    assert lib.mxl_rmsnorm_fwd(p, None, f32(1e-5), 4, 256, p, p, None) == -1         # y without a weight
+    assert lib.mxl_rmsnorm_fwd(p, None, f32(1e-5), 0, 256, None, None, None) == 0    # no rows: nothing to do
+    assert lib.mxl_rmsnorm_bwd_workspace_bytes(4, 256) == 4 * 256 * 4
+    assert lib.mxl_rmsnorm_bwd_workspace_bytes(100000, 4096) == 1024 * 4096 * 4     # capped number of partial rows
+    assert lib.mxl_rmsnorm_bwd_workspace_bytes(4, 100) == -1
+    assert lib.mxl_rmsnorm_bwd(p, p, p, p, 4, 256, p, None, p, 4096, None) == -1     # no dw
+    assert lib.mxl_rmsnorm_quantize(p, None, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 0, None) == -1   # no weight
+    assert lib.mxl_rmsnorm_quantize(p, p, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 8, None) == -1      # unknown flag
+    assert lib.mxl_rmsnorm_quantize(p, p, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 0, None) == -3
+    # tensor-wise scaling
+    assert lib.mxl_amax(p, -1, p, None) == -1
+    assert lib.mxl_amax(p, 64, None, None) == -1
+    assert lib.mxl_amax(p, 64, p, None) == -3
+    assert lib.mxl_quantize_tensorwise(p, 128, 128, 128, _lib.FMT_E2M1, p, None, 0, p, p, None, None, p, 0, None) == -1   # FP8 only
+    assert lib.mxl_quantize_tensorwise(p, 128, 128, 128, _lib.FMT_E5M2, None, None, 0, p, p, None, None, p, 0, None) == -1  # no amax
+    assert lib.mxl_quantize_tensorwise(p, 128, 128, 128, _lib.FMT_E5M2, p, None, 0, p, p, None, None, p, 0, None) == -3
+    assert lib.mxl_quantize_weight_tensorwise(p, 1, 128, 128, 128, 128, 7, p, p, p, None, None, p, 0, None) == -1
+    # scaled GEMMs and the accumulating wgrad
+    assert lib.mxl_grouped_gemm_nt_scaled(p, p, 0, p, p, 0, p, None, 1, 128, 128, 128, None, p, 0, None) == -1    # one factor missing
+    assert lib.mxl_grouped_gemm_nt_scaled(p, p, 0, p, p, 0, p, None, 1, 128, 128, 128, p, p, 0, None) == -3
+    assert lib.mxl_grouped_gemm_nt_ex(p, p, _lib.FMT_E5M2, p, p, 0, p, None, 1, 128, 128, 128, 0, None) in (-1, -3)
+    assert lib.mxl_grouped_gemm_wgrad_ex(p, p, 0, p, p, 0, p, None, 0, 128, 128, 128, _lib.GF_ACCUM_F32, None) == -1   # needs KCHUNK
+    assert lib.mxl_grouped_gemm_wgrad_ex(p, p, 0, p, p, 0, p, None, 0, 128, 128, 128, 64, None) == -1                   # unknown flag
+    assert lib.mxl_grouped_gemm_wgrad_ex(p, p, 0, p, p, 0, p, None, 0, 128, 128, 128, _lib.GF_ACCUM_F32 | _lib.GF_KCHUNK, None) == -3

@@ -243,3 +243,66 @@ def test_full_size_mixtral_every_output_bit_exact(gpu):
         a, b = int(offs[g]), int(offs[g + 1])
         want = (dyf[a:b].T @ xf1[a:b]).bfloat16()
         assert torch.equal(dw[g], want), g
+
+
+def _chunk(codes):
+    """Row-major codes [rows, k] -> K-chunk-major [k / 128, rows, 128] (FP8: one byte per element)."""
+    rows, k = codes.shape
+    return codes.view(torch.uint8).reshape(rows, k // 128, 128).permute(1, 0, 2).contiguous().view(codes.dtype)
+
+
+def test_full_size_mixtral_chunked_scaled_and_accumulating_bit_exact(gpu):
+    """The same full-size case through the later kernel variants: K-chunk-major operands, the scaled GEMM
+    with E5M2 x E4M3 operands and per-tensor factors, and the wgrad that adds into a float32 buffer --
+    every output element exact (small-integer codes, power-of-two factors, integer buffer contents)."""
+    from primus_amd.pytorch import kernels as K
+
+    spec = bench.WORKLOADS["mixtral_8x7b_moe_mxfp8"]
+    lens = bench.route(spec)
+    G, M, k, n = spec["G"], sum(lens), spec["hidden"], spec["fc1_out"]
+    gen = torch.Generator(device=gpu).manual_seed(78)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    e5 = torch.tensor([0x00, 0x3C, 0x40, 0x42, 0x44, 0xBC, 0xC0, 0xC2], dtype=torch.uint8, device=gpu)   # 0, +-1, +-2, +-3, 4
+    e5val = torch.tensor([0.0, 1.0, 2.0, 3.0, 4.0, -1.0, -2.0, -3.0], device=gpu)
+
+    def unit(rows, cols):
+        return torch.full((rows, cols // 32), 127, dtype=torch.uint8, device=gpu).view(torch.float8_e8m0fnu)
+
+    # forward-shaped: a = E5M2 codes [M, k] (chunked), b = E4M3 weights [G, n, k] (chunked), factors 0.5 and 0.25
+    idx = torch.randint(0, 8, (M, k), generator=gen, device=gpu)
+    a_codes, af = e5[idx].view(torch.float8_e5m2), e5val[idx]
+    wq, _ = _exact_codes(gen, G * n, k, gpu)
+    wf = K.dequantize_mx_impl(wq, unit(G * n, k)).float().view(G, n, k)
+    sa, sb = torch.tensor([0.5], device=gpu), torch.tensor([0.25], device=gpu)
+    y = K.gemm_tw_nt_impl(_chunk(a_codes), unit(M, k), sa, _chunk(wq), unit(G * n, k).view(G, n, k // 32), sb, gl, kchunk=True)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        assert torch.equal(y[a:b], ((af[a:b] @ wf[g].T) * 0.125).bfloat16()), g
+    del y, wq, wf, idx
+
+    # wgrad-shaped, accumulating: buf[g] += dY_g^T . X_g for a 512-column slice of dY, MX entry point
+    W = K.padded_width(M, G)
+    _, poffs = o.segment_layout(lens)
+    nd = 512
+    dq, _ = _exact_codes(gen, M, nd, gpu)
+    xq, _ = _exact_codes(gen, M, k, gpu)
+
+    def transposed_chunked(codes_rows):
+        cols = codes_rows.shape[1]
+        qT = torch.zeros(cols, W, dtype=torch.uint8, device=gpu)
+        for g in range(G):
+            a, b, p = int(offs[g]), int(offs[g + 1]), int(poffs[g])
+            qT[:, p : p + (b - a)] = codes_rows.view(torch.uint8)[a:b].T
+        return _chunk(qT.view(torch.float8_e4m3fn)), unit(cols, W)
+
+    dyf = K.dequantize_mx_impl(dq, unit(M, nd)).float()
+    xf = K.dequantize_mx_impl(xq, unit(M, k)).float()
+    before = torch.randint(-1000, 1000, (G, nd, k), generator=gen, device=gpu).float()
+    buf = before.clone()
+    dqT, dsT = transposed_chunked(dq)
+    xqT, xsT = transposed_chunked(xq)
+    K.grouped_gemm_mx_wgrad_impl(dqT, dsT, xqT, xsT, gl, M, kchunk=True, accum_into=buf)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        assert torch.equal(buf[g], before[g] + dyf[a:b].T @ xf[a:b]), g

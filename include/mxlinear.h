@@ -102,6 +102,13 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
  *                  row-major layout.  The GEMM entry points take such operands with MXL_GF_KCHUNK.  This is
  *                  the role the reference's pre-shuffled layouts play for its kernels (use_preshuffle,
  *                  primus_turbo_mxfp4_local.py:184-198); the arrangement itself is this library's own.
+ *   MXL_QF_KSTEP   K-step-major layout of codes AND scales for both copies (FP8 formats only; excludes
+ *                  MXL_QF_KCHUNK): codes [ld / 64][rows][64] -- the 64 elements one MFMA K step consumes --
+ *                  and scales [ceil(ld / 512)][rows][16], i.e. the 16 scale bytes (8 K steps) of a row stay
+ *                  together and consecutive rows follow each other.  Every request of the ring GEMM kernel
+ *                  (MXL_GF_KSTEP) then reads whole consecutive cache lines: 64 rows of a K step are 4 KiB,
+ *                  the scales of 256 rows for 8 K steps are 4 KiB.  Needs row_ld % 128 == 0; a scale array
+ *                  holds ceil(ld / 512) * rows * 16 bytes (bytes past ld / 32 of a row are not written).
  *
  * and, for fmt = MXL_FMT_E2M1 only, the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
  * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288):
@@ -127,6 +134,7 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
 #define MXL_QF_SR 1u
 #define MXL_QF_RHT_COL 2u
 #define MXL_QF_KCHUNK 4u
+#define MXL_QF_KSTEP 8u
 int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                     const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                     void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);
@@ -192,6 +200,10 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * of a and num_groups * n rows of b in the forward / dgrad GEMM; n rows of a and k rows of b over the padded
  * token width in wgrad).  Scales stay row-major.  Same results bit for bit; an operand must stay below 4 GiB. */
 #define MXL_GF_KCHUNK 1u
+/* MXL_GF_KSTEP (instead of MXL_GF_KCHUNK): codes and scales of both operands are K-step-major, as written by the
+ * quantisers with MXL_QF_KSTEP.  FP8-format operands, at most 128 groups, bf16 output (no MXL_GF_ACCUM_F32);
+ * anything else returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit. */
+#define MXL_GF_KSTEP 4u
 /* mxl_grouped_gemm_wgrad_ex / _scaled only, together with MXL_GF_KCHUNK: c_bf16 points to FLOAT32 [g, n, k] and the
  * result is ADDED to it in fp32 (no rounding to bf16).  This is the gradient-accumulation fusion of the reference
  * (fuse_bgrad_accum_pattern = "megatron": the GEMM's beta = 1 epilogue adds into weight.main_grad,

@@ -85,6 +85,7 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, int64_t bytes) {
     return r;
 }
 __device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
+    asm volatile("" : "+s"(soff));   // the scalar offset has to sit in a register, also when it is a known constant
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_off), "v"(voff), "s"(rsrc), "s"(soff)
@@ -554,6 +555,445 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 #undef MXL_RD_B
 }
 
+// ---------------------------------------------------------------------------------------------------
+// 4-slot ring kernel (FP8-family operands in the K-step-major layout, at most RING_MAX_GROUPS groups).
+//
+// Same tiling, MFMA schedule and epilogue idea as mx_gemm_kernel; what differs is how operands travel:
+//   * a ring slot holds ONE MFMA K step (K = 64: 64-byte row pieces, 16 KiB per operand), four slots;
+//   * the 8 load rounds of K step s+4 go out during step s, one per two MFMAs (six after the step's
+//     barrier, the last two at the start of the next step), into the slot step s has just released:
+//     a request has between two and three K steps to land, and the request stream never pauses or bunches;
+//   * the wait in front of a step's barrier is partial: vmcnt(16) lets the requests of the two youngest
+//     steps stay in flight (loads return in order, so anything older has landed whatever else is pending);
+//   * the stream runs across tile boundaries: the last four steps of a tile request the first four steps of
+//     the workgroup's next tile.  Only the 6 requests that would overwrite the slot the epilogue stages its
+//     output in are held back until the epilogue has left it.
+// Measured on cache-shared operands with this discipline the MFMA pipe never waits for operands; with the
+// 2-slot ring of mx_gemm_kernel (one K = 128 slot in flight, everything waited for) it idles 12 % and more.
+// ---------------------------------------------------------------------------------------------------
+constexpr int RING_SLOTS = 4;
+constexpr int RING_STAGE = 2 * 256 * BK;          // both operands, K = 64, FP8: 32 KiB
+constexpr int RING_MAX_GROUPS = 128;
+constexpr int RING_PANEL = 256 * 16;              // scale panel of one operand: 16 bytes per row = 8 K steps
+constexpr int RING_PANEL_BUFS = 3;
+constexpr int RING_TBL = RING_MAX_GROUPS + 2;
+
+constexpr int ring_lds_bytes() {
+    return RING_SLOTS * RING_STAGE + RING_PANEL_BUFS * 2 * RING_PANEL + RING_TBL * 4 + RING_TBL * 8 + RING_TBL * 4;
+}
+
+template <int AFMT, int BFMT, int MODE, bool ALPHA>
+__global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
+    static_assert(AFMT != kFmtE2M1 && BFMT != kFmtE2M1, "FP8-family operands only");
+    constexpr int A_BYTES = 256 * BK;                 // 16 KiB
+    constexpr int STAGE = RING_STAGE;
+    constexpr int PANEL = RING_PANEL;
+    constexpr int CB = BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE5M2 ? 1 : 0;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* panels = smem + RING_SLOTS * STAGE;
+    int* pre_tiles = (int*)(panels + RING_PANEL_BUFS * 2 * PANEL);
+    int64_t* pre_rows = (int64_t*)(pre_tiles + RING_TBL);
+    int* pre_pan = (int*)(pre_rows + RING_TBL);                      // [G+1] prefix of scale panels (WGRAD)
+
+    const int t = threadIdx.x;
+    const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l = t & 63, lr = l & 31, g = l >> 5;
+    const int wm = w >> 1, wn = w & 1;
+    const int G = p.num_groups;
+    const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
+
+    // ---- per-workgroup group tables (as in mx_gemm_kernel, plus the scale-panel prefix) ----
+    for (int i = t; i < G; i += GTHREADS) pre_rows[i + 1] = p.group_lens ? p.group_lens[i] : p.total_m;
+    __syncthreads();
+    if (t == 0) {
+        int tiles = 0, pans = 0;
+        int64_t rows = 0;
+        const int64_t cap = (MODE == MODE_FWD) ? p.total_m : p.k;
+        pre_tiles[0] = 0;
+        pre_rows[0] = 0;
+        pre_pan[0] = 0;
+        for (int i = 0; i < G; ++i) {
+            int64_t len = pre_rows[i + 1];
+            len = len < 0 ? 0 : len;
+            if (MODE == MODE_FWD) {
+                len = len > cap - rows ? cap - rows : len;
+                tiles += (int)((len + BM - 1) / BM);
+                rows += len;
+            } else {
+                int64_t seg = (len + MXL_SEG_ALIGN - 1) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
+                seg = seg > cap - rows ? cap - rows : seg;
+                rows += seg;
+                pans += (int)((seg + 511) / 512);
+            }
+            pre_tiles[i + 1] = tiles;
+            pre_rows[i + 1] = rows;
+            pre_pan[i + 1] = pans;
+        }
+    }
+    __syncthreads();
+
+    const int tiles_n = (int)((p.n + BN - 1) / BN);
+    int tiles_m, total_tiles;
+    if (MODE == MODE_FWD) {
+        tiles_m = pre_tiles[G];
+        total_tiles = tiles_m * tiles_n;
+    } else {
+        tiles_m = (int)((p.m + BM - 1) / BM);
+        total_tiles = G * tiles_m * tiles_n;
+    }
+    const int nwg = gridDim.x;
+    const int per_xcd = nwg >> 3;
+    const int vwg = (nwg & 7) ? (int)blockIdx.x : ((int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3));
+
+    const int64_t a_rows_total = (MODE == MODE_FWD) ? p.total_m : p.m;
+    const int64_t b_rows_total = (MODE == MODE_FWD) ? (int64_t)G * p.n : p.n;
+    // K-step-major codes: [k / 64][rows][64]; scales: [ceil(k / 512)][rows][16] (16 bytes = 8 K steps of a row)
+    const uint32_t a_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * BK));
+    const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * BK));
+    const uint32_t a_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * 16));
+    const uint32_t b_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * 16));
+    // panels in a scale array: a contraction that is split into groups restarts its panels at every group
+    const int64_t n_panels = (p.k + 511) / 512 + ((MODE == MODE_WGRAD && p.group_lens) ? G + 1 : 0);
+    // a load round covers 64 consecutive rows = 4 KiB: thread -> (row t / 4, 16-byte piece t % 4); the XOR swizzle of
+    // the piece index is applied on the global side so that the LDS image (64-byte rows) reads without bank conflicts
+    const int ld_row = t >> 2;
+    const uint32_t ld_voff = (uint32_t)(ld_row * BK + 16 * ((t & 3) ^ ((ld_row >> 2) & 3)));
+    const uint32_t s_voff = (uint32_t)(t * 16);     // scale panel: row t of the tile, 16 bytes
+
+    struct Tile {
+        v4i ra, rb, rsa, rsb;
+        uint32_t ca0, cb0;         // byte offset of the first K step of each operand
+        uint32_t pa0, pb0;         // byte offset of the scale panel of the first K step
+        uint32_t cal, cbl;         // byte offset of the LAST K step of the contraction range (requests never pass it)
+        int nst, nst_real;         // K steps of 64 to run (>= 4, even) and how many of them multiply (2 or nst)
+        int m_valid, n_valid;
+        int64_t c_off;
+    };
+    auto decode = [&](int tile) __attribute__((always_inline)) {
+        Tile d;
+        int grp = 0, pid_m, pid_n;
+        int tl = tile;
+        if (MODE == MODE_WGRAD) {
+            grp = tl / (tiles_m * tiles_n);
+            tl -= grp * tiles_m * tiles_n;
+        }
+        {
+            const int width = GROUP_M * tiles_n;
+            const int gid = tl / width;
+            const int first = gid * GROUP_M;
+            const int gsz = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
+            pid_m = first + (tl % width) % gsz;
+            pid_n = (tl % width) / gsz;
+        }
+        int64_t a_row0, b_row0, c_row0, k0, k1;
+        if (MODE == MODE_FWD) {
+            int lo = 0, hi = G;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (pre_tiles[mid] <= pid_m) lo = mid; else hi = mid;
+            }
+            grp = lo;
+            const int64_t g_row0 = pre_rows[grp], g_rows = pre_rows[grp + 1] - g_row0;
+            const int64_t r = (int64_t)(pid_m - pre_tiles[grp]) * BM;
+            a_row0 = g_row0 + r;
+            d.m_valid = (g_rows - r) < BM ? (int)(g_rows - r) : BM;
+            b_row0 = (int64_t)grp * p.n + (int64_t)pid_n * BN;
+            c_row0 = a_row0;
+            k0 = 0;
+            k1 = p.k;
+        } else {
+            a_row0 = (int64_t)pid_m * BM;
+            d.m_valid = (p.m - a_row0) < BM ? (int)(p.m - a_row0) : BM;
+            b_row0 = (int64_t)pid_n * BN;
+            c_row0 = (int64_t)grp * p.m + a_row0;
+            k0 = pre_rows[grp];
+            k1 = pre_rows[grp + 1];
+        }
+        const int64_t n0 = (int64_t)pid_n * BN;
+        d.n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
+        d.c_off = c_row0 * p.n + n0;
+        const int nreal = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BK));   // even: the range is a multiple of 128
+        d.nst_real = nreal;
+        d.nst = nreal < 4 ? 4 : nreal;
+        // descriptors anchored at the tile's first row inside K step 0 / panel 0; readable up to the operand's end
+        d.ra = make_rsrc(p.a + a_row0 * BK, a_rows_total * p.k - a_row0 * BK);
+        d.rb = make_rsrc(p.b + b_row0 * BK, b_rows_total * p.k - b_row0 * BK);
+        d.rsa = make_rsrc(p.sa + a_row0 * 16, a_rows_total * n_panels * 16 - a_row0 * 16);
+        d.rsb = make_rsrc(p.sb + b_row0 * 16, b_rows_total * n_panels * 16 - b_row0 * 16);
+        const uint32_t st0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(k0 / BK));
+        d.ca0 = st0 * a_cstride;
+        d.cb0 = st0 * b_cstride;
+        d.cal = d.ca0 + (uint32_t)(nreal - 1) * a_cstride;
+        d.cbl = d.cb0 + (uint32_t)(nreal - 1) * b_cstride;
+        // scale panels restart at every group of a ragged contraction (wgrad): panel 0 of a tile is its group's first
+        const uint32_t pan0 = (MODE == MODE_WGRAD) ? (uint32_t)__builtin_amdgcn_readfirstlane(pre_pan[grp]) : 0u;
+        d.pa0 = pan0 * a_pstride;
+        d.pb0 = pan0 * b_pstride;
+        return d;
+    };
+
+    // ---- the request stream ----
+    // Requests are issued in K-step groups of 8 rounds (A rows 0-63, 64-127, 128-191, 192-255, then B likewise).
+    // lra / lrb: descriptors of the tile the stream is in; lca / lcb: byte offset of the K chunk the next group
+    // starts in; ga / gb: byte offset (chunk + half) of the group in flight.
+    v4i lra, lrb, crb;
+    uint32_t lca, lcb, lla, llb, ga = 0, gb = 0, cgb = 0;
+    auto stream_enter = [&](const Tile& d) __attribute__((always_inline)) {
+        lra = d.ra; lrb = d.rb; lca = d.ca0; lcb = d.cb0; lla = d.cal; llb = d.cbl;
+    };
+    // start the group of the stream's next K step: fixes ga / gb and moves the stream on.  A step past the tile's
+    // contraction range (a range of two steps is padded to four) requests the range's last step again: every
+    // request stays inside the operand, its data is never multiplied.
+    auto group_begin = [&]() __attribute__((always_inline)) {
+        ga = lca < lla ? lca : lla;
+        gb = lcb < llb ? lcb : llb;
+        lca += a_cstride;
+        lcb += b_cstride;
+        // rounds 6 and 7 of this group go out at the start of the next step, possibly after the stream has
+        // moved on to the next tile: they keep their own copy of the descriptor and offset
+        crb = lrb;
+        cgb = gb;
+    };
+    // round e (0 .. 7) of the group in flight into ring slot `slot` (0 .. 3, run time)
+    auto issue_e = [&](int e, uint32_t slot_base) __attribute__((always_inline)) {
+        if (e < 4) dma16(lra, slot_base + (uint32_t)((e * 4 + w) * 1024), ld_voff, ga + (uint32_t)(e * 64 * BK));
+        else if (e >= 6) dma16(crb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff, cgb + (uint32_t)((e - 4) * 64 * BK));
+        else dma16(lrb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff, gb + (uint32_t)((e - 4) * 64 * BK));
+    };
+    // scale panel pn of tile d (its K steps 8 pn .. 8 pn + 7) into panel buffer `buf`: 4 KiB per operand
+    auto issue_s = [&](const Tile& d, int pn, int buf) __attribute__((always_inline)) {
+        const uint32_t base = smem_base + (uint32_t)(RING_SLOTS * STAGE + buf * 2 * PANEL);
+        dma16(d.rsa, base + w * 1024, s_voff, d.pa0 + (uint32_t)pn * a_pstride);
+        dma16(d.rsb, base + PANEL + w * 1024, s_voff, d.pb0 + (uint32_t)pn * b_pstride);
+    };
+    auto next3 = [](int b) { return b == 2 ? 0 : b + 1; };
+
+#define MXL_MFMA(F, I, J) \
+    do { if (MF) acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I]); } while (0)
+#define MXL_PIN __builtin_amdgcn_sched_barrier(0)
+    // fragment (+ scale byte) reads of the K step in ring slot at `sn`, panel bytes at `pan`
+#define MXL_RD_A(F, I) \
+    do { const uint8_t* r_ = sn + a_frag + (I) * (32 * BK); \
+         const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
+         F.a[I][0] = lo_.x; F.a[I][1] = lo_.y; F.a[I][2] = lo_.z; F.a[I][3] = lo_.w; \
+         F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; \
+         F.sa[I] = pan[a_sc + (I) * (32 * 16)]; } while (0)
+#define MXL_RD_B(F, J) \
+    do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * BK); \
+         const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
+         F.b[J][0] = lo_.x; F.b[J][1] = lo_.y; F.b[J][2] = lo_.z; F.b[J][3] = lo_.w; \
+         F.b[J][4] = hi_.x; F.b[J][5] = hi_.y; F.b[J][6] = hi_.z; F.b[J][7] = hi_.w; \
+         F.sb[J] = pan[PANEL + b_sc + (J) * (32 * 16)]; } while (0)
+    // per-lane constants of the fragment reads: 64-byte rows, piece index XOR (row / 4) % 4
+    const int sw = (lr >> 2) & 3;
+    const int a_frag = (wm * 128 + lr) * BK, b_frag = (wn * 128 + lr) * BK;
+    const int a_lo = 16 * (g ^ sw), a_hi = 16 * ((2 + g) ^ sw);
+    const int a_sc = (wm * 128 + lr) * 16 + g, b_sc = (wn * 128 + lr) * 16 + g;
+
+    // The workgroup's tiles: vwg, vwg + nwg, ...  A tile whose contraction range is empty (wgrad of a group without
+    // tokens) never enters the pipeline: its output is zero-filled on the spot and the sequence moves on.
+    auto next_tile = [&](int tl) __attribute__((always_inline)) {
+        if (MODE == MODE_WGRAD) {
+            while (tl < total_tiles) {
+                const int grp = tl / (tiles_m * tiles_n);
+                if (pre_rows[grp + 1] > pre_rows[grp]) break;
+                const int rem = tl - grp * tiles_m * tiles_n;
+                const int width = GROUP_M * tiles_n;
+                const int first = (rem / width) * GROUP_M;
+                const int gsz = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
+                const int64_t row0 = (int64_t)(first + (rem % width) % gsz) * BM, col0 = (int64_t)((rem % width) / gsz) * BN;
+                uint16_t* ct = p.c + ((int64_t)grp * p.m + row0) * p.n + col0;
+                const int mv = (p.m - row0) < BM ? (int)(p.m - row0) : BM, nv = (p.n - col0) < BN ? (int)(p.n - col0) : BN;
+                for (int r = t >> 5; r < mv; r += GTHREADS / 32) {
+                    const int c = (t & 31) * 8;
+                    if (c < nv) store16_streaming((uint8_t*)(ct + (int64_t)r * p.n + c), make_uint4(0u, 0u, 0u, 0u));
+                }
+                tl += nwg;
+            }
+        }
+        return tl;
+    };
+    int tile = next_tile(vwg);
+    if (tile >= total_tiles) return;
+    int tile_n = next_tile(tile + nwg);
+    Tile d = decode(tile);
+    // past the last tile the stream requests the last tile's first steps again (nobody reads them)
+    Tile dn = decode(tile_n < total_tiles ? tile_n : tile);
+    int gs = 0;          // K steps run so far by this workgroup (ring slot of a step = its number & 3)
+    int pb_rd = 0;       // panel buffer of the scales being read
+    int pb_is = 0;       // panel buffer of the most recent panel request
+    // prologue: panel 0 and K steps 0, 1, 2 of the first tile, and the first six rounds of step 3
+    stream_enter(d);
+    issue_s(d, 0, 0);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        group_begin();
+#pragma unroll
+        for (int e = 0; e < (s < 3 ? 8 : 6); ++e) issue_e(e, smem_base + (uint32_t)(s * STAGE));
+    }
+    wait_vm<22>();       // everything up to K step 0 has landed
+    __syncthreads();
+
+    while (true) {
+        v16f acc[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        Frags f0, f1;
+        const int nst = d.nst, nst_real = d.nst_real;
+        {   // fragments of K step 0
+            const uint8_t* sn = smem + (gs & 3) * STAGE;
+            const uint8_t* pan = panels + pb_rd * 2 * PANEL;
+            MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
+            MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
+        }
+        // One K step s (local number, parity PAR) of 16 MFMAs.  MF: multiply (false for the padding steps of a
+        // tile whose contraction range is shorter than four steps).  LAST: the tile's last step; the six rounds
+        // that would go into the slot the epilogue is about to use are issued after the epilogue instead.
+        auto kstep = [&](auto par_tag, auto mf_tag, auto last_tag, int s, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
+            constexpr int PAR = decltype(par_tag)::value;
+            constexpr bool MF = decltype(mf_tag)::value;
+            constexpr bool LAST = decltype(last_tag)::value;
+            const uint32_t slot_prev = smem_base + (uint32_t)(((gs + 3) & 3) * STAGE);   // group of step gs + 3
+            const uint32_t slot_new = smem_base + (uint32_t)((gs & 3) * STAGE);          // group of step gs + 4
+            MXL_MFMA(cur, 0, 0); issue_e(6, slot_prev); MXL_PIN;
+            MXL_MFMA(cur, 1, 0); MXL_PIN;
+            MXL_MFMA(cur, 2, 0); issue_e(7, slot_prev); MXL_PIN;
+            MXL_MFMA(cur, 3, 0); MXL_PIN;
+            wait_vm<16>();       // the group of step gs + 1 has landed (two younger groups may be in flight)
+            __syncthreads();
+            MXL_PIN;
+            // bookkeeping between the barrier and the first read: panel of the next step, stream hand-over
+            const int s1 = s + 1;
+            pb_rd = ((s1 & 7) == 0 && s1 < nst) ? next3(pb_rd) : pb_rd;
+            if (!LAST) group_begin();
+            const uint8_t* sn = smem + ((gs + 1) & 3) * STAGE;
+            const uint8_t* pan = panels + pb_rd * 2 * PANEL + 2 * (s1 & 7);
+            MXL_PIN;
+            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(0, slot_new); MXL_PIN;
+            MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1);  MXL_PIN;
+            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1);  if (!LAST) issue_e(1, slot_new); MXL_PIN;
+            MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1);  MXL_PIN;
+            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2);  if (!LAST) issue_e(2, slot_new); MXL_PIN;
+            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2);  MXL_PIN;
+            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(3, slot_new); MXL_PIN;
+            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2);  MXL_PIN;
+            MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(4, slot_new); MXL_PIN;
+            MXL_MFMA(cur, 1, 3); MXL_PIN;
+            MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(5, slot_new); MXL_PIN;
+            MXL_MFMA(cur, 3, 3); MXL_PIN;
+            ++gs;
+        };
+        using P0 = std::integral_constant<int, 0>;
+        using P1 = std::integral_constant<int, 1>;
+        using Yes = std::integral_constant<bool, true>;
+        using No = std::integral_constant<bool, false>;
+        if (nst_real >= 4) {
+            for (int s = 0; s < nst - 2; s += 2) {
+                if (s == nst - 4) {
+                    // the request stream moves on to the workgroup's next tile: its scale panel 0 first
+                    pb_is = next3(pb_is);
+                    issue_s(dn, 0, pb_is);
+                    stream_enter(dn);
+                } else if ((s & 7) == 4 && s + 4 < nst) {
+                    // this tile's next scale panel (K steps s + 4 ...): first read three barriers from here
+                    pb_is = next3(pb_is);
+                    issue_s(d, (s >> 3) + 1, pb_is);
+                }
+                kstep(P0{}, Yes{}, No{}, s, f0, f1);
+                kstep(P1{}, Yes{}, No{}, s + 1, f1, f0);
+            }
+            kstep(P0{}, Yes{}, No{}, nst - 2, f0, f1);
+            kstep(P1{}, Yes{}, Yes{}, nst - 1, f1, f0);
+        } else {
+            // a contraction range of two steps: four steps run, the last two without multiplying
+            pb_is = next3(pb_is);
+            issue_s(dn, 0, pb_is);
+            stream_enter(dn);
+            kstep(P0{}, Yes{}, No{}, 0, f0, f1);
+            kstep(P1{}, Yes{}, No{}, 1, f1, f0);
+            kstep(P0{}, No{}, No{}, 2, f0, f1);
+            kstep(P1{}, No{}, Yes{}, 3, f1, f0);
+        }
+        // K step 0 of the next tile (and its scale panel) has landed; every wave is done reading the ring
+        wait_vm<16>();
+        __syncthreads();
+        MXL_PIN;
+
+        // ---- epilogue: fp32 -> bf16 through a wave-private LDS patch of 32 rows x 128 bytes in the ring slot of
+        // the step that has just finished, so that the global stores are 16 bytes per lane, 8 rows x 128
+        // contiguous bytes per instruction.  The patch is not padded (the four patches fill half a slot);
+        // 16-byte pieces are XOR-swizzled by (row / 2) % 8 and the 8-byte halves swapped in rows 16-31:
+        // conflict-free for the 8-byte writes (a lane owns a row) and the 16-byte reads (8 lanes per row).
+        {
+            const int m_valid = d.m_valid, n_valid = d.n_valid;
+            uint16_t* ctile = p.c + d.c_off;
+            uint8_t* stg = smem + ((gs + 3) & 3) * STAGE + w * (32 * 128);
+            uint8_t* wr = stg + lr * 128 + 8 * (g ^ (lr >> 4));
+            const int wsw = (lr >> 1) & 7;
+            const int rrow = l >> 3, rch = l & 7;
+            // rows 8u + rrow: (row / 2) % 8 = (4 (u & 1) + rrow / 2) % 8
+            const uint8_t* rd0 = stg + rrow * 128 + 16 * (rch ^ (rrow >> 1));
+            const uint8_t* rd1 = stg + rrow * 128 + 16 * (rch ^ (4 + (rrow >> 1)));
+            const bool full = (m_valid == BM) && (n_valid == BN);
+            float alpha = 1.f;
+            if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int jh = 0; jh < 2; ++jh) {
+#pragma unroll
+                    for (int jl = 0; jl < 2; ++jl)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int j = 2 * jh + jl;
+                            if (ALPHA) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] *= alpha;
+                            }
+                            v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
+                                      (__bf16)acc[i][j][4 * q + 3]};
+                            *(v4bf*)(wr + 16 * ((4 * jl + q) ^ wsw)) = o;
+                        }
+                    uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32 + rrow) * p.n + wn * 128 + jh * 64 + rch * 8);
+                    const int cc = wn * 128 + jh * 64 + rch * 8;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        uint4 v = *(const uint4*)(((u & 1) ? rd1 : rd0) + u * (8 * 128));
+                        if (u >= 2) v = make_uint4(v.z, v.w, v.x, v.y);
+                        if (full || (wm * 128 + i * 32 + 8 * u + rrow < m_valid && cc < n_valid))
+                            store16_streaming(rowbase + (int64_t)(8 * u) * p.n * 2, v);
+                    }
+                }
+                MXL_PIN;
+            }
+        }
+        if (tile_n >= total_tiles) break;
+        __syncthreads();      // every wave has left the patch: its slot takes K step 3 of the next tile
+        // (the stream entered the next tile four steps ago; the group of its step 3 begins here)
+        group_begin();
+        {
+            const uint32_t slot_new = smem_base + (uint32_t)(((gs + 3) & 3) * STAGE);
+#pragma unroll
+            for (int e = 0; e < 6; ++e) issue_e(e, slot_new);
+        }
+        d = dn;
+        tile = tile_n;
+        tile_n = next_tile(tile + nwg);
+        dn = decode(tile_n < total_tiles ? tile_n : tile);
+        pb_rd = next3(pb_rd);
+        MXL_PIN;
+    }
+    wait_vm<0>();   // nothing may still be writing this workgroup's LDS when it ends
+#undef MXL_MFMA
+#undef MXL_PIN
+#undef MXL_RD_A
+#undef MXL_RD_B
+}
+
 constexpr int gemm_lds_bytes(int afmt, int bfmt) {
     return NSLOT * (256 * (afmt == kFmtE2M1 ? BKP / 2 : BKP) + 256 * (bfmt == kFmtE2M1 ? BKP / 2 : BKP)) + 4 * 256 * 16 +
            (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
@@ -596,6 +1036,41 @@ static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
+template <int AFMT, int BFMT, int MODE, bool ALPHA>
+static int launch_gemm_ring(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    constexpr int lds = ring_lds_bytes();
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    static std::atomic<bool> attr_set[64];
+    const int slot = current_device_slot();
+    auto kern = mx_gemm_ring_kernel<AFMT, BFMT, MODE, ALPHA>;
+    if (!attr_set[slot].load(std::memory_order_acquire)) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+            return MXL_ELAUNCH;
+        attr_set[slot].store(true, std::memory_order_release);
+    }
+    int64_t grid = num_cus(slot);
+    if (max_tiles < grid) grid = max_tiles;
+    if (grid <= 0) return MXL_OK;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(GTHREADS), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
+
+// The 4-slot ring kernel serves FP8-family operands in the K-step-major layout with at most RING_MAX_GROUPS groups.
+template <int MODE>
+static bool ring_serves(int afmt, int bfmt, const GemmArgs& a) {
+    if (a.num_groups > RING_MAX_GROUPS) return false;
+    if (a.alpha_a != nullptr) return bfmt == MXL_FMT_E4M3 && (afmt == MXL_FMT_E4M3 || afmt == MXL_FMT_E5M2);
+    return afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3;
+}
+template <int MODE>
+static int dispatch_gemm_ring(int afmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    if (a.alpha_a != nullptr) {
+        if (afmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
+        return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
+    }
+    return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, false>(a, max_tiles, st);
+}
+
 template <int MODE, int LAYOUT>
 static int dispatch_gemm_l(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, LAYOUT>(a, max_tiles, st);
@@ -632,9 +1107,17 @@ static int dispatch_wgrad_accum(int afmt, int bfmt, const GemmArgs& a, int64_t m
 }
 
 // a_rows / b_rows: rows of the whole operands (for the 4 GiB bound of the chunk-major layout)
+// layout: 0 row-major codes, 1 K-chunk-major codes, 2 K-step-major codes and scales
 template <int MODE>
-static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, bool kchunk, int64_t a_rows, int64_t b_rows,
+static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, int layout, int64_t a_rows, int64_t b_rows,
                          hipStream_t st, bool accum = false) {
+    const bool kchunk = layout == 1;
+    if (layout == 2) {
+        if (accum || !ring_serves<MODE>(afmt, bfmt, a)) return MXL_EINVAL;
+        // offsets inside an operand are 32-bit
+        if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
+        return dispatch_gemm_ring<MODE>(afmt, a, max_tiles, st);
+    }
     if (accum) {
         if (MODE != MODE_WGRAD || !kchunk) return MXL_EINVAL;
         if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
@@ -664,7 +1147,8 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t w
 static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes, const void* b_scales,
                            int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
                            int64_t k, const float* alpha_a, const float* alpha_b, uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)MXL_GF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP)) return MXL_EINVAL;
+    if ((flags & MXL_GF_KCHUNK) && (flags & MXL_GF_KSTEP)) return MXL_EINVAL;
     if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
     if (k > MAX_CONTRACTION) return MXL_EINVAL;   // tile-relative byte offsets are 32-bit
@@ -687,7 +1171,7 @@ static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt,
     a.alpha_a = alpha_a;
     a.alpha_b = alpha_b;
     const int64_t max_tiles = (total_m / BM + num_groups) * ((n + BN - 1) / BN);
-    return dispatch_gemm<MODE_FWD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, total_m,
+    return dispatch_gemm<MODE_FWD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KSTEP) ? 2 : (flags & MXL_GF_KCHUNK) ? 1 : 0, total_m,
                                    (int64_t)num_groups * n, (hipStream_t)stream);
 }
 
@@ -724,7 +1208,8 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
                               const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups,
                               int64_t total_m, int64_t n, int64_t k, const float* alpha_a, const float* alpha_b,
                               uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_ACCUM_F32)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP | MXL_GF_ACCUM_F32)) return MXL_EINVAL;
+    if ((flags & MXL_GF_KCHUNK) && (flags & MXL_GF_KSTEP)) return MXL_EINVAL;
     const bool accum = (flags & MXL_GF_ACCUM_F32) != 0;
     if (accum && !(flags & MXL_GF_KCHUNK)) return MXL_EINVAL;
     if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
@@ -766,7 +1251,8 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
     a.alpha_a = alpha_a;
     a.alpha_b = alpha_b;
     const int64_t max_tiles = (int64_t)G * ((n + BM - 1) / BM) * ((k + BN - 1) / BN);
-    return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KCHUNK) != 0, n, k, (hipStream_t)stream, accum);
+    return dispatch_gemm<MODE_WGRAD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KSTEP) ? 2 : (flags & MXL_GF_KCHUNK) ? 1 : 0, n, k,
+                                     (hipStream_t)stream, accum);
 }
 
 extern "C" int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,

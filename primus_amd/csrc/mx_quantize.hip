@@ -76,6 +76,7 @@ struct QuantArgs {
     // the 128 elements of a row that one GEMM K slot consumes stay together and consecutive rows follow
     // each other, so a GEMM tile's slot is one contiguous block and this kernel writes 128 x 128-element
     // pieces contiguously.  chunk_rows_row / chunk_rows_col: rows of the whole row-wise / transposed operand.
+    // 2: K-step-major (FP8 only): codes [ld / 64][rows][64], scales [ceil(ld / 512)][rows][16].
     int kchunk;
     int64_t chunk_rows_row, chunk_rows_col;
     uint64_t sr_seed;       // SR kernels: seed of the stochastic rounding
@@ -156,6 +157,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     int64_t src_row0 = 0;
     int rows_valid = 0;
     int64_t batch_off_rows = 0;  // TWOD: first row of this matrix in the flattened input
+    // K-step-major scales of a grouped transposed copy: the 16-byte scale panels restart at every group
+    int64_t seg_pan0 = 0;        // panels of the groups in front of this tile's group
+    int seg_tile = -1;           // this tile's number inside its group's padded segment (-1: not grouped)
     if (TWOD) {
         // grid.x enumerates (matrix, row tile); matrices are independent.
         const int tiles_per_mat = (int)((a.mat_rows + QT - 1) / QT);
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         int64_t rem = a.rows - src_row0;
         rows_valid = rem <= 0 ? 0 : (rem < QT ? (int)rem : QT);
     } else {
-        int64_t off = 0;
+        int64_t off = 0, ppo = 0;
         int pto = 0;
         for (int g = 0; g < a.num_groups; ++g) {
             // clamped to the rows that exist, so that lens which do not match the buffer cannot read outside it
@@ -180,10 +184,17 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                 const int64_t r = (int64_t)(pt - pto) * QT;
                 src_row0 = off + r;
                 rows_valid = (len - r) < QT ? (int)(len - r) : QT;
+                seg_pan0 = ppo;
+                seg_tile = pt - pto;
                 break;
             }
             off += len;
             pto += nt;
+            ppo += (nt + 3) / 4;
+        }
+        if (seg_tile < 0) {   // a padding tile behind the last group: its scales go behind the last group's panels
+            seg_pan0 = ppo;
+            seg_tile = pt - pto;
         }
     }
 
@@ -298,8 +309,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o.y = nonfinite4_e4m3(d[it].z, d[it].w);
                 }
                 if (out_ok && r < rows_valid) {
-                    const int64_t at = a.kchunk ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
-                                                : (src_row0 + r) * a.row_ld + col;
+                    const int64_t at = a.kchunk == 2 ? ((int64_t)(2 * ct + (c16 >> 3)) * a.chunk_rows_row + src_row0 + r) * (QT / 2) + 8 * (c16 & 7)
+                                     : a.kchunk  ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
+                                                 : (src_row0 + r) * a.row_ld + col;
                     store8_streaming(a.q_row + at, o);
                 }
             } else {
@@ -437,7 +449,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         const int64_t nb = (a.row_ld - col0) / 32;  // valid blocks in this tile row
         uint8_t* dst = a.s_row + (src_row0 + t) * sld + col0 / 32;
         const uint32_t v = srow_tile[t];
-        if (nb >= 4 && (sld & 3) == 0) {
+        if (a.kchunk == 2) {
+            *(uint32_t*)(a.s_row + ((int64_t)(ct >> 2) * a.chunk_rows_row + src_row0 + t) * 16 + (ct & 3) * 4) = v;
+        } else if (nb >= 4 && (sld & 3) == 0) {
             *(uint32_t*)dst = v;
         } else {
             for (int b = 0; b < 4 && b < nb; ++b) dst[b] = (uint8_t)(v >> (8 * b));
@@ -450,7 +464,10 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             uint8_t* dst = a.s_colT + (out_rows_base + col0 + t) * (a.W / 32) + m0 / 32;
             const uint32_t v = scol_tile[t];
             const int64_t nb = (a.W - m0) / 32;
-            if (nb >= 4 && ((a.W / 32) & 3) == 0) {
+            if (a.kchunk == 2) {
+                const int64_t mt = seg_tile >= 0 ? (int64_t)seg_tile : m0 / QT;
+                *(uint32_t*)(a.s_colT + ((seg_pan0 + mt / 4) * a.chunk_rows_col + out_rows_base + col0 + t) * 16 + (mt & 3) * 4) = v;
+            } else if (nb >= 4 && ((a.W / 32) & 3) == 0) {
                 *(uint32_t*)dst = v;
             } else {
                 for (int b = 0; b < 4 && b < nb; ++b) dst[b] = (uint8_t)(v >> (8 * b));
@@ -467,8 +484,10 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             const int ch = t % LPR;
             if (col0 + c < a.cols && 16 * ch < avail) {
                 const uint4 v = *(const uint4*)(t_tile + c * TPITCH + 16 * ch);
-                const int64_t at = a.kchunk ? ((m0 / QT) * a.chunk_rows_col + out_rows_base + col0 + c) * ROWB + 16 * ch
-                                            : (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch;
+                const int64_t at = (!FP4 && a.kchunk == 2)
+                                       ? ((2 * (m0 / QT) + (ch >> 2)) * a.chunk_rows_col + out_rows_base + col0 + c) * (QT / 2) + 16 * (ch & 3)
+                                   : a.kchunk ? ((m0 / QT) * a.chunk_rows_col + out_rows_base + col0 + c) * ROWB + 16 * ch
+                                              : (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch;
                 store16_streaming(a.q_colT + at, v);
             }
         }
@@ -637,13 +656,20 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
     return (total_rows + (int64_t)(MXL_SEG_ALIGN - 1) * num_groups) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
 }
 
+// code layout selected by the flags: 0 row-major, 1 K-chunk-major, 2 K-step-major, -1 both requested
+static int qf_layout(uint32_t flags) {
+    if ((flags & MXL_QF_KCHUNK) && (flags & MXL_QF_KSTEP)) return -1;
+    return (flags & MXL_QF_KSTEP) ? 2 : (flags & MXL_QF_KCHUNK) ? 1 : 0;
+}
+
 static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                        const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT, void* s_colT,
                        int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
                        bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0,
-                       bool kchunk = false, const void* norm_w = nullptr, const void* tensor_amax = nullptr,
+                       int kchunk = 0, const void* norm_w = nullptr, const void* tensor_amax = nullptr,
                        void* scale_inv_out = nullptr) {
     if (row_ld == 0) row_ld = cols;
+    if (kchunk < 0 || (kchunk == 2 && fmt == MXL_FMT_E2M1)) return MXL_EINVAL;   // both layout flags; K-step-major is FP8 only
     if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
     if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
     if (rht && !q_colT) return MXL_EINVAL;   // the transform belongs to the transposed copy
@@ -673,7 +699,7 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.scale_inv_out = (float*)scale_inv_out;
     a.sr_seed = sr_seed;
     a.rht_signs = rht_signs & 0xFFFFu;
-    a.kchunk = kchunk ? 1 : 0;
+    a.kchunk = kchunk;
     a.chunk_rows_row = rows;
     a.chunk_rows_col = cols;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
@@ -703,10 +729,10 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
 extern "C" int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                                const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                                void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream) {
-    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT,
                        s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, (flags & MXL_QF_SR) != 0, sr_seed,
-                       (flags & MXL_QF_RHT_COL) != 0, rht_signs, (flags & MXL_QF_KCHUNK) != 0);
+                       (flags & MXL_QF_RHT_COL) != 0, rht_signs, qf_layout(flags));
 }
 
 extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
@@ -716,26 +742,27 @@ extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int
     if (act != MXL_ACT_SILU && act != MXL_ACT_GELU) return MXL_EINVAL;
     if (probs_dtype != MXL_PROBS_F32 && probs_dtype != MXL_PROBS_BF16) return MXL_EINVAL;
     if (rows > 0 && !probs) return MXL_EINVAL;
-    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, f, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT, act,
-                       probs, probs_dtype, row_mask, stream, false, 0, false, 0, (flags & MXL_QF_KCHUNK) != 0);
+                       probs, probs_dtype, row_mask, stream, false, 0, false, 0, qf_layout(flags));
 }
 
 extern "C" int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows, int64_t k,
                                     int64_t row_ld, int fmt, int scale_mode, const int64_t* group_lens, int num_groups,
                                     void* q_row, void* s_row, void* q_colT, void* s_colT, uint32_t flags, void* stream) {
     if (!w_bf16 || (rows > 0 && !rstd_f32)) return MXL_EINVAL;
-    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, k, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
                        PRO_RMSNORM, rstd_f32, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
-                       (flags & MXL_QF_KCHUNK) != 0, w_bf16);
+                       qf_layout(flags), w_bf16);
 }
 
 static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld, int64_t n_ld, int fmt,
-                              int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT, bool kchunk,
+                              int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT, int kchunk,
                               void* stream, const void* tensor_amax = nullptr, void* scale_inv_out = nullptr) {
     if (k_ld == 0) k_ld = k;
     if (n_ld == 0) n_ld = n;
+    if (kchunk < 0 || (kchunk == 2 && fmt == MXL_FMT_E2M1)) return MXL_EINVAL;
     if (kchunk && ((q_row && k_ld % QT != 0) || (q_colT && n_ld % QT != 0))) return MXL_EINVAL;   // whole chunks
     if (k_ld < k || n_ld < n || k_ld % MXL_BLOCK != 0 || n_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if (n_ld > (n + QT - 1) / QT * QT) return MXL_EINVAL;  // padding of the transposed copy stays inside the last tile
@@ -763,7 +790,7 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
     a.scale_inv_out = (float*)scale_inv_out;
     a.sr_seed = 0;
     a.rht_signs = 0;
-    a.kchunk = kchunk ? 1 : 0;
+    a.kchunk = kchunk;
     a.chunk_rows_row = batch * n;   // the batch is one operand of batch * n rows (resp. batch * k for the transposed copy)
     a.chunk_rows_col = batch * k;
     const int64_t gx = batch * ((n + QT - 1) / QT);
@@ -781,9 +808,9 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
 extern "C" int mxl_quantize_weight_2d_ex(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
                                          int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
                                          void* s_colT, uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, scale_mode, q_row, s_row, q_colT, s_colT,
-                              (flags & MXL_QF_KCHUNK) != 0, stream);
+                              qf_layout(flags), stream);
 }
 
 extern "C" int mxl_quantize_tensorwise(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt,
@@ -791,10 +818,10 @@ extern "C" int mxl_quantize_tensorwise(const void* x_bf16, int64_t rows, int64_t
                                        void* s_row, void* q_colT, void* s_colT, void* scale_inv_f32, uint32_t flags,
                                        void* stream) {
     if (!amax_f32 || (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
-    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, cols, row_ld, fmt, MXL_SCALE_OCP_FLOOR, group_lens, num_groups, q_row, s_row, q_colT,
                        s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
-                       (flags & MXL_QF_KCHUNK) != 0, nullptr, amax_f32, scale_inv_f32);
+                       qf_layout(flags), nullptr, amax_f32, scale_inv_f32);
 }
 
 extern "C" int mxl_quantize_weight_tensorwise(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
@@ -802,9 +829,9 @@ extern "C" int mxl_quantize_weight_tensorwise(const void* w_bf16, int64_t batch,
                                               void* q_colT, void* s_colT, void* scale_inv_f32, uint32_t flags,
                                               void* stream) {
     if (!amax_f32 || (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
-    if (flags & ~(uint32_t)MXL_QF_KCHUNK) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, MXL_SCALE_OCP_FLOOR, q_row, s_row, q_colT, s_colT,
-                              (flags & MXL_QF_KCHUNK) != 0, stream, amax_f32, scale_inv_f32);
+                              qf_layout(flags), stream, amax_f32, scale_inv_f32);
 }
 
 extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,

@@ -68,7 +68,7 @@ class QuantizedTensor(torch.Tensor):
         # tensor-wise scaled payload: float32 reciprocal scale of the whole tensor (one element, on the device);
         # ``scales`` then holds unit E8M0 bytes, which only make the codes acceptable to the GEMM kernels
         self._tensor_scale_inv = tensor_scale_inv
-        self._kchunk = bool(kchunk)
+        self._kchunk = 2 if (kchunk == 2 and kchunk is not True) else int(bool(kchunk))
         self._codes = codes
         self._scales = scales
         self._axis = axis
@@ -95,7 +95,8 @@ class QuantizedTensor(torch.Tensor):
         return self._use_2d_block
 
     @property
-    def kchunk(self) -> bool:
+    def kchunk(self) -> int:
+        """Storage layout: 0 row-major, 1 K-chunk-major codes, 2 K-step-major codes and scales."""
         return self._kchunk
 
     @property
@@ -108,6 +109,16 @@ class QuantizedTensor(torch.Tensor):
             return self._codes
         flat = K.unchunk(self._codes)
         return flat.view(tuple(self.shape[:-1]) + (flat.shape[-1],))
+
+    def rowmajor_scales(self) -> torch.Tensor:
+        """The scales as ``[..., rows, ld / 32]`` whatever layout they are stored in (a copy if K-step-major)."""
+        if self._kchunk != 2:
+            return self._scales
+        if self._segment_lens is not None:
+            raise NotImplementedError("row-major scales of a K-step-major copy that is split into groups")
+        blocks = self._codes.shape[0] * self._codes.shape[2] // _lib.BLOCK
+        flat = K.unpanel(self._scales.view(torch.uint8), blocks).view(self._scales.dtype)
+        return flat.view(tuple(self.shape[:-1]) + (blocks,))
 
     @property
     def fmt(self) -> int:
@@ -207,7 +218,7 @@ class QuantizedTensor(torch.Tensor):
     def dequantize(self) -> torch.Tensor:
         """Back to the original dtype in the payload's orientation.  For a
         transposed copy of ``rows`` tokens the padding columns are dropped."""
-        out = K.dequantize_mx_impl(self.rowmajor_codes(), self._scales, self.dtype)
+        out = K.dequantize_mx_impl(self.rowmajor_codes(), self.rowmajor_scales(), self.dtype)
         if self._tensor_scale_inv is not None:
             out = (out.float() * self._tensor_scale_inv).to(self.dtype)   # FP8 values are exact in bf16: one rounding
         if self._axis == -2 and not self._use_2d_block and self._segment_lens is not None:
@@ -268,8 +279,8 @@ def create_quantized_weight(
                                   tensor_scale_inv=si)
         return row, col
     if kchunk is None:
-        kchunk = K.kchunk_default() and K.kchunk_fits(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1,
-                                                      w.shape[-2], w.shape[-1])
+        kchunk = K.pick_layout(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1, w.shape[-2], w.shape[-1],
+                               fp8=fmt != _lib.FMT_E2M1)
     q_row, s_row, q_col, s_col = K.quantize_mx_weight_2d_impl(
         w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN,
         kchunk=kchunk,

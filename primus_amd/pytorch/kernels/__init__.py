@@ -80,10 +80,62 @@ def _round_up(x: int, m: int) -> int:
 
 
 KCHUNK = 128   # elements of a row that stay together in the K-chunk-major code layout (one GEMM K slot)
+KSTEP = 64     # ... in the K-step-major layout (one MFMA K step); its scales travel in 16-byte panels (512 elements)
+PANEL = 512
+
+# Storage layouts of quantised operands, the value of the ``kchunk`` arguments below:
+#   0 / False  row-major codes [rows, ld] and scales [rows, ld / 32]
+#   1 / True   K-chunk-major codes [ld / 128, rows, 128 elements], row-major scales
+#   2          K-step-major codes [ld / 64, rows, 64] and scales [panels, rows, 16] (FP8 formats only): what the
+#              ring GEMM kernel reads; a transposed copy that is split into groups has its scale panels restart
+#              at every group (ceil(ld / 512) + groups + 1 panels are allocated)
+LAYOUT_ROWMAJOR, LAYOUT_KCHUNK, LAYOUT_KSTEP = 0, 1, 2
+RING_MAX_GROUPS = 128   # the ring GEMM kernel keeps its group tables for at most this many groups
 
 
-def _code_shape(rows: int, ld: int, per: int, kchunk: bool):
-    return (ld // KCHUNK, rows, KCHUNK // per) if kchunk else (rows, ld // per)
+def _layout(kchunk) -> int:
+    return LAYOUT_KSTEP if (kchunk == 2 and kchunk is not True) else (LAYOUT_KCHUNK if kchunk else LAYOUT_ROWMAJOR)
+
+
+def _code_shape(rows: int, ld: int, per: int, kchunk):
+    lay = _layout(kchunk)
+    if lay == LAYOUT_KSTEP:
+        return (ld // KSTEP, rows, KSTEP // per)
+    return (ld // KCHUNK, rows, KCHUNK // per) if lay else (rows, ld // per)
+
+
+def _scale_shape(rows: int, ld: int, kchunk, groups: int = 0):
+    if _layout(kchunk) == LAYOUT_KSTEP:
+        return ((ld + PANEL - 1) // PANEL + (groups + 1 if groups else 0), rows, 16)
+    return (rows, ld // BLOCK)
+
+
+def _qflag(kchunk) -> int:
+    return (0, _lib.QF_KCHUNK, _lib.QF_KSTEP)[_layout(kchunk)]
+
+
+def _gflag(kchunk) -> int:
+    return (0, _lib.GF_KCHUNK, _lib.GF_KSTEP)[_layout(kchunk)]
+
+
+def pick_layout(groups: int, n: int, k: int, rows: int = 0, fp8: bool = True, accum: bool = False) -> int:
+    """Layout the differentiable operators store their quantised operands in: K-step-major when every operand
+    is FP8, the groups fit the ring kernel and the weight gradient is not accumulated in the GEMM; otherwise
+    K-chunk-major; row-major when the layouts are switched off or an operand reaches 4 GiB."""
+    if not (kchunk_default() and kchunk_fits(groups, n, k, rows)):
+        return LAYOUT_ROWMAJOR
+    if fp8 and groups <= RING_MAX_GROUPS and not accum and _kstep_default:
+        return LAYOUT_KSTEP
+    return LAYOUT_KCHUNK
+
+
+_kstep_default = True
+
+
+def set_kstep_default(enabled: bool) -> None:
+    """Whether ``pick_layout`` may choose the K-step-major layout (default) or stops at K-chunk-major."""
+    global _kstep_default
+    _kstep_default = bool(enabled)
 
 
 _kchunk_default = True
@@ -112,10 +164,19 @@ def kchunk_fits(groups: int, n: int, k: int, rows: int = 0) -> bool:
 
 
 def unchunk(codes: torch.Tensor) -> torch.Tensor:
-    """K-chunk-major codes ``[ld / 128, rows, 128]`` as a row-major ``[rows, ld]`` tensor (a copy)."""
+    """K-chunk-major ``[ld / 128, rows, 128]`` or K-step-major ``[ld / 64, rows, 64]`` codes as a row-major
+    ``[rows, ld]`` tensor (a copy)."""
     if codes.dim() != 3:
         raise ValueError("expected 3-D K-chunk-major codes")
     return codes.permute(1, 0, 2).reshape(codes.shape[1], codes.shape[0] * codes.shape[2])
+
+
+def unpanel(scales: torch.Tensor, blocks: int) -> torch.Tensor:
+    """K-step-major scales ``[panels, rows, 16]`` of an operand that is NOT split into groups as row-major
+    ``[rows, blocks]`` (a copy)."""
+    if scales.dim() != 3 or scales.shape[2] != 16:
+        raise ValueError("expected 3-D K-step-major scales [panels, rows, 16]")
+    return scales.permute(1, 0, 2).reshape(scales.shape[1], scales.shape[0] * 16)[:, :blocks].contiguous()
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -194,7 +255,7 @@ def quantize_mx_impl(
     pad_to: int = 1,
     sr_seed: Optional[int] = None,
     rht_signs: Optional[int] = None,
-    kchunk: bool = False,
+    kchunk=False,
 ):
     """MX-quantise bf16 ``x[rows, cols]``.
 
@@ -237,11 +298,11 @@ def quantize_mx_impl(
     row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
         q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-        s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
         q_col = torch.empty(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty((cols, W // BLOCK), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
         row_ok = rows > 0
@@ -252,7 +313,7 @@ def quantize_mx_impl(
                 rc = _lib.load().mxl_quantize(*args, _stream())
             else:
                 flags = ((_lib.QF_SR if sr_seed is not None else 0) | (_lib.QF_RHT_COL if rht_signs is not None else 0)
-                         | (_lib.QF_KCHUNK if kchunk else 0))
+                         | _qflag(kchunk))
                 rc = _lib.load().mxl_quantize_ex(
                     *args, flags, int(sr_seed or 0) & 0xFFFFFFFFFFFFFFFF, int(rht_signs or 0) & 0xFFFF, _stream())
         _lib.check(rc, "mxl_quantize")
@@ -269,7 +330,7 @@ def quantize_mx_weight_2d_impl(
     rowwise: bool = True,
     colwise: bool = True,
     pad_to: int = 1,
-    kchunk: bool = False,
+    kchunk=False,
 ):
     """2-D (32x32 tile) MX quantisation of ``w[n, k]`` or ``w[G, n, k]``;
     returns ``(q_row [.., n, k], s_row [.., n, k/32], q_colT [.., k, n],
@@ -291,17 +352,19 @@ def quantize_mx_weight_2d_impl(
     q_row = s_row = q_col = s_col = None
     k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     if rowwise:
-        shape = _code_shape(batch * n, k_ld, per, True) if kchunk else lead + (n, k_ld // per)
+        shape = _code_shape(batch * n, k_ld, per, kchunk) if kchunk else lead + (n, k_ld // per)
         q_row = torch.empty(shape, dtype=torch.uint8, device=dev)
-        s_row = torch.empty(lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
+        sshape = _scale_shape(batch * n, k_ld, kchunk) if _layout(kchunk) == LAYOUT_KSTEP else lead + (n, k_ld // BLOCK)
+        s_row = torch.empty(sshape, dtype=torch.uint8, device=dev)
     if colwise:
-        shape = _code_shape(batch * k, n_ld, per, True) if kchunk else lead + (k, n_ld // per)
+        shape = _code_shape(batch * k, n_ld, per, kchunk) if kchunk else lead + (k, n_ld // per)
         q_col = torch.empty(shape, dtype=torch.uint8, device=dev)
-        s_col = torch.empty(lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
+        sshape = _scale_shape(batch * k, n_ld, kchunk) if _layout(kchunk) == LAYOUT_KSTEP else lead + (k, n_ld // BLOCK)
+        s_col = torch.empty(sshape, dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_2d_ex(
             _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
-            _lib.QF_KCHUNK if kchunk else 0, _stream()
+            _qflag(kchunk), _stream()
         )
     _lib.check(rc, "mxl_quantize_weight_2d")
     cd = _code_dtype(fmt)
@@ -348,20 +411,31 @@ def _check_out_dtype(out_dtype) -> None:
         raise ValueError("the MX GEMMs produce bfloat16 output")
 
 
-def _chunked_dims(codes: torch.Tensor, fmt: int):
-    """(rows, k) of K-chunk-major codes [k / 128, rows, 128]."""
-    if codes.dim() != 3 or codes.shape[2] * _per_byte(fmt) != KCHUNK or not codes.is_contiguous():
-        raise ValueError("K-chunk-major codes must be a contiguous [k / 128, rows, 128-element] tensor")
-    return codes.shape[1], codes.shape[0] * KCHUNK
+def _chunked_dims(codes: torch.Tensor, fmt: int, kchunk=True):
+    """(rows, k) of K-chunk-major codes [k / 128, rows, 128] or K-step-major codes [k / 64, rows, 64]."""
+    step = KSTEP if _layout(kchunk) == LAYOUT_KSTEP else KCHUNK
+    if codes.dim() != 3 or codes.shape[2] * _per_byte(fmt) != step or not codes.is_contiguous():
+        raise ValueError(f"chunked codes must be a contiguous [k / {step}, rows, {step}-element] tensor")
+    return codes.shape[1], codes.shape[0] * step
 
 
-def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk: bool = False) -> torch.Tensor:
+def _check_scales(scales: torch.Tensor, rows: int, k: int, kchunk, what: str) -> None:
+    if _layout(kchunk) == LAYOUT_KSTEP:
+        ok = scales.dim() == 3 and scales.shape[1] == rows and scales.shape[2] == 16 and scales.shape[0] * PANEL >= k
+    else:
+        ok = scales.numel() == rows * (k // BLOCK) and scales.shape[-1] == k // BLOCK
+    if not ok or not scales.is_contiguous():
+        raise ValueError(f"{what}: scale shape {tuple(scales.shape)} does not match {rows} rows x {k} elements")
+
+
+def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=False) -> torch.Tensor:
     """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T.  ``kchunk``: both code tensors are K-chunk-major."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
     if kchunk:
-        return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale.unsqueeze(0), None, kchunk=True)
+        return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _layout(kchunk) == LAYOUT_KSTEP else b_scale.unsqueeze(0),
+                                       None, kchunk=kchunk)
     m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
     n, kb = b.shape[0], b.shape[1] * _per_byte(b_fmt)
     if k != kb:
@@ -377,7 +451,7 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk: bo
     return c
 
 
-def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16, kchunk: bool = False) -> torch.Tensor:
+def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16, kchunk=False) -> torch.Tensor:
     """Forward / dgrad grouped GEMM: rows of ``a[total_m, k]`` split by
     ``group_lens``; ``b`` is ``[G, n, k]``.  ``kchunk``: both code tensors are K-chunk-major,
     ``a [k / 128, total_m, 128]`` and ``b [k / 128, G * n, 128]``; ``b_scale`` is ``[G, n, k / 32]`` as always."""
@@ -386,19 +460,26 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
     G = _check_group_lens(group_lens, a.device)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
     if kchunk:
-        total_m, k = _chunked_dims(a, a_fmt)
-        b_rows, kb = _chunked_dims(b, b_fmt)
+        total_m, k = _chunked_dims(a, a_fmt, kchunk)
+        b_rows, kb = _chunked_dims(b, b_fmt, kchunk)
         groups = max(G, 1)
-        if b_scale.dim() != 3 or b_scale.shape[0] != groups or b_scale.shape[0] * b_scale.shape[1] != b_rows:
-            raise ValueError("b_scale must be [num_groups, n, k/32] and match the rows of b")
-        n = b_scale.shape[1]
-        if k != kb or tuple(a_scale.shape) != (total_m, k // BLOCK) or b_scale.shape[2] != k // BLOCK:
-            raise ValueError("contraction dims / scale shapes do not match")
+        if _layout(kchunk) == LAYOUT_KSTEP:
+            if b_rows % groups:
+                raise ValueError("the rows of b do not split into num_groups weights")
+            n = b_rows // groups
+        else:
+            if b_scale.dim() != 3 or b_scale.shape[0] != groups or b_scale.shape[0] * b_scale.shape[1] != b_rows:
+                raise ValueError("b_scale must be [num_groups, n, k/32] and match the rows of b")
+            n = b_scale.shape[1]
+        if k != kb:
+            raise ValueError("contraction dims do not match")
+        _check_scales(a_scale, total_m, k, kchunk, "a_scale")
+        _check_scales(b_scale, b_rows, k, kchunk, "b_scale")
         c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
         with _hooked("grouped_gemm_nt" if G else "gemm_nt", m=total_m, n=n, k=k):
             rc = _lib.load().mxl_grouped_gemm_nt_ex(
                 _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), groups, total_m, n, k,
-                _lib.GF_KCHUNK, _stream()
+                _gflag(kchunk), _stream()
             )
         _lib.check(rc, "mxl_grouped_gemm_nt_ex")
         return c
@@ -423,7 +504,7 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
 
 def _accum_target(accum_into, shape, kchunk, device):
     """Checks the float32 buffer a wgrad GEMM is to add its result to."""
-    if not kchunk:
+    if _layout(kchunk) != LAYOUT_KCHUNK:
         raise ValueError("accumulating wgrad needs K-chunk-major operands")
     if (accum_into.dtype != torch.float32 or tuple(accum_into.shape) != tuple(shape) or not accum_into.is_contiguous()
             or accum_into.device != device):
@@ -432,7 +513,7 @@ def _accum_target(accum_into, shape, kchunk, device):
 
 
 def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total_m, out_dtype=torch.bfloat16,
-                               kchunk: bool = False, accum_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+                               kchunk=False, accum_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Variable-K (wgrad) grouped GEMM on segment-padded transposed operands:
     ``a_t`` = dY^T codes ``[n, W]``, ``b_t`` = X^T codes ``[k, W]``; returns
     ``[G, n, k]`` (``[n, k]`` when ``group_lens`` is None).  An expert with no
@@ -443,17 +524,21 @@ def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total
     a_fmt, b_fmt = fmt_of(a_t), fmt_of(b_t)
     W = padded_width(total_m, G)
     if kchunk:
-        (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt), _chunked_dims(b_t, b_fmt)
+        (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt, kchunk), _chunked_dims(b_t, b_fmt, kchunk)
         if wa != W or wb != W:
             raise ValueError(f"transposed operands must have padded width {W}")
     else:
         n, k = a_t.shape[0], b_t.shape[0]
         if a_t.shape[1] * _per_byte(a_fmt) != W or b_t.shape[1] * _per_byte(b_fmt) != W:
             raise ValueError(f"transposed operands must have padded width {W}")
-    if tuple(a_t_scale.shape) != (n, W // BLOCK) or tuple(b_t_scale.shape) != (k, W // BLOCK):
+    if _layout(kchunk) == LAYOUT_KSTEP:
+        for sc, r in ((a_t_scale, n), (b_t_scale, k)):
+            if tuple(sc.shape) != _scale_shape(r, W, kchunk, G) or not sc.is_contiguous():
+                raise ValueError("K-step-major scales of the transposed operands must be [panels, rows, 16]")
+    elif tuple(a_t_scale.shape) != (n, W // BLOCK) or tuple(b_t_scale.shape) != (k, W // BLOCK):
         raise ValueError("scale shapes must be [rows, W/32]")
     shape = (n, k) if group_lens is None else (G, n, k)
-    flags = _lib.GF_KCHUNK if kchunk else 0
+    flags = _gflag(kchunk)
     if accum_into is not None:
         # the result is added, in float32, to accum_into (which is returned)
         c = _accum_target(accum_into, shape, kchunk, a_t.device)
@@ -523,7 +608,7 @@ def glu_with_probs_bwd_impl(dy, x, probs, row_mask, activation: str):
 
 def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *,
                                  colwise: bool = False, group_lens: Optional[torch.Tensor] = None, pad_to: int = 1,
-                                 kchunk: bool = False):
+                                 kchunk=False):
     """``quantize_mx_impl(glu_with_probs_fwd_impl(x, ...))`` in one pass over ``x [tokens, 2F]``, the
     activated tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
     act, pd, row_mask = _glu_args(x, probs, row_mask, activation)
@@ -539,19 +624,19 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
     dev = x.device
     row_ld = _round_up(f, KCHUNK if kchunk else pad_to)
     q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-    s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+    s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, G)
         q_col = torch.empty(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty((f, W // BLOCK), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(f, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         row_ok = rows > 0
         with _hooked("glu_probs_quantize", rows=rows, cols=f, fmt=fmt, rowwise=True, colwise=colwise):
             rc = _lib.load().mxl_glu_probs_quantize(
                 _ptr(x) if row_ok else None, _ptr(probs), pd, _ptr(row_mask), rows, f, row_ld, act, fmt, scale_mode,
                 _ptr(group_lens), G, _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col),
-                _ptr(s_col), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+                _ptr(s_col), _qflag(kchunk), _stream(),
             )
         _lib.check(rc, "mxl_glu_probs_quantize")
     cd = _code_dtype(fmt)
@@ -782,7 +867,7 @@ def rmsnorm_bwd_impl(dy, x, weight, rstd):
 
 
 def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *, colwise: bool = False,
-                          pad_to: int = 1, kchunk: bool = False):
+                          pad_to: int = 1, kchunk=False):
     """``quantize_mx_impl(rmsnorm_fwd_impl(x, weight, eps)[0])`` in one pass over ``x`` given ``rstd``, the
     normalised tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
     _norm_args(x, weight)
@@ -798,16 +883,16 @@ def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCAL
     dev = x.device
     row_ld = _round_up(k, KCHUNK if kchunk else pad_to)
     q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-    s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+    s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, 0)
         q_col = torch.empty(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty((k, W // BLOCK), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(k, W, kchunk), dtype=torch.uint8, device=dev)
     with _hooked("rmsnorm_quantize", rows=rows, cols=k, fmt=fmt, rowwise=True, colwise=colwise):
         rc = _lib.load().mxl_rmsnorm_quantize(
             _ptr(x), _ptr(weight), _ptr(rstd), rows, k, row_ld, fmt, scale_mode, None, 0, _ptr(q_row), _ptr(s_row),
-            _ptr(q_col), _ptr(s_col), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+            _ptr(q_col), _ptr(s_col), _qflag(kchunk), _stream(),
         )
     _lib.check(rc, "mxl_rmsnorm_quantize")
     cd = _code_dtype(fmt)

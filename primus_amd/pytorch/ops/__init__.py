@@ -111,10 +111,23 @@ def _accum_from(b, pattern):
     return main_grad, b
 
 
-def _cached_codes(q: QuantizedTensor, kchunk: bool) -> torch.Tensor:
-    """Codes of a cached weight copy in the layout this call's GEMMs use.  A K-chunk-major cache is
+def _cached_codes(q: QuantizedTensor, kchunk) -> torch.Tensor:
+    """Codes of a cached weight copy in the layout this call's GEMMs use.  A chunked cache is
     rearranged (one pass over the weight) only when this call cannot use that layout."""
-    return q.codes if q.kchunk == kchunk else q.rowmajor_codes()
+    return q.codes if int(q.kchunk) == int(kchunk) else q.rowmajor_codes()
+
+
+def _cached_scales(q: QuantizedTensor, kchunk) -> torch.Tensor:
+    return q.scales if int(q.kchunk) == int(kchunk) else q.rowmajor_scales()
+
+
+def _cache_layout(b: QuantizedTensor, b_t, kc: int, fp8: bool, groups: int) -> int:
+    """Layout of a call on cached weight copies: the cache's own, row-major when the pair disagrees or
+    this call cannot read that layout."""
+    lay = int(b.kchunk) if (b_t is None or int(b_t.kchunk) == int(b.kchunk)) else 0
+    if lay == K.LAYOUT_KSTEP and not (fp8 and groups <= K.RING_MAX_GROUPS):
+        lay = 0
+    return lay if kc else 0
 
 
 class _MXLinearFunction(torch.autograd.Function):
@@ -135,9 +148,10 @@ class _MXLinearFunction(torch.autograd.Function):
         # Every operand of the three GEMMs is stored in one layout, K-chunk-major unless an operand is
         # too large for it (or the layout is switched off): same codes, same results, faster loads.
         groups = b.shape[0] if grouped else 1
-        kc = K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])
-        if isinstance(b, QuantizedTensor):   # cached copies decide: row-major caches are used as they are
-            kc = kc and b.kchunk and (b_t is None or b_t.kchunk)
+        fp8 = act_fmt != _lib.FMT_E2M1 and w_fmt != _lib.FMT_E2M1
+        kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, accum=accum is not None)
+        if isinstance(b, QuantizedTensor):   # cached copies decide: the call uses the layout they are stored in
+            kc = _cache_layout(b, b_t, kc, fp8, groups)
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
         # (row-wise copies are padded to the GEMM's K granularity, like the reference pads its
         # MXFP4 operands to 128: primus_turbo_mxfp4_local.py:119-124)
@@ -163,14 +177,14 @@ class _MXLinearFunction(torch.autograd.Function):
                 raise ValueError("the forward weight copy must be quantised along axis=-1")
             if b.tensor_scale_inv is not None:
                 raise ValueError("the cached weight copy is tensor-wise scaled, the operator's config is an MX recipe")
-            w_row, w_rs = _cached_codes(b, kc), b.scales
+            w_row, w_rs = _cached_codes(b, kc), _cached_scales(b, kc)
             w_col = w_cs = None
             if need_dgrad:
                 if b_t is None:
                     raise ValueError("dgrad needs the transposed weight copy (QuantizedTensorPair.data_t)")
                 if b_t.axis != -2:
                     raise ValueError("QuantizedTensorPair.data_t must be quantised along axis=-2")
-                w_col, w_cs = _cached_codes(b_t, kc), b_t.scales
+                w_col, w_cs = _cached_codes(b_t, kc), _cached_scales(b_t, kc)
         else:
             w_row, w_rs, w_col, w_cs = K.quantize_mx_weight_2d_impl(
                 b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
@@ -223,7 +237,7 @@ class _MXLinearFunction(torch.autograd.Function):
                 grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
-            fused = target is not None and kc          # the GEMM's epilogue adds into the float32 buffer
+            fused = target is not None and kc == K.LAYOUT_KCHUNK   # the GEMM's epilogue adds into the float32 buffer
 
             def wgrad():
                 return K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc,

@@ -105,7 +105,7 @@ def test_newer_entry_points_validate_before_they_touch_the_device(lib):
     assert lib.mxl_rmsnorm_bwd_workspace_bytes(4, 100) == -1
     assert lib.mxl_rmsnorm_bwd(p, p, p, p, 4, 256, p, None, p, 4096, None) == -1     # no dw
     assert lib.mxl_rmsnorm_quantize(p, None, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 0, None) == -1   # no weight
-    assert lib.mxl_rmsnorm_quantize(p, p, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 8, None) == -1      # unknown flag
+    assert lib.mxl_rmsnorm_quantize(p, p, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 64, None) == -1     # unknown flag
     assert lib.mxl_rmsnorm_quantize(p, p, p, 4, 256, 256, 0, 0, None, 0, p, p, None, None, 0, None) == -3
     # tensor-wise scaling
     assert lib.mxl_amax(p, -1, p, None) == -1

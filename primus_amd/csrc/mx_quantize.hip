@@ -290,6 +290,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
 
     // ---- row-wise copy ----
     if (ROW) {
+        uint2 o_even = make_uint2(0u, 0u);   // FP8: codes of the even row of a row pair, kept until its partner is done
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
             const int r = 32 * w + 8 * rg + it;
@@ -308,11 +309,25 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                     o.x = nonfinite4_e4m3(d[it].x, d[it].y);
                     o.y = nonfinite4_e4m3(d[it].z, d[it].w);
                 }
-                if (out_ok && r < rows_valid) {
-                    const int64_t at = a.kchunk == 2 ? ((int64_t)(2 * ct + (c16 >> 3)) * a.chunk_rows_row + src_row0 + r) * (QT / 2) + 8 * (c16 & 7)
-                                     : a.kchunk  ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
-                                                 : (src_row0 + r) * a.row_ld + col;
-                    store8_streaming(a.q_row + at, o);
+                // Two rows at a time, 16 bytes per lane: a lane pair swaps one 8-byte piece, after which the even lane
+                // holds 16 consecutive codes of the even row and the odd lane 16 of the odd row.  Half the store
+                // instructions, and in the K-step-major layout (64-byte row pieces, two rows to a cache line) an
+                // instruction then writes whole lines.
+                if ((it & 1) == 0) {
+                    o_even = o;
+                } else {
+                    const bool odd = (c16 & 1) != 0;
+                    const uint2 send = odd ? o_even : o;
+                    const uint2 recv = make_uint2(dpp_xor1(send.x), dpp_xor1(send.y));
+                    const uint4 out = odd ? make_uint4(recv.x, recv.y, o.x, o.y) : make_uint4(o_even.x, o_even.y, recv.x, recv.y);
+                    const int rr = odd ? r : r - 1;
+                    const int cc = c16 & ~1;          // the pair's first 8-column piece
+                    if (out_ok && rr < rows_valid) {
+                        const int64_t at = a.kchunk == 2 ? ((int64_t)(2 * ct + (cc >> 3)) * a.chunk_rows_row + src_row0 + rr) * (QT / 2) + 8 * (cc & 7)
+                                         : a.kchunk  ? ((int64_t)ct * a.chunk_rows_row + src_row0 + rr) * QT + 8 * cc
+                                                     : (src_row0 + rr) * a.row_ld + col0 + 8 * cc;
+                        store16_streaming(a.q_row + at, out);
+                    }
                 }
             } else {
                 uint32_t o;

@@ -32,6 +32,7 @@ extern "C" {
 #define MXL_EINVAL (-1)  /* bad shape / alignment / enum / null pointer */
 #define MXL_ELAUNCH (-2) /* HIP reported an error at launch */
 #define MXL_ENODEV (-3)  /* current device is not gfx950 */
+#define MXL_ESCRATCH (-4) /* the problem needs more scratch memory than an allocation-free entry point owns */
 
 #define MXL_FMT_E4M3 0
 #define MXL_FMT_E2M1 1
@@ -297,6 +298,19 @@ int mxl_rmsnorm_fwd(const void* x_bf16, const void* w_bf16, float eps, int64_t r
 int64_t mxl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t k);
 int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows,
                     int64_t k, void* dx_bf16, void* dw_bf16, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* mxl_rmsnorm_bwd for callers that cannot allocate or hand over a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  Same arguments minus the
+ * workspace, same kernels, same results bit for bit; the partial column sums go through a static device array of
+ * mxl_rmsnorm_bwd_noalloc_max_bytes() = 8 MiB that every GPU the library runs on holds until the process ends.
+ * A problem with mxl_rmsnorm_bwd_workspace_bytes(rows, k) above that returns MXL_ESCRATCH (e.g. k = 4096 with
+ * more than 512 rows; k <= 1024 always fits).  Calls no hipMalloc / hipFree or other allocating routine.  All
+ * calls on one GPU share the array: calls that overlap on a GPU (two streams, two threads) race; calls on one
+ * stream are ordered.  Nothing in the array has to be cleared between calls (every word read was written by
+ * the same call). */
+int64_t mxl_rmsnorm_bwd_noalloc_max_bytes(void);
+int mxl_rmsnorm_bwd_noalloc(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows,
+                            int64_t k, void* dx_bf16, void* dw_bf16, void* stream);
 
 /* The normalisation feeding the MX quantiser directly: what mxl_quantize would produce for
  * y = mxl_rmsnorm_fwd(x, w, ...) (bit for bit) from x, w and rstd (mxl_rmsnorm_fwd with y_bf16 = NULL), without

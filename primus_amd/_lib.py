@@ -52,6 +52,8 @@ EXPORTS = (
     "mxl_rmsnorm_fwd",
     "mxl_rmsnorm_bwd",
     "mxl_rmsnorm_bwd_workspace_bytes",
+    "mxl_rmsnorm_bwd_noalloc",
+    "mxl_rmsnorm_bwd_noalloc_max_bytes",
     "mxl_rmsnorm_quantize",
     "mxl_amax",
     "mxl_quantize_tensorwise",
@@ -125,6 +127,10 @@ def load() -> ctypes.CDLL:
         lib.mxl_rmsnorm_bwd_workspace_bytes.argtypes = [i64, i64]
         lib.mxl_rmsnorm_bwd.restype = i32
         lib.mxl_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i64, vp]
+        lib.mxl_rmsnorm_bwd_noalloc.restype = i32
+        lib.mxl_rmsnorm_bwd_noalloc.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp]
+        lib.mxl_rmsnorm_bwd_noalloc_max_bytes.restype = i64
+        lib.mxl_rmsnorm_bwd_noalloc_max_bytes.argtypes = []
         lib.mxl_rmsnorm_quantize.restype = i32
         lib.mxl_rmsnorm_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, u32, vp]
         lib.mxl_amax.restype = i32

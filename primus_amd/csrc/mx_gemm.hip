@@ -1287,6 +1287,7 @@ extern "C" const char* mxl_error_string(int code) {
         case MXL_EINVAL: return "invalid argument (shape, alignment, enum or null pointer)";
         case MXL_ELAUNCH: return "HIP launch error";
         case MXL_ENODEV: return "device is not gfx950";
+        case MXL_ESCRATCH: return "the problem needs more scratch memory than this allocation-free entry point owns";
         default: return "unknown error";
     }
 }

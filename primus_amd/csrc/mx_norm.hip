@@ -210,9 +210,10 @@ extern "C" int64_t mxl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t k) {
     return (int64_t)norm_bwd_blocks(rows, k) * k * 4;
 }
 
-extern "C" int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32,
-                               int64_t rows, int64_t k, void* dx_bf16, void* dw_bf16, void* workspace,
-                               int64_t workspace_bytes, void* stream) {
+// shared by the two backward entry points; `workspace` is the caller's buffer or this device's static scratch
+static int rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32,
+                       int64_t rows, int64_t k, void* dx_bf16, void* dw_bf16, void* workspace,
+                       int64_t workspace_bytes, void* stream) {
     if (!norm_shape_ok(rows, k) || !dw_bf16) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
     hipStream_t st = (hipStream_t)stream;
@@ -238,4 +239,47 @@ extern "C" int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const vo
     hipLaunchKernelGGL(rmsnorm_dw_kernel, dim3((unsigned)grid), dim3(NTHREADS), 0, st, (const float*)workspace, blocks, k,
                        (uint16_t*)dw_bf16);
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
+
+extern "C" int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32,
+                               int64_t rows, int64_t k, void* dx_bf16, void* dw_bf16, void* workspace,
+                               int64_t workspace_bytes, void* stream) {
+    return rmsnorm_bwd(dy_bf16, x_bf16, w_bf16, rstd_f32, rows, k, dx_bf16, dw_bf16, workspace, workspace_bytes, stream);
+}
+
+// ---- the same without a workspace argument and without any allocation ----
+// The partial column sums go through a file-scope device array.  Each GPU holds its own copy of it at its own
+// address (from the moment the library's code is loaded there until the process ends); the address is asked
+// for once per device, with that device current, and kept.  Host code must never hand the array's NAME to a
+// kernel: on the host that name is a stand-in, not a device address.
+constexpr int64_t NORM_SCRATCH_BYTES = (int64_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[NORM_SCRATCH_BYTES];
+
+static int norm_scratch_ptr(void** out) {
+    constexpr int MAXDEV = 64;
+    static std::atomic<void*> ptrs[MAXDEV];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MXL_ELAUNCH;
+    void* ptr = (dev >= 0 && dev < MAXDEV) ? ptrs[dev].load(std::memory_order_acquire) : nullptr;
+    if (!ptr) {
+        if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MXL_ELAUNCH;
+        if (dev >= 0 && dev < MAXDEV) ptrs[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return MXL_OK;
+}
+
+extern "C" int64_t mxl_rmsnorm_bwd_noalloc_max_bytes(void) { return NORM_SCRATCH_BYTES; }
+
+extern "C" int mxl_rmsnorm_bwd_noalloc(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32,
+                                       int64_t rows, int64_t k, void* dx_bf16, void* dw_bf16, void* stream) {
+    if (!norm_shape_ok(rows, k) || !dw_bf16) return MXL_EINVAL;
+    // same partial-sum geometry as mxl_rmsnorm_bwd (hence the same bits); a problem whose partial sums do not
+    // fit the static array is refused
+    if ((int64_t)norm_bwd_blocks(rows, k) * k * 4 > NORM_SCRATCH_BYTES) return MXL_ESCRATCH;
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    void* ptr = nullptr;
+    const int rc = norm_scratch_ptr(&ptr);
+    if (rc != MXL_OK) return rc;
+    return rmsnorm_bwd(dy_bf16, x_bf16, w_bf16, rstd_f32, rows, k, dx_bf16, dw_bf16, ptr, NORM_SCRATCH_BYTES, stream);
 }

@@ -485,20 +485,24 @@ class _LowPrecisionGemm:
         assert norm is None or not grouped, "the normalisation prologue exists for the dense linears only"
 
         def run(op_dense, op_grouped, a, b, fuse_pattern, **kw):
+            # the prologues are folded into the MX quantisers only: under the tensor-wise (current scaling) recipe,
+            # as outside a low-precision autocast, the normalisation / activation runs as an operator of its own
+            # in front of the GEMM, which is what the reference does (primus_turbo.py:1689-1741)
+            mx = "config" in kw and kw["config"].granularity == ScalingGranularity.MX_BLOCKWISE
             if norm is not None:
                 norm_weight, eps = norm
-                if op_dense is ops.gemm:               # outside a low-precision autocast: two plain operators
+                if not mx:
                     return op_dense(ops.rmsnorm(a, norm_weight, eps), b, trans_a=False, trans_b=True, out_dtype=None,
-                                    fuse_bgrad_accum_pattern=fuse_pattern)
+                                    fuse_bgrad_accum_pattern=fuse_pattern, **kw)
                 fused = ops.rmsnorm_gemm_fp8 if op_dense is ops.gemm_fp8 else ops.rmsnorm_gemm_fp4
                 return fused(a, norm_weight, eps, b, trans_a=False, trans_b=True, out_dtype=None,
                              fuse_bgrad_accum_pattern=fuse_pattern, **kw)
             if glu is not None:
                 probs, row_mask, activation = glu
-                if op_grouped is ops.grouped_gemm:     # outside a low-precision autocast: two plain operators
+                if not mx:
                     act = ops.swiglu_with_probs if activation == "silu" else ops.geglu_with_probs
                     return op_grouped(act(a, probs, row_mask), b, group_lens, trans_b=True,
-                                      fuse_bgrad_accum_pattern=fuse_pattern)
+                                      fuse_bgrad_accum_pattern=fuse_pattern, **kw)
                 fused = ops.glu_grouped_gemm_fp8 if op_grouped is ops.grouped_gemm_fp8 else ops.glu_grouped_gemm_fp4
                 return fused(a, probs, b, group_lens, activation=activation, row_mask=row_mask, trans_b=True,
                              fuse_bgrad_accum_pattern=fuse_pattern, **kw)

@@ -46,8 +46,7 @@ def _unsupported(**flags) -> None:
         raise NotImplementedError(f"quantize_mxfp4_dual: no kernel for {', '.join(on)}")
 
 
-@torch.library.custom_op("primus_amd::quantize_mxfp4_dual", mutates_args=(), device_types="cuda")
-def _quantize_mxfp4_dual_op(
+def _quantize_mxfp4_dual_impl(
     x: torch.Tensor,
     out_dtype: torch.dtype,
     padding_align_size: int,
@@ -93,7 +92,6 @@ def _quantize_mxfp4_dual_op(
     return q, s, qt, st
 
 
-@_quantize_mxfp4_dual_op.register_fake
 def _quantize_mxfp4_dual_fake(
     x, out_dtype, padding_align_size, rowwise_use_2d_block, rowwise_use_sr, rowwise_use_rht, colwise_use_2d_block,
     colwise_use_sr, colwise_use_rht, shuffle_rowwise_scale, shuffle_rowwise, shuffle_colwise_scale, shuffle_colwise,
@@ -118,6 +116,20 @@ def _quantize_mxfp4_dual_fake(
         u8(N, M_pad // 2).view(_FP4_DTYPE),
         u8(*scale_shape(N, M_pad, shuffle_colwise_scale)).view(float8_e8m0),
     )
+
+
+# The op under two names: this package's own namespace and the one the reference's call sites use,
+# torch.ops.primus_turbo_cpp_extension.quantize_mxfp4_dual (primus_turbo_mxfp4_local.py:147-161), so that
+# code written against the reference's C++ extension finds it unchanged.
+_quantize_mxfp4_dual_op = torch.library.custom_op(
+    "primus_amd::quantize_mxfp4_dual", _quantize_mxfp4_dual_impl, mutates_args=(), device_types="cuda")
+_quantize_mxfp4_dual_op.register_fake(_quantize_mxfp4_dual_fake)
+try:
+    _quantize_mxfp4_dual_ref_name = torch.library.custom_op(
+        "primus_turbo_cpp_extension::quantize_mxfp4_dual", _quantize_mxfp4_dual_impl, mutates_args=(), device_types="cuda")
+    _quantize_mxfp4_dual_ref_name.register_fake(_quantize_mxfp4_dual_fake)
+except RuntimeError:   # the real extension is loaded in this process and owns the name
+    _quantize_mxfp4_dual_ref_name = None
 
 
 _quantize_mxfp4_dual_op.register_autograd(lambda ctx, *grads: (None,) * 13, setup_context=lambda ctx, inputs, output: None)

@@ -940,12 +940,21 @@ def grouped_gemm_fp8_variable_k_impl(a, b, a_scale_inv, b_scale_inv, group_lens,
     """grouped_gemm_fp8_variable_k_impl of the reference (zbpp_gemm.py:710-724):
     ``a`` = X col-wise copy ``[k, W]``, ``b`` = dY col-wise copy ``[n, W]``
     (both transposed, segment-padded); with ``trans_c=True`` (weights stored
-    ``[n, k]``, i.e. trans_b=True in the forward) returns ``[G, n, k]``."""
+    ``[n, k]``, i.e. trans_b=True in the forward) returns ``[G, n, k]``.
+    ``total_m`` (ours, optional) is the token count; without it the padded width is taken from the operands."""
     _require_mx(granularity)
     if not trans_a or trans_b:
         raise ValueError("variable-K grouped GEMM expects trans_a=True, trans_b=False")
     if total_m is None:
-        raise ValueError("total_m (number of tokens) is required: the padded width alone does not determine it")
+        # The reference's call (13 arguments) does not carry the token count.  The kernels need it only for the
+        # padded width of the transposed operands, which the operand states itself: any count with that padded
+        # width describes the same buffers (the groups come from group_lens, on the device).
+        G = _check_group_lens(group_lens, a.device)
+        per = _per_byte(fmt_of(a))
+        width = a.shape[0] * a.shape[2] * per if a.dim() == 3 else a.shape[-1] * per
+        total_m = max(width - (_lib.SEG_ALIGN - 1) * max(G, 1), 0)
+        if padded_width(total_m, G) != width:
+            raise ValueError(f"the operands' last dim ({width}) is not a padded width for {G} groups")
     if trans_c:
         return grouped_gemm_mx_wgrad_impl(b, b_scale_inv, a, a_scale_inv, group_lens, total_m, out_dtype)
     return grouped_gemm_mx_wgrad_impl(a, a_scale_inv, b, b_scale_inv, group_lens, total_m, out_dtype)

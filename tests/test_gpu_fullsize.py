@@ -36,6 +36,14 @@ def _bf(t):
     return o.bf16_bits_to_f32(t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
 
 
+def _elementwise_bound(want, absdot, k):
+    """|got - want| allowed per element: bf16 rounding of the output (2^-8 relative) plus the accumulation error,
+    (k + 1024) * 2^-23 * sum |a_i b_i|: k fp32 additions, and a floor of 2^-13 for the MFMA's 64-term dot product,
+    whose products are aligned to a common exponent in a finite datapath (measured: at most 2^-16 of sum |a_i b_i|
+    beyond the output rounding, at k = 128 as at k = 14336)."""
+    return 2.0 ** -8 * np.abs(want) + (k + 1024) * 2.0 ** -23 * absdot + 1e-30
+
+
 def _sample_rows(lens, rng, per_group=2):
     """Row indices: first and last row of every non-empty expert plus random interior rows."""
     rows, off = [], 0
@@ -149,6 +157,7 @@ def test_full_size_linear(gpu, workload, layer):
     d_rows = _deq_rows(_u8(dq)[ridx].cpu().numpy(), _u8(ds)[ridx].cpu().numpy(), a_fmt)        # [R, np]
     y_s, dx_s = _bf(y[ridx][:, cn]), _bf(dx[ridx][:, ck])
     want_y, want_dx = np.zeros_like(y_s), np.zeros_like(dx_s)
+    abs_y, abs_dx = np.zeros_like(y_s), np.zeros_like(dx_s)      # sum |a_i b_i| of every sampled output
     cache = {}
     for i, r in enumerate(rows):
         g, _ = _group_of(r, glens)
@@ -159,8 +168,13 @@ def test_full_size_linear(gpu, workload, layer):
             cache[g] = (b_fwd, b_bwd)
         want_y[i] = cache[g][0] @ a_rows[i]
         want_dx[i] = cache[g][1] @ d_rows[i]
+        abs_y[i] = np.abs(cache[g][0]) @ np.abs(a_rows[i])
+        abs_dx[i] = np.abs(cache[g][1]) @ np.abs(d_rows[i])
     assert np.abs(y_s - want_y).max() <= tol * np.abs(want_y).max()
     assert np.abs(dx_s - want_dx).max() <= tol * np.abs(want_dx).max()
+    # per element: the output's own bf16 rounding plus the accumulation-order error of the contraction
+    assert (np.abs(y_s - want_y) <= _elementwise_bound(want_y, abs_y, kp)).all()
+    assert (np.abs(dx_s - want_dx) <= _elementwise_bound(want_dx, abs_dx, d_rows.shape[1])).all()
 
     # wgrad: sampled (n, k) positions of up to three experts, contraction over the expert's padded segment
     for g in sorted(set(picked))[:3]:
@@ -171,6 +185,7 @@ def test_full_size_linear(gpu, workload, layer):
         want = a_t @ b_t.T
         got = _bf((dw if dense else dw[g])[cn][:, ck])
         assert np.abs(got - want).max() <= tol * np.abs(want).max(), (workload, g)
+        assert (np.abs(got - want) <= _elementwise_bound(want, np.abs(a_t) @ np.abs(b_t).T, wpad)).all(), (workload, g)
 
     # ---- (3) properties ----
     if not dense:

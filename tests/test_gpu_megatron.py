@@ -455,6 +455,77 @@ def test_linear_and_grouped_linear_under_the_tensorwise_recipe(mg, gpu, hybrid, 
     assert not wg[1].any() and wg[0].abs().sum() > 0
 
 
+@pytest.mark.parametrize("microbatches", [1, 2])
+def test_fused_prologue_modules_under_the_tensorwise_recipe(mg, gpu, microbatches):
+    """The modules that fold RMSNorm / the gated activation into the MX quantiser still work under the tensor-wise
+    recipe: there the prologue runs as an operator of its own in front of the FP8 GEMM (the reference's sequence,
+    primus_turbo.py:1689-1741 and the GroupedMLP forward), with the switches for the folded forms left on."""
+    pt = mg
+    from primus_amd.megatron import runtime
+    from primus_amd.pytorch.core import Format, ScalingGranularity
+
+    runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                     turbo_grouped_gemm_without_padding=True, use_turbo_fused_act_with_probs=True,
+                     turbo_fuse_norm_into_quantize=True)
+    runtime.set_num_microbatches(microbatches)
+    qc = pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.TENSORWISE, format=Format.E4M3)
+
+    def autocast():
+        return pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc)
+
+    torch.manual_seed(31)
+    ln = pt.PrimusTurboLayerNormColumnParallelLinear(256, 160, config=_cfg(), bias=True)
+    assert ln.fuse_norm_into_quantize
+    with torch.no_grad():
+        ln.layer_norm_weight.copy_(1 + 0.1 * torch.randn(256))
+    ln.weight.main_grad = torch.zeros_like(ln.weight, dtype=torch.float32)
+    ln.weight.grad_added_to_main_grad = False
+    x = torch.randn(12, 8, 256, device=gpu).bfloat16().requires_grad_()
+    dy = torch.randn(12, 8, 160, device=gpu).bfloat16()
+    with autocast():
+        y, _ = ln(x)
+    y.backward(dy)
+    xr = x.detach().clone().requires_grad_()
+    wr, gr = ln.weight.detach().clone().requires_grad_(), ln.layer_norm_weight.detach().clone().requires_grad_()
+    yr = torch.nn.functional.linear(torch.nn.functional.rms_norm(xr, [256], gr, 1e-5), wr, ln.bias.detach())
+    yr.backward(dy)
+    wgrad = ln.weight.main_grad if microbatches > 1 else ln.weight.grad
+    assert _cos(y, yr) > 0.998 and _cos(x.grad, xr.grad) > 0.998
+    assert _cos(wgrad, wr.grad) > 0.998 and _cos(ln.layer_norm_weight.grad, gr.grad) > 0.998
+
+    mlp = _mlp(pt, gpu, 4, 256, 384)
+    assert mlp.fuse_act_into_fc2
+    lens = [100, 0, 37, 55]
+    tpe = torch.tensor(lens, device=gpu)
+    xm = torch.randn(sum(lens), 256, device=gpu).bfloat16()
+    probs = torch.rand(sum(lens), device=gpu)
+    dym = torch.randn(sum(lens), 256, device=gpu).bfloat16()
+
+    def run(ctx):
+        mlp.zero_grad(set_to_none=True)
+        for lin in (mlp.linear_fc1, mlp.linear_fc2):
+            lin.weights.main_grad = torch.zeros_like(lin.weights, dtype=torch.float32)
+            lin.weights.grad_added_to_main_grad = False
+            lin.set_is_first_microbatch()                    # every run is the first microbatch of a new step
+        xi, pi = xm.clone().requires_grad_(), probs.clone().requires_grad_()
+        with ctx:
+            out, _ = mlp(xi, tpe, pi)
+        out.backward(dym)
+        grads = [(lin.weights.main_grad if microbatches > 1 and ctx is not plain else lin.weights.grad).float().clone()
+                 for lin in (mlp.linear_fc1, mlp.linear_fc2)]
+        return [out.detach(), xi.grad, pi.grad] + grads
+
+    import contextlib
+
+    plain = contextlib.nullcontext()
+    want = run(plain)
+    got = run(autocast())
+    for name, a, b in zip(("y", "dx", "dprobs", "dw1", "dw2"), got, want):
+        assert torch.isfinite(a.float()).all(), name
+        assert _cos(a, b) > 0.995, (name, _cos(a, b))
+    assert not got[3][1].any() and not got[4][1].any()       # the expert without tokens has no gradient
+
+
 @pytest.mark.parametrize("recipe", ["bf16", "tensorwise", "mxfp8"])
 def test_gradient_accumulation_fusion_adds_into_main_grad(mg, gpu, recipe):
     """config.gradient_accumulation_fusion: the wgrad GEMM adds into weight.main_grad itself

@@ -322,6 +322,31 @@ int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, const void* rst
                          int64_t row_ld, int fmt, int scale_mode, const int64_t* group_lens, int num_groups,
                          void* q_row, void* s_row, void* q_colT, void* s_colT, uint32_t flags, void* stream);
 
+/* Expert groups padded to the quantisation alignment without a host read of the counts.  Replaces the
+ * tokens_per_expert.tolist() + per-expert split / zero-append of the reference's expert MLP
+ * (primus/backends/megatron/core/transformer/experts.py:196-209) and its inverse (:262-264); the alignment is the
+ * reference's pad_multiple (primus/backends/megatron/core/extensions/primus_turbo.py:2344-2353: 32 for MX, else 16).
+ *
+ *   x           : [rows, row_bytes] bytes, rows of the groups back to back (sum(group_lens) == rows; rows of x the
+ *                 counts do not cover are dropped)
+ *   group_lens  : int64[num_groups] on the device, 1 <= num_groups <= 1024; negative counts read as 0
+ *   out         : [out_rows, row_bytes]; group g starts at the sum of the padded lengths before it, holds its rows
+ *                 and then zero rows up to a multiple of align; every row behind the last group's padding is a zero
+ *                 row as well.  out_rows >= mxl_padded_rows_bound(rows, num_groups, align), the largest total the
+ *                 counts can produce, since the host does not know them.
+ *   padded_lens : int64[num_groups] (may be NULL): ceil(len / align) * align, the last one enlarged by the rows
+ *                 behind its padding so that the lengths sum to out_rows exactly.
+ *
+ * mxl_unpad_groups is the inverse (and the gradient of mxl_pad_groups, as mxl_pad_groups is of it): row i of group
+ * g of `out` [rows, row_bytes] is row i of that group in the padded `y` [padded_rows, row_bytes]; rows of `out`
+ * behind sum(group_lens) are zero.  Any row_bytes >= 1; rows move 16 bytes per lane when pointers and row_bytes
+ * are multiples of 16. */
+int64_t mxl_padded_rows_bound(int64_t rows, int num_groups, int align);
+int mxl_pad_groups(const void* x, int64_t rows, int64_t row_bytes, const int64_t* group_lens, int num_groups, int align,
+                   void* out, int64_t out_rows, int64_t* padded_lens, void* stream);
+int mxl_unpad_groups(const void* y, int64_t padded_rows, int64_t row_bytes, const int64_t* group_lens, int num_groups,
+                     int align, void* out, int64_t rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -92,6 +92,13 @@ Parity status
   Primus-Turbo C++ op whose source is absent: the float32 product used here is **parity unpinned**
   against that op.
 
+* ``pad_groups`` / ``unpad_groups`` (expert groups padded with zero rows to the quantisation alignment,
+  experts.py:196-209 and :262-264; alignment from primus_turbo.py:2344-2353): index work, written with numpy
+  slices per group; pinned in tests/ against the reference's own sequence (split per expert, append zero rows,
+  concatenate) written as a row-by-row Python loop, and by unpad(pad(x)) == x.  The rows behind the last group's
+  padding in a buffer sized for the worst case (zero rows counted into the last group) have no counterpart in
+  the reference, whose buffer has the exact size because it reads the counts on the host.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -813,3 +820,44 @@ def tensorwise_gemm_nt_ref(a_codes, a_scale_inv, b_codes, b_scale_inv, a_fmt=FMT
     acc = _matmul_nt_f32(decode_fp8(a_codes, a_fmt), decode_fp8(b_codes, b_fmt))
     c = (acc * (np.float32(a_scale_inv) * np.float32(b_scale_inv))).astype(np.float32)
     return f32_to_bf16_bits(c) if out_bf16 else c
+
+
+# --------------------------------------------------------------------------
+# expert groups padded to the quantisation alignment
+# --------------------------------------------------------------------------
+def padded_rows_bound(rows: int, num_groups: int, align: int) -> int:
+    """Largest sum of padded group lengths that ``num_groups`` counts summing to ``rows`` can produce."""
+    return (rows + num_groups * (align - 1)) // align * align
+
+
+def pad_groups(x: np.ndarray, group_lens, align: int, out_rows=None):
+    """``(out, padded_lens)``: every group's rows followed by zero rows up to a multiple of ``align``
+    (experts.py:196-209).  ``out_rows`` None gives the exact size, which is the reference's result; a larger
+    buffer ends in zero rows that are counted into the last group."""
+    lens = [max(int(n), 0) for n in group_lens]
+    padded = [(n + align - 1) // align * align for n in lens]
+    total = sum(padded)
+    out_rows = total if out_rows is None else int(out_rows)
+    assert out_rows >= total
+    out = np.zeros((out_rows,) + x.shape[1:], dtype=x.dtype)
+    src = dst = 0
+    for n, m in zip(lens, padded):
+        out[dst:dst + n] = x[src:src + n]
+        src += n
+        dst += m
+    padded[-1] += out_rows - total
+    return out, np.asarray(padded, dtype=np.int64)
+
+
+def unpad_groups(y: np.ndarray, group_lens, align: int, rows=None) -> np.ndarray:
+    """Inverse of ``pad_groups`` (experts.py:262-264): the first ``len`` rows of every padded group, back to back;
+    rows of the result behind ``sum(group_lens)`` are zero."""
+    lens = [max(int(n), 0) for n in group_lens]
+    rows = sum(lens) if rows is None else int(rows)
+    out = np.zeros((rows,) + y.shape[1:], dtype=y.dtype)
+    src = dst = 0
+    for n in lens:
+        out[dst:dst + n] = y[src:src + n]
+        dst += n
+        src += (n + align - 1) // align * align
+    return out

@@ -60,6 +60,9 @@ EXPORTS = (
     "mxl_quantize_weight_tensorwise",
     "mxl_grouped_gemm_nt_scaled",
     "mxl_grouped_gemm_wgrad_scaled",
+    "mxl_padded_rows_bound",
+    "mxl_pad_groups",
+    "mxl_unpad_groups",
 )
 
 
@@ -143,6 +146,12 @@ def load() -> ctypes.CDLL:
         lib.mxl_grouped_gemm_nt_scaled.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp, vp, u32, vp]
         lib.mxl_grouped_gemm_wgrad_scaled.restype = i32
         lib.mxl_grouped_gemm_wgrad_scaled.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp, vp, u32, vp]
+        lib.mxl_padded_rows_bound.restype = i64
+        lib.mxl_padded_rows_bound.argtypes = [i64, i32, i32]
+        lib.mxl_pad_groups.restype = i32
+        lib.mxl_pad_groups.argtypes = [vp, i64, i64, vp, i32, i32, vp, i64, vp, vp]
+        lib.mxl_unpad_groups.restype = i32
+        lib.mxl_unpad_groups.argtypes = [vp, i64, i64, vp, i32, i32, vp, i64, vp]
         _lib = lib
     return _lib
 

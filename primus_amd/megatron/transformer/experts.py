@@ -163,8 +163,19 @@ class PrimusGroupedMLP(torch.nn.Module):
     def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor,
                 permuted_probs: torch.Tensor) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         pad = self._use_explicit_quantization_padding()
-        if pad:
-            # the only host read-back of the path; the router-side padding or the ragged GEMMs avoid it
+        on_device = pad and tokens_per_expert.is_cuda
+        if on_device:
+            # the counts stay on the device: both tensors go into buffers sized for the worst case, whose zero rows
+            # behind the last expert's padding count as that expert's (no host read-back, unlike the reference)
+            from ...pytorch import ops
+
+            actual_rows = permuted_local_hidden_states.shape[0]
+            actual = tokens_per_expert.to(torch.int64).contiguous()
+            align = get_align_size_for_quantization(self.config)
+            permuted_local_hidden_states, tokens_per_expert = ops.pad_groups(permuted_local_hidden_states, actual, align)
+            permuted_probs, _ = ops.pad_groups(permuted_probs.unsqueeze(-1), actual, align)
+        elif pad:
+            # counts that already live on the host: the reference's sequence as it stands
             actual: List[int] = [int(v) for v in tokens_per_expert.tolist()]
             permuted_local_hidden_states, padded = self.quantization_padding(permuted_local_hidden_states, actual)
             permuted_probs, _ = self.quantization_padding(permuted_probs.unsqueeze(-1), actual)
@@ -188,6 +199,8 @@ class PrimusGroupedMLP(torch.nn.Module):
         else:
             act = self.bias_act_func_with_mask(fc1_output, bias1, permuted_probs, tokens_per_expert)
             output, _ = self.linear_fc2(act, tokens_per_expert)
-        if pad:
+        if on_device:
+            output = ops.unpad_groups(output, actual, align, actual_rows)
+        elif pad:
             output = self.quantization_unpadding(output, actual)
         return output, None

@@ -903,6 +903,58 @@ def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCAL
 # --------------------------------------------------------------------------
 # reference-named low-level entry points (MX granularity only)
 # --------------------------------------------------------------------------
+# --------------------------------------------------------------------------
+# expert groups padded to the quantisation alignment
+# --------------------------------------------------------------------------
+def padded_rows_bound(rows: int, groups: int, align: int) -> int:
+    """Rows of the buffer ``pad_groups_impl`` fills: the largest total the counts can produce."""
+    return (rows + groups * (align - 1)) // align * align
+
+
+def _pad_args(x, group_lens, align):
+    _require_cuda(x, group_lens)
+    if x.dim() < 1 or not x.is_contiguous():
+        raise ValueError("x must be a contiguous tensor with the rows of the groups along dim 0")
+    if int(align) < 1:
+        raise ValueError("align must be positive")
+    groups = _check_group_lens(group_lens, x.device)
+    if groups > 1024:
+        raise ValueError("at most 1024 groups")
+    row_bytes = x.element_size()
+    for d in x.shape[1:]:
+        row_bytes *= int(d)
+    if row_bytes < 1:
+        raise ValueError("rows must not be empty")
+    return groups, row_bytes
+
+
+def pad_groups_impl(x, group_lens, align: int):
+    """``(padded, padded_lens)``: each group's rows of ``x`` followed by zero rows up to a multiple of ``align``
+    (experts.py:196-209 without the host read of the counts).  ``padded`` has ``padded_rows_bound`` rows; the zero
+    rows behind the last group's padding are counted into ``padded_lens[-1]``."""
+    groups, row_bytes = _pad_args(x, group_lens, align)
+    rows = x.shape[0]
+    out_rows = padded_rows_bound(rows, groups, int(align))
+    out = torch.empty((out_rows,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+    padded_lens = torch.empty_like(group_lens)
+    with _hooked("pad_groups", rows=rows, out_rows=out_rows, row_bytes=row_bytes):
+        rc = _lib.load().mxl_pad_groups(_ptr(x), rows, row_bytes, _ptr(group_lens), groups, int(align), _ptr(out),
+                                        out_rows, _ptr(padded_lens), _stream())
+    _lib.check(rc, "mxl_pad_groups")
+    return out, padded_lens
+
+
+def unpad_groups_impl(y, group_lens, align: int, rows: int):
+    """Inverse of ``pad_groups_impl`` (experts.py:262-264): ``[rows, ...]`` from the padded ``y``."""
+    groups, row_bytes = _pad_args(y, group_lens, align)
+    out = torch.empty((int(rows),) + tuple(y.shape[1:]), dtype=y.dtype, device=y.device)
+    with _hooked("unpad_groups", rows=int(rows), padded_rows=y.shape[0], row_bytes=row_bytes):
+        rc = _lib.load().mxl_unpad_groups(_ptr(y), y.shape[0], row_bytes, _ptr(group_lens), groups, int(align),
+                                          _ptr(out), int(rows), _stream())
+    _lib.check(rc, "mxl_unpad_groups")
+    return out
+
+
 def _require_mx(granularity) -> None:
     val = getattr(granularity, "value", granularity)
     if val != ScalingGranularity.MX_BLOCKWISE.value:

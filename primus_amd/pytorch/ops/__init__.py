@@ -37,7 +37,7 @@ from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
 __all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
            "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask", "glu_grouped_gemm_fp8",
-           "glu_grouped_gemm_fp4", "manual_sr_seed", "set_kchunk_layout", "rmsnorm", "rmsnorm_gemm_fp8", "rmsnorm_gemm_fp4"]
+           "glu_grouped_gemm_fp4", "manual_sr_seed", "set_kchunk_layout", "rmsnorm", "rmsnorm_gemm_fp8", "rmsnorm_gemm_fp4", "pad_groups", "unpad_groups"]
 
 # dgrad and wgrad of one linear are independent once dY is quantised.  Both GEMMs are persistent
 # kernels with one workgroup per CU, so launching wgrad on a second stream lets its workgroups move in
@@ -669,3 +669,48 @@ def swiglu_with_probs(x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[t
 def geglu_with_probs(x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Same with the (erf) GELU as the gate activation."""
     return _glu_with_probs(x, probs, row_mask, "gelu")
+
+
+class _PadGroups(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, group_lens, align):
+        out, padded_lens = K.pad_groups_impl(x.contiguous(), group_lens, align)
+        ctx.save_for_backward(group_lens)
+        ctx.align, ctx.rows = align, x.shape[0]
+        ctx.mark_non_differentiable(padded_lens)
+        return out, padded_lens
+
+    @staticmethod
+    def backward(ctx, dout, _):
+        (group_lens,) = ctx.saved_tensors
+        return K.unpad_groups_impl(dout.contiguous(), group_lens, ctx.align, ctx.rows), None, None
+
+
+class _UnpadGroups(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, y, group_lens, align, rows):
+        ctx.save_for_backward(group_lens)
+        ctx.align, ctx.padded_rows = align, y.shape[0]
+        return K.unpad_groups_impl(y.contiguous(), group_lens, align, rows)
+
+    @staticmethod
+    def backward(ctx, dout):
+        (group_lens,) = ctx.saved_tensors
+        dy, _ = K.pad_groups_impl(dout.contiguous(), group_lens, ctx.align)
+        assert dy.shape[0] == ctx.padded_rows, "unpad_groups takes the buffer pad_groups made for the same counts"
+        return dy, None, None, None
+
+
+def pad_groups(x: torch.Tensor, group_lens: torch.Tensor, align: int):
+    """``(padded, padded_lens)``: the rows of every expert followed by zero rows up to a multiple of ``align``,
+    with the counts staying on the device (the reference reads them back and concatenates per expert,
+    experts.py:196-209).  ``padded`` is sized for the worst case, ``(rows + G * (align - 1)) // align * align`` rows;
+    the zero rows behind the last expert's padding count into ``padded_lens[-1]``, so ``padded_lens`` always
+    describes the whole buffer.  Differentiable in ``x``."""
+    return _PadGroups.apply(x, group_lens, int(align))
+
+
+def unpad_groups(y: torch.Tensor, group_lens: torch.Tensor, align: int, rows: int) -> torch.Tensor:
+    """The ``rows`` live rows of a buffer made by ``pad_groups`` for the same counts (experts.py:262-264).
+    Differentiable in ``y``: padding rows get a zero gradient."""
+    return _UnpadGroups.apply(y, group_lens, int(align), int(rows))

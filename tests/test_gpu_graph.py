@@ -169,3 +169,73 @@ def test_tensorwise_norm_and_fused_accumulation_replay(gpu, recipe):
         for a, b in zip(got, want):
             assert _same(a, b), (new_lens, seed)
         assert got[-1].abs().sum() > 0
+
+
+def test_expert_mlp_with_explicit_padding_replays_with_new_routing(gpu):
+    """The expert MLP on its explicit-padding route (groups padded to 32 rows on the device, fc1, the activation, fc2,
+    unpadding) captured once and replayed with other tokens and other tokens-per-expert: nothing in it reads the
+    counts on the host."""
+    from types import SimpleNamespace
+
+    from primus_amd.megatron import runtime
+    from primus_amd.megatron.extensions import primus_turbo as pt
+    from primus_amd.megatron.transformer.experts import PrimusGroupedMLP
+    from primus_amd.pytorch.core import Format, ScaleDtype, ScalingGranularity
+
+    pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+    runtime.bind()
+    runtime.set_num_microbatches(1)
+    runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                     turbo_grouped_gemm_without_padding=False, use_turbo_fused_act_with_probs=True)
+    try:
+        torch.manual_seed(23)
+        cfg = SimpleNamespace(params_dtype=torch.bfloat16, use_cpu_initialization=False, perform_initialization=True,
+                              tensor_model_parallel_size=1, gradient_accumulation_fusion=False, normalization="RMSNorm",
+                              layernorm_epsilon=1e-5, hidden_size=256, ffn_hidden_size=384, moe_ffn_hidden_size=384,
+                              gated_linear_unit=True, fp8="e4m3", fp8_recipe="mxfp8", fp4=None, add_bias_linear=False)
+        mlp = PrimusGroupedMLP(4, cfg)
+        assert mlp._use_explicit_quantization_padding()
+        qc = pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.MX_BLOCKWISE, format=Format.E4M3, block_size=32,
+                                       scale_dtype=ScaleDtype.E8M0)
+        rows = 500
+        gen = torch.Generator().manual_seed(4)
+        x = torch.randn(rows, 256, generator=gen).bfloat16().to(gpu).requires_grad_()
+        probs = torch.rand(rows, generator=gen).to(gpu).requires_grad_()
+        dy = torch.randn(rows, 256, generator=gen).bfloat16().to(gpu)
+        lens = torch.tensor([100, 0, 143, 257], dtype=torch.int64, device=gpu)
+        params = [mlp.linear_fc1.weights, mlp.linear_fc2.weights]
+
+        def step():
+            for lin in (mlp.linear_fc1, mlp.linear_fc2):
+                lin.set_is_first_microbatch()
+            with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc):
+                y, _ = mlp(x, lens, probs)
+            return (y,) + torch.autograd.grad(y, [x, probs] + params, dy)
+
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            step()
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = step()
+        for new_lens, seed in [([100, 0, 143, 257], 1), ([0, 0, 0, 500], 2), ([125, 125, 125, 125], 3), ([499, 1, 0, 0], 4)]:
+            g2 = torch.Generator().manual_seed(seed)
+            with torch.no_grad():
+                x.copy_(torch.randn(rows, 256, generator=g2).bfloat16())
+                probs.copy_(torch.rand(rows, generator=g2))
+                dy.copy_(torch.randn(rows, 256, generator=g2).bfloat16())
+                lens.copy_(torch.tensor(new_lens, dtype=torch.int64))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [t.clone() for t in outs]
+            want = step()
+            torch.cuda.synchronize()
+            for a, b in zip(got, want):
+                assert _same(a, b), (new_lens, seed)
+            assert got[0].abs().sum() > 0
+    finally:
+        pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+        runtime.set_args()

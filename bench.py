@@ -175,7 +175,20 @@ def cpu_baseline(spec, lens, sample_div=16):
             del y, dx, dw
             flops += 6.0 * slens[e] * n * k
     dt_s = time.perf_counter() - t0
+    # the reference's own CPU-runnable case at full size: X [4096, 4096] ~ N(0, 1), W [4096, 4096] ~ N(0, 0.02),
+    # MXFP8 quantise both, dequantise, fp32 matmul, bf16 output (forward only)
+    g1 = torch.Generator().manual_seed(1001)
+    x1 = o.to_bf16_bits(torch.randn(4096, 4096, generator=g1).bfloat16())
+    w1 = o.to_bf16_bits((torch.randn(4096, 4096, generator=g1) * 0.02).bfloat16())
+    t1 = time.perf_counter()
+    xq1, xs1 = C.quantize_rowwise(x1, o.FMT_E4M3)
+    wq1, ws1, _, _ = C.quantize_2d(w1[None], o.FMT_E4M3)
+    y1 = (torch.from_numpy(C.dequantize(xq1, xs1, o.FMT_E4M3)) @ torch.from_numpy(C.dequantize(wq1[0], ws1[0], o.FMT_E4M3)).t()).bfloat16()
+    cfg1_s = time.perf_counter() - t1
+    del y1
     return {
+        "cfg1_dense_4096": {"value": round(2.0 * 4096 ** 3 / cfg1_s / 1e12, 6), "unit": "TFLOP/s", "seconds": round(cfg1_s, 3),
+                            "sample": "full size: quantise X and W (C oracle), dequantise, torch CPU fp32 matmul, bf16 output"},
         "value": round(flops / dt_s / 1e12, 6),
         "unit": "TFLOP/s",
         "cores": threads,
@@ -183,6 +196,52 @@ def cpu_baseline(spec, lens, sample_div=16):
         "sample": f"same workload with tokens-per-expert divided by {sample_div} ({m} routed rows), full-size weights; "
         f"C oracle quantise/dequantise + torch CPU fp32 matmul; {dt_s:.1f} s",
     }
+
+
+def board_sample(run_step, seconds):
+    """Socket power and shader clocks (``amd-smi metric --power --clock``) sampled while ``run_step`` loops for
+    ``seconds``: says how far below the 2.4 GHz that the MFMA peak is quoted at the chip clocks under this load.
+    None when the tool is missing or prints something else."""
+    import subprocess
+    import threading
+
+    import torch
+
+    rows, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                r = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--csv"], capture_output=True, text=True, timeout=10)
+                lines = [ln for ln in r.stdout.strip().splitlines() if ln.strip()]
+                head, vals = lines[0].split(","), lines[1].split(",")
+                rows.append(dict(zip(head, vals)))
+            except Exception:
+                return
+            time.sleep(0.05)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    t_end = time.perf_counter() + seconds
+    run_step()
+    torch.cuda.synchronize()
+    th.start()
+    while time.perf_counter() < t_end:
+        run_step()
+        torch.cuda.synchronize()
+    stop.set()
+    th.join(timeout=15)
+    try:
+        # the first and the last sample may straddle the loop's ends
+        use = rows[1:-1] if len(rows) > 3 else rows
+        power = [float(r["socket_power"]) for r in use]
+        clocks = [float(v) for r in use for k, v in r.items() if k.startswith("gfx_") and k.endswith("_clk") and k.count("_") == 2]
+        if not power or not clocks:
+            return None
+        return {"socket_power_w": round(sum(power) / len(power), 1), "gfx_clk_mhz_mean": round(sum(clocks) / len(clocks), 1),
+                "gfx_clk_mhz_min": min(clocks), "gfx_clk_mhz_max": max(clocks), "gfx_clk_mhz_peak": 2400.0,
+                "samples": len(use), "seconds": seconds, "source": "amd-smi metric --power --clock, sampled while the step loops"}
+    except Exception:
+        return None
 
 
 def main():
@@ -194,6 +253,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-wgrad-overlap", action="store_true",
                     help="keep wgrad on the launch stream behind dgrad (per-kernel durations are then undisturbed)")
+    ap.add_argument("--board-seconds", type=float, default=2.0,
+                    help="after the timed region, loop the step for this long while sampling socket power and shader "
+                         "clocks with amd-smi (0: skip)")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="launch one plain 1 GiB-in / 1 GiB-out elementwise kernel first, so that a hardware-counter "
                          "run of this command also reads the counters for a kernel of known HBM traffic")
@@ -371,6 +433,9 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
     }
+    if args.board_seconds > 0:
+        pt.ops.set_wgrad_overlap(not args.no_wgrad_overlap)
+        out["board"] = board_sample(step, args.board_seconds)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(spec, lens)
     print(json.dumps(out))

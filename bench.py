@@ -49,12 +49,13 @@ WORKLOADS = {
 }
 
 
-# HBM bytes per launch of the forward/dgrad grouped GEMM, measured with hardware counters
-# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; KiB per dispatch averaged over the four launches of a
-# step, each scaled by what the same counter reads for a 1 GiB -> 1 GiB elementwise kernel: 2.000 and
-# 1.000).  The counter summary is committed as profiles/bench_mixtral_mxfp8_hbm_traffic.txt.
+# Bytes per launch that cross between the L2s and the memory side (memory-side cache or HBM) for the forward/dgrad
+# grouped GEMM, measured with hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; KiB per dispatch
+# averaged over the four launches of a step, each scaled by what the same counter reads for a 1 GiB -> 1 GiB
+# elementwise kernel: 2.000 and 1.000).  The counter summary is committed as
+# profiles/bench_mixtral_mxfp8_hbm_traffic.txt.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "mixtral_8x7b_moe_mxfp8": (2802905.4 * 2.000 + 836113.3 * 1.000) * 1024,
+    "mixtral_8x7b_moe_mxfp8": (3257550.1 * 2.000 + 826636.6 * 1.000) * 1024,
 }
 
 
@@ -377,8 +378,10 @@ def main():
     gk = acc[fwd_name]
     gemm_tflops = gk["flops"] / gk["sec"] / 1e12
     roofline = {
-        "kernel": "mx_gemm_kernel<%s,%s,fwd/dgrad%s> (%s)" % ("e4m3|e5m2" if spec.get("tensorwise") else "e4m3", "e2m1" if spec["fp4"] else "e4m3",
-                                                               ",alpha" if spec.get("tensorwise") else "", fwd_name),
+        # MXFP8 x MXFP8 operands run on the 4-slot ring kernel; FP4 operands and the tensor-wise recipe on the 2-slot kernel
+        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_kernel" if spec["fp4"] or spec.get("tensorwise") else "mx_gemm_ring_kernel",
+                                                   "e4m3|e5m2" if spec.get("tensorwise") else "e4m3", "e2m1" if spec["fp4"] else "e4m3",
+                                                   ",alpha" if spec.get("tensorwise") else "", fwd_name),
         "bound": "mfma",
         "achieved": round(gemm_tflops, 2),
         "peak": FP8_PEAK_TFLOPS,

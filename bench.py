@@ -436,6 +436,25 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
     }
+    # what a plain streaming kernel reaches on this board: 1 GiB read + 1 GiB written by torch's elementwise add,
+    # the practical ceiling the quantisers' GB/s are to be read against (their HBM traffic is the algorithmic one)
+    src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        torch.add(src, 1, out=dst)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        torch.add(src, 1, out=dst)
+    e1.record()
+    torch.cuda.synchronize()
+    stream_gbs = 10 * 2.0 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del src, dst
+    out["hbm_stream_calibration"] = {"kernel": "torch.add(int32[2^28], 1, out=...): 1 GiB read, 1 GiB written", "GB/s": round(stream_gbs, 1),
+                                     "frac_hbm_peak": round(stream_gbs / HBM_PEAK_GBS, 4)}
+    for name in ("quantize", "quantize_weight_2d"):
+        if name in kernels and "GB/s" in kernels[name]:
+            kernels[name]["frac_of_stream_calibration"] = round(kernels[name]["GB/s"] / stream_gbs, 4)
     if args.board_seconds > 0:
         pt.ops.set_wgrad_overlap(not args.no_wgrad_overlap)
         out["board"] = board_sample(step, args.board_seconds)

@@ -99,6 +99,16 @@ Parity status
   padding in a buffer sized for the worst case (zero rows counted into the last group) have no counterpart in
   the reference, whose buffer has the exact size because it reads the counts on the host.
 
+* ``quantize_blockwise`` / ``quantize_blockwise_2d`` / ``blockwise_gemm_nt_ref`` (the 128-blockwise FP8 recipe:
+  operand flow at primus_turbo_float8_local.py:1019-1087, admitted by rocm_arg_validation.py:145): per block the
+  formula the reference restates for its tensor-wise quantiser (:194-207), scale = fp8_max / max(amax, 1e-12),
+  codes = cast(clamp(x * scale)), scale_inv = 1 / scale in float32; the GEMM adds the K blocks' float32 partial
+  products times both blocks' scale_inv.  Pinned in tests/ against the same formula evaluated with torch ops on
+  reshaped blocks and torch's float8 casts (library routines), by "one block == the tensor-wise quantiser", block
+  independence and the dequantisation error bound; the GEMM against float64 arithmetic on the decoded operands.
+  The Primus-Turbo ops behind ``quant_fp8_blockwise_impl`` are absent: whether they use this formula or another
+  (e.g. amax / fp8_max without the clamp at 1e-12) is **parity unpinned**.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -861,3 +871,71 @@ def unpad_groups(y: np.ndarray, group_lens, align: int, rows=None) -> np.ndarray
         dst += n
         src += (n + align - 1) // align * align
     return out
+
+
+# --------------------------------------------------------------------------
+# the 128-blockwise FP8 recipe
+# --------------------------------------------------------------------------
+BW_BLOCK = 128
+
+
+def _quantize_blocks(xf: np.ndarray, amax: np.ndarray, fmt: int):
+    """codes of xf and scale_inv per entry of amax (broadcastable to xf): the tensor-wise formula per block."""
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        scale = (np.float32(_FP8_MAX[fmt]) / np.maximum(amax.astype(np.float32), np.float32(1e-12))).astype(np.float32)
+        scale_inv = (np.float32(1.0) / scale).astype(np.float32)
+        y = (xf * scale).astype(np.float32)
+    codes = cast_e5m2(y) if fmt == FMT_E5M2 else cast_e4m3(y)
+    codes = np.where(np.isfinite(np.broadcast_to(amax, xf.shape)), codes, np.uint8(0x7F)).astype(np.uint8)
+    return codes, scale_inv
+
+
+def quantize_blockwise(x, fmt: int = FMT_E4M3, axis: int = -1, block: int = BW_BLOCK):
+    """quant_fp8_blockwise_impl(x, dtype, axis, block_size) (primus_turbo_float8_local.py:1019, :1053-1059):
+    1-D blocks of ``block`` along ``axis`` of the 2-D ``x``.
+    axis -1 / 1: ``(codes [rows, cols], scale_inv [rows, cols / block])``; cols must be a multiple of the block.
+    axis -2 / 0: blocks along the rows, returned TRANSPOSED and zero-padded as the NT GEMM consumes the copy:
+    ``(codes [cols, rows_pad], scale_inv [cols, rows_pad / block])``; a block that reaches past the last row takes its
+    scale from the rows it has."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x))
+    rows, cols = xf.shape
+    if axis in (-2, 0):
+        pad = (-rows) % block
+        xt = np.concatenate([xf, np.zeros((pad, cols), np.float32)]).T.copy()      # [cols, rows_pad]
+        return quantize_blockwise(f32_to_bf16_bits(xt), fmt, -1, block)
+    assert cols % block == 0
+    blocks = xf.reshape(rows, cols // block, block)
+    amax = np.abs(blocks).max(axis=2, keepdims=True)
+    codes, scale_inv = _quantize_blocks(blocks, amax, fmt)
+    return codes.reshape(rows, cols), scale_inv.reshape(rows, cols // block)
+
+
+def quantize_blockwise_2d(w, fmt: int = FMT_E4M3, block: int = BW_BLOCK):
+    """quant_fp8_blockwise_for_weight_impl (primus_turbo_float8_local.py:1020, :1060): one scale per block x block
+    tile of ``w [n, k]``.  ``(codes [n, k], scale_inv [n / block, k / block], codes_T [k, n], scale_inv_T)``."""
+    wf = bf16_bits_to_f32(to_bf16_bits(w))
+    n, k = wf.shape
+    assert n % block == 0 and k % block == 0
+    tiles = wf.reshape(n // block, block, k // block, block)
+    amax = np.abs(tiles).max(axis=(1, 3), keepdims=True)
+    codes, scale_inv = _quantize_blocks(tiles, amax, fmt)
+    codes = codes.reshape(n, k)
+    scale_inv = scale_inv.reshape(n // block, k // block)
+    return codes, scale_inv, codes.T.copy(), scale_inv.T.copy()
+
+
+def blockwise_gemm_nt_ref(a_codes, a_sinv, b_codes, b_sinv, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, block: int = BW_BLOCK, out_bf16=True):
+    """c[m, n] = sum over K blocks of a_sinv[m, kb] * b_sinv[n (or n / block), kb] * (a[m, kb] . b[n, kb]) in float32
+    (gemm_fp8_impl with blockwise granularity, primus_turbo_float8_local.py:1022-1033).  ``b_sinv`` has one row per
+    row of b or one per ``block`` rows (weights)."""
+    a = decode_fp8(a_codes, a_fmt)
+    b = decode_fp8(b_codes, b_fmt)
+    m, k = a.shape
+    n = b.shape[0]
+    sb = np.repeat(b_sinv, block, axis=0) if b_sinv.shape[0] != n else b_sinv
+    acc = np.zeros((m, n), np.float32)
+    for kb in range(k // block):
+        sl = slice(kb * block, (kb + 1) * block)
+        part = _matmul_nt_f32(a[:, sl], b[:, sl])
+        acc = (acc + part * (a_sinv[:, kb][:, None] * sb[:, kb][None, :]).astype(np.float32)).astype(np.float32)
+    return f32_to_bf16_bits(acc) if out_bf16 else acc

@@ -516,7 +516,10 @@ class _LowPrecisionGemm:
             assert qc.mxfp8_scaling() or qc.current_scaling() or qc.block_scaling(), (
                 "Turbo FP8 is enabled but quant config is not mxfp8, current scaling, or block scaling."
             )
-            if one_microbatch:
+            # the 128-blockwise operator quantises from the bf16 weight at every call, whatever the number of
+            # microbatches (same codes as a cached copy; its backward needs the bf16 weight for the other format anyway,
+            # primus_turbo_float8_local.py:1059-1062)
+            if one_microbatch or qc.block_scaling():
                 return run(ops.gemm_fp8, ops.grouped_gemm_fp8, x, weight,
                            _fuse_wgrad_accum_pattern(self.config, weight), config=qc.data())
             x, pair, fuse_pattern = self._quantized(

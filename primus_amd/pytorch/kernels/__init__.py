@@ -955,6 +955,102 @@ def unpad_groups_impl(y, group_lens, align: int, rows: int):
     return out
 
 
+# --------------------------------------------------------------------------
+# the 128-blockwise FP8 recipe
+# --------------------------------------------------------------------------
+BW_BLOCK = 128
+
+
+def _bw_check(x, fmt, what):
+    _require_cuda(x)
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError(f"{what} must be a contiguous 2-D bfloat16 tensor")
+    if fmt not in (_lib.FMT_E4M3, _lib.FMT_E5M2):
+        raise ValueError("blockwise scaling is defined for the FP8 formats E4M3 and E5M2")
+    if x.shape[1] % BW_BLOCK != 0:
+        raise ValueError(f"the blockwise recipe needs the last dimension to be a multiple of {BW_BLOCK} (got {x.shape[1]})")
+
+
+def quantize_blockwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool = False):
+    """``quant_fp8_blockwise_impl`` for both axes in one launch (primus_turbo_float8_local.py:1019, :1053-1059):
+    ``(codes [rows, cols], scale_inv f32 [rows, cols / 128], codes_T [cols, rows_pad], scale_inv_T f32
+    [cols, rows_pad / 128])``; the row-wise copy has 1 x 128 blocks along the columns, the transposed one 128 x 1
+    blocks along the rows (``rows_pad``: rows rounded up to 128, zero codes).  Copies not asked for are None."""
+    _bw_check(x, fmt, "x")
+    if not (rowwise or colwise):
+        raise ValueError("at least one copy must be requested")
+    rows, cols = x.shape
+    rows_pad = _round_up(rows, BW_BLOCK)
+    dt = _code_dtype(fmt) if fmt != _lib.FMT_E5M2 else torch.float8_e5m2
+    q = s = qt = st = None
+    if rowwise:
+        q = torch.empty((rows, cols), dtype=torch.uint8, device=x.device)
+        s = torch.empty((rows, cols // BW_BLOCK), dtype=torch.float32, device=x.device)
+    if colwise:
+        qt = torch.empty((cols, rows_pad), dtype=torch.uint8, device=x.device)
+        st = torch.empty((cols, rows_pad // BW_BLOCK), dtype=torch.float32, device=x.device)
+    with _hooked("quantize_blockwise", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
+        rc = _lib.load().mxl_quantize_blockwise(_ptr(x), rows, cols, fmt, _ptr(q), _ptr(s), _ptr(qt), _ptr(st), _stream())
+    _lib.check(rc, "mxl_quantize_blockwise")
+    return (q.view(dt) if q is not None else None), s, (qt.view(dt) if qt is not None else None), st
+
+
+def quantize_blockwise_weight_impl(w, fmt: int, *, rowwise: bool = True, colwise: bool = False):
+    """``quant_fp8_blockwise_for_weight_impl`` (primus_turbo_float8_local.py:1020, :1060): one scale per 128 x 128
+    block of ``w [n, k]``.  ``(codes [n, k], scale_inv f32 [n / 128, k / 128], codes_T [k, n], scale_inv_T)``."""
+    _bw_check(w, fmt, "w")
+    n, k = w.shape
+    if n % BW_BLOCK != 0:
+        raise ValueError(f"the blockwise recipe needs weight dimensions that are multiples of {BW_BLOCK} (got {n})")
+    if not (rowwise or colwise):
+        raise ValueError("at least one copy must be requested")
+    dt = _code_dtype(fmt) if fmt != _lib.FMT_E5M2 else torch.float8_e5m2
+    q = s = qt = st = None
+    if rowwise:
+        q = torch.empty((n, k), dtype=torch.uint8, device=w.device)
+        s = torch.empty((n // BW_BLOCK, k // BW_BLOCK), dtype=torch.float32, device=w.device)
+    if colwise:
+        qt = torch.empty((k, n), dtype=torch.uint8, device=w.device)
+        st = torch.empty((k // BW_BLOCK, n // BW_BLOCK), dtype=torch.float32, device=w.device)
+    with _hooked("quantize_blockwise_weight", rows=n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
+        rc = _lib.load().mxl_quantize_blockwise_weight(_ptr(w), n, k, fmt, _ptr(q), _ptr(s), _ptr(qt), _ptr(st), _stream())
+    _lib.check(rc, "mxl_quantize_blockwise_weight")
+    return (q.view(dt) if q is not None else None), s, (qt.view(dt) if qt is not None else None), st
+
+
+def _fp8_fmt_of(codes: torch.Tensor) -> int:
+    if codes.dtype == torch.float8_e5m2:
+        return _lib.FMT_E5M2
+    if codes.dtype in (torch.float8_e4m3fn, torch.uint8):
+        return _lib.FMT_E4M3
+    raise ValueError(f"not an FP8 code tensor: {codes.dtype}")
+
+
+def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv) -> torch.Tensor:
+    """``gemm_fp8_impl(..., granularity=BLOCKWISE)`` in NT form (primus_turbo_float8_local.py:1022-1033):
+    ``c[m, n] = sum_kb a_scale_inv[m, kb] * b_scale_inv[n or n / 128, kb] * (a[m, kb] . b[n, kb])``, bf16.
+    ``b_scale_inv`` has one row per row of ``b`` (an activation copy) or one per 128 rows (a weight)."""
+    _require_cuda(a, a_scale_inv, b, b_scale_inv)
+    m, k = a.shape
+    n = b.shape[0]
+    if b.shape[1] != k or k % BW_BLOCK != 0 or n % BW_BLOCK != 0:
+        raise ValueError("blockwise GEMM: contraction lengths must agree and k, n must be multiples of 128")
+    kb = k // BW_BLOCK
+    if a_scale_inv.dtype != torch.float32 or tuple(a_scale_inv.shape) != (m, kb) or not a_scale_inv.is_contiguous():
+        raise ValueError("a_scale_inv must be contiguous float32 [m, k / 128]")
+    if b_scale_inv.dtype != torch.float32 or not b_scale_inv.is_contiguous() or tuple(b_scale_inv.shape) not in ((n, kb), (n // BW_BLOCK, kb)):
+        raise ValueError("b_scale_inv must be contiguous float32 [n, k / 128] or [n / 128, k / 128]")
+    per = 1 if (b_scale_inv.shape[0] == n and n != n // BW_BLOCK) else BW_BLOCK
+    if not (a.is_contiguous() and b.is_contiguous()):
+        raise ValueError("code tensors must be contiguous")
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    with _hooked("gemm_blockwise_nt", m=m, n=n, k=k):
+        rc = _lib.load().mxl_gemm_nt_blockwise(_ptr(a), _ptr(a_scale_inv), _fp8_fmt_of(a), _ptr(b), _ptr(b_scale_inv),
+                                               _fp8_fmt_of(b), per, _ptr(c), m, n, k, _stream())
+    _lib.check(rc, "mxl_gemm_nt_blockwise")
+    return c
+
+
 def _require_mx(granularity) -> None:
     val = getattr(granularity, "value", granularity)
     if val != ScalingGranularity.MX_BLOCKWISE.value:

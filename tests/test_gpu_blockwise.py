@@ -1,0 +1,207 @@
+"""The 128-blockwise FP8 recipe on the GPU through the C-ABI: the quantisers' codes and reciprocal scales against the
+oracle bit for bit (1 x 128 blocks, the transposed 128 x 1 copy, 128 x 128 weight blocks; E4M3 and E5M2), the GEMM
+against the oracle within one bf16 rounding plus the float32 accumulation bound, and the operator / Megatron module
+under the recipe against bf16 arithmetic."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as o
+
+pytestmark = pytest.mark.gpu
+DT = {0: torch.float8_e4m3fn, 2: torch.float8_e5m2}
+
+
+def _u8(t):
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def _f(t):
+    return o.bf16_bits_to_f32(t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16))
+
+
+def _x(seed, rows, cols, spread=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(rows, cols, generator=g) * spread * torch.logspace(-2, 1, cols)[None, :]).bfloat16()
+
+
+@pytest.mark.parametrize("fmt", [0, 2])
+@pytest.mark.parametrize("rows,cols", [(1, 128), (37, 256), (128, 128), (200, 384), (513, 1024)])
+def test_quantiser_equals_the_oracle(gpu, fmt, rows, cols):
+    from primus_amd.pytorch import kernels as K
+
+    x = _x(rows * 7 + cols + fmt, rows, cols, 2.0)
+    x[rows // 2, 3] = 0.0
+    q, s, qt, st = K.quantize_blockwise_impl(x.to(gpu), fmt, rowwise=True, colwise=True)
+    wq, ws = o.quantize_blockwise(x, fmt, axis=-1)
+    wqt, wst = o.quantize_blockwise(x, fmt, axis=0)
+    assert q.dtype == DT[fmt] and np.array_equal(_u8(q), wq) and np.array_equal(s.cpu().numpy(), ws)
+    assert tuple(qt.shape) == wqt.shape and np.array_equal(_u8(qt), wqt) and np.array_equal(st.cpu().numpy(), wst)
+    # one copy at a time gives the same bytes
+    q1, s1, n1, n2 = K.quantize_blockwise_impl(x.to(gpu), fmt, rowwise=True, colwise=False)
+    assert n1 is None and n2 is None and torch.equal(q1.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s1, s)
+    n1, n2, qt1, st1 = K.quantize_blockwise_impl(x.to(gpu), fmt, rowwise=False, colwise=True)
+    assert n1 is None and torch.equal(qt1.view(torch.uint8), qt.view(torch.uint8)) and torch.equal(st1, st)
+
+
+@pytest.mark.parametrize("fmt", [0, 2])
+@pytest.mark.parametrize("n,k", [(128, 128), (256, 384), (384, 1024)])
+def test_weight_quantiser_equals_the_oracle(gpu, fmt, n, k):
+    from primus_amd.pytorch import kernels as K
+
+    w = (_x(n + k + fmt, n, k) * 0.02).bfloat16()
+    q, s, qt, st = K.quantize_blockwise_weight_impl(w.to(gpu), fmt, rowwise=True, colwise=True)
+    wq, ws, wqt, wst = o.quantize_blockwise_2d(w, fmt)
+    assert np.array_equal(_u8(q), wq) and np.array_equal(s.cpu().numpy(), ws)
+    assert np.array_equal(_u8(qt), wqt) and np.array_equal(st.cpu().numpy(), wst)
+
+
+def test_zero_and_nonfinite_blocks(gpu):
+    from primus_amd.pytorch import kernels as K
+
+    x = torch.zeros(4, 256).bfloat16()
+    x[1, 130] = float("inf")
+    x[2, 5] = 3.0
+    x[3, 200] = float("nan")
+    q, s, _, _ = K.quantize_blockwise_impl(x.to(gpu), 0)
+    wq, ws = o.quantize_blockwise(x, 0)
+    assert np.array_equal(_u8(q), wq)
+    fin = np.ones((4, 2), bool)
+    fin[3, 1] = False                                        # the reciprocal scale of a block with a NaN is not specified
+    assert np.array_equal(s.cpu().numpy()[fin], ws[fin])
+
+
+def _bound(a_codes, sa, b_codes, sb, a_fmt, b_fmt, want32):
+    da = np.abs(o.decode_fp8(a_codes, a_fmt)).astype(np.float64) * np.repeat(np.abs(sa).astype(np.float64), 128, axis=1)
+    sbr = sb if sb.shape[0] == b_codes.shape[0] else np.repeat(sb, 128, axis=0)
+    db = np.abs(o.decode_fp8(b_codes, b_fmt)).astype(np.float64) * np.repeat(np.abs(sbr).astype(np.float64), 128, axis=1)
+    k = a_codes.shape[1]
+    return 2.0 ** -8 * np.abs(want32) + (k + 1024) * 2.0 ** -23 * (da @ db.T) + 1e-30
+
+
+@pytest.mark.parametrize("a_fmt,b_fmt", [(0, 0), (2, 2), (2, 0), (0, 2)])
+@pytest.mark.parametrize("m,n,k,per_row", [(70, 128, 128, False), (300, 256, 384, False), (129, 384, 1024, True), (1, 128, 256, True)])
+def test_gemm_against_the_oracle(gpu, a_fmt, b_fmt, m, n, k, per_row):
+    from primus_amd.pytorch import kernels as K
+
+    x = _x(m + n + k, m, k)
+    w = (_x(n * 3 + k, n, k) * 0.05).bfloat16()
+    a, sa = o.quantize_blockwise(x, a_fmt)
+    if per_row:
+        b, sb = o.quantize_blockwise(w, b_fmt)
+    else:
+        b, sb, _, _ = o.quantize_blockwise_2d(w, b_fmt)
+    want32 = o.blockwise_gemm_nt_ref(a, sa, b, sb, a_fmt, b_fmt, out_bf16=False)
+    dev = lambda arr, dt=None: (torch.from_numpy(arr).to(gpu) if dt is None else torch.from_numpy(arr).to(gpu).view(dt))
+    got = K.gemm_blockwise_nt_impl(dev(a, DT[a_fmt]), dev(sa), dev(b, DT[b_fmt]), dev(sb))
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (m, n)
+    err = np.abs(_f(got).astype(np.float64) - want32)
+    assert np.all(err <= _bound(a, sa, b, sb, a_fmt, b_fmt, want32))
+    assert err.max() <= 1e-2 * np.abs(want32).max()
+
+
+def test_gemm_is_exact_where_the_arithmetic_is(gpu):
+    """Small integers times power-of-two scales: every product and every sum is exact in float32 and in bf16."""
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator().manual_seed(5)
+    m, n, k = 200, 256, 512
+    a = torch.randint(-2, 3, (m, k), generator=g).float()
+    b = torch.randint(-2, 3, (n, k), generator=g).float()
+    sa = torch.tensor([0.5, 1.0, 2.0, 4.0])[torch.randint(0, 4, (m, k // 128), generator=g)]
+    sb = torch.tensor([0.25, 1.0, 2.0])[torch.randint(0, 3, (n // 128, k // 128), generator=g)]
+    want = ((a * sa.repeat_interleave(128, 1)) @ (b * sb.repeat_interleave(128, 0).repeat_interleave(128, 1)).t())
+    assert want.abs().max() < 256 * 128                      # stays on bf16's integer grid? checked below
+    got = K.gemm_blockwise_nt_impl(a.to(torch.float8_e4m3fn).to(gpu), sa.contiguous().to(gpu),
+                                   b.to(torch.float8_e4m3fn).to(gpu), sb.contiguous().to(gpu))
+    assert torch.equal(got.float().cpu(), want.bfloat16().float())
+
+
+def _cos(a, b):
+    return torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item()
+
+
+@pytest.mark.parametrize("hybrid", [False, True])
+def test_operator_forward_and_backward_follow_the_oracle_and_bf16(gpu, hybrid):
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import Float8QuantConfig, Format, ScalingGranularity
+
+    cfg = Float8QuantConfig(format=Format.HYBRID if hybrid else Format.E4M3, granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+    bwd = o.FMT_E5M2 if hybrid else o.FMT_E4M3
+    x = _x(1, 300, 256).to(gpu).requires_grad_()
+    w = (_x(2, 384, 256) * 0.05).bfloat16().to(gpu).requires_grad_()
+    dy = _x(3, 300, 384).to(gpu)
+    y = turbo.ops.gemm_fp8(x, w, config=cfg)
+    dx, dw = torch.autograd.grad(y, [x, w], dy)
+    # forward: X row-wise x W in 2-D blocks; dgrad: dY row-wise x W^T; wgrad: dY^T x X^T, blocks along the tokens
+    xa, xs = o.quantize_blockwise(x.detach().cpu(), o.FMT_E4M3)
+    wq, ws, _, _ = o.quantize_blockwise_2d(w.detach().cpu(), o.FMT_E4M3)
+    want_y = o.blockwise_gemm_nt_ref(xa, xs, wq, ws, out_bf16=False)
+    da, ds = o.quantize_blockwise(dy.cpu(), bwd)
+    _, _, wt, wts = o.quantize_blockwise_2d(w.detach().cpu(), bwd)
+    want_dx = o.blockwise_gemm_nt_ref(da, ds, wt, wts, bwd, bwd, out_bf16=False)
+    dt_, dts = o.quantize_blockwise(dy.cpu(), bwd, axis=0)
+    xt, xts = o.quantize_blockwise(x.detach().cpu(), bwd, axis=0)
+    want_dw = o.blockwise_gemm_nt_ref(dt_, dts, xt, xts, bwd, bwd, out_bf16=False)
+    for got, want in ((y, want_y), (dx, want_dx), (dw, want_dw)):
+        assert tuple(got.shape) == want.shape
+        assert np.abs(_f(got) - want).max() <= 1e-2 * np.abs(want).max()
+    xr, wr = x.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+    yr = xr @ wr.t()
+    dxr, dwr = torch.autograd.grad(yr, [xr, wr], dy)
+    bar = 0.99 if hybrid else 0.998
+    assert _cos(y, yr) > 0.998 and _cos(dx, dxr) > bar and _cos(dw, dwr) > bar
+
+
+def test_operator_refuses_what_the_recipe_does_not_cover(gpu):
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import Float8QuantConfig, Format, ScalingGranularity
+
+    cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+    x = torch.zeros(8, 96, device=gpu).bfloat16()
+    w = torch.zeros(128, 96, device=gpu).bfloat16()
+    with pytest.raises(ValueError):
+        turbo.ops.gemm_fp8(x, w, config=cfg)                       # K is not a multiple of 128
+    wg = torch.zeros(2, 128, 128, device=gpu).bfloat16()
+    with pytest.raises(NotImplementedError):
+        turbo.ops.grouped_gemm_fp8(torch.zeros(8, 128, device=gpu).bfloat16(), wg, torch.tensor([4, 4], device=gpu), config=cfg)
+
+
+@pytest.mark.parametrize("microbatches", [1, 2])
+def test_megatron_linear_under_the_blockwise_recipe(gpu, microbatches):
+    from types import SimpleNamespace
+
+    from primus_amd.megatron import runtime
+    from primus_amd.megatron.extensions import primus_turbo as pt
+    from primus_amd.pytorch.core import Format, ScalingGranularity
+
+    pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+    runtime.bind()
+    runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                     turbo_grouped_gemm_without_padding=True)
+    runtime.set_num_microbatches(microbatches)
+    try:
+        qc = pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.BLOCKWISE, format=Format.E4M3, block_size=128)
+        assert qc.block_scaling() and not qc.mxfp8_scaling() and not qc.current_scaling()
+        torch.manual_seed(3)
+        cfg = SimpleNamespace(params_dtype=torch.bfloat16, use_cpu_initialization=False, perform_initialization=True,
+                              tensor_model_parallel_size=1, gradient_accumulation_fusion=False, normalization="RMSNorm",
+                              layernorm_epsilon=1e-5)
+        lin = pt.PrimusTurboLinear(256, 384, parallel_mode=None, config=cfg, bias=False, skip_bias_add=False)
+        lin.weight.main_grad = torch.zeros_like(lin.weight, dtype=torch.float32)
+        lin.weight.grad_added_to_main_grad = False
+        x = torch.randn(16, 8, 256, device=gpu).bfloat16().requires_grad_()
+        dy = torch.randn(16, 8, 384, device=gpu).bfloat16()
+        with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc):
+            y, _ = lin(x)
+        y.backward(dy)
+        xr = x.detach().clone().requires_grad_()
+        wr = lin.weight.detach().clone().requires_grad_()
+        yr = torch.nn.functional.linear(xr, wr)
+        yr.backward(dy)
+        assert _cos(y, yr) > 0.998 and _cos(x.grad, xr.grad) > 0.998 and _cos(lin.weight.grad, wr.grad) > 0.998
+    finally:
+        pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+        runtime.set_args()
+        runtime.set_num_microbatches(1)

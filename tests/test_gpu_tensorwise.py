@@ -268,6 +268,6 @@ def test_operator_argument_errors(gpu):
     with pytest.raises(NotImplementedError):
         turbo.ops.gemm_fp8(x, w, config=Float8QuantConfig(format=Format.E5M2, granularity=ScalingGranularity.TENSORWISE))
     with pytest.raises(NotImplementedError):
-        turbo.ops.gemm_fp8(x, w, config=Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.BLOCKWISE, block_size=128))
+        turbo.ops.gemm_fp8(x, w, config=Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.ROWWISE))
     with pytest.raises(NotImplementedError):
         turbo.ops.rmsnorm_gemm_fp8(x, torch.ones(64, device=gpu).bfloat16(), 1e-5, w, config=_tw_cfg(False))

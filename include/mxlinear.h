@@ -160,7 +160,8 @@ int mxl_quantize_weight_2d_ex(const void* w_bf16, int64_t batch, int64_t n, int6
                               void* s_colT, uint32_t flags, void* stream);
 
 /* Row-wise dequantise to bf16 (QuantizedTensor.dequantize(),
- * weight_deosc.py:155-168): out[rows, k] = decode(codes) * 2^(scale-127). */
+ * weight_deosc.py:155-168): out[rows, k] = decode(codes) * 2^(scale-127).  fmt: MXL_FMT_E4M3, MXL_FMT_E2M1 or
+ * MXL_FMT_E5M2 (the codes of the tensor-wise and blockwise recipes; their scale bytes are 127). */
 int mxl_dequantize(const void* codes, const void* scales, int64_t rows, int64_t k, int fmt,
                    void* out_bf16, void* stream);
 

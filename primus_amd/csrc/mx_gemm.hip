@@ -84,6 +84,10 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, int64_t bytes) {
     r[3] = 0x00020000;
     return r;
 }
+// The statement writes M0 (the LDS address of an LDS-direct load).  M0 cannot be named in the clobber list: the
+// compiler diagnoses clobbers of reserved registers.  Nothing else in these kernels lives in M0: LDS instructions do
+// not take it on gfx950 and the kernels use no relative moves, messages or interpolation, and every use here
+// reloads it first.
 __device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
     asm volatile("" : "+s"(soff));   // the scalar offset has to sit in a register, also when it is a known constant
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"

@@ -524,6 +524,10 @@ __device__ __forceinline__ float dec_e4m3(uint32_t c) {
         v = __uint_as_float(((e + 120u) << 23) | (m << 20));
     return __uint_as_float(__float_as_uint(v) | s);
 }
+// E5M2 is the upper byte of an IEEE half: exact through the half -> float conversion (NaN and infinity included)
+__device__ __forceinline__ float dec_e5m2(uint32_t c) {
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)(c << 8));
+}
 __device__ __forceinline__ float dec_e2m1(uint32_t c) {
     const uint32_t s = (c & 8u) << 28, e = (c >> 1) & 3u, m = c & 1u;
     const uint32_t bits = e ? (((e + 126u) << 23) | (m << 22)) : (m ? 0x3F000000u : 0u);
@@ -541,12 +545,12 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t* q, const
     // fp32 holds 2^(byte-127) exactly (subnormal for byte 0); multiply in two steps to stay exact
     const float sc = (byte == 255u) ? __uint_as_float(0x7FC00000u) : fwd_scale(byte);
     float v[8];
-    if (FMT == kFmtE4M3) {
+    if (FMT == kFmtE4M3 || FMT == kFmtE5M2) {
         const uint2 c = *(const uint2*)(q + i * 8);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            v[k] = dec_e4m3((c.x >> (8 * k)) & 0xFFu);
-            v[4 + k] = dec_e4m3((c.y >> (8 * k)) & 0xFFu);
+            v[k] = FMT == kFmtE5M2 ? dec_e5m2((c.x >> (8 * k)) & 0xFFu) : dec_e4m3((c.x >> (8 * k)) & 0xFFu);
+            v[4 + k] = FMT == kFmtE5M2 ? dec_e5m2((c.y >> (8 * k)) & 0xFFu) : dec_e4m3((c.y >> (8 * k)) & 0xFFu);
         }
     } else {
         const uint32_t c = *(const uint32_t*)(q + i * 4);
@@ -857,9 +861,12 @@ extern "C" int mxl_dequantize(const void* codes, const void* scales, int64_t row
     const int64_t threads = nblocks * 4;
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7FFFFFFF) return MXL_EINVAL;
-    if (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E2M1) return MXL_EINVAL;
+    if (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E2M1 && fmt != MXL_FMT_E5M2) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
-    if (fmt == MXL_FMT_E4M3)
+    if (fmt == MXL_FMT_E5M2)
+        hipLaunchKernelGGL((mx_dequant_kernel<MXL_FMT_E5M2>), dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                           (const uint8_t*)codes, (const uint8_t*)scales, (uint16_t*)out_bf16, nblocks);
+    else if (fmt == MXL_FMT_E4M3)
         hipLaunchKernelGGL((mx_dequant_kernel<MXL_FMT_E4M3>), dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
                            (const uint8_t*)codes, (const uint8_t*)scales, (uint16_t*)out_bf16, nblocks);
     else if (fmt == MXL_FMT_E2M1)

@@ -436,15 +436,16 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=Fal
     if kchunk:
         return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _layout(kchunk) == LAYOUT_KSTEP else b_scale.unsqueeze(0),
                                        None, kchunk=kchunk)
-    m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
-    n, kb = b.shape[0], b.shape[1] * _per_byte(b_fmt)
+    # operands may arrive with or without the padding of K to 128 (the operators pad activations, a copy made by
+    # QuantizedTensor.quantize does not): the contraction lengths are compared after padding both
+    a, a_scale, k = _pad_k(a, a_scale, a_fmt)
+    b, b_scale, kb = _pad_k(b, b_scale, b_fmt)
+    m, n = a.shape[0], b.shape[0]
     if k != kb:
         raise ValueError(f"contraction dims differ: {k} vs {kb}")
     if tuple(a_scale.shape) != (m, k // BLOCK) or tuple(b_scale.shape) != (n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-    a, a_scale, _ = _pad_k(a, a_scale, a_fmt)
-    b, b_scale, k = _pad_k(b, b_scale, b_fmt)
     with _hooked("gemm_nt", m=m, n=n, k=k):
         rc = _lib.load().mxl_gemm_nt(_ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), m, n, k, _stream())
     _lib.check(rc, "mxl_gemm_nt")
@@ -485,15 +486,14 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
         return c
     if b.dim() != 3 or b.shape[0] != G:
         raise ValueError("grouped GEMM expects weights of shape [num_groups, n, k]")
-    total_m, k = a.shape[0], a.shape[1] * _per_byte(a_fmt)
-    n, kb = b.shape[1], b.shape[2] * _per_byte(b_fmt)
+    a, a_scale, k = _pad_k(a, a_scale, a_fmt)
+    b, b_scale, kb = _pad_k(b, b_scale, b_fmt)
+    total_m, n = a.shape[0], b.shape[1]
     if k != kb:
         raise ValueError(f"contraction dims differ: {k} vs {kb}")
     if tuple(a_scale.shape) != (total_m, k // BLOCK) or tuple(b_scale.shape) != (G, n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
-    a, a_scale, _ = _pad_k(a, a_scale, a_fmt)
-    b, b_scale, k = _pad_k(b, b_scale, b_fmt)
     with _hooked("grouped_gemm_nt", m=total_m, n=n, k=k):
         rc = _lib.load().mxl_grouped_gemm_nt(
             _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), G, total_m, n, k, _stream()

@@ -106,9 +106,15 @@ def _accum_from(b, pattern):
     main_grad = getattr(b, "main_grad", None)
     if main_grad is None or not hasattr(b, "grad_added_to_main_grad"):
         raise ValueError("fuse_bgrad_accum_pattern='megatron' needs main_grad and grad_added_to_main_grad on the weight operand")
-    if main_grad.dtype != torch.float32 or tuple(main_grad.shape) != tuple(b.shape) or not main_grad.is_contiguous():
-        raise ValueError("main_grad must be a contiguous float32 tensor of the weight's shape")
+    if tuple(main_grad.shape) != tuple(b.shape):
+        raise ValueError("main_grad must have the weight's shape")
+    # any dtype is accepted, as by the reference's bridge (primus_turbo.py:166-240); only a contiguous float32
+    # buffer can be the target of the GEMM's own accumulating epilogue, anything else is added to after the GEMM
     return main_grad, b
+
+
+def _fusable(target) -> bool:
+    return target is not None and target.dtype == torch.float32 and target.is_contiguous()
 
 
 def _cached_codes(q: QuantizedTensor, kchunk) -> torch.Tensor:
@@ -149,7 +155,7 @@ class _MXLinearFunction(torch.autograd.Function):
         # too large for it (or the layout is switched off): same codes, same results, faster loads.
         groups = b.shape[0] if grouped else 1
         fp8 = act_fmt != _lib.FMT_E2M1 and w_fmt != _lib.FMT_E2M1
-        kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, accum=accum is not None)
+        kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, accum=accum is not None and _fusable(accum[0]))
         if isinstance(b, QuantizedTensor):   # cached copies decide: the call uses the layout they are stored in
             kc = _cache_layout(b, b_t, kc, fp8, groups)
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
@@ -237,7 +243,7 @@ class _MXLinearFunction(torch.autograd.Function):
                 grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
-            fused = target is not None and kc == K.LAYOUT_KCHUNK   # the GEMM's epilogue adds into the float32 buffer
+            fused = _fusable(target) and kc == K.LAYOUT_KCHUNK   # the GEMM's epilogue adds into the float32 buffer
 
             def wgrad():
                 return K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc,
@@ -341,7 +347,7 @@ class _TWLinearFunction(torch.autograd.Function):
             grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
-            fused = target is not None and kc
+            fused = _fusable(target) and bool(kc)
 
             def wgrad():
                 return K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc,

@@ -114,7 +114,7 @@ def test_pattern_argument_errors(gpu):
         turbo.ops.gemm_fp8(x, w, config=cfg, fuse_bgrad_accum_pattern="megatron")     # no main_grad on the weight
     with pytest.raises(ValueError):
         turbo.ops.gemm_fp8(x, w, config=cfg, fuse_bgrad_accum_pattern="other")
-    w.main_grad = torch.zeros(32, 64, device=gpu, dtype=torch.bfloat16)
+    w.main_grad = torch.zeros(16, 64, device=gpu, dtype=torch.float32)
     w.grad_added_to_main_grad = False
     with pytest.raises(ValueError):
-        turbo.ops.gemm_fp8(x, w, config=cfg, fuse_bgrad_accum_pattern="megatron")     # main_grad must be float32
+        turbo.ops.gemm_fp8(x, w, config=cfg, fuse_bgrad_accum_pattern="megatron")     # main_grad must have the weight's shape

@@ -204,7 +204,9 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
 #define MXL_GF_KCHUNK 1u
 /* MXL_GF_KSTEP (instead of MXL_GF_KCHUNK): codes and scales of both operands are K-step-major, as written by the
  * quantisers with MXL_QF_KSTEP.  FP8-format operands, at most 128 groups, bf16 output (no MXL_GF_ACCUM_F32);
- * anything else returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit. */
+ * anything else returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
+ * With either layout flag the kernels request whole 256-row tiles of a K chunk: a code or scale array whose row count
+ * is not a multiple of 256 must be followed by 32 KiB of readable memory (the values read there are never used). */
 #define MXL_GF_KSTEP 4u
 /* mxl_grouped_gemm_wgrad_ex / _scaled only, together with MXL_GF_KCHUNK: c_bf16 points to FLOAT32 [g, n, k] and the
  * result is ADDED to it in fp32 (no rounding to bf16).  This is the gradient-accumulation fusion of the reference

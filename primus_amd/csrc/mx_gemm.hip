@@ -583,7 +583,7 @@ constexpr int RING_PANEL_BUFS = 3;
 constexpr int RING_TBL = RING_MAX_GROUPS + 2;
 
 constexpr int ring_lds_bytes() {
-    return RING_SLOTS * RING_STAGE + RING_PANEL_BUFS * 2 * RING_PANEL + RING_TBL * 4 + RING_TBL * 8 + RING_TBL * 4;
+    return RING_SLOTS * RING_STAGE + RING_PANEL_BUFS * 2 * RING_PANEL + RING_TBL * 4 + RING_TBL * 8 + RING_TBL * 4 + RING_TBL * 4;
 }
 
 template <int AFMT, int BFMT, int MODE, bool ALPHA>
@@ -598,6 +598,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     int* pre_tiles = (int*)(panels + RING_PANEL_BUFS * 2 * PANEL);
     int64_t* pre_rows = (int64_t*)(pre_tiles + RING_TBL);
     int* pre_pan = (int*)(pre_rows + RING_TBL);                      // [G+1] prefix of scale panels (WGRAD)
+    int* by_len = pre_pan + RING_TBL;                                // [G] groups by descending contraction length (WGRAD)
 
     const int t = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -635,6 +636,23 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         }
     }
     __syncthreads();
+
+    // wgrad: the tiles of a group all run that group's contraction length, and lengths differ widely between
+    // groups.  The tile order goes through the groups from the longest to the shortest (ties by index; groups
+    // without tokens come last), and the workgroups walk it in a serpentine (below): every workgroup then gets
+    // nearly the same number of K steps instead of whatever mix of groups its stride happens to hit.
+    if (MODE == MODE_WGRAD) {
+        for (int i = t; i < G; i += GTHREADS) {
+            const int64_t len = pre_rows[i + 1] - pre_rows[i];
+            int rank = 0;
+            for (int j = 0; j < G; ++j) {
+                const int64_t lj = pre_rows[j + 1] - pre_rows[j];
+                rank += (lj > len || (lj == len && j < i)) ? 1 : 0;
+            }
+            by_len[rank] = i;
+        }
+        __syncthreads();
+    }
 
     const int tiles_n = (int)((p.n + BN - 1) / BN);
     int tiles_m, total_tiles;
@@ -678,8 +696,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         int grp = 0, pid_m, pid_n;
         int tl = tile;
         if (MODE == MODE_WGRAD) {
-            grp = tl / (tiles_m * tiles_n);
-            tl -= grp * tiles_m * tiles_n;
+            const int pos = tl / (tiles_m * tiles_n);
+            tl -= pos * tiles_m * tiles_n;
+            grp = __builtin_amdgcn_readfirstlane(by_len[pos]);
         }
         {
             const int width = GROUP_M * tiles_n;
@@ -794,14 +813,22 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     const int a_lo = 16 * (g ^ sw), a_hi = 16 * ((2 + g) ^ sw);
     const int a_sc = (wm * 128 + lr) * 16 + g, b_sc = (wn * 128 + lr) * 16 + g;
 
-    // The workgroup's tiles: vwg, vwg + nwg, ...  A tile whose contraction range is empty (wgrad of a group without
-    // tokens) never enters the pipeline: its output is zero-filled on the spot and the sequence moves on.
-    auto next_tile = [&](int tl) __attribute__((always_inline)) {
+    // The workgroup's tiles: one per round of nwg tiles, at position vwg of the round -- in wgrad at position
+    // nwg - 1 - vwg in odd rounds (the serpentine; an XCD's workgroups still hold a contiguous run of the order).
+    // A tile whose contraction range is empty (wgrad of a group without tokens) never enters the pipeline: its
+    // output is zero-filled on the spot and the sequence moves on.
+    auto tile_at = [&](int round) __attribute__((always_inline)) {
+        return round * nwg + ((MODE == MODE_WGRAD && (round & 1)) ? nwg - 1 - vwg : vwg);
+    };
+    int round = 0;
+    auto next_tile = [&]() __attribute__((always_inline)) {
+        int tl = tile_at(round);
         if (MODE == MODE_WGRAD) {
             while (tl < total_tiles) {
-                const int grp = tl / (tiles_m * tiles_n);
-                if (pre_rows[grp + 1] > pre_rows[grp]) break;
-                const int rem = tl - grp * tiles_m * tiles_n;
+                const int pos = tl / (tiles_m * tiles_n);
+                const int grp = __builtin_amdgcn_readfirstlane(by_len[pos]);
+                if (__builtin_amdgcn_readfirstlane((int)(pre_rows[grp + 1] > pre_rows[grp]))) break;   // uniform by construction
+                const int rem = tl - pos * tiles_m * tiles_n;
                 const int width = GROUP_M * tiles_n;
                 const int first = (rem / width) * GROUP_M;
                 const int gsz = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
@@ -812,14 +839,15 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                     const int c = (t & 31) * 8;
                     if (c < nv) store16_streaming((uint8_t*)(ct + (int64_t)r * p.n + c), make_uint4(0u, 0u, 0u, 0u));
                 }
-                tl += nwg;
+                tl = tile_at(++round);
             }
         }
-        return tl;
+        ++round;
+        return __builtin_amdgcn_readfirstlane(tl);
     };
-    int tile = next_tile(vwg);
+    int tile = next_tile();
     if (tile >= total_tiles) return;
-    int tile_n = next_tile(tile + nwg);
+    int tile_n = next_tile();
     Tile d = decode(tile);
     // past the last tile the stream requests the last tile's first steps again (nobody reads them)
     Tile dn = decode(tile_n < total_tiles ? tile_n : tile);
@@ -986,7 +1014,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         }
         d = dn;
         tile = tile_n;
-        tile_n = next_tile(tile + nwg);
+        tile_n = next_tile();
         dn = decode(tile_n < total_tiles ? tile_n : tile);
         pb_rd = next3(pb_rd);
         MXL_PIN;

@@ -110,6 +110,21 @@ def _scale_shape(rows: int, ld: int, kchunk, groups: int = 0):
     return (rows, ld // BLOCK)
 
 
+OPERAND_TAIL = 32 * 1024
+
+
+def _empty_tail(shape, dtype, device):
+    """A code or scale buffer followed by ``OPERAND_TAIL`` bytes the GEMMs may read (never use).  In the chunked
+    layouts the GEMMs request whole 256-row tiles of a K chunk; for an operand whose row count is not a multiple of
+    256 the last tile's requests in the last chunk reach up to 32 KiB past the last code (the values land in tile
+    rows that are never stored).  The tail keeps those reads inside the allocation."""
+    n = 1
+    for d in shape:
+        n *= int(d)
+    flat = torch.empty((n + OPERAND_TAIL,), dtype=dtype, device=device)
+    return flat[:n].view(shape)
+
+
 def _qflag(kchunk) -> int:
     return (0, _lib.QF_KCHUNK, _lib.QF_KSTEP)[_layout(kchunk)]
 
@@ -297,12 +312,12 @@ def quantize_mx_impl(
     q_row = s_row = q_col = s_col = None
     row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
-        q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-        s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+        q_row = _empty_tail(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+        s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        q_col = torch.empty(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
         row_ok = rows > 0
@@ -353,14 +368,14 @@ def quantize_mx_weight_2d_impl(
     k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     if rowwise:
         shape = _code_shape(batch * n, k_ld, per, kchunk) if kchunk else lead + (n, k_ld // per)
-        q_row = torch.empty(shape, dtype=torch.uint8, device=dev)
+        q_row = _empty_tail(shape, dtype=torch.uint8, device=dev)
         sshape = _scale_shape(batch * n, k_ld, kchunk) if _layout(kchunk) == LAYOUT_KSTEP else lead + (n, k_ld // BLOCK)
-        s_row = torch.empty(sshape, dtype=torch.uint8, device=dev)
+        s_row = _empty_tail(sshape, dtype=torch.uint8, device=dev)
     if colwise:
         shape = _code_shape(batch * k, n_ld, per, kchunk) if kchunk else lead + (k, n_ld // per)
-        q_col = torch.empty(shape, dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(shape, dtype=torch.uint8, device=dev)
         sshape = _scale_shape(batch * k, n_ld, kchunk) if _layout(kchunk) == LAYOUT_KSTEP else lead + (k, n_ld // BLOCK)
-        s_col = torch.empty(sshape, dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(sshape, dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_2d_ex(
             _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
@@ -406,6 +421,13 @@ def _pad_k(codes: torch.Tensor, scales: torch.Tensor, fmt: int):
     return c, s, kp
 
 
+def _check_contraction(k: int, kb: int) -> None:
+    """The two contraction lengths agree, or one is the other padded to the GEMM's granularity (the operators pad
+    activations, a copy made by ``QuantizedTensor.quantize`` is not padded)."""
+    if k != kb and max(k, kb) != _round_up(min(k, kb), GEMM_K_ALIGN):
+        raise ValueError(f"contraction dims differ: {k} vs {kb}")
+
+
 def _check_out_dtype(out_dtype) -> None:
     if out_dtype not in (None, torch.bfloat16):
         raise ValueError("the MX GEMMs produce bfloat16 output")
@@ -436,13 +458,10 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=Fal
     if kchunk:
         return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _layout(kchunk) == LAYOUT_KSTEP else b_scale.unsqueeze(0),
                                        None, kchunk=kchunk)
-    # operands may arrive with or without the padding of K to 128 (the operators pad activations, a copy made by
-    # QuantizedTensor.quantize does not): the contraction lengths are compared after padding both
+    _check_contraction(a.shape[-1] * _per_byte(a_fmt), b.shape[-1] * _per_byte(b_fmt))
     a, a_scale, k = _pad_k(a, a_scale, a_fmt)
     b, b_scale, kb = _pad_k(b, b_scale, b_fmt)
     m, n = a.shape[0], b.shape[0]
-    if k != kb:
-        raise ValueError(f"contraction dims differ: {k} vs {kb}")
     if tuple(a_scale.shape) != (m, k // BLOCK) or tuple(b_scale.shape) != (n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
@@ -486,11 +505,10 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
         return c
     if b.dim() != 3 or b.shape[0] != G:
         raise ValueError("grouped GEMM expects weights of shape [num_groups, n, k]")
+    _check_contraction(a.shape[-1] * _per_byte(a_fmt), b.shape[-1] * _per_byte(b_fmt))
     a, a_scale, k = _pad_k(a, a_scale, a_fmt)
     b, b_scale, kb = _pad_k(b, b_scale, b_fmt)
     total_m, n = a.shape[0], b.shape[1]
-    if k != kb:
-        raise ValueError(f"contraction dims differ: {k} vs {kb}")
     if tuple(a_scale.shape) != (total_m, k // BLOCK) or tuple(b_scale.shape) != (G, n, k // BLOCK):
         raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
@@ -623,13 +641,13 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
     per = _per_byte(fmt)
     dev = x.device
     row_ld = _round_up(f, KCHUNK if kchunk else pad_to)
-    q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-    s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+    q_row = _empty_tail(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+    s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, G)
-        q_col = torch.empty(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty(_scale_shape(f, W, kchunk, G), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(f, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         row_ok = rows > 0
         with _hooked("glu_probs_quantize", rows=rows, cols=f, fmt=fmt, rowwise=True, colwise=colwise):
@@ -688,11 +706,11 @@ def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool
     q_row = s_row = q_col = s_col = None
     row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
-        q_row = torch.empty(_code_shape(rows, row_ld, 1, kchunk), dtype=torch.uint8, device=dev)
+        q_row = _empty_tail(_code_shape(rows, row_ld, 1, kchunk), dtype=torch.uint8, device=dev)
         s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        q_col = torch.empty(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
         s_col = torch.empty((cols, W // BLOCK), dtype=torch.uint8, device=dev)
     if rows == 0 and not (colwise and q_col.numel()):
         scale_inv.fill_(1e-12 / (448.0 if fmt == _lib.FMT_E4M3 else 57344.0))
@@ -729,10 +747,10 @@ def quantize_weight_tensorwise_impl(w, fmt: int, *, rowwise: bool = True, colwis
     k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     q_row = s_row = q_col = s_col = None
     if rowwise:
-        q_row = torch.empty(_code_shape(batch * n, k_ld, 1, True) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
+        q_row = _empty_tail(_code_shape(batch * n, k_ld, 1, True) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
         s_row = torch.empty(lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
-        q_col = torch.empty(_code_shape(batch * k, n_ld, 1, True) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(batch * k, n_ld, 1, True) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
         s_col = torch.empty(lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_tensorwise", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_tensorwise(
@@ -882,13 +900,13 @@ def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCAL
     per = _per_byte(fmt)
     dev = x.device
     row_ld = _round_up(k, KCHUNK if kchunk else pad_to)
-    q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-    s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+    q_row = _empty_tail(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+    s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, 0)
-        q_col = torch.empty(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty(_scale_shape(k, W, kchunk), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(k, W, kchunk), dtype=torch.uint8, device=dev)
     with _hooked("rmsnorm_quantize", rows=rows, cols=k, fmt=fmt, rowwise=True, colwise=colwise):
         rc = _lib.load().mxl_rmsnorm_quantize(
             _ptr(x), _ptr(weight), _ptr(rstd), rows, k, row_ld, fmt, scale_mode, None, 0, _ptr(q_row), _ptr(s_row),

@@ -378,8 +378,8 @@ def main():
     gk = acc[fwd_name]
     gemm_tflops = gk["flops"] / gk["sec"] / 1e12
     roofline = {
-        # MXFP8 x MXFP8 operands run on the 4-slot ring kernel; FP4 operands and the tensor-wise recipe on the 2-slot kernel
-        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_kernel" if spec["fp4"] or spec.get("tensorwise") else "mx_gemm_ring_kernel",
+        # FP8 x FP8 operands (MX or tensor-wise scaled) run on the 4-slot ring kernel, FP4 operands on the 2-slot kernel
+        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_kernel" if spec["fp4"] else "mx_gemm_ring_kernel",
                                                    "e4m3|e5m2" if spec.get("tensorwise") else "e4m3", "e2m1" if spec["fp4"] else "e4m3",
                                                    ",alpha" if spec.get("tensorwise") else "", fwd_name),
         "bound": "mfma",

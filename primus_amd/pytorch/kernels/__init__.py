@@ -707,11 +707,11 @@ def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool
     row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
         q_row = _empty_tail(_code_shape(rows, row_ld, 1, kchunk), dtype=torch.uint8, device=dev)
-        s_row = torch.empty((rows, row_ld // BLOCK), dtype=torch.uint8, device=dev)
+        s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
         q_col = _empty_tail(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
-        s_col = torch.empty((cols, W // BLOCK), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows == 0 and not (colwise and q_col.numel()):
         scale_inv.fill_(1e-12 / (448.0 if fmt == _lib.FMT_E4M3 else 57344.0))
     else:
@@ -719,7 +719,7 @@ def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool
             rc = _lib.load().mxl_quantize_tensorwise(
                 _ptr(x) if rows else None, rows, cols, row_ld if rowwise else 0, fmt, _ptr(amax),
                 _ptr(group_lens) if colwise else None, G, _ptr(q_row) if rows else None, _ptr(s_row) if rows else None,
-                _ptr(q_col), _ptr(s_col), _ptr(scale_inv), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+                _ptr(q_col), _ptr(s_col), _ptr(scale_inv), _qflag(kchunk), _stream(),
             )
         _lib.check(rc, "mxl_quantize_tensorwise")
     cd = _code_dtype(fmt)
@@ -746,16 +746,17 @@ def quantize_weight_tensorwise_impl(w, fmt: int, *, rowwise: bool = True, colwis
     scale_inv = torch.empty((1,), dtype=torch.float32, device=dev)
     k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     q_row = s_row = q_col = s_col = None
+    kstep = _layout(kchunk) == LAYOUT_KSTEP
     if rowwise:
-        q_row = _empty_tail(_code_shape(batch * n, k_ld, 1, True) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
-        s_row = torch.empty(lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
+        q_row = _empty_tail(_code_shape(batch * n, k_ld, 1, kchunk) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
+        s_row = _empty_tail(_scale_shape(batch * n, k_ld, kchunk) if kstep else lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
-        q_col = _empty_tail(_code_shape(batch * k, n_ld, 1, True) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
-        s_col = torch.empty(lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(batch * k, n_ld, 1, kchunk) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(batch * k, n_ld, kchunk) if kstep else lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_tensorwise", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_tensorwise(
             _ptr(w), batch, n, k, k_ld, n_ld, fmt, _ptr(amax), _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
-            _ptr(scale_inv), _lib.QF_KCHUNK if kchunk else 0, _stream(),
+            _ptr(scale_inv), _qflag(kchunk), _stream(),
         )
     _lib.check(rc, "mxl_quantize_weight_tensorwise")
     cd = _code_dtype(fmt)
@@ -779,22 +780,32 @@ def gemm_tw_nt_impl(a, a_unit, a_scale_inv, b, b_unit, b_scale_inv, group_lens=N
     G = _check_group_lens(group_lens, a.device)
     groups = max(G, 1)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    kstep = _layout(kchunk) == LAYOUT_KSTEP
     if kchunk:
-        total_m, k = _chunked_dims(a, a_fmt)
-        b_rows, kb = _chunked_dims(b, b_fmt)
+        total_m, k = _chunked_dims(a, a_fmt, kchunk)
+        b_rows, kb = _chunked_dims(b, b_fmt, kchunk)
     else:
         total_m, k = a.shape
         b_rows, kb = b.numel() // b.shape[-1], b.shape[-1]
-    n = b_unit.shape[-2]
-    if k != kb or k % _lib.GEMM_K_ALIGN or b_rows != groups * n or b_unit.numel() != b_rows * (k // BLOCK):
-        raise ValueError("operand shapes do not match (the contraction dim must be padded to 128)")
-    if tuple(a_unit.shape) != (total_m, k // BLOCK):
-        raise ValueError("scale shapes must be [rows, k/32]")
+    if kstep:
+        if b_rows % groups:
+            raise ValueError("the rows of b do not split into num_groups weights")
+        n = b_rows // groups
+        if k != kb or k % _lib.GEMM_K_ALIGN:
+            raise ValueError("operand shapes do not match (the contraction dim must be padded to 128)")
+        _check_scales(a_unit, total_m, k, kchunk, "a_unit")
+        _check_scales(b_unit, b_rows, k, kchunk, "b_unit")
+    else:
+        n = b_unit.shape[-2]
+        if k != kb or k % _lib.GEMM_K_ALIGN or b_rows != groups * n or b_unit.numel() != b_rows * (k // BLOCK):
+            raise ValueError("operand shapes do not match (the contraction dim must be padded to 128)")
+        if tuple(a_unit.shape) != (total_m, k // BLOCK):
+            raise ValueError("scale shapes must be [rows, k/32]")
     c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
     with _hooked("grouped_gemm_nt" if G else "gemm_nt", m=total_m, n=n, k=k):
         rc = _lib.load().mxl_grouped_gemm_nt_scaled(
             _ptr(a), _ptr(a_unit), a_fmt, _ptr(b), _ptr(b_unit), b_fmt, _ptr(c), _ptr(group_lens), groups, total_m, n, k,
-            _ptr(a_scale_inv), _ptr(b_scale_inv), _lib.GF_KCHUNK if kchunk else 0, _stream(),
+            _ptr(a_scale_inv), _ptr(b_scale_inv), _gflag(kchunk), _stream(),
         )
     _lib.check(rc, "mxl_grouped_gemm_nt_scaled")
     return c
@@ -809,16 +820,23 @@ def gemm_tw_wgrad_impl(a_t, a_t_unit, a_scale_inv, b_t, b_t_unit, b_scale_inv, g
     G = _check_group_lens(group_lens, a_t.device)
     a_fmt, b_fmt = fmt_of(a_t), fmt_of(b_t)
     W = padded_width(total_m, G)
+    kstep = _layout(kchunk) == LAYOUT_KSTEP
     if kchunk:
-        (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt), _chunked_dims(b_t, b_fmt)
+        (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt, kchunk), _chunked_dims(b_t, b_fmt, kchunk)
     else:
         (n, wa), (k, wb) = a_t.shape, b_t.shape
     if wa != W or wb != W:
         raise ValueError(f"transposed operands must have padded width {W}")
-    if tuple(a_t_unit.shape) != (n, W // BLOCK) or tuple(b_t_unit.shape) != (k, W // BLOCK):
+    if kstep:
+        if accum_into is not None:
+            raise ValueError("the accumulating wgrad epilogue takes K-chunk-major operands")
+        for sc, r, what in ((a_t_unit, n, "a_t_unit"), (b_t_unit, k, "b_t_unit")):
+            if tuple(sc.shape) != _scale_shape(r, W, kchunk, G) or not sc.is_contiguous():
+                raise ValueError(f"{what} must be the K-step-major scale array of its operand")
+    elif tuple(a_t_unit.shape) != (n, W // BLOCK) or tuple(b_t_unit.shape) != (k, W // BLOCK):
         raise ValueError("scale shapes must be [rows, W/32]")
     shape = (n, k) if group_lens is None else (G, n, k)
-    flags = _lib.GF_KCHUNK if kchunk else 0
+    flags = _gflag(kchunk)
     if accum_into is not None:
         c = _accum_target(accum_into, shape, kchunk, a_t.device)
         flags |= _lib.GF_ACCUM_F32

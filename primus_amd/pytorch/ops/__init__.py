@@ -304,9 +304,13 @@ class _TWLinearFunction(torch.autograd.Function):
         need_wgrad = b.requires_grad
         grouped = group_lens is not None
         groups = b.shape[0] if grouped else 1
-        kc = K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])
         if isinstance(b, QuantizedTensor):
-            kc = kc and b.kchunk and (b_t is None or b_t.kchunk)
+            # cached copies are stored row-major or K-chunk-major
+            kc = K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])
+            kc = int(bool(kc and b.kchunk and (b_t is None or b_t.kchunk)))
+        else:
+            kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=True,
+                               accum=accum is not None and _fusable(accum[0]))
         a_row, a_ru, a_col, a_cu, a_si = K.quantize_tensorwise_impl(
             a, fwd_fmt, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
         if isinstance(b, QuantizedTensor):
@@ -347,7 +351,7 @@ class _TWLinearFunction(torch.autograd.Function):
             grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
-            fused = _fusable(target) and bool(kc)
+            fused = _fusable(target) and kc == K.LAYOUT_KCHUNK
 
             def wgrad():
                 return K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc,

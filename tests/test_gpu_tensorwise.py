@@ -45,7 +45,7 @@ def test_amax(gpu, n):
 @pytest.mark.parametrize("fmt", [0, 2])
 @pytest.mark.parametrize("rows,cols,lens", [(37, 32, None), (300, 160, None), (257, 4096, None),
                                             (256, 96, [33, 0, 130, 1, 92]), (600, 256, [300, 300])])
-@pytest.mark.parametrize("kchunk", [False, True])
+@pytest.mark.parametrize("kchunk", [False, True, 2])
 def test_quantiser_equals_the_oracle(gpu, fmt, rows, cols, lens, kchunk):
     from primus_amd.pytorch import kernels as K
 
@@ -60,7 +60,12 @@ def test_quantiser_equals_the_oracle(gpu, fmt, rows, cols, lens, kchunk):
     row = _u8(K.unchunk(qr) if kchunk else qr)
     assert row.shape[0] == rows and row.shape[1] % 128 == 0
     assert np.array_equal(row[:, :cols], want) and not row[:, cols:].any()
-    assert np.all(_u8(sr) == 127) and np.all(_u8(sc) == 127)
+    if kchunk == 2:
+        # K-step-major scale panels: the entries of the row-wise copy's K blocks hold the unit byte (the transposed
+        # copy's panels restart per expert segment and are covered by the GEMM test below)
+        assert np.all(_u8(K.unpanel(sr.view(torch.uint8), row.shape[1] // 32)) == 127)
+    else:
+        assert np.all(_u8(sr) == 127) and np.all(_u8(sc) == 127)
     # transposed copy: per expert segment, padded to 128 tokens with zero codes
     col = _u8(K.unchunk(qc) if kchunk else qc)
     lens_ = [rows] if lens is None else lens
@@ -102,7 +107,7 @@ def test_quantiser_special_tensors(gpu, fmt):
 
 @pytest.mark.parametrize("fmt", [0, 2])
 @pytest.mark.parametrize("shape", [(96, 160), (3, 256, 128), (2, 416, 288)])
-@pytest.mark.parametrize("kchunk", [False, True])
+@pytest.mark.parametrize("kchunk", [False, True, 2])
 def test_weight_quantiser_equals_the_oracle(gpu, fmt, shape, kchunk):
     from primus_amd.pytorch import kernels as K
 
@@ -121,7 +126,7 @@ def test_weight_quantiser_equals_the_oracle(gpu, fmt, shape, kchunk):
 
 @pytest.mark.parametrize("afmt", [0, 2])
 @pytest.mark.parametrize("lens,n,k", [(None, 96, 160), ([33, 0, 130, 1, 92], 160, 96), ([300, 212], 384, 256), (None, 512, 1024)])
-@pytest.mark.parametrize("kchunk", [False, True])
+@pytest.mark.parametrize("kchunk", [False, True, 2])
 def test_scaled_gemms_vs_oracle(gpu, afmt, lens, n, k, kchunk):
     from primus_amd.pytorch import kernels as K
 

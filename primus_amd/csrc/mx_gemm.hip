@@ -328,16 +328,18 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         for (int r = 0; r < LPT; ++r) issue_1(d, 0, 0, r);
     };
 
+    // NA: how many of this wave's four 32-row fragments hold rows of the tile (see `live` below); the MFMAs and
+    // fragment reads of the others are left out
 #define MXL_MFMA(F, I, J) \
-    acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I])
+    do { if ((I) < NA) acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I]); } while (0)
 #define MXL_PIN __builtin_amdgcn_sched_barrier(0)
     // read one fragment (+ its scale byte) of the K step described by (sn, pan, ks_n)
 #define MXL_RD_A(F, I) \
-    F.a[I] = read_frag<AFMT>(sn, wm * 128 + (I) * 32 + lr, ks_n, g); \
-    F.sa[I] = pan[16 * (wm * 128 + (I) * 32 + lr)]
+    do { if ((I) < NA) { F.a[I] = read_frag<AFMT>(sn, wm * 128 + (I) * 32 + lr, ks_n, g); \
+                         F.sa[I] = pan[16 * (wm * 128 + (I) * 32 + lr)]; } } while (0)
 #define MXL_RD_B(F, J) \
-    F.b[J] = read_frag<BFMT>(sn + A_BYTES, wn * 128 + (J) * 32 + lr, ks_n, g); \
-    F.sb[J] = pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]
+    do { if (NA > 0) { F.b[J] = read_frag<BFMT>(sn + A_BYTES, wn * 128 + (J) * 32 + lr, ks_n, g); \
+                       F.sb[J] = pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]; } } while (0)
 
     int tile = vwg;
     if (tile >= total_tiles) return;
@@ -366,6 +368,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             const uint8_t* sn = smem;
             const uint8_t* pan = panels + g;
             constexpr int ks_n = 0;
+            constexpr int NA = 4;
             MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
             MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
         }
@@ -374,9 +377,10 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         // slot is dead, so the requests for K slot kp+2 start to go out.
         // The body is written in its final instruction order and pinned with scheduling
         // barriers; each LDS fragment read sits next to an MFMA that hides it.
-        auto kstep = [&](auto ks_tag, auto sub_tag, int kp, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
+        auto kstep = [&](auto ks_tag, auto sub_tag, auto na_tag, int kp, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
             constexpr int KS = decltype(ks_tag)::value;
             constexpr int SUB = decltype(sub_tag)::value;      // kp & 3, known at compile time
+            constexpr int NA = decltype(na_tag)::value;
             constexpr int slot = SUB & 1;
             constexpr int ks_n = 1 - KS;                       // K step (within its slot) of the fragments read here
             const int st_n = 2 * kp + KS + 1;                  // its global K-step index
@@ -421,23 +425,34 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         using I1 = std::integral_constant<int, 1>;
         using I2 = std::integral_constant<int, 2>;
         using I3 = std::integral_constant<int, 3>;
+        using I4 = std::integral_constant<int, 4>;
         const int np = d.np;
-        for (int kp = 0; kp < np; kp += 4) {
-            kstep(I0{}, I0{}, kp, f0, f1);
-            kstep(I1{}, I0{}, kp, f1, f0);
-            if (kp + 1 < np) {
-                kstep(I0{}, I1{}, kp + 1, f0, f1);
-                kstep(I1{}, I1{}, kp + 1, f1, f0);
+        auto kloop = [&](auto na) __attribute__((always_inline)) {
+            for (int kp = 0; kp < np; kp += 4) {
+                kstep(I0{}, I0{}, na, kp, f0, f1);
+                kstep(I1{}, I0{}, na, kp, f1, f0);
+                if (kp + 1 < np) {
+                    kstep(I0{}, I1{}, na, kp + 1, f0, f1);
+                    kstep(I1{}, I1{}, na, kp + 1, f1, f0);
+                }
+                if (kp + 2 < np) {
+                    kstep(I0{}, I2{}, na, kp + 2, f0, f1);
+                    kstep(I1{}, I2{}, na, kp + 2, f1, f0);
+                }
+                if (kp + 3 < np) {
+                    kstep(I0{}, I3{}, na, kp + 3, f0, f1);
+                    kstep(I1{}, I3{}, na, kp + 3, f1, f0);
+                }
             }
-            if (kp + 2 < np) {
-                kstep(I0{}, I2{}, kp + 2, f0, f1);
-                kstep(I1{}, I2{}, kp + 2, f1, f0);
-            }
-            if (kp + 3 < np) {
-                kstep(I0{}, I3{}, kp + 3, f0, f1);
-                kstep(I1{}, I3{}, kp + 3, f1, f0);
-            }
-        }
+        };
+        // Rows of this wave's 128 that lie inside the tile.  In the forward / dgrad GEMM a group's last row tile is
+        // ragged (an expert with 500 tokens: its second tile has 244 rows, a third would have a handful), and the
+        // fragments past its end would multiply another group's rows into accumulators that are never stored: a wave
+        // runs the loop variant for 4, 2 or 0 live fragments.  Loads and barriers are the same in all of them.
+        const int live = (MODE == MODE_FWD && !ACCUM) ? d.m_valid - wm * 128 : 128;
+        if (live > 64) kloop(I4{});
+        else if (live > 0) kloop(I2{});
+        else kloop(I0{});
         // Drain the look-ahead requests (they target the ring) and make sure every wave is done
         // reading it; then the next tile's first requests go out and overlap with the epilogue.
         wait_vm<0>();

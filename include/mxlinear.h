@@ -356,28 +356,42 @@ int mxl_unpad_groups(const void* y, int64_t padded_rows, int64_t row_bytes, cons
  * fmt is MXL_FMT_E4M3 or MXL_FMT_E5M2; every scale is an fp32 scale_inv = 1 / (fp8_max / max(amax, 1e-12)) of its block,
  * codes = cast(clamp(x * scale)), fp32 arithmetic (the formula the reference restates at :194-207, per block).
  *
- * mxl_quantize_blockwise replaces quant_fp8_blockwise_impl(x, dtype, axis, block_size = 128) (:1019, :1053-1059):
+ * mxl_quantize_blockwise replaces quant_fp8_blockwise_impl(x, dtype, axis, block_size = 128) (:1019, :1053-1059) and, with
+ * group_lens, quant_fp8_blockwise_segment_m_row_col_impl (primus/backends/megatron/core/extensions/zbpp_gemm.py:633, :785):
  *   x          : bf16 [rows, cols], cols % 128 == 0, 16-byte aligned
+ *   group_lens : int64[num_groups] on the device (<= 1024 groups) or NULL / 0: the rows of x are split into groups
  *   q_row      : [rows, cols] codes, 1 x 128 blocks along the columns (axis = 1 / -1); sinv_row fp32 [rows, cols / 128]
  *   q_colT     : the copy with 128 x 1 blocks along the rows (axis = 0 / -2), stored TRANSPOSED as the NT GEMM consumes
- *                it: [cols, rows_pad] codes, rows_pad = rows rounded up to 128 (zero codes), sinv_colT fp32
- *                [cols, rows_pad / 128].  Either copy may be left out (both pointers NULL).
- * mxl_quantize_blockwise_weight replaces quant_fp8_blockwise_for_weight_impl (:1020, :1060): w bf16 [n, k], both
- * multiples of 128, one scale per 128 x 128 block; q [n, k] with sinv [n / 128, k / 128] and / or the transposed copy
- * q_T [k, n] with sinv_T [k / 128, n / 128] (the same scales, transposed).
+ *                it: [cols, W] codes, sinv_colT fp32 [cols, W / 128].  Without groups W = rows rounded up to 128; with
+ *                groups W = mxl_padded_width(rows, num_groups) and group g owns columns [poff_g, poff_g + len_g), poff =
+ *                prefix sum of the lens rounded up to 128, so the blocks restart at every group.  Padding: zero codes.
+ *                Either copy may be left out (both pointers NULL).
+ * mxl_quantize_blockwise_weight replaces quant_fp8_blockwise_for_weight_impl (:1020, :1060): w bf16 [batch, n, k], n and
+ * k multiples of 128, one scale per 128 x 128 block; q [batch, n, k] with sinv [batch, n / 128, k / 128] and / or the
+ * transposed copies q_T [batch, k, n] with sinv_T [batch, k / 128, n / 128] (the same scales, transposed).
  *
  * mxl_gemm_nt_blockwise replaces gemm_fp8_impl(..., granularity = BLOCKWISE) (:1022-1033, :1064-1087), always in NT
  * form on the copies above:  c[m, n] (bf16) = sum over kb of a_sinv[m, kb] * b_sinv[n / b_rows_per_scale, kb] *
  * (a[m, 128 kb ..] . b[n, 128 kb ..]), fp32 accumulation.  a [m, k] codes, b [n, k] codes, k % 128 == 0, n % 128 == 0;
  * b_rows_per_scale is 128 (b is a weight: b_sinv [n / 128, k / 128]) or 1 (b_sinv [n, k / 128], the wgrad GEMM, whose
  * two operands are transposed activation copies).  forward: a = q_row(X), b = q(W); dgrad: a = q_row(dY), b = q_T(W);
- * wgrad: a = q_colT(dY), b = q_colT(X), k = rows_pad. */
-int mxl_quantize_blockwise(const void* x_bf16, int64_t rows, int64_t cols, int fmt, void* q_row, void* sinv_row,
-                           void* q_colT, void* sinv_colT, void* stream);
-int mxl_quantize_blockwise_weight(const void* w_bf16, int64_t n, int64_t k, int fmt, void* q, void* sinv, void* q_T,
-                                  void* sinv_T, void* stream);
+ * wgrad: a = q_colT(dY), b = q_colT(X), k = rows_pad.
+ * mxl_grouped_gemm_nt_blockwise (grouped_gemm_fp8_impl with blockwise granularity, zbpp_gemm.py:608-630): the rows of
+ * a [total_m, k] are split by group_lens, b is [num_groups, n, k] with b_sinv [num_groups, n / 128, k / 128].
+ * mxl_grouped_gemm_wgrad_blockwise (grouped_gemm_fp8_variable_k_impl, zbpp_gemm.py:757-800): a = q_colT(dY) [n, W],
+ * b = q_colT(X) [k, W] with their per-row factors, c [num_groups, n, k]; a group without tokens yields zeros. */
+int mxl_quantize_blockwise(const void* x_bf16, int64_t rows, int64_t cols, int fmt, const int64_t* group_lens, int num_groups,
+                           void* q_row, void* sinv_row, void* q_colT, void* sinv_colT, void* stream);
+int mxl_quantize_blockwise_weight(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int fmt, void* q, void* sinv,
+                                  void* q_T, void* sinv_T, void* stream);
 int mxl_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,
                           int b_fmt, int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k, void* stream);
+int mxl_grouped_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,
+                                  int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m,
+                                  int64_t n, int64_t k, void* stream);
+int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,
+                                     int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m,
+                                     int64_t n, int64_t k, void* stream);
 
 #ifdef __cplusplus
 }

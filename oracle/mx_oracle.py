@@ -939,3 +939,56 @@ def blockwise_gemm_nt_ref(a_codes, a_sinv, b_codes, b_sinv, a_fmt=FMT_E4M3, b_fm
         part = _matmul_nt_f32(a[:, sl], b[:, sl])
         acc = (acc + part * (a_sinv[:, kb][:, None] * sb[:, kb][None, :]).astype(np.float32)).astype(np.float32)
     return f32_to_bf16_bits(acc) if out_bf16 else acc
+
+
+def quantize_blockwise_segmented(x, group_lens, fmt: int = FMT_E4M3, block: int = BW_BLOCK):
+    """The copy with blocks along the rows for a tensor whose rows are split into groups
+    (quant_fp8_blockwise_segment_m_row_col_impl, zbpp_gemm.py:633, :785), in the layout the wgrad GEMM consumes:
+    transposed and segment-padded, ``(codes [cols, W], scale_inv [cols, W / block])`` with ``W = padded_width(rows,
+    G, block)``; group g owns columns ``[poff_g, poff_g + len_g)``, so the blocks restart at every group.  Padding is
+    zero codes; the scale_inv of a block that holds nothing is the one of an all-zero block."""
+    xf = bf16_bits_to_f32(to_bf16_bits(x))
+    rows, cols = xf.shape
+    lens = [max(int(n), 0) for n in group_lens]
+    W = padded_width(rows, len(lens), block)
+    codes = np.zeros((cols, W), np.uint8)
+    empty = np.float32(1.0) / (np.float32(_FP8_MAX[fmt]) / np.float32(1e-12))
+    sinv = np.full((cols, W // block), empty, np.float32)
+    src = dst = 0
+    for n in lens:
+        if n:
+            c, s = quantize_blockwise(f32_to_bf16_bits(xf[src:src + n]), fmt, 0, block)
+            codes[:, dst:dst + c.shape[1]] = c
+            sinv[:, dst // block:dst // block + s.shape[1]] = s
+        src += n
+        dst += (n + block - 1) // block * block
+    return codes, sinv
+
+
+def grouped_blockwise_gemm_nt_ref(a_codes, a_sinv, b_codes, b_sinv, group_lens, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, out_bf16=True):
+    """Rows of a split by group_lens, b [G, n, k] with b_sinv [G, n / 128, k / 128] (grouped_gemm_fp8_impl with blockwise
+    granularity, zbpp_gemm.py:608-630)."""
+    outs, pos = [], 0
+    for g, n in enumerate(max(int(v), 0) for v in group_lens):
+        outs.append(blockwise_gemm_nt_ref(a_codes[pos:pos + n], a_sinv[pos:pos + n], b_codes[g], b_sinv[g], a_fmt, b_fmt,
+                                          out_bf16=out_bf16))
+        pos += n
+    dt = np.uint16 if out_bf16 else np.float32
+    return np.concatenate(outs) if outs else np.zeros((0, b_codes.shape[1]), dt)
+
+
+def grouped_blockwise_wgrad_ref(a_codes, a_sinv, b_codes, b_sinv, group_lens, a_fmt=FMT_E4M3, b_fmt=FMT_E4M3, block: int = BW_BLOCK,
+                                out_bf16=True):
+    """c[g] = a[:, seg_g] . b[:, seg_g]^T on the segment-padded transposed copies (grouped_gemm_fp8_variable_k_impl,
+    zbpp_gemm.py:757-800); a group without tokens yields zeros."""
+    outs, pos = [], 0
+    for n in (max(int(v), 0) for v in group_lens):
+        w = (n + block - 1) // block * block
+        if w:
+            outs.append(blockwise_gemm_nt_ref(a_codes[:, pos:pos + w], a_sinv[:, pos // block:(pos + w) // block],
+                                              b_codes[:, pos:pos + w], b_sinv[:, pos // block:(pos + w) // block], a_fmt, b_fmt,
+                                              out_bf16=out_bf16))
+        else:
+            outs.append(np.zeros((a_codes.shape[0], b_codes.shape[0]), np.uint16 if out_bf16 else np.float32))
+        pos += w
+    return np.stack(outs)

@@ -66,6 +66,8 @@ EXPORTS = (
     "mxl_quantize_blockwise",
     "mxl_quantize_blockwise_weight",
     "mxl_gemm_nt_blockwise",
+    "mxl_grouped_gemm_nt_blockwise",
+    "mxl_grouped_gemm_wgrad_blockwise",
 )
 
 
@@ -156,9 +158,13 @@ def load() -> ctypes.CDLL:
         lib.mxl_unpad_groups.restype = i32
         lib.mxl_unpad_groups.argtypes = [vp, i64, i64, vp, i32, i32, vp, i64, vp]
         lib.mxl_quantize_blockwise.restype = i32
-        lib.mxl_quantize_blockwise.argtypes = [vp, i64, i64, i32, vp, vp, vp, vp, vp]
+        lib.mxl_quantize_blockwise.argtypes = [vp, i64, i64, i32, vp, i32, vp, vp, vp, vp, vp]
         lib.mxl_quantize_blockwise_weight.restype = i32
-        lib.mxl_quantize_blockwise_weight.argtypes = [vp, i64, i64, i32, vp, vp, vp, vp, vp]
+        lib.mxl_quantize_blockwise_weight.argtypes = [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp]
+        lib.mxl_grouped_gemm_nt_blockwise.restype = i32
+        lib.mxl_grouped_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        lib.mxl_grouped_gemm_wgrad_blockwise.restype = i32
+        lib.mxl_grouped_gemm_wgrad_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
         lib.mxl_gemm_nt_blockwise.restype = i32
         lib.mxl_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, i32, vp, i64, i64, i64, vp]
         _lib = lib

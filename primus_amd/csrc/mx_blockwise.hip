@@ -41,7 +41,70 @@ struct BwQuantArgs {
     float* sinv_row;
     uint8_t* q_colT;
     float* sinv_colT;
+    // grouped activations (1-D blocks only): the transposed copy is segment-padded like the MX one -- group g owns the
+    // columns [poff_g, poff_g + len_g) of its W = mxl_padded_width(rows, G) columns, poff = prefix sum of the lens
+    // rounded up to 128 -- so that the blocks along the tokens restart at every group
+    // (quant_fp8_blockwise_segment_m_row_col_impl, primus/backends/megatron/core/extensions/zbpp_gemm.py:633, :785)
+    const int64_t* group_lens;
+    int num_groups;
+    int64_t W;
 };
+
+constexpr int BW_MAX_GROUPS = 1024;
+
+// Which group holds tile `y` when every group is cut into tiles of 128 rows (a group's last tile may be ragged):
+// `pre` (LDS, BW_MAX_GROUPS + 1 ints) receives the prefix sum of the groups' tile counts, `red` (LDS, 4 words of 8
+// bytes) is scratch.  Returns the group (or -1 behind the last tile); tile_in_group, the rows in front of the group
+// and its length come back through the references.  Negative lens read as 0.  All threads of the workgroup call it.
+__device__ __forceinline__ int bw_locate(const int64_t* lens, int groups, int y, int* pre, int64_t* red, int& tile_in_group,
+                                         int64_t& rows_before, int64_t& len) {
+    const int t = threadIdx.x;
+    if (t == 0) pre[0] = 0;
+    for (int j = t; j < groups; j += BW_THREADS) {
+        const int64_t l = lens[j] > 0 ? lens[j] : 0;
+        pre[j + 1] = (int)((l + BW - 1) / BW);
+    }
+    __syncthreads();
+    if (t < 64) {   // in-place inclusive scan of pre[1 .. groups], a run of consecutive entries per lane
+        const int per = (groups + 63) / 64, j0 = 1 + t * per;
+        int sum = 0;
+        for (int i = 0; i < per; ++i)
+            if (j0 + i <= groups) sum += pre[j0 + i];
+        int incl = sum;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int o = __shfl_up(incl, d);
+            if (t >= d) incl += o;
+        }
+        int run = incl - sum;
+        for (int i = 0; i < per; ++i)
+            if (j0 + i <= groups) {
+                run += pre[j0 + i];
+                pre[j0 + i] = run;
+            }
+    }
+    __syncthreads();
+    int g = -1;
+    if (y < pre[groups]) {
+        int lo = 0, hi = groups;   // first index in (0, groups] whose prefix exceeds y
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (pre[mid] > y) hi = mid;
+            else lo = mid + 1;
+        }
+        g = lo - 1;
+    }
+    tile_in_group = g >= 0 ? y - pre[g] : 0;
+    int64_t part = 0;
+    for (int j = t; j < g; j += BW_THREADS) part += lens[j] > 0 ? lens[j] : 0;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) part += __shfl_xor(part, d);
+    if ((t & 63) == 0) red[t >> 6] = part;
+    __syncthreads();
+    rows_before = red[0] + red[1] + red[2] + red[3];
+    len = g >= 0 ? (lens[g] > 0 ? lens[g] : 0) : 0;
+    return g;
+}
 
 constexpr int BW_PITCH = 130;
 
@@ -52,16 +115,34 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
     __shared__ uint16_t tile[BW * BW_PITCH];
     __shared__ uint32_t amax_r[BW], amax_c[BW];
     __shared__ uint32_t amax_tile;
+    __shared__ int grp_pre[BW_MAX_GROUPS + 1];
+    __shared__ int64_t grp_red[4];
     const int t = threadIdx.x;
-    const int64_t row0 = (int64_t)blockIdx.y * BW, col0 = (int64_t)blockIdx.x * BW;
-    const int64_t rows_pad = (a.rows + BW - 1) / BW * BW;
+    const int64_t col0 = (int64_t)blockIdx.x * BW;
+    // the tile's rows: rows [row0, row0 + valid) of this matrix land in columns [prow0, prow0 + 128) of the transposed copy
+    const int64_t zoff = TWOD ? (int64_t)blockIdx.z : 0;          // matrix of a batch of weights
+    int64_t row0 = (int64_t)blockIdx.y * BW, prow0 = row0, rows_pad = (a.rows + BW - 1) / BW * BW;
+    int64_t valid = a.rows - row0 < BW ? a.rows - row0 : BW;
+    if (!TWOD && a.group_lens != nullptr) {
+        int tile_in_group;
+        int64_t before, len;
+        const int grp = bw_locate(a.group_lens, a.num_groups, (int)blockIdx.y, grp_pre, grp_red, tile_in_group, before, len);
+        // bw_locate counts tiles per group exactly as the padded layout counts 128-column pieces per segment
+        row0 = before + (int64_t)tile_in_group * BW;
+        valid = grp >= 0 ? len - (int64_t)tile_in_group * BW : 0;
+        valid = valid > BW ? BW : valid;
+        valid = row0 + valid > a.rows ? a.rows - row0 : valid;     // lens that claim more rows than there are
+        valid = valid < 0 ? 0 : valid;
+        rows_pad = a.W;
+    }
+    const uint16_t* xin = a.x + zoff * a.rows * a.cols;
     const int64_t kb_cols = a.cols / BW, kb_rows = rows_pad / BW;
     // load: 2048 pieces of 8 elements, 8 per thread; rows past the end read as zero
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int pc = i * BW_THREADS + t, r = pc >> 4, c8 = (pc & 15) * 8;
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + r < a.rows) v = *(const uint4*)(a.x + (row0 + r) * a.cols + col0 + c8);
+        if (r < valid) v = *(const uint4*)(xin + (row0 + r) * a.cols + col0 + c8);
         uint32_t* d = (uint32_t*)(tile + r * BW_PITCH + c8);   // pitch 130 elements: 4-byte aligned
         d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
     }
@@ -101,9 +182,9 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
         const float sc = scale_of(am);
         const bool bad = am >= 0x7F80u;
         const int64_t r = row0 + own;
-        if (r < a.rows) {
+        if (own < valid) {
             const uint32_t* p = (const uint32_t*)(tile + own * BW_PITCH + half * 64);
-            uint8_t* dst = a.q_row + r * a.cols + col0 + half * 64;
+            uint8_t* dst = a.q_row + (zoff * a.rows + r) * a.cols + col0 + half * 64;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 uint4 o;
@@ -115,7 +196,7 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
             }
             if (!TWOD && half == 0) a.sinv_row[r * kb_cols + blockIdx.x] = 1.0f / sc;
         }
-        if (TWOD && t == 0) a.sinv_row[(int64_t)blockIdx.y * kb_cols + blockIdx.x] = 1.0f / sc;
+        if (TWOD && t == 0) a.sinv_row[(zoff * kb_rows + blockIdx.y) * kb_cols + blockIdx.x] = 1.0f / sc;
     }
     // ---- transposed copy: half a column, 64 codes of row (col0 + own) of the output; rows past the end give zero codes ----
     if (a.q_colT != nullptr) {
@@ -123,7 +204,7 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
         const float sc = scale_of(am);
         const bool bad = am >= 0x7F80u;
         const uint16_t* q = tile + (half * 64) * BW_PITCH + own;
-        uint8_t* dst = a.q_colT + (col0 + own) * rows_pad + row0 + half * 64;
+        uint8_t* dst = a.q_colT + (zoff * a.cols + col0 + own) * rows_pad + prow0 + half * 64;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t w[4];
@@ -137,7 +218,7 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
             *(uint4*)(dst + 16 * i) = make_uint4(w[0], w[1], w[2], w[3]);
         }
         if (!TWOD && half == 0) a.sinv_colT[(col0 + own) * kb_rows + blockIdx.y] = 1.0f / sc;
-        if (TWOD && t == 0) a.sinv_colT[(int64_t)blockIdx.x * kb_rows + blockIdx.y] = 1.0f / sc;
+        if (TWOD && t == 0) a.sinv_colT[(zoff * kb_cols + blockIdx.x) * kb_rows + blockIdx.y] = 1.0f / sc;
     }
 }
 
@@ -155,6 +236,13 @@ struct BwGemmArgs {
     uint16_t* c;
     int64_t m, n, k;
     int sb_shift;
+    // mode 0: one dense GEMM.  mode 1 (forward / dgrad of a grouped linear): the rows of a are split by group_lens, b is
+    // [num_groups, n, k] with its factors per group, a row tile belongs to one group.  mode 2 (wgrad of a grouped
+    // linear): a [m, k] and b [n, k] are transposed segment-padded copies, group z = blockIdx.z contracts over its
+    // segment of k only and writes c[z] (zeros for a group without tokens).
+    int mode;
+    const int64_t* group_lens;
+    int num_groups;
 };
 
 constexpr int BW_GEMM_LDS = 2 * 2 * BW * BW + 2 * 2 * BW * 4;
@@ -165,20 +253,48 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t bw_smem[];
     uint8_t (*ops)[2][BW * BW] = (uint8_t (*)[2][BW * BW])bw_smem;                     // [stage][operand][row * 128 + swizzled piece]
     float (*fac)[2][BW] = (float (*)[2][BW])(bw_smem + 2 * 2 * BW * BW);               // [stage][operand][row]
+    __shared__ int grp_pre[BW_MAX_GROUPS + 1];
+    __shared__ int64_t grp_red[4];
     const int t = threadIdx.x;
     const int w = t >> 6, l = t & 63, lr = l & 31, g = l >> 5, wm = w >> 1, wn = w & 1;
-    const int64_t row0 = (int64_t)blockIdx.y * BW, col0 = (int64_t)blockIdx.x * BW;
+    int64_t row0 = (int64_t)blockIdx.y * BW;
+    const int64_t col0 = (int64_t)blockIdx.x * BW;
     const int64_t kb_n = p.k / BW;   // (the argument block itself is only read here and in the copies below)
+    int64_t m_end = p.m, b_group = 0, c_group = 0, kb0 = 0, kb1 = kb_n;
+    if (p.mode == 1) {
+        int tile_in_group;
+        int64_t before, len;
+        const int grp = bw_locate(p.group_lens, p.num_groups, (int)blockIdx.y, grp_pre, grp_red, tile_in_group, before, len);
+        if (grp < 0) return;                     // the grid is sized for the worst case (every group with a ragged tile)
+        row0 = before + (int64_t)tile_in_group * BW;
+        m_end = before + len < p.m ? before + len : p.m;
+        if (row0 >= m_end) return;
+        b_group = grp;
+    } else if (p.mode == 2) {
+        // this group's segment of the contraction: [sum of the padded lens in front, + its own padded len), in blocks
+        const int grp = (int)blockIdx.z;
+        int64_t part = 0;
+        for (int j = t; j < grp; j += BW_THREADS) part += ((p.group_lens[j] > 0 ? p.group_lens[j] : 0) + BW - 1) / BW;
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) part += __shfl_xor(part, d);
+        if ((t & 63) == 0) grp_red[t >> 6] = part;
+        __syncthreads();
+        kb0 = grp_red[0] + grp_red[1] + grp_red[2] + grp_red[3];
+        kb1 = kb0 + ((p.group_lens[grp] > 0 ? p.group_lens[grp] : 0) + BW - 1) / BW;
+        kb0 = kb0 > kb_n ? kb_n : kb0;           // lens that claim more than the operands hold
+        kb1 = kb1 > kb_n ? kb_n : kb1;
+        c_group = grp;
+    }
     // loader geometry: piece pc = i * 256 + t of an operand's 1024 pieces: row pc / 8 = 32 i + t / 8, piece t % 8.
     // Everything the loop needs from the argument block is copied to locals first (and the loader is written as
     // macros over scalars): a lambda that captures the block or an array by reference puts it on the stack.
-    const uint8_t* const pa = p.a;
-    const uint8_t* const pb = p.b;
-    const float* const psa = p.sa;
-    const float* const psb = p.sb;
-    const int64_t pm = p.m, pk = p.k, pn = p.n;
-    uint16_t* const pc_out = p.c;
+    const int64_t pm = m_end, pk = p.k, pn = p.n;
     const int sb_shift = p.sb_shift;
+    const uint8_t* const pa = p.a;
+    const uint8_t* const pb = p.b + b_group * pn * pk;
+    const float* const psa = p.sa;
+    const float* const psb = p.sb + b_group * (pn >> sb_shift) * kb_n;
+    uint16_t* const pc_out = p.c + c_group * p.m * pn;
     const int lrow = t >> 3, lpc = t & 7;
     const int lds_off = lrow * BW + 16 * (lpc ^ (lrow & 7));      // rows 32 i + lrow share (row & 7)
     const uint8_t* ga = pa + (row0 + lrow) * pk + lpc * 16;
@@ -220,12 +336,14 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-    MXL_BW_FETCH(0);
-    MXL_BW_STASH(0);
+    if (kb0 < kb1) {
+        MXL_BW_FETCH(kb0);
+        MXL_BW_STASH(0);
+    }
     __syncthreads();
-    for (int64_t kb = 0; kb < kb_n; ++kb) {
-        const int st = (int)(kb & 1);
-        if (kb + 1 < kb_n) MXL_BW_FETCH(kb + 1);
+    for (int64_t kb = kb0; kb < kb1; ++kb) {
+        const int st = (int)((kb - kb0) & 1);
+        if (kb + 1 < kb1) MXL_BW_FETCH(kb + 1);
         bv16f part[2][2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -269,7 +387,7 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
                     acc[i][j][4 * q + 3] = fmaf(part[i][j][4 * q + 3], sa * sb.w, acc[i][j][4 * q + 3]);
                 }
         }
-        if (kb + 1 < kb_n) MXL_BW_STASH(st ^ 1);   // the other stage was last read before the previous iteration's barrier
+        if (kb + 1 < kb1) MXL_BW_STASH(st ^ 1);   // the other stage was last read before the previous iteration's barrier
         __syncthreads();
     }
 #undef MXL_BW_FETCH
@@ -290,54 +408,52 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
 }
 
 template <bool TWOD>
-static int launch_bw_quant(const BwQuantArgs& a, int fmt, hipStream_t st) {
-    const dim3 grid((unsigned)(a.cols / BW), (unsigned)((a.rows + BW - 1) / BW));
+static int launch_bw_quant(const BwQuantArgs& a, int fmt, int64_t row_tiles, int batch, hipStream_t st) {
+    const dim3 grid((unsigned)(a.cols / BW), (unsigned)row_tiles, (unsigned)batch);
     if (fmt == MXL_FMT_E4M3) hipLaunchKernelGGL((bw_quant_kernel<MXL_FMT_E4M3, TWOD>), grid, dim3(BW_THREADS), 0, st, a);
     else hipLaunchKernelGGL((bw_quant_kernel<MXL_FMT_E5M2, TWOD>), grid, dim3(BW_THREADS), 0, st, a);
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
-static int bw_quant(const void* x, int64_t rows, int64_t cols, int fmt, void* q_row, void* sinv_row, void* q_colT,
-                    void* sinv_colT, bool twod, void* stream) {
+static int bw_quant(const void* x, int64_t rows, int64_t cols, int fmt, const int64_t* group_lens, int num_groups, int batch,
+                    void* q_row, void* sinv_row, void* q_colT, void* sinv_colT, bool twod, void* stream) {
     if (rows < 0 || cols <= 0 || cols % BW != 0 || (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
     if ((q_row == nullptr) != (sinv_row == nullptr) || (q_colT == nullptr) != (sinv_colT == nullptr)) return MXL_EINVAL;
     if (!q_row && !q_colT) return MXL_EINVAL;
-    if (twod && rows % BW != 0) return MXL_EINVAL;
-    if (rows == 0) return MXL_OK;
-    if (!x || ((uintptr_t)x & 15) != 0 || (rows + BW - 1) / BW > 65535) return MXL_EINVAL;
+    if (batch < 1 || batch > 65535 || (twod && rows % BW != 0) || (!twod && batch != 1)) return MXL_EINVAL;
+    if (num_groups < 0 || num_groups > BW_MAX_GROUPS || (num_groups > 0) != (group_lens != nullptr) || (twod && num_groups)) return MXL_EINVAL;
+    const int64_t W = num_groups ? mxl_padded_width(rows, num_groups) : (rows + BW - 1) / BW * BW;
+    const int64_t row_tiles = W / BW;       // with groups: the 128-column pieces of the padded transposed copy
+    if (row_tiles == 0) return MXL_OK;
+    if (!x && rows > 0) return MXL_EINVAL;
+    if (((uintptr_t)x & 15) != 0 || row_tiles > 65535) return MXL_EINVAL;
     if ((((uintptr_t)q_row | (uintptr_t)q_colT) & 15) != 0) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
-    BwQuantArgs a{(const uint16_t*)x, rows, cols, (uint8_t*)q_row, (float*)sinv_row, (uint8_t*)q_colT, (float*)sinv_colT};
-    return twod ? launch_bw_quant<true>(a, fmt, (hipStream_t)stream) : launch_bw_quant<false>(a, fmt, (hipStream_t)stream);
+    BwQuantArgs a{(const uint16_t*)x, rows, cols, (uint8_t*)q_row, (float*)sinv_row, (uint8_t*)q_colT, (float*)sinv_colT,
+                  group_lens, num_groups, W};
+    return twod ? launch_bw_quant<true>(a, fmt, row_tiles, batch, (hipStream_t)stream)
+                : launch_bw_quant<false>(a, fmt, row_tiles, 1, (hipStream_t)stream);
 }
 
-}  // namespace mxl
-
-using namespace mxl;
-
-extern "C" int mxl_quantize_blockwise(const void* x_bf16, int64_t rows, int64_t cols, int fmt, void* q_row, void* sinv_row,
-                                      void* q_colT, void* sinv_colT, void* stream) {
-    return bw_quant(x_bf16, rows, cols, fmt, q_row, sinv_row, q_colT, sinv_colT, false, stream);
-}
-
-extern "C" int mxl_quantize_blockwise_weight(const void* w_bf16, int64_t n, int64_t k, int fmt, void* q, void* sinv, void* q_T,
-                                             void* sinv_T, void* stream) {
-    return bw_quant(w_bf16, n, k, fmt, q, sinv, q_T, sinv_T, true, stream);
-}
-
-extern "C" int mxl_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,
-                                     int b_fmt, int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k,
-                                     void* stream) {
-    if (m < 0 || n <= 0 || k <= 0 || n % BW != 0 || k % BW != 0) return MXL_EINVAL;
+static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv, int b_fmt,
+                   int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k, int mode, const int64_t* group_lens,
+                   int num_groups, void* stream) {
+    if (m < 0 || n <= 0 || k < 0 || n % BW != 0 || k % BW != 0) return MXL_EINVAL;
     if (b_rows_per_scale != 1 && b_rows_per_scale != BW) return MXL_EINVAL;
     if ((a_fmt != MXL_FMT_E4M3 && a_fmt != MXL_FMT_E5M2) || (b_fmt != MXL_FMT_E4M3 && b_fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
+    if (mode != 0 && (!group_lens || num_groups < 1 || num_groups > BW_MAX_GROUPS)) return MXL_EINVAL;
     if (m == 0) return MXL_OK;
-    if (!a_codes || !a_sinv || !b_codes || !b_sinv || !c_bf16 || (m + BW - 1) / BW > 65535) return MXL_EINVAL;
-    if ((((uintptr_t)a_codes | (uintptr_t)b_codes) & 15) != 0 || ((uintptr_t)c_bf16 & 7) != 0) return MXL_EINVAL;
+    if (!c_bf16 || ((uintptr_t)c_bf16 & 7) != 0) return MXL_EINVAL;
+    if (k > 0 && (!a_codes || !a_sinv || !b_codes || !b_sinv)) return MXL_EINVAL;
+    if (k == 0 && mode != 2) return MXL_EINVAL;
+    if ((((uintptr_t)a_codes | (uintptr_t)b_codes) & 15) != 0) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
+    // row tiles: exact for a dense GEMM and for wgrad; at most one ragged tile per group in the grouped forward
+    const int64_t row_tiles = mode == 1 ? m / BW + num_groups : (m + BW - 1) / BW;
+    if (row_tiles > 65535 || (mode == 2 && num_groups > 65535)) return MXL_EINVAL;
     BwGemmArgs g{(const uint8_t*)a_codes, (const float*)a_sinv, (const uint8_t*)b_codes, (const float*)b_sinv, (uint16_t*)c_bf16,
-                 m, n, k, b_rows_per_scale == 1 ? 0 : 7};
-    const dim3 grid((unsigned)(n / BW), (unsigned)((m + BW - 1) / BW));
+                 m, n, k, b_rows_per_scale == 1 ? 0 : 7, mode, group_lens, num_groups};
+    const dim3 grid((unsigned)(n / BW), (unsigned)row_tiles, (unsigned)(mode == 2 ? num_groups : 1));
     hipStream_t st = (hipStream_t)stream;
     // the dynamic LDS size is above the default limit: the attribute is set at every launch (a host-side table write)
 #define MXL_BW_GEMM(A, B)                                                                                                \
@@ -353,4 +469,42 @@ extern "C" int mxl_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, in
     else MXL_BW_GEMM(MXL_FMT_E5M2, MXL_FMT_E5M2);
 #undef MXL_BW_GEMM
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
+
+}  // namespace mxl
+
+using namespace mxl;
+
+extern "C" int mxl_quantize_blockwise(const void* x_bf16, int64_t rows, int64_t cols, int fmt, const int64_t* group_lens,
+                                      int num_groups, void* q_row, void* sinv_row, void* q_colT, void* sinv_colT, void* stream) {
+    return bw_quant(x_bf16, rows, cols, fmt, group_lens, num_groups, 1, q_row, sinv_row, q_colT, sinv_colT, false, stream);
+}
+
+extern "C" int mxl_quantize_blockwise_weight(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int fmt, void* q, void* sinv,
+                                             void* q_T, void* sinv_T, void* stream) {
+    if (batch < 1 || batch > 65535) return MXL_EINVAL;
+    return bw_quant(w_bf16, n, k, fmt, nullptr, 0, (int)batch, q, sinv, q_T, sinv_T, true, stream);
+}
+
+extern "C" int mxl_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,
+                                     int b_fmt, int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k,
+                                     void* stream) {
+    if (k <= 0) return MXL_EINVAL;
+    return bw_gemm(a_codes, a_sinv, a_fmt, b_codes, b_sinv, b_fmt, b_rows_per_scale, c_bf16, m, n, k, 0, nullptr, 0, stream);
+}
+
+extern "C" int mxl_grouped_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes,
+                                             const void* b_sinv, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                             int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
+    if (k <= 0) return MXL_EINVAL;
+    return bw_gemm(a_codes, a_sinv, a_fmt, b_codes, b_sinv, b_fmt, BW, c_bf16, total_m, n, k, 1, group_lens, num_groups, stream);
+}
+
+extern "C" int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes,
+                                                const void* b_sinv, int b_fmt, void* c_bf16, const int64_t* group_lens,
+                                                int num_groups, int64_t total_m, int64_t n, int64_t k, void* stream) {
+    if (total_m < 0 || num_groups < 1) return MXL_EINVAL;
+    // a: dY^T [n, W], b: X^T [k, W], W = mxl_padded_width(total_m, num_groups); c [num_groups, n, k]
+    return bw_gemm(a_codes, a_sinv, a_fmt, b_codes, b_sinv, b_fmt, 1, c_bf16, n, k, mxl_padded_width(total_m, num_groups), 2,
+                   group_lens, num_groups, stream);
 }

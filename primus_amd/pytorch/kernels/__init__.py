@@ -1007,35 +1007,48 @@ def _bw_check(x, fmt, what):
         raise ValueError(f"the blockwise recipe needs the last dimension to be a multiple of {BW_BLOCK} (got {x.shape[1]})")
 
 
-def quantize_blockwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool = False):
+def quantize_blockwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool = False,
+                            group_lens: Optional[torch.Tensor] = None):
     """``quant_fp8_blockwise_impl`` for both axes in one launch (primus_turbo_float8_local.py:1019, :1053-1059):
-    ``(codes [rows, cols], scale_inv f32 [rows, cols / 128], codes_T [cols, rows_pad], scale_inv_T f32
-    [cols, rows_pad / 128])``; the row-wise copy has 1 x 128 blocks along the columns, the transposed one 128 x 1
-    blocks along the rows (``rows_pad``: rows rounded up to 128, zero codes).  Copies not asked for are None."""
+    ``(codes [rows, cols], scale_inv f32 [rows, cols / 128], codes_T [cols, W], scale_inv_T f32 [cols, W / 128])``;
+    the row-wise copy has 1 x 128 blocks along the columns, the transposed one 128 x 1 blocks along the rows.
+    Without ``group_lens`` W is rows rounded up to 128 (zero codes); with it the rows are split into groups and the
+    transposed copy is segment-padded, ``W = padded_width(rows, G)``, blocks restarting at every group
+    (``quant_fp8_blockwise_segment_m_row_col_impl``, zbpp_gemm.py:633, :785).  Copies not asked for are None."""
     _bw_check(x, fmt, "x")
     if not (rowwise or colwise):
         raise ValueError("at least one copy must be requested")
     rows, cols = x.shape
-    rows_pad = _round_up(rows, BW_BLOCK)
+    G = _check_group_lens(group_lens, x.device) if colwise else 0
+    W = padded_width(rows, G) if G else _round_up(rows, BW_BLOCK)
     dt = _code_dtype(fmt) if fmt != _lib.FMT_E5M2 else torch.float8_e5m2
     q = s = qt = st = None
     if rowwise:
         q = torch.empty((rows, cols), dtype=torch.uint8, device=x.device)
         s = torch.empty((rows, cols // BW_BLOCK), dtype=torch.float32, device=x.device)
     if colwise:
-        qt = torch.empty((cols, rows_pad), dtype=torch.uint8, device=x.device)
-        st = torch.empty((cols, rows_pad // BW_BLOCK), dtype=torch.float32, device=x.device)
+        qt = torch.empty((cols, W), dtype=torch.uint8, device=x.device)
+        st = torch.empty((cols, W // BW_BLOCK), dtype=torch.float32, device=x.device)
     with _hooked("quantize_blockwise", rows=rows, cols=cols, fmt=fmt, rowwise=rowwise, colwise=colwise):
-        rc = _lib.load().mxl_quantize_blockwise(_ptr(x), rows, cols, fmt, _ptr(q), _ptr(s), _ptr(qt), _ptr(st), _stream())
+        rc = _lib.load().mxl_quantize_blockwise(_ptr(x), rows, cols, fmt, _ptr(group_lens) if G else None, G, _ptr(q), _ptr(s),
+                                                _ptr(qt), _ptr(st), _stream())
     _lib.check(rc, "mxl_quantize_blockwise")
     return (q.view(dt) if q is not None else None), s, (qt.view(dt) if qt is not None else None), st
 
 
 def quantize_blockwise_weight_impl(w, fmt: int, *, rowwise: bool = True, colwise: bool = False):
     """``quant_fp8_blockwise_for_weight_impl`` (primus_turbo_float8_local.py:1020, :1060): one scale per 128 x 128
-    block of ``w [n, k]``.  ``(codes [n, k], scale_inv f32 [n / 128, k / 128], codes_T [k, n], scale_inv_T)``."""
-    _bw_check(w, fmt, "w")
-    n, k = w.shape
+    block of ``w [n, k]`` or of every matrix of ``w [G, n, k]``.  ``(codes [.., n, k], scale_inv f32 [.., n / 128,
+    k / 128], codes_T [.., k, n], scale_inv_T)``."""
+    if w.dim() == 3:
+        _bw_check(w[0] if w.shape[0] else w.reshape(-1, w.shape[-1]), fmt, "w")
+        if not w.is_contiguous():
+            raise ValueError("w must be contiguous")
+    else:
+        _bw_check(w, fmt, "w")
+    lead = tuple(w.shape[:-2])
+    batch = lead[0] if lead else 1
+    n, k = w.shape[-2], w.shape[-1]
     if n % BW_BLOCK != 0:
         raise ValueError(f"the blockwise recipe needs weight dimensions that are multiples of {BW_BLOCK} (got {n})")
     if not (rowwise or colwise):
@@ -1043,14 +1056,15 @@ def quantize_blockwise_weight_impl(w, fmt: int, *, rowwise: bool = True, colwise
     dt = _code_dtype(fmt) if fmt != _lib.FMT_E5M2 else torch.float8_e5m2
     q = s = qt = st = None
     if rowwise:
-        q = torch.empty((n, k), dtype=torch.uint8, device=w.device)
-        s = torch.empty((n // BW_BLOCK, k // BW_BLOCK), dtype=torch.float32, device=w.device)
+        q = torch.empty(lead + (n, k), dtype=torch.uint8, device=w.device)
+        s = torch.empty(lead + (n // BW_BLOCK, k // BW_BLOCK), dtype=torch.float32, device=w.device)
     if colwise:
-        qt = torch.empty((k, n), dtype=torch.uint8, device=w.device)
-        st = torch.empty((k // BW_BLOCK, n // BW_BLOCK), dtype=torch.float32, device=w.device)
-    with _hooked("quantize_blockwise_weight", rows=n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
-        rc = _lib.load().mxl_quantize_blockwise_weight(_ptr(w), n, k, fmt, _ptr(q), _ptr(s), _ptr(qt), _ptr(st), _stream())
-    _lib.check(rc, "mxl_quantize_blockwise_weight")
+        qt = torch.empty(lead + (k, n), dtype=torch.uint8, device=w.device)
+        st = torch.empty(lead + (k // BW_BLOCK, n // BW_BLOCK), dtype=torch.float32, device=w.device)
+    if batch:
+        with _hooked("quantize_blockwise_weight", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
+            rc = _lib.load().mxl_quantize_blockwise_weight(_ptr(w), batch, n, k, fmt, _ptr(q), _ptr(s), _ptr(qt), _ptr(st), _stream())
+        _lib.check(rc, "mxl_quantize_blockwise_weight")
     return (q.view(dt) if q is not None else None), s, (qt.view(dt) if qt is not None else None), st
 
 
@@ -1062,28 +1076,70 @@ def _fp8_fmt_of(codes: torch.Tensor) -> int:
     raise ValueError(f"not an FP8 code tensor: {codes.dtype}")
 
 
-def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv) -> torch.Tensor:
-    """``gemm_fp8_impl(..., granularity=BLOCKWISE)`` in NT form (primus_turbo_float8_local.py:1022-1033):
+def _bw_scales(t, shape, what):
+    if t.dtype != torch.float32 or tuple(t.shape) != tuple(shape) or not t.is_contiguous():
+        raise ValueError(f"{what} must be contiguous float32 {tuple(shape)}")
+
+
+def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv, group_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gemm_fp8_impl`` / ``grouped_gemm_fp8_impl`` with ``granularity=BLOCKWISE`` in NT form
+    (primus_turbo_float8_local.py:1022-1033, zbpp_gemm.py:608-630):
     ``c[m, n] = sum_kb a_scale_inv[m, kb] * b_scale_inv[n or n / 128, kb] * (a[m, kb] . b[n, kb])``, bf16.
-    ``b_scale_inv`` has one row per row of ``b`` (an activation copy) or one per 128 rows (a weight)."""
-    _require_cuda(a, a_scale_inv, b, b_scale_inv)
+    Dense: ``b [n, k]``, ``b_scale_inv`` with one row per row of ``b`` (an activation copy) or one per 128 rows (a
+    weight).  Grouped: the rows of ``a`` are split by ``group_lens``, ``b [G, n, k]``, ``b_scale_inv [G, n / 128, k / 128]``."""
+    _require_cuda(a, a_scale_inv, b, b_scale_inv, group_lens)
+    G = _check_group_lens(group_lens, a.device)
     m, k = a.shape
-    n = b.shape[0]
-    if b.shape[1] != k or k % BW_BLOCK != 0 or n % BW_BLOCK != 0:
+    n = b.shape[-2]
+    if b.shape[-1] != k or k % BW_BLOCK != 0 or n % BW_BLOCK != 0 or k == 0:
         raise ValueError("blockwise GEMM: contraction lengths must agree and k, n must be multiples of 128")
-    kb = k // BW_BLOCK
-    if a_scale_inv.dtype != torch.float32 or tuple(a_scale_inv.shape) != (m, kb) or not a_scale_inv.is_contiguous():
-        raise ValueError("a_scale_inv must be contiguous float32 [m, k / 128]")
-    if b_scale_inv.dtype != torch.float32 or not b_scale_inv.is_contiguous() or tuple(b_scale_inv.shape) not in ((n, kb), (n // BW_BLOCK, kb)):
-        raise ValueError("b_scale_inv must be contiguous float32 [n, k / 128] or [n / 128, k / 128]")
-    per = 1 if (b_scale_inv.shape[0] == n and n != n // BW_BLOCK) else BW_BLOCK
     if not (a.is_contiguous() and b.is_contiguous()):
         raise ValueError("code tensors must be contiguous")
+    kb = k // BW_BLOCK
+    _bw_scales(a_scale_inv, (m, kb), "a_scale_inv")
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    lib = _lib.load()
+    if G:
+        if b.dim() != 3 or b.shape[0] != G:
+            raise ValueError("grouped blockwise GEMM expects weights of shape [num_groups, n, k]")
+        _bw_scales(b_scale_inv, (G, n // BW_BLOCK, kb), "b_scale_inv")
+        with _hooked("grouped_gemm_blockwise_nt", m=m, n=n, k=k):
+            rc = lib.mxl_grouped_gemm_nt_blockwise(_ptr(a), _ptr(a_scale_inv), _fp8_fmt_of(a), _ptr(b), _ptr(b_scale_inv),
+                                                   _fp8_fmt_of(b), _ptr(c), _ptr(group_lens), G, m, n, k, _stream())
+        _lib.check(rc, "mxl_grouped_gemm_nt_blockwise")
+        return c
+    if b.dim() != 2:
+        raise ValueError("dense blockwise GEMM expects b [n, k]")
+    if b_scale_inv.dtype != torch.float32 or not b_scale_inv.is_contiguous() or tuple(b_scale_inv.shape) not in ((n, kb), (n // BW_BLOCK, kb)):
+        raise ValueError("b_scale_inv must be contiguous float32 [n, k / 128] or [n / 128, k / 128]")
+    per = 1 if b_scale_inv.shape[0] == n else BW_BLOCK
     with _hooked("gemm_blockwise_nt", m=m, n=n, k=k):
-        rc = _lib.load().mxl_gemm_nt_blockwise(_ptr(a), _ptr(a_scale_inv), _fp8_fmt_of(a), _ptr(b), _ptr(b_scale_inv),
-                                               _fp8_fmt_of(b), per, _ptr(c), m, n, k, _stream())
+        rc = lib.mxl_gemm_nt_blockwise(_ptr(a), _ptr(a_scale_inv), _fp8_fmt_of(a), _ptr(b), _ptr(b_scale_inv),
+                                       _fp8_fmt_of(b), per, _ptr(c), m, n, k, _stream())
     _lib.check(rc, "mxl_gemm_nt_blockwise")
+    return c
+
+
+def grouped_gemm_blockwise_wgrad_impl(a_t, a_t_scale_inv, b_t, b_t_scale_inv, group_lens, total_m: int) -> torch.Tensor:
+    """``grouped_gemm_fp8_variable_k_impl`` with blockwise granularity (zbpp_gemm.py:757-800) on the segment-padded
+    transposed copies: ``a_t = q_colT(dY) [n, W]``, ``b_t = q_colT(X) [k, W]`` with their ``[rows, W / 128]`` factors;
+    ``c [G, n, k]``, zeros for a group without tokens."""
+    _require_cuda(a_t, a_t_scale_inv, b_t, b_t_scale_inv, group_lens)
+    G = _check_group_lens(group_lens, a_t.device)
+    if not G:
+        raise ValueError("group_lens is required")
+    W = padded_width(int(total_m), G)
+    n, k = a_t.shape[0], b_t.shape[0]
+    if a_t.shape[1] != W or b_t.shape[1] != W or n % BW_BLOCK or k % BW_BLOCK or not (a_t.is_contiguous() and b_t.is_contiguous()):
+        raise ValueError(f"transposed operands must be contiguous [rows, {W}] with rows a multiple of 128")
+    _bw_scales(a_t_scale_inv, (n, W // BW_BLOCK), "a_t_scale_inv")
+    _bw_scales(b_t_scale_inv, (k, W // BW_BLOCK), "b_t_scale_inv")
+    c = torch.empty((G, n, k), dtype=torch.bfloat16, device=a_t.device)
+    with _hooked("grouped_gemm_blockwise_wgrad", m=int(total_m), n=n, k=k):
+        rc = _lib.load().mxl_grouped_gemm_wgrad_blockwise(_ptr(a_t), _ptr(a_t_scale_inv), _fp8_fmt_of(a_t), _ptr(b_t),
+                                                          _ptr(b_t_scale_inv), _fp8_fmt_of(b_t), _ptr(c), _ptr(group_lens), G,
+                                                          int(total_m), n, k, _stream())
+    _lib.check(rc, "mxl_grouped_gemm_wgrad_blockwise")
     return c
 
 

@@ -371,38 +371,43 @@ class _TWLinearFunction(torch.autograd.Function):
 
 
 class _BWLinearFunction(torch.autograd.Function):
-    """Y = X . W^T under the 128-blockwise FP8 recipe (FP8LinearBlockwiseFunction,
-    primus_turbo_float8_local.py:993-1089): X in 1 x 128 blocks, W in 128 x 128 blocks, forward format; like the
-    reference the backward starts from the bf16 tensors again and quantises dY (both axes), X (along the tokens) and
-    W in the backward format (E5M2 for Format.HYBRID).  Every GEMM is NT on the transposed copies the quantisers write."""
+    """Y = X . W^T under the 128-blockwise FP8 recipe, dense (FP8LinearBlockwiseFunction,
+    primus_turbo_float8_local.py:993-1089) or grouped (zbpp_gemm.py:590-640, :757-800): X in 1 x 128 blocks, W in
+    128 x 128 blocks, forward format; like the reference the backward starts from the bf16 tensors again and quantises
+    dY (both axes), X (along the tokens, blocks restarting at every group) and W in the backward format (E5M2 for
+    Format.HYBRID).  Every GEMM is NT on the transposed copies the quantisers write."""
 
     @staticmethod
-    def forward(ctx, a, b, fwd_fmt, bwd_fmt, accum=None):
+    def forward(ctx, a, b, group_lens, fwd_fmt, bwd_fmt, accum=None):
         a_row, a_s, _, _ = K.quantize_blockwise_impl(a, fwd_fmt, rowwise=True, colwise=False)
         w_row, w_s, _, _ = K.quantize_blockwise_weight_impl(b.detach(), fwd_fmt, rowwise=True, colwise=False)
-        y = K.gemm_blockwise_nt_impl(a_row, a_s, w_row, w_s)
-        ctx.save_for_backward(a, b)
+        y = K.gemm_blockwise_nt_impl(a_row, a_s, w_row, w_s, group_lens)
+        ctx.save_for_backward(a, b, group_lens)
         ctx.cfg = (bwd_fmt, a.requires_grad, b.requires_grad)
         ctx.accum = accum
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        a, b = ctx.saved_tensors
+        a, b, group_lens = ctx.saved_tensors
         bwd_fmt, need_dgrad, need_wgrad = ctx.cfg
         dy = dy.contiguous()
         if dy.dtype != torch.bfloat16:
             dy = dy.to(torch.bfloat16)
-        d_row, d_s, d_col, d_cs = K.quantize_blockwise_impl(dy, bwd_fmt, rowwise=need_dgrad, colwise=need_wgrad)
+        d_row, d_s, d_col, d_cs = K.quantize_blockwise_impl(dy, bwd_fmt, rowwise=need_dgrad, colwise=need_wgrad,
+                                                            group_lens=group_lens)
         grad_a = grad_b = None
         if need_dgrad:
             _, _, w_col, w_cs = K.quantize_blockwise_weight_impl(b.detach(), bwd_fmt, rowwise=False, colwise=True)
-            grad_a = K.gemm_blockwise_nt_impl(d_row, d_s, w_col, w_cs)
+            grad_a = K.gemm_blockwise_nt_impl(d_row, d_s, w_col, w_cs, group_lens)
         if need_wgrad:
-            _, _, a_col, a_cs = K.quantize_blockwise_impl(a.detach(), bwd_fmt, rowwise=False, colwise=True)
-            grad_b = K.gemm_blockwise_nt_impl(d_col, d_cs, a_col, a_cs)
+            _, _, a_col, a_cs = K.quantize_blockwise_impl(a.detach(), bwd_fmt, rowwise=False, colwise=True, group_lens=group_lens)
+            if group_lens is None:
+                grad_b = K.gemm_blockwise_nt_impl(d_col, d_cs, a_col, a_cs)
+            else:
+                grad_b = K.grouped_gemm_blockwise_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, a.shape[0])
             grad_b = _finish_wgrad(grad_b, ctx.accum, False, tuple(b.shape))
-        return grad_a, grad_b, None, None, None
+        return grad_a, grad_b, None, None, None, None
 
 
 def _tensorwise_formats(config):
@@ -442,8 +447,8 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
     tensorwise = (not fp4) and isinstance(config, Float8QuantConfig) and config.granularity == ScalingGranularity.TENSORWISE
     blockwise = (not fp4) and isinstance(config, Float8QuantConfig) and config.granularity == ScalingGranularity.BLOCKWISE
     if blockwise:
-        if group_lens is not None or glu is not None or norm is not None or not torch.is_tensor(b):
-            raise NotImplementedError("the 128-blockwise recipe is built for the dense linear on a bfloat16 weight")
+        if glu is not None or norm is not None or not torch.is_tensor(b):
+            raise NotImplementedError("the 128-blockwise recipe runs on a bfloat16 weight, without the fused prologues")
         if config.block_size not in (None, 128):
             raise NotImplementedError(f"blockwise scaling is built for block_size 128 (got {config.block_size})")
     if tensorwise or blockwise:
@@ -479,9 +484,9 @@ def _run(a, b, group_lens, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum
     # accumulates for every recipe
     accum = _accum_from(b, fuse_bgrad_accum_pattern)
     if blockwise:
-        if a.shape[-1] % 128 != 0 or b.shape[0] % 128 != 0:
+        if a.shape[-1] % 128 != 0 or b.shape[-2] % 128 != 0:
             raise ValueError("the 128-blockwise recipe needs K and N to be multiples of 128")
-        return _BWLinearFunction.apply(a, b, fwd_fmt, bwd_fmt, accum)
+        return _BWLinearFunction.apply(a, b, group_lens, fwd_fmt, bwd_fmt, accum)
     if tensorwise:
         if glu is not None or norm is not None:
             raise NotImplementedError("the activation / normalisation prologues exist for the MX recipes only")

@@ -163,9 +163,12 @@ def test_operator_refuses_what_the_recipe_does_not_cover(gpu):
     w = torch.zeros(128, 96, device=gpu).bfloat16()
     with pytest.raises(ValueError):
         turbo.ops.gemm_fp8(x, w, config=cfg)                       # K is not a multiple of 128
-    wg = torch.zeros(2, 128, 128, device=gpu).bfloat16()
+    wg = torch.zeros(2, 96, 128, device=gpu).bfloat16()
+    with pytest.raises(ValueError):
+        turbo.ops.grouped_gemm_fp8(torch.zeros(8, 128, device=gpu).bfloat16(), wg, torch.tensor([4, 4], device=gpu), config=cfg)   # N = 96
     with pytest.raises(NotImplementedError):
-        turbo.ops.grouped_gemm_fp8(torch.zeros(8, 128, device=gpu).bfloat16(), wg, torch.tensor([4, 4], device=gpu), config=cfg)
+        turbo.ops.rmsnorm_gemm_fp8(torch.zeros(8, 128, device=gpu).bfloat16(), torch.ones(128, device=gpu).bfloat16(), 1e-5,
+                                   torch.zeros(128, 128, device=gpu).bfloat16(), config=cfg)
 
 
 @pytest.mark.parametrize("microbatches", [1, 2])
@@ -201,6 +204,133 @@ def test_megatron_linear_under_the_blockwise_recipe(gpu, microbatches):
         yr = torch.nn.functional.linear(xr, wr)
         yr.backward(dy)
         assert _cos(y, yr) > 0.998 and _cos(x.grad, xr.grad) > 0.998 and _cos(lin.weight.grad, wr.grad) > 0.998
+    finally:
+        pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+        runtime.set_args()
+        runtime.set_num_microbatches(1)
+
+
+GROUPS = [([5, 0, 130, 64, 0, 1], 256), ([128, 128], 128), ([300], 384), ([0, 0, 7], 128), ([1] * 40 + [0] * 5 + [200], 256)]
+
+
+@pytest.mark.parametrize("fmt", [0, 2])
+@pytest.mark.parametrize("lens,cols", GROUPS)
+def test_grouped_quantiser_equals_the_oracle(gpu, fmt, lens, cols):
+    """The copy with blocks along the tokens of a grouped tensor: transposed, segment-padded, blocks restarting at
+    every group; the row-wise copy of the same launch is the ungrouped one."""
+    from primus_amd.pytorch import kernels as K
+
+    rows = sum(lens)
+    x = _x(rows + cols + fmt, rows, cols, 2.0)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    q, s, qt, st = K.quantize_blockwise_impl(x.to(gpu), fmt, rowwise=True, colwise=True, group_lens=gl)
+    wq, ws = o.quantize_blockwise(x, fmt, axis=-1)
+    wqt, wst = o.quantize_blockwise_segmented(x, lens, fmt)
+    assert np.array_equal(_u8(q), wq) and np.array_equal(s.cpu().numpy(), ws)
+    assert tuple(qt.shape) == wqt.shape == (cols, o.padded_width(rows, len(lens), 128))
+    assert np.array_equal(_u8(qt), wqt) and np.array_equal(st.cpu().numpy(), wst)
+
+
+@pytest.mark.parametrize("fmt", [0, 2])
+def test_weight_batch_equals_the_oracle(gpu, fmt):
+    from primus_amd.pytorch import kernels as K
+
+    w = (_x(9 + fmt, 3 * 256, 384) * 0.02).bfloat16().reshape(3, 256, 384)
+    q, s, qt, st = K.quantize_blockwise_weight_impl(w.to(gpu), fmt, rowwise=True, colwise=True)
+    for e in range(3):
+        wq, ws, wqt, wst = o.quantize_blockwise_2d(w[e], fmt)
+        assert np.array_equal(_u8(q[e]), wq) and np.array_equal(s[e].cpu().numpy(), ws)
+        assert np.array_equal(_u8(qt[e]), wqt) and np.array_equal(st[e].cpu().numpy(), wst)
+
+
+@pytest.mark.parametrize("a_fmt,b_fmt", [(0, 0), (2, 2)])
+@pytest.mark.parametrize("lens,k", GROUPS)
+def test_grouped_gemms_against_the_oracle(gpu, a_fmt, b_fmt, lens, k):
+    from primus_amd.pytorch import kernels as K
+
+    rows, G, n = sum(lens), len(lens), 256
+    x = _x(rows + k, rows, k)
+    w = (_x(n * G + k, G * n, k) * 0.05).bfloat16().reshape(G, n, k)
+    dy = _x(rows + n + 1, rows, n)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    dev = lambda arr, dt=None: (torch.from_numpy(arr).to(gpu) if dt is None else torch.from_numpy(arr).to(gpu).view(dt))
+    # forward shape: rows of a grouped, one weight per group
+    a, sa = o.quantize_blockwise(x, a_fmt)
+    bq = [o.quantize_blockwise_2d(w[e], b_fmt) for e in range(G)]
+    b, sb = np.stack([t[0] for t in bq]), np.stack([t[1] for t in bq])
+    want = o.grouped_blockwise_gemm_nt_ref(a, sa, b, sb, lens, a_fmt, b_fmt, out_bf16=False)
+    got = K.gemm_blockwise_nt_impl(dev(a, DT[a_fmt]), dev(sa), dev(b, DT[b_fmt]), dev(sb), gl)
+    assert tuple(got.shape) == (rows, n)
+    err = np.abs(_f(got).astype(np.float64) - want)
+    assert err.max() <= 1e-2 * max(np.abs(want).max(), 1e-30)
+    pos = 0
+    for e, ln in enumerate(lens):
+        if ln:
+            assert np.all(err[pos:pos + ln] <= _bound(a[pos:pos + ln], sa[pos:pos + ln], b[e], sb[e], a_fmt, b_fmt, want[pos:pos + ln]))
+        pos += ln
+    # wgrad shape: contraction over each group's token segment
+    at, sat = o.quantize_blockwise_segmented(dy, lens, a_fmt)
+    bt, sbt = o.quantize_blockwise_segmented(x, lens, b_fmt)
+    want_w = o.grouped_blockwise_wgrad_ref(at, sat, bt, sbt, lens, a_fmt, b_fmt, out_bf16=False)
+    got_w = K.grouped_gemm_blockwise_wgrad_impl(dev(at, DT[a_fmt]), dev(sat), dev(bt, DT[b_fmt]), dev(sbt), gl, rows)
+    assert tuple(got_w.shape) == (G, n, k)
+    gw = _f(got_w).reshape(G, n, k)
+    for e, ln in enumerate(lens):
+        if ln == 0:
+            assert not gw[e].any()
+        else:
+            assert np.abs(gw[e] - want_w[e]).max() <= 1e-2 * np.abs(want_w[e]).max()
+
+
+@pytest.mark.parametrize("hybrid", [False, True])
+def test_grouped_operator_follows_bf16(gpu, hybrid):
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import Float8QuantConfig, Format, ScalingGranularity
+
+    cfg = Float8QuantConfig(format=Format.HYBRID if hybrid else Format.E4M3, granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+    lens = [100, 0, 257, 27]
+    x = _x(1, sum(lens), 256).to(gpu).requires_grad_()
+    w = (_x(2, 4 * 384, 256) * 0.05).bfloat16().reshape(4, 384, 256).to(gpu).requires_grad_()
+    dy = _x(3, sum(lens), 384).to(gpu)
+    gl = torch.tensor(lens, device=gpu)
+    y = turbo.ops.grouped_gemm_fp8(x, w, gl, config=cfg)
+    dx, dw = torch.autograd.grad(y, [x, w], dy)
+    xr, wr = x.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+    yr = torch.cat([xs @ wr[e].t() for e, xs in enumerate(torch.split(xr, lens))])
+    dxr, dwr = torch.autograd.grad(yr, [xr, wr], dy)
+    bar = 0.99 if hybrid else 0.998
+    assert _cos(y, yr) > 0.998 and _cos(dx, dxr) > bar and _cos(dw, dwr) > bar
+    assert not dw[1].any()
+
+
+def test_megatron_grouped_linear_under_the_blockwise_recipe(gpu):
+    from types import SimpleNamespace
+
+    from primus_amd.megatron import runtime
+    from primus_amd.megatron.extensions import primus_turbo as pt
+    from primus_amd.pytorch.core import Format, ScalingGranularity
+
+    pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
+    runtime.bind()
+    runtime.set_args(enable_primus_turbo=True, use_turbo_gemm=True, use_turbo_grouped_gemm=True,
+                     turbo_grouped_gemm_without_padding=True)
+    runtime.set_num_microbatches(2)
+    try:
+        qc = pt.PrimusTurboQuantConfig(granularity=ScalingGranularity.BLOCKWISE, format=Format.E4M3, block_size=128)
+        torch.manual_seed(4)
+        cfg = SimpleNamespace(params_dtype=torch.bfloat16, use_cpu_initialization=False, perform_initialization=True,
+                              tensor_model_parallel_size=1, gradient_accumulation_fusion=False, normalization="RMSNorm",
+                              layernorm_epsilon=1e-5)
+        lens = [33, 0, 130, 1, 92]
+        gl = pt.PrimusTurboColumnParallelGroupedLinear(5, 128, 256, config=cfg)
+        xg = torch.randn(sum(lens), 128, device=gpu).bfloat16().requires_grad_()
+        dyg = torch.randn(sum(lens), 256, device=gpu).bfloat16()
+        with pt.primus_turbo_fp8_autocast(enabled=False, enabled_turbo=True, turbo_quant_config=qc):
+            yg, _ = gl(xg, torch.tensor(lens))
+        yg.backward(dyg)
+        want = torch.cat([xs @ gl.weights[e].detach().t() for e, xs in enumerate(torch.split(xg.detach(), lens))])
+        assert _cos(yg, want) > 0.998
+        assert not gl.weights.grad[1].any() and gl.weights.grad[0].abs().sum() > 0
     finally:
         pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
         runtime.set_args()

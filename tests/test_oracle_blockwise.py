@@ -113,3 +113,29 @@ def test_gemm_reference_against_float64(per_row):
     # and the dequantised operands are the input to FP8 precision, so the product is the bf16 product to ~2^-3 of |x||w|
     ref = x.double().numpy() @ w.double().numpy().T
     assert np.abs(got - ref).max() <= 0.08 * (np.abs(x.double().numpy()) @ np.abs(w.double().numpy()).T).max()
+
+
+def test_segmented_copy_is_the_groups_side_by_side():
+    lens = [5, 0, 130, 64]
+    x = _x(21, sum(lens), 256, 2.0)
+    codes, sinv = o.quantize_blockwise_segmented(x, lens, o.FMT_E4M3)
+    assert codes.shape == (256, o.padded_width(sum(lens), 4, 128)) and sinv.shape == (256, codes.shape[1] // 128)
+    pos = src = 0
+    for n in lens:
+        w = -(-n // 128) * 128
+        if n:
+            c, s = o.quantize_blockwise(x[src:src + n], o.FMT_E4M3, axis=0)
+            assert np.array_equal(codes[:, pos:pos + w], c) and np.array_equal(sinv[:, pos // 128:(pos + w) // 128], s)
+        pos += w
+        src += n
+    assert not codes[:, pos:].any()
+    # the wgrad reference over the segments equals per-group products of the dequantised pieces
+    dy = _x(22, sum(lens), 128)
+    at, sat = o.quantize_blockwise_segmented(dy, lens, o.FMT_E4M3)
+    got = o.grouped_blockwise_wgrad_ref(at, sat, codes, sinv, lens, out_bf16=False)
+    assert got.shape == (4, 128, 256) and not got[1].any()
+    da = o.decode_fp8(at, o.FMT_E4M3).astype(np.float64) * np.repeat(sat.astype(np.float64), 128, axis=1)
+    db = o.decode_fp8(codes, o.FMT_E4M3).astype(np.float64) * np.repeat(sinv.astype(np.float64), 128, axis=1)
+    seg3 = slice(128 + 256, 128 + 256 + 128)
+    ref = da[:, seg3] @ db[:, seg3].T
+    assert np.allclose(got[3], ref, rtol=1e-5, atol=1e-5 * np.abs(ref).max())

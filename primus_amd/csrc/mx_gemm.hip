@@ -603,11 +603,15 @@ constexpr int ring_lds_bytes() {
 
 template <int AFMT, int BFMT, int MODE, bool ALPHA>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
-    static_assert(AFMT != kFmtE2M1 && BFMT != kFmtE2M1, "FP8-family operands only");
+    static_assert(AFMT != kFmtE2M1, "the row operand is FP8");
+    static_assert(BFMT != kFmtE2M1 || (MODE == MODE_FWD && !ALPHA), "an E2M1 weight operand: forward / dgrad of the MX recipe");
+    constexpr bool B4 = BFMT == kFmtE2M1;             // the weight operand is FP4: 32 bytes per row and K step
+    constexpr int B_ROW = B4 ? BK / 2 : BK;           // bytes of a row of b in a K step
+    constexpr int ROUNDS = B4 ? 6 : 8;                // load rounds of 4 KiB per K step: 4 of a, 2 or 4 of b
     constexpr int A_BYTES = 256 * BK;                 // 16 KiB
     constexpr int STAGE = RING_STAGE;
     constexpr int PANEL = RING_PANEL;
-    constexpr int CB = BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE5M2 ? 1 : 0;
+    constexpr int CB = B4 ? 4 : BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE5M2 ? 1 : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* panels = smem + RING_SLOTS * STAGE;
     int* pre_tiles = (int*)(panels + RING_PANEL_BUFS * 2 * PANEL);
@@ -686,7 +690,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     const int64_t b_rows_total = (MODE == MODE_FWD) ? (int64_t)G * p.n : p.n;
     // K-step-major codes: [k / 64][rows][64]; scales: [ceil(k / 512)][rows][16] (16 bytes = 8 K steps of a row)
     const uint32_t a_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * BK));
-    const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * BK));
+    const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * B_ROW));
     const uint32_t a_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * 16));
     const uint32_t b_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * 16));
     // panels in a scale array: a contraction that is split into groups restarts its panels at every group
@@ -695,6 +699,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     // the piece index is applied on the global side so that the LDS image (64-byte rows) reads without bank conflicts
     const int ld_row = t >> 2;
     const uint32_t ld_voff = (uint32_t)(ld_row * BK + 16 * ((t & 3) ^ ((ld_row >> 2) & 3)));
+    // FP4 rows are 32 bytes: a round covers 128 rows, thread -> (row t / 2, piece t % 2), pieces swapped in every
+    // second group of 8 rows so that the 16-byte fragment reads of 16 consecutive rows cover all banks
+    const uint32_t ld_voff_b = B4 ? (uint32_t)((t >> 1) * B_ROW + 16 * ((t & 1) ^ ((t >> 4) & 1))) : ld_voff;
     const uint32_t s_voff = (uint32_t)(t * 16);     // scale panel: row t of the tile, 16 bytes
 
     struct Tile {
@@ -755,7 +762,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         d.nst = nreal < 4 ? 4 : nreal;
         // descriptors anchored at the tile's first row inside K step 0 / panel 0; readable up to the operand's end
         d.ra = make_rsrc(p.a + a_row0 * BK, a_rows_total * p.k - a_row0 * BK);
-        d.rb = make_rsrc(p.b + b_row0 * BK, b_rows_total * p.k - b_row0 * BK);
+        d.rb = make_rsrc(p.b + b_row0 * B_ROW, b_rows_total * (p.k / BK) * B_ROW - b_row0 * B_ROW);
         d.rsa = make_rsrc(p.sa + a_row0 * 16, a_rows_total * n_panels * 16 - a_row0 * 16);
         d.rsb = make_rsrc(p.sb + b_row0 * 16, b_rows_total * n_panels * 16 - b_row0 * 16);
         const uint32_t st0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(k0 / BK));
@@ -795,8 +802,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     // round e (0 .. 7) of the group in flight into ring slot `slot` (0 .. 3, run time)
     auto issue_e = [&](int e, uint32_t slot_base) __attribute__((always_inline)) {
         if (e < 4) dma16(lra, slot_base + (uint32_t)((e * 4 + w) * 1024), ld_voff, ga + (uint32_t)(e * 64 * BK));
-        else if (e >= 6) dma16(crb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff, cgb + (uint32_t)((e - 4) * 64 * BK));
-        else dma16(lrb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff, gb + (uint32_t)((e - 4) * 64 * BK));
+        else if (e >= 6) dma16(crb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff_b, cgb + (uint32_t)((e - 4) * 4096));
+        else dma16(lrb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff_b, gb + (uint32_t)((e - 4) * 4096));
     };
     // scale panel pn of tile d (its K steps 8 pn .. 8 pn + 7) into panel buffer `buf`: 4 KiB per operand
     auto issue_s = [&](const Tile& d, int pn, int buf) __attribute__((always_inline)) {
@@ -817,14 +824,21 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
          F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; \
          F.sa[I] = pan[a_sc + (I) * (32 * 16)]; } while (0)
 #define MXL_RD_B(F, J) \
-    do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * BK); \
-         const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
-         F.b[J][0] = lo_.x; F.b[J][1] = lo_.y; F.b[J][2] = lo_.z; F.b[J][3] = lo_.w; \
-         F.b[J][4] = hi_.x; F.b[J][5] = hi_.y; F.b[J][6] = hi_.z; F.b[J][7] = hi_.w; \
+    do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * B_ROW); \
+         if (B4) { \
+             const uint4 lo_ = *(const uint4*)(r_ + b4_lo); \
+             F.b[J][0] = lo_.x; F.b[J][1] = lo_.y; F.b[J][2] = lo_.z; F.b[J][3] = lo_.w; \
+             F.b[J][4] = 0; F.b[J][5] = 0; F.b[J][6] = 0; F.b[J][7] = 0; \
+         } else { \
+             const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
+             F.b[J][0] = lo_.x; F.b[J][1] = lo_.y; F.b[J][2] = lo_.z; F.b[J][3] = lo_.w; \
+             F.b[J][4] = hi_.x; F.b[J][5] = hi_.y; F.b[J][6] = hi_.z; F.b[J][7] = hi_.w; \
+         } \
          F.sb[J] = pan[PANEL + b_sc + (J) * (32 * 16)]; } while (0)
     // per-lane constants of the fragment reads: 64-byte rows, piece index XOR (row / 4) % 4
     const int sw = (lr >> 2) & 3;
-    const int a_frag = (wm * 128 + lr) * BK, b_frag = (wn * 128 + lr) * BK;
+    const int a_frag = (wm * 128 + lr) * BK, b_frag = (wn * 128 + lr) * B_ROW;
+    const int b4_lo = 16 * (g ^ ((lr >> 3) & 1));      // FP4: lane (row, g) holds elements 32 g .. 32 g + 31 of the K step
     const int a_lo = 16 * (g ^ sw), a_hi = 16 * ((2 + g) ^ sw);
     const int a_sc = (wm * 128 + lr) * 16 + g, b_sc = (wn * 128 + lr) * 16 + g;
 
@@ -876,9 +890,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     for (int s = 0; s < 4; ++s) {
         group_begin();
 #pragma unroll
-        for (int e = 0; e < (s < 3 ? 8 : 6); ++e) issue_e(e, smem_base + (uint32_t)(s * STAGE));
+        for (int e = 0; e < (s < 3 ? ROUNDS : 6); ++e) issue_e(e, smem_base + (uint32_t)(s * STAGE));
     }
-    wait_vm<22>();       // everything up to K step 0 has landed
+    wait_vm<2 * ROUNDS + 6>();       // everything up to K step 0 has landed
     __syncthreads();
 
     while (true) {
@@ -906,11 +920,11 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             constexpr bool LAST = decltype(last_tag)::value;
             const uint32_t slot_prev = smem_base + (uint32_t)(((gs + 3) & 3) * STAGE);   // group of step gs + 3
             const uint32_t slot_new = smem_base + (uint32_t)((gs & 3) * STAGE);          // group of step gs + 4
-            MXL_MFMA(cur, 0, 0); issue_e(6, slot_prev); MXL_PIN;
+            MXL_MFMA(cur, 0, 0); if (ROUNDS == 8) issue_e(6, slot_prev); MXL_PIN;
             MXL_MFMA(cur, 1, 0); MXL_PIN;
-            MXL_MFMA(cur, 2, 0); issue_e(7, slot_prev); MXL_PIN;
+            MXL_MFMA(cur, 2, 0); if (ROUNDS == 8) issue_e(7, slot_prev); MXL_PIN;
             MXL_MFMA(cur, 3, 0); MXL_PIN;
-            wait_vm<16>();       // the group of step gs + 1 has landed (two younger groups may be in flight)
+            wait_vm<2 * ROUNDS>();       // the group of step gs + 1 has landed (two younger groups may be in flight)
             __syncthreads();
             MXL_PIN;
             // bookkeeping between the barrier and the first read: panel of the next step, stream hand-over
@@ -966,7 +980,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             kstep(P1{}, No{}, Yes{}, 3, f1, f0);
         }
         // K step 0 of the next tile (and its scale panel) has landed; every wave is done reading the ring
-        wait_vm<16>();
+        wait_vm<2 * ROUNDS>();
         __syncthreads();
         MXL_PIN;
 
@@ -1102,18 +1116,23 @@ static int launch_gemm_ring(const GemmArgs& a, int64_t max_tiles, hipStream_t st
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
-// The 4-slot ring kernel serves FP8-family operands in the K-step-major layout with at most RING_MAX_GROUPS groups.
+// The 4-slot ring kernel serves operands in the K-step-major layout with at most RING_MAX_GROUPS groups: FP8 x FP8,
+// and FP8 rows against an FP4 weight operand in the forward / dgrad GEMM.
 template <int MODE>
 static bool ring_serves(int afmt, int bfmt, const GemmArgs& a) {
     if (a.num_groups > RING_MAX_GROUPS) return false;
     if (a.alpha_a != nullptr) return bfmt == MXL_FMT_E4M3 && (afmt == MXL_FMT_E4M3 || afmt == MXL_FMT_E5M2);
-    return afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3;
+    // MX: E4M3 x E4M3, and in the forward / dgrad GEMM E4M3 activations against E2M1 weights
+    return afmt == MXL_FMT_E4M3 && (bfmt == MXL_FMT_E4M3 || (bfmt == MXL_FMT_E2M1 && MODE == MODE_FWD));
 }
 template <int MODE>
-static int dispatch_gemm_ring(int afmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+static int dispatch_gemm_ring(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     if (a.alpha_a != nullptr) {
         if (afmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
         return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
+    }
+    if constexpr (MODE == MODE_FWD) {
+        if (bfmt == MXL_FMT_E2M1) return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E2M1, MODE_FWD, false>(a, max_tiles, st);
     }
     return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, false>(a, max_tiles, st);
 }
@@ -1163,7 +1182,7 @@ static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tile
         if (accum || !ring_serves<MODE>(afmt, bfmt, a)) return MXL_EINVAL;
         // offsets inside an operand are 32-bit
         if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
-        return dispatch_gemm_ring<MODE>(afmt, a, max_tiles, st);
+        return dispatch_gemm_ring<MODE>(afmt, bfmt, a, max_tiles, st);
     }
     if (accum) {
         if (MODE != MODE_WGRAD || !kchunk) return MXL_EINVAL;

@@ -347,7 +347,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                         (nonfinite2_e2m1(d[it].w) << 24);
                 }
                 if (out_ok && r < rows_valid) {
-                    const int64_t at = a.kchunk ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
+                    // element offsets; K-step-major: 64 elements (32 bytes) of a row per K step
+                    const int64_t at = a.kchunk == 2 ? ((int64_t)(2 * ct + (c16 >> 3)) * a.chunk_rows_row + src_row0 + r) * (QT / 2) + 8 * (c16 & 7)
+                                     : a.kchunk ? ((int64_t)ct * a.chunk_rows_row + src_row0 + r) * QT + 8 * c16
                                                 : (src_row0 + r) * a.row_ld + col;
                     store4_streaming(a.q_row + at / 2, o);
                 }
@@ -499,7 +501,9 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             const int ch = t % LPR;
             if (col0 + c < a.cols && 16 * ch < avail) {
                 const uint4 v = *(const uint4*)(t_tile + c * TPITCH + 16 * ch);
-                const int64_t at = (!FP4 && a.kchunk == 2)
+                const int64_t at = (FP4 && a.kchunk == 2)
+                                       ? ((2 * (m0 / QT) + (ch >> 1)) * a.chunk_rows_col + out_rows_base + col0 + c) * (QT / 4) + 16 * (ch & 1)
+                                   : a.kchunk == 2
                                        ? ((2 * (m0 / QT) + (ch >> 2)) * a.chunk_rows_col + out_rows_base + col0 + c) * (QT / 2) + 16 * (ch & 3)
                                    : a.kchunk ? ((m0 / QT) * a.chunk_rows_col + out_rows_base + col0 + c) * ROWB + 16 * ch
                                               : (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch;
@@ -688,7 +692,7 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
                        int kchunk = 0, const void* norm_w = nullptr, const void* tensor_amax = nullptr,
                        void* scale_inv_out = nullptr) {
     if (row_ld == 0) row_ld = cols;
-    if (kchunk < 0 || (kchunk == 2 && fmt == MXL_FMT_E2M1)) return MXL_EINVAL;   // both layout flags; K-step-major is FP8 only
+    if (kchunk < 0 || (kchunk == 2 && fmt == MXL_FMT_E2M1)) return MXL_EINVAL;   // both layout flags; activations: K-step-major is FP8 only
     if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
     if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
     if (rht && !q_colT) return MXL_EINVAL;   // the transform belongs to the transposed copy
@@ -781,7 +785,7 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
                               void* stream, const void* tensor_amax = nullptr, void* scale_inv_out = nullptr) {
     if (k_ld == 0) k_ld = k;
     if (n_ld == 0) n_ld = n;
-    if (kchunk < 0 || (kchunk == 2 && fmt == MXL_FMT_E2M1)) return MXL_EINVAL;
+    if (kchunk < 0) return MXL_EINVAL;
     if (kchunk && ((q_row && k_ld % QT != 0) || (q_colT && n_ld % QT != 0))) return MXL_EINVAL;   // whole chunks
     if (k_ld < k || n_ld < n || k_ld % MXL_BLOCK != 0 || n_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if (n_ld > (n + QT - 1) / QT * QT) return MXL_EINVAL;  // padding of the transposed copy stays inside the last tile

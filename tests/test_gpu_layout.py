@@ -82,12 +82,13 @@ def test_gemms_give_identical_results_on_either_layout(gpu, afmt, wfmt, lens, n,
     w = (torch.randn(G, n, k, generator=g) * 0.05).bfloat16().to(gpu)
     gl = None if lens is None else torch.tensor(lens, dtype=torch.int64, device=gpu)
     res = []
-    for kc in (False, True):
+    # 2: K-step-major codes and scales (the 4-slot ring kernel): FP8 activations against FP8 or FP4 weights
+    for kc in (False, True) + ((2,) if afmt == 0 else ()):
         xq = K.quantize_mx_impl(x, afmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kc)
         dq = K.quantize_mx_impl(dy, afmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kc)
         wq = K.quantize_mx_weight_2d_impl(w, wfmt, rowwise=True, colwise=True, pad_to=128, kchunk=kc)
         if lens is None:
-            ws_row, ws_col = wq[1][0], wq[3][0]
+            ws_row, ws_col = (wq[1], wq[3]) if kc == 2 else (wq[1][0], wq[3][0])
             w_row = wq[0] if kc else wq[0][0]
             w_col = wq[2] if kc else wq[2][0]
             y = K.gemm_mx_nt_impl(xq[0], xq[1], w_row, ws_row, kchunk=kc)
@@ -97,8 +98,9 @@ def test_gemms_give_identical_results_on_either_layout(gpu, afmt, wfmt, lens, n,
             dx = K.grouped_gemm_mx_nt_impl(dq[0], dq[1], wq[2], wq[3], gl, kchunk=kc)
         dw = K.grouped_gemm_mx_wgrad_impl(dq[2], dq[3], xq[2], xq[3], gl, m, kchunk=kc)
         res.append((y, dx[:, :k], dw))
-    for a, b in zip(*res):
-        assert a.shape == b.shape and torch.equal(a, b)
+    for other in res[1:]:
+        for a, b in zip(res[0], other):
+            assert a.shape == b.shape and torch.equal(a, b)
 
 
 def test_kchunk_argument_checks(gpu):

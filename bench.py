@@ -199,6 +199,66 @@ def cpu_baseline(spec, lens, sample_div=16):
     }
 
 
+def gemm_calibration(fp4_weights, dev):
+    """What this board's matrix cores deliver, measured in the same process, to read the GEMM figures against
+    (the published peak assumes the 2.4 GHz boost clock; under load the board sits at its power limit):
+    the library's register-only loop of the GEMM's own scaled MFMA (no memory traffic: the ceiling of any GEMM here),
+    and torch's vendor-library GEMMs on a dense problem of the benchmark's size (M 32768, N 28672, K 4096): FP8 with one
+    scale per tensor (no block scales) and, where torch supports it, MXFP8 with E8M0 block scales.  About 2 s."""
+    import torch
+
+    from primus_amd import _lib
+
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+
+    def rate(fn, flops, seconds=0.6):
+        fn()
+        torch.cuda.synchronize()
+        t_end = time.perf_counter() + 0.2
+        while time.perf_counter() < t_end:      # bring the board to its steady clocks first
+            fn()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n, t_end = 0, time.perf_counter() + seconds
+        e0.record()
+        while time.perf_counter() < t_end:
+            fn()
+            n += 1
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(n * flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+
+    iters = 4096
+    flops = float(lib.mxl_calibrate_mfma_flops(iters))
+    for name, (fa, fb) in (("fp8_x_fp8", (_lib.FMT_E4M3, _lib.FMT_E4M3)),) + ((("fp8_x_fp4", (_lib.FMT_E4M3, _lib.FMT_E2M1)),) if fp4_weights else ()):
+        def loop(fa=fa, fb=fb):
+            _lib.check(lib.mxl_calibrate_mfma(fa, fb, iters, st), "mxl_calibrate_mfma")
+        out["mfma_only_loop_%s_TFLOP/s" % name] = rate(loop, flops)
+    out["mfma_only_loop"] = "mxl_calibrate_mfma: 256 workgroups x 4 waves, 16 scaled MFMAs 32x32x64 per K step on register operands, no memory traffic"
+    try:
+        M, N, Kd = 32768, 28672, 4096
+        a8 = (torch.randn(M, Kd, device=dev) * 100).to(torch.float8_e4m3fn)
+        b8 = (torch.randn(N, Kd, device=dev) * 100).to(torch.float8_e4m3fn)
+        one = torch.ones((), device=dev)
+        out["vendor_gemm_shape_mnk"] = [M, N, Kd]
+        out["torch_scaled_mm_fp8_per_tensor_scale_TFLOP/s"] = rate(
+            lambda: torch._scaled_mm(a8, b8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 2.0 * M * N * Kd)
+        try:
+            sa = torch.full((M, Kd // 32), 127, dtype=torch.uint8, device=dev).view(torch.float8_e8m0fnu)
+            sb = torch.full((N, Kd // 32), 127, dtype=torch.uint8, device=dev).view(torch.float8_e8m0fnu)
+            out["torch_scaled_mm_mxfp8_block_scales_TFLOP/s"] = rate(
+                lambda: torch._scaled_mm(a8, b8.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16), 2.0 * M * N * Kd)
+        except Exception as ex:   # this torch build may not carry the MX path
+            out["torch_scaled_mm_mxfp8_block_scales_TFLOP/s"] = None
+            out["torch_scaled_mm_mxfp8_error"] = type(ex).__name__
+    except Exception as ex:
+        out["torch_scaled_mm_error"] = type(ex).__name__
+    return out
+
+
 def board_sample(run_step, seconds):
     """Socket power and shader clocks (``amd-smi metric --power --clock``) sampled while ``run_step`` loops for
     ``seconds``: says how far below the 2.4 GHz that the MFMA peak is quoted at the chip clocks under this load.
@@ -252,6 +312,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="mixtral_8x7b_moe_mxfp8", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm-calibration", action="store_true",
+                    help="skip the matrix-core calibration (register-only MFMA loop, torch's vendor GEMMs)")
     ap.add_argument("--no-wgrad-overlap", action="store_true",
                     help="keep wgrad on the launch stream behind dgrad (per-kernel durations are then undisturbed)")
     ap.add_argument("--board-seconds", type=float, default=2.0,
@@ -455,6 +517,12 @@ def main():
     for name in ("quantize", "quantize_weight_2d"):
         if name in kernels and "GB/s" in kernels[name]:
             kernels[name]["frac_of_stream_calibration"] = round(kernels[name]["GB/s"] / stream_gbs, 4)
+    if not args.no_gemm_calibration:
+        out["mfma_calibration"] = cal = gemm_calibration(spec["fp4"], dev)
+        ceiling = cal.get("mfma_only_loop_fp8_x_fp4_TFLOP/s" if spec["fp4"] else "mfma_only_loop_fp8_x_fp8_TFLOP/s")
+        for name, entry in kernels.items():
+            if "gemm" in name and "TFLOP/s" in entry and ceiling:
+                entry["frac_of_mfma_only_loop"] = round(entry["TFLOP/s"] / ceiling, 4)
     if args.board_seconds > 0:
         pt.ops.set_wgrad_overlap(not args.no_wgrad_overlap)
         out["board"] = board_sample(step, args.board_seconds)

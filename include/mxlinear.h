@@ -393,6 +393,15 @@ int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, in
                                      int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m,
                                      int64_t n, int64_t k, void* stream);
 
+/* ---- calibration (no counterpart in the reference: a measuring aid of this library's benchmark) ----
+ *
+ * mxl_calibrate_mfma launches a register-only loop of the GEMM kernels' scaled MFMA (32 x 32 x 64; a_fmt / b_fmt:
+ * MXL_FMT_E4M3 or MXL_FMT_E2M1) on 256 workgroups of 4 waves, `iters` K steps of 16 MFMAs per wave, with no memory
+ * traffic at all: its rate is what the matrix cores of the board sustain under its power limit, the ceiling for any
+ * GEMM on it.  mxl_calibrate_mfma_flops(iters) = the floating-point operations of one such launch. */
+int mxl_calibrate_mfma(int a_fmt, int b_fmt, int64_t iters, void* stream);
+int64_t mxl_calibrate_mfma_flops(int64_t iters);
+
 #ifdef __cplusplus
 }
 #endif

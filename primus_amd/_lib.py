@@ -68,6 +68,8 @@ EXPORTS = (
     "mxl_gemm_nt_blockwise",
     "mxl_grouped_gemm_nt_blockwise",
     "mxl_grouped_gemm_wgrad_blockwise",
+    "mxl_calibrate_mfma",
+    "mxl_calibrate_mfma_flops",
 )
 
 
@@ -165,6 +167,10 @@ def load() -> ctypes.CDLL:
         lib.mxl_grouped_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
         lib.mxl_grouped_gemm_wgrad_blockwise.restype = i32
         lib.mxl_grouped_gemm_wgrad_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        lib.mxl_calibrate_mfma.restype = i32
+        lib.mxl_calibrate_mfma.argtypes = [i32, i32, i64, vp]
+        lib.mxl_calibrate_mfma_flops.restype = i64
+        lib.mxl_calibrate_mfma_flops.argtypes = [i64]
         lib.mxl_gemm_nt_blockwise.restype = i32
         lib.mxl_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, i32, vp, i64, i64, i64, vp]
         _lib = lib

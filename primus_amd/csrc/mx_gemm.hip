@@ -821,8 +821,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     do { const uint8_t* r_ = sn + a_frag + (I) * (32 * BK); \
          const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
          F.a[I][0] = lo_.x; F.a[I][1] = lo_.y; F.a[I][2] = lo_.z; F.a[I][3] = lo_.w; \
-         F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; \
-         F.sa[I] = pan[a_sc + (I) * (32 * 16)]; } while (0)
+         F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; } while (0)
 #define MXL_RD_B(F, J) \
     do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * B_ROW); \
          if (B4) { \
@@ -833,14 +832,25 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
              const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
              F.b[J][0] = lo_.x; F.b[J][1] = lo_.y; F.b[J][2] = lo_.z; F.b[J][3] = lo_.w; \
              F.b[J][4] = hi_.x; F.b[J][5] = hi_.y; F.b[J][6] = hi_.z; F.b[J][7] = hi_.w; \
-         } \
-         F.sb[J] = pan[PANEL + b_sc + (J) * (32 * 16)]; } while (0)
+         } } while (0)
+    // the scale byte of step `psh / 8` of the panel, for fragment I of A / J of B (one shift each; they are spread
+    // over the second half of a step's MFMAs so that the panel reads have long landed)
+#define MXL_SC_A(F, I) do { F.sa[I] = (int)(uint32_t)(psa[I] >> psh); } while (0)
+#define MXL_SC_B(F, J) do { F.sb[J] = (int)(uint32_t)(psb[J] >> psh); } while (0)
     // per-lane constants of the fragment reads: 64-byte rows, piece index XOR (row / 4) % 4
     const int sw = (lr >> 2) & 3;
     const int a_frag = (wm * 128 + lr) * BK, b_frag = (wn * 128 + lr) * B_ROW;
     const int b4_lo = 16 * (g ^ ((lr >> 3) & 1));      // FP4: lane (row, g) holds elements 32 g .. 32 g + 31 of the K step
     const int a_lo = 16 * (g ^ sw), a_hi = 16 * ((2 + g) ^ sw);
-    const int a_sc = (wm * 128 + lr) * 16 + g, b_sc = (wn * 128 + lr) * 16 + g;
+    // Scale bytes: a panel row holds [g][K step] = 2 x 8 bytes, so the 8 bytes at (row, g) are the lane's scale
+    // bytes of the panel's 8 K steps.  They are read once per panel (8 reads of 8 bytes per wave, 512 consecutive
+    // bytes each) and the byte of a step is shifted down in registers: the MFMA takes byte 0 of its scale operand.
+    const int a_sc = (wm * 128 + lr) * 16 + 8 * g, b_sc = (wn * 128 + lr) * 16 + 8 * g;
+    uint64_t psa[4], psb[4];
+#define MXL_RD_PANEL(PAN) \
+    do { _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) { \
+             psa[i_] = *(const uint64_t*)((PAN) + a_sc + i_ * (32 * 16)); \
+             psb[i_] = *(const uint64_t*)((PAN) + PANEL + b_sc + i_ * (32 * 16)); } } while (0)
 
     // The workgroup's tiles: one per round of nwg tiles, at position vwg of the round -- in wgrad at position
     // nwg - 1 - vwg in odd rounds (the serpentine; an XCD's workgroups still hold a contiguous run of the order).
@@ -907,9 +917,12 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         const int nst = d.nst, nst_real = d.nst_real;
         {   // fragments of K step 0
             const uint8_t* sn = smem + (gs & 3) * STAGE;
-            const uint8_t* pan = panels + pb_rd * 2 * PANEL;
+            MXL_RD_PANEL(panels + pb_rd * 2 * PANEL);
+            const int psh = 0;
             MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
             MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
+            MXL_SC_B(f0, 0); MXL_SC_B(f0, 1); MXL_SC_B(f0, 2); MXL_SC_B(f0, 3);
+            MXL_SC_A(f0, 0); MXL_SC_A(f0, 1); MXL_SC_A(f0, 2); MXL_SC_A(f0, 3);
         }
         // One K step s (local number, parity PAR) of 16 MFMAs.  MF: multiply (false for the padding steps of a
         // tile whose contraction range is shorter than four steps).  LAST: the tile's last step; the six rounds
@@ -929,23 +942,26 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             MXL_PIN;
             // bookkeeping between the barrier and the first read: panel of the next step, stream hand-over
             const int s1 = s + 1;
-            pb_rd = ((s1 & 7) == 0 && s1 < nst) ? next3(pb_rd) : pb_rd;
+            if ((s1 & 7) == 0 && s1 < nst) {
+                pb_rd = next3(pb_rd);
+                MXL_RD_PANEL(panels + pb_rd * 2 * PANEL);
+            }
             if (!LAST) group_begin();
             const uint8_t* sn = smem + ((gs + 1) & 3) * STAGE;
-            const uint8_t* pan = panels + pb_rd * 2 * PANEL + 2 * (s1 & 7);
+            const int psh = 8 * (s1 & 7);
             MXL_PIN;
             MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(0, slot_new); MXL_PIN;
             MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1);  MXL_PIN;
             MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1);  if (!LAST) issue_e(1, slot_new); MXL_PIN;
             MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1);  MXL_PIN;
             MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2);  if (!LAST) issue_e(2, slot_new); MXL_PIN;
-            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2);  MXL_PIN;
-            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(3, slot_new); MXL_PIN;
-            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2);  MXL_PIN;
-            MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(4, slot_new); MXL_PIN;
-            MXL_MFMA(cur, 1, 3); MXL_PIN;
-            MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(5, slot_new); MXL_PIN;
-            MXL_MFMA(cur, 3, 3); MXL_PIN;
+            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2);  MXL_SC_B(nxt, 0); MXL_PIN;
+            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(3, slot_new); MXL_SC_A(nxt, 0); MXL_PIN;
+            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2);  MXL_SC_A(nxt, 1); MXL_PIN;
+            MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(4, slot_new); MXL_SC_A(nxt, 2); MXL_PIN;
+            MXL_MFMA(cur, 1, 3); MXL_SC_A(nxt, 3); MXL_SC_B(nxt, 1); MXL_PIN;
+            MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(5, slot_new); MXL_SC_B(nxt, 2); MXL_PIN;
+            MXL_MFMA(cur, 3, 3); MXL_SC_B(nxt, 3); MXL_PIN;
             ++gs;
         };
         using P0 = std::integral_constant<int, 0>;
@@ -1053,6 +1069,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
 #undef MXL_PIN
 #undef MXL_RD_A
 #undef MXL_RD_B
+#undef MXL_RD_PANEL
+#undef MXL_SC_A
+#undef MXL_SC_B
 }
 
 constexpr int gemm_lds_bytes(int afmt, int bfmt) {

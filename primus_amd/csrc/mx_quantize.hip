@@ -126,6 +126,15 @@ template <int FMT, int SMODE> __device__ __forceinline__ uint32_t block_byte(uin
     }
 }
 
+// K-step-major scales: a row's 16 bytes of a panel (512 elements = 8 MFMA K steps of two blocks) are ordered
+// [block parity][K step], so that the 8 bytes a GEMM lane needs for the panel's 8 steps are adjacent (the lanes
+// 0-31 of an MFMA supply the scales of the even blocks, the lanes 32-63 those of the odd ones).  `v` = the scale
+// bytes of the four blocks of 128-element tile `quarter` of the panel.
+__device__ __forceinline__ void store_panel_scales(uint8_t* row16, int quarter, uint32_t v) {
+    *(uint16_t*)(row16 + 2 * quarter) = (uint16_t)((v & 0xFFu) | ((v >> 8) & 0xFF00u));
+    *(uint16_t*)(row16 + 8 + 2 * quarter) = (uint16_t)(((v >> 8) & 0xFFu) | ((v >> 16) & 0xFF00u));
+}
+
 template <int FMT, int SMODE, bool ROW, bool COL, bool TWOD, int ACT = -1, bool SR = false, bool RHT = false>
 __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
     constexpr bool FP4 = (FMT == kFmtE2M1);
@@ -467,7 +476,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         uint8_t* dst = a.s_row + (src_row0 + t) * sld + col0 / 32;
         const uint32_t v = srow_tile[t];
         if (a.kchunk == 2) {
-            *(uint32_t*)(a.s_row + ((int64_t)(ct >> 2) * a.chunk_rows_row + src_row0 + t) * 16 + (ct & 3) * 4) = v;
+            store_panel_scales(a.s_row + ((int64_t)(ct >> 2) * a.chunk_rows_row + src_row0 + t) * 16, ct & 3, v);
         } else if (nb >= 4 && (sld & 3) == 0) {
             *(uint32_t*)dst = v;
         } else {
@@ -483,7 +492,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             const int64_t nb = (a.W - m0) / 32;
             if (a.kchunk == 2) {
                 const int64_t mt = seg_tile >= 0 ? (int64_t)seg_tile : m0 / QT;
-                *(uint32_t*)(a.s_colT + ((seg_pan0 + mt / 4) * a.chunk_rows_col + out_rows_base + col0 + t) * 16 + (mt & 3) * 4) = v;
+                store_panel_scales(a.s_colT + ((seg_pan0 + mt / 4) * a.chunk_rows_col + out_rows_base + col0 + t) * 16, (int)(mt & 3), v);
             } else if (nb >= 4 && ((a.W / 32) & 3) == 0) {
                 *(uint32_t*)dst = v;
             } else {

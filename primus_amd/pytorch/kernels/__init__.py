@@ -191,7 +191,10 @@ def unpanel(scales: torch.Tensor, blocks: int) -> torch.Tensor:
     ``[rows, blocks]`` (a copy)."""
     if scales.dim() != 3 or scales.shape[2] != 16:
         raise ValueError("expected 3-D K-step-major scales [panels, rows, 16]")
-    return scales.permute(1, 0, 2).reshape(scales.shape[1], scales.shape[0] * 16)[:, :blocks].contiguous()
+    panels, rows = scales.shape[0], scales.shape[1]
+    # a panel row is [block parity][K step]: block 2 s + g of the panel sits at byte 8 g + s
+    by_block = scales.reshape(panels, rows, 2, 8).permute(1, 0, 3, 2)
+    return by_block.reshape(rows, panels * 16)[:, :blocks].contiguous()
 
 
 def _ptr(t: Optional[torch.Tensor]):

@@ -43,6 +43,12 @@ def test_host_only_entry_points(lib):
         assert lib.mxl_error_string(code).decode()
     for rows, groups in [(0, 0), (1, 1), (128, 1), (129, 1), (32768, 8), (65536, 128), (5, 0)]:
         assert _lib.padded_width(rows, groups) == o.padded_width(rows, groups)
+    # the calibration loop: 256 workgroups x 4 waves x iters x 16 MFMAs of 2 * 32 * 32 * 64 flops
+    assert lib.mxl_calibrate_mfma_flops(1) == 256 * 4 * 16 * 2 * 32 * 32 * 64
+    assert lib.mxl_calibrate_mfma_flops(4096) == 4096 * lib.mxl_calibrate_mfma_flops(1)
+    assert lib.mxl_calibrate_mfma_flops(-1) == -1
+    assert lib.mxl_calibrate_mfma(_lib.FMT_E4M3, _lib.FMT_E4M3, 0, None) == -1      # no iterations
+    assert lib.mxl_calibrate_mfma(7, _lib.FMT_E4M3, 16, None) == -1                 # unknown format
 
 
 def test_constants_match_the_header():

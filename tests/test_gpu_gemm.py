@@ -400,3 +400,15 @@ def test_fp4_fp4_repeated_launches_are_identical(gpu, mode):
     for _ in range(400):
         bad += int(not torch.equal(launch().view(torch.int16), want_t))
     assert bad == 0, f"{bad} of 400 launches differ from the oracle"
+
+
+def test_calibration_loop_runs_for_every_operand_mix():
+    """The register-only MFMA loop of the benchmark's calibration launches and finishes for the four operand mixes."""
+    from primus_amd import _lib
+
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    for fa in (_lib.FMT_E4M3, _lib.FMT_E2M1):
+        for fb in (_lib.FMT_E4M3, _lib.FMT_E2M1):
+            assert lib.mxl_calibrate_mfma(fa, fb, 8, st) == 0
+    torch.cuda.synchronize()

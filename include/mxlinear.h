@@ -393,6 +393,21 @@ int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, in
                                      int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m,
                                      int64_t n, int64_t k, void* stream);
 
+/* ---- pre-shuffled MXFP4 layouts ----
+ *
+ * The byte orders behind the shuffle_rowwise / shuffle_colwise (codes) and shuffle_*_scale flags of the reference's
+ * quantize_mxfp4_dual (primus_turbo_mxfp4_local.py:147-161; output shapes :184-198) and behind
+ * gemm_fp4_impl(..., preshuffled=True) (:319-331), which the reference describes as the AITER pre-shuffle path.
+ * mxl_shuffle_codes:  packed FP4 codes [rows, row_bytes], rows % 16 == 0, row_bytes % 32 == 0, same shape out: every
+ *   block of 16 rows x 32 bytes becomes 512 consecutive bytes ([16-byte half][row][byte]), blocks in row-major order.
+ * mxl_shuffle_scales: E8M0 bytes [rows, cols] -> [ceil(rows / 256) * 256, ceil(cols / 8) * 8] with zero bytes in the
+ *   padding: every 32 rows x 8 columns become 256 consecutive bytes ([col % 4][row % 16][(col / 4) % 2][(row / 16) % 2]).
+ * inverse != 0 converts back (src is the shuffled array, dst [rows, row_bytes] / [rows, cols]).  src and dst must not
+ * overlap; code arrays must be 16-byte aligned.  The GEMM entry points read the plain layouts: a caller holding
+ * pre-shuffled operands converts them back first (the Python boundary does). */
+int mxl_shuffle_codes(const void* src, int64_t rows, int64_t row_bytes, void* dst, int inverse, void* stream);
+int mxl_shuffle_scales(const void* src, int64_t rows, int64_t cols, void* dst, int inverse, void* stream);
+
 /* ---- calibration (no counterpart in the reference: a measuring aid of this library's benchmark) ----
  *
  * mxl_calibrate_mfma launches a register-only loop of the GEMM kernels' scaled MFMA (32 x 32 x 64; a_fmt / b_fmt:

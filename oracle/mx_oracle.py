@@ -109,6 +109,19 @@ Parity status
   The Primus-Turbo ops behind ``quant_fp8_blockwise_impl`` are absent: whether they use this formula or another
   (e.g. amax / fp8_max without the clamp at 1e-12) is **parity unpinned**.
 
+* ``shuffle_codes_16x16`` / ``shuffle_e8m0`` and their inverses (the "pre-shuffled" MXFP4 layouts, the
+  ``shuffle_*`` flags of ``quantize_mxfp4_dual`` and ``gemm_fp4_impl(preshuffled=True)``,
+  primus_turbo_mxfp4_local.py:147-161, :184-198, :319-331; the reference calls it the AITER preshuffle fast
+  path, :39-99): pure byte permutations.  The permutation itself lives in the third-party AITER package
+  (ROCm/aiter; no version is pinned in the reference tree: it comes in through Primus-Turbo), which is absent:
+  restated here from its published ``shuffle_weight(x, layout=(16, 16))`` (16 rows x 32 bytes blocks, stored as
+  two halves of 16 rows x 16 bytes) and ``e8m0_shuffle`` (scales padded to 256 x 8, then
+  ``view(m/32, 2, 16, n/8, 2, 4).permute(0, 3, 5, 2, 4, 1)``).  Written below as explicit index arithmetic;
+  pinned in tests/ against the view / permute formulation evaluated by torch (a library routine doing the
+  permutation another way), by inverse(shuffle(x)) == x and by the scale shapes the reference's own shape
+  function states for the shuffled outputs (:184-187, :192-195: rows to 256, blocks to 8).  Whether Primus-Turbo's
+  C++ op writes exactly these byte orders is **parity unpinned**.
+
 All scale arithmetic is integer arithmetic on fp32 bit patterns (no log2), so
 results are reproducible bit-for-bit on any host.
 """
@@ -992,3 +1005,62 @@ def grouped_blockwise_wgrad_ref(a_codes, a_sinv, b_codes, b_sinv, group_lens, a_
             outs.append(np.zeros((a_codes.shape[0], b_codes.shape[0]), np.uint16 if out_bf16 else np.float32))
         pos += w
     return np.stack(outs)
+
+
+# --------------------------------------------------------------------------
+# pre-shuffled MXFP4 layouts (byte permutations; see the header)
+# --------------------------------------------------------------------------
+def _shuffle_codes_index(rows: int, row_bytes: int) -> np.ndarray:
+    """dst flat byte offset of source byte (r, b): blocks of 16 rows x 32 bytes, each stored as
+    [half of 16 bytes][row in block][byte]."""
+    if rows % 16 or row_bytes % 32:
+        raise ValueError("the shuffled code layout needs rows % 16 == 0 and row bytes % 32 == 0")
+    r = np.arange(rows, dtype=np.int64)[:, None]
+    b = np.arange(row_bytes, dtype=np.int64)[None, :]
+    block = (r // 16) * (row_bytes // 32) + b // 32
+    return block * 512 + ((b % 32) // 16) * 256 + (r % 16) * 16 + b % 16
+
+
+def shuffle_codes_16x16(codes: np.ndarray) -> np.ndarray:
+    """``codes`` uint8 [rows, row_bytes] (packed FP4: two elements a byte) -> the same shape, shuffled."""
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    idx = _shuffle_codes_index(*codes.shape)
+    out = np.empty(codes.size, dtype=np.uint8)
+    out[idx.ravel()] = codes.ravel()
+    return out.reshape(codes.shape)
+
+
+def unshuffle_codes_16x16(shuffled: np.ndarray) -> np.ndarray:
+    shuffled = np.ascontiguousarray(shuffled, dtype=np.uint8)
+    idx = _shuffle_codes_index(*shuffled.shape)
+    return shuffled.ravel()[idx.ravel()].reshape(shuffled.shape)
+
+
+def shuffled_scale_shape(rows: int, blocks: int):
+    return (rows + 255) // 256 * 256, (blocks + 7) // 8 * 8
+
+
+def _shuffle_scale_index(rows: int, blocks: int, ld: int) -> np.ndarray:
+    """dst flat offset of scale (m, n) in the padded [.., ld] array: 32 rows x 8 blocks form one 256-byte group
+    stored as [block % 4][row % 16][(block / 4) % 2][(row / 16) % 2]."""
+    m = np.arange(rows, dtype=np.int64)[:, None]
+    n = np.arange(blocks, dtype=np.int64)[None, :]
+    group = (m // 32) * (ld // 8) + n // 8
+    return group * 256 + (n % 4) * 64 + (m % 16) * 4 + ((n // 4) % 2) * 2 + (m // 16) % 2
+
+
+def shuffle_e8m0(scales: np.ndarray) -> np.ndarray:
+    """``scales`` uint8 [rows, blocks] -> [ceil(rows / 256) * 256, ceil(blocks / 8) * 8], zero bytes in the padding."""
+    scales = np.ascontiguousarray(scales, dtype=np.uint8)
+    rows, blocks = scales.shape
+    pr, pb = shuffled_scale_shape(rows, blocks)
+    out = np.zeros(pr * pb, dtype=np.uint8)
+    out[_shuffle_scale_index(rows, blocks, pb).ravel()] = scales.ravel()
+    return out.reshape(pr, pb)
+
+
+def unshuffle_e8m0(shuffled: np.ndarray, rows: int, blocks: int) -> np.ndarray:
+    shuffled = np.ascontiguousarray(shuffled, dtype=np.uint8)
+    if tuple(shuffled.shape) != shuffled_scale_shape(rows, blocks):
+        raise ValueError("shuffled scales have the wrong shape")
+    return shuffled.ravel()[_shuffle_scale_index(rows, blocks, shuffled.shape[1]).ravel()].reshape(rows, blocks)

@@ -68,6 +68,8 @@ EXPORTS = (
     "mxl_gemm_nt_blockwise",
     "mxl_grouped_gemm_nt_blockwise",
     "mxl_grouped_gemm_wgrad_blockwise",
+    "mxl_shuffle_codes",
+    "mxl_shuffle_scales",
     "mxl_calibrate_mfma",
     "mxl_calibrate_mfma_flops",
 )
@@ -167,6 +169,10 @@ def load() -> ctypes.CDLL:
         lib.mxl_grouped_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
         lib.mxl_grouped_gemm_wgrad_blockwise.restype = i32
         lib.mxl_grouped_gemm_wgrad_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        lib.mxl_shuffle_codes.restype = i32
+        lib.mxl_shuffle_codes.argtypes = [vp, i64, i64, vp, i32, vp]
+        lib.mxl_shuffle_scales.restype = i32
+        lib.mxl_shuffle_scales.argtypes = [vp, i64, i64, vp, i32, vp]
         lib.mxl_calibrate_mfma.restype = i32
         lib.mxl_calibrate_mfma.argtypes = [i32, i32, i64, vp]
         lib.mxl_calibrate_mfma_flops.restype = i64

@@ -1165,14 +1165,17 @@ static int dispatch_gemm_l(int afmt, int bfmt, const GemmArgs& a, int64_t max_ti
     return MXL_EINVAL;
 }
 
-// tensor-wise scaled operands: E4M3 x E4M3 (forward, or every GEMM of the E4M3 format) and E5M2 x E4M3
-// (gradient times weight / activation of the HYBRID format), output times *alpha_a * *alpha_b
+// tensor-wise scaled operands: E4M3 x E4M3 (forward, or every GEMM of the E4M3 format), E5M2 x E4M3 (gradient
+// times weight / activation of the HYBRID format) and E5M2 x E5M2 (the FP8 backward of the MXFP4 linear, which
+// re-quantises all three tensors to the gradient format); output times *alpha_a * *alpha_b
 template <int MODE, int LAYOUT>
 static int dispatch_gemm_alpha_l(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3)
         return launch_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, LAYOUT, true>(a, max_tiles, st);
     if (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E4M3)
         return launch_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE, LAYOUT, true>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E5M2)
+        return launch_gemm<MXL_FMT_E5M2, MXL_FMT_E5M2, MODE, LAYOUT, true>(a, max_tiles, st);
     return MXL_EINVAL;
 }
 

@@ -69,13 +69,14 @@ class MXScalingRecipe:
     """Per-operand options of MX quantisation (primus_turbo.py:305-319)."""
 
     use_2d_block: bool = False  # one scale per 32x32 tile (weights)
-    shuffle_scale: bool = False  # pre-shuffled scale layout (not implemented)
-    shuffle_out: bool = False  # pre-shuffled data layout (not implemented)
+    # Pre-shuffled scale / data layouts (primus_turbo.py:305-311).  In the reference they ask the quantiser for the
+    # byte order its FP4 GEMM back end wants.  Here the storage of a QuantizedTensor is private to the library (its
+    # GEMMs read the K-chunk-major layout the quantisers write directly), so the flags are accepted and change
+    # nothing an operator computes; the pre-shuffled byte orders themselves are available through
+    # ``QuantizedTensor.preshuffled_codes()`` / ``preshuffled_scales()`` and the flags of ``quantize_mxfp4_dual``.
+    shuffle_scale: bool = False
+    shuffle_out: bool = False
     scale_mode: ScaleMode = ScaleMode.OCP_FLOOR
-
-    def __post_init__(self):
-        if self.shuffle_scale or self.shuffle_out:
-            raise NotImplementedError("pre-shuffled MX layouts are not implemented")
 
 
 # older name of the same class (primus_turbo.py:57-62)
@@ -109,6 +110,8 @@ class Float4QuantConfig:
     scale_dtype: ScaleDtype = ScaleDtype.E8M0
     block_size: Optional[int] = MX_BLOCK_SIZE
     use_gradient_sr: bool = False  # stochastic rounding of E2M1 gradients
+    # Accepted for the reference's configs (primus_turbo.py:304-311): the operators already keep FP4 weights in the
+    # layout their GEMM reads fastest, so the switch changes no result here (see MXScalingRecipe).
     use_preshuffle: bool = False
     scale_mode: ScaleMode = ScaleMode.OCP_FLOOR
     # Element format of activations and gradients.  E2M1_X2 is plain MXFP4;
@@ -129,8 +132,6 @@ class Float4QuantConfig:
             raise ValueError(f"MX block size must be {MX_BLOCK_SIZE}, got {self.block_size}")
         if self.activation_format not in (Format.E2M1_X2, Format.E4M3):
             raise ValueError("activation_format must be E2M1_X2 or E4M3")
-        if self.use_preshuffle:
-            raise NotImplementedError("pre-shuffled FP4 layouts are not implemented")
 
 
 def _gfx950_reason() -> Tuple[bool, str]:

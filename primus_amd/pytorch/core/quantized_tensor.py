@@ -120,6 +120,19 @@ class QuantizedTensor(torch.Tensor):
         flat = K.unpanel(self._scales.view(torch.uint8), blocks).view(self._scales.dtype)
         return flat.view(tuple(self.shape[:-1]) + (blocks,))
 
+    def preshuffled_codes(self) -> torch.Tensor:
+        """The payload of a 2-D MXFP4 tensor in the pre-shuffled byte order of the reference's FP4 GEMM back end
+        (``shuffle_out`` of the scaling recipe, primus_turbo.py:305-311): a copy."""
+        if self.fmt != _lib.FMT_E2M1 or self.dim() != 2:
+            raise ValueError("the pre-shuffled layout is defined for 2-D MXFP4 tensors")
+        return K.shuffle_codes_impl(self.rowmajor_codes())
+
+    def preshuffled_scales(self) -> torch.Tensor:
+        """The scales of a 2-D tensor in the pre-shuffled order (``shuffle_scale``), padded to 256 rows x 8 blocks."""
+        if self.dim() != 2 or self._tensor_scale_inv is not None:
+            raise ValueError("the pre-shuffled scale layout is defined for 2-D MX tensors")
+        return K.shuffle_scales_impl(self.rowmajor_scales())
+
     @property
     def fmt(self) -> int:
         return dtype_to_fmt_code(self._codes.dtype)

@@ -1162,10 +1162,68 @@ def gemm_fp8_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, t
     return gemm_mx_nt_impl(a, a_scale_inv, b, b_scale_inv, out_dtype)
 
 
+# --------------------------------------------------------------------------
+# pre-shuffled MXFP4 layouts (the shuffle_* flags of quantize_mxfp4_dual,
+# primus_turbo_mxfp4_local.py:147-161, :184-198)
+# --------------------------------------------------------------------------
+def shuffled_scale_shape(rows: int, blocks: int) -> Tuple[int, int]:
+    """Shape of a pre-shuffled scale array: rows to 256, blocks to 8 (primus_turbo_mxfp4_local.py:184-187)."""
+    return _round_up(rows, 256), _round_up(blocks, 8)
+
+
+def shuffle_codes_impl(codes: torch.Tensor, inverse: bool = False) -> torch.Tensor:
+    """Packed FP4 codes ``[rows, row_bytes]`` in the pre-shuffled byte order (16 x 32-byte blocks made contiguous), or
+    back with ``inverse=True``.  Same shape and dtype; rows must be a multiple of 16, row bytes of 32."""
+    _require_cuda(codes)
+    if codes.dim() != 2:
+        raise ValueError("expected 2-D codes [rows, row_bytes]")
+    u8 = _codes_u8(codes)
+    rows, rb = u8.shape
+    if rows % 16 or rb % 32:
+        raise ValueError(f"the pre-shuffled code layout needs rows % 16 == 0 and row bytes % 32 == 0 (got {rows} x {rb})")
+    out = torch.empty_like(u8)
+    rc = _lib.load().mxl_shuffle_codes(_ptr(u8), rows, rb, _ptr(out), int(bool(inverse)), _stream())
+    _lib.check(rc, "mxl_shuffle_codes")
+    return out.view(codes.dtype)
+
+
+def shuffle_scales_impl(scales: torch.Tensor) -> torch.Tensor:
+    """E8M0 scales ``[rows, blocks]`` -> pre-shuffled ``[ceil(rows/256)*256, ceil(blocks/8)*8]`` (zero bytes in the
+    padding)."""
+    _require_cuda(scales)
+    if scales.dim() != 2:
+        raise ValueError("expected 2-D scales [rows, blocks]")
+    u8 = scales.view(torch.uint8)
+    rows, blocks = u8.shape
+    out = torch.empty(shuffled_scale_shape(rows, blocks), dtype=torch.uint8, device=scales.device)
+    rc = _lib.load().mxl_shuffle_scales(_ptr(u8), rows, blocks, _ptr(out), 0, _stream())
+    _lib.check(rc, "mxl_shuffle_scales")
+    return out.view(scales.dtype)
+
+
+def unshuffle_scales_impl(shuffled: torch.Tensor, rows: int, blocks: int) -> torch.Tensor:
+    """The inverse of ``shuffle_scales_impl`` for an operand of ``rows`` rows and ``blocks`` blocks a row."""
+    _require_cuda(shuffled)
+    if tuple(shuffled.shape) != shuffled_scale_shape(rows, blocks):
+        raise ValueError(f"pre-shuffled scales of a [{rows}, {blocks}] operand must be {shuffled_scale_shape(rows, blocks)}")
+    u8 = shuffled.view(torch.uint8)
+    out = torch.empty((rows, blocks), dtype=torch.uint8, device=shuffled.device)
+    rc = _lib.load().mxl_shuffle_scales(_ptr(u8), rows, blocks, _ptr(out), 1, _stream())
+    _lib.check(rc, "mxl_shuffle_scales")
+    return out.view(shuffled.dtype)
+
+
 def gemm_fp4_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity=None, default_backend=None, preshuffled=False):
-    """gemm_fp4_impl of the reference (primus_turbo_mxfp4_local.py:319-331)."""
+    """gemm_fp4_impl of the reference (primus_turbo_mxfp4_local.py:319-331).  ``preshuffled``: the operands are
+    what the reference's MXFP4 linear hands over with its pre-shuffle switch on (:234-288): ``a`` plain codes with
+    pre-shuffled scales, ``b`` pre-shuffled codes and scales.  The GEMM kernels read the plain layouts, so the three
+    arrays are converted back first (byte permutations, one pass over half a byte per element)."""
     if preshuffled:
-        raise NotImplementedError("pre-shuffled FP4 layouts are not implemented")
+        _require_mx(granularity)
+        k_blocks = a.shape[-1] * _per_byte(fmt_of(a)) // BLOCK
+        a_scale_inv = unshuffle_scales_impl(a_scale_inv, a.shape[0], k_blocks)
+        b_scale_inv = unshuffle_scales_impl(b_scale_inv, b.shape[0], b.shape[-1] * _per_byte(fmt_of(b)) // BLOCK)
+        b = shuffle_codes_impl(b, inverse=True)
     return gemm_fp8_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity, default_backend)
 
 

@@ -306,8 +306,19 @@ def test_mxfp4_dual_quantize_op_matches_oracle_bytes(mg, gpu):
     assert np.array_equal(wcs.view(torch.uint8).cpu().numpy()[:, :2], st)
     with pytest.raises(NotImplementedError, match="rowwise_use_rht"):
         m4._quantize_mxfp4_dual_op(x, m4._FP4_DTYPE, 128, False, False, True, False, False, True, False, False, False, False)
-    with pytest.raises(NotImplementedError, match="shuffle_rowwise_scale"):
-        m4._quantize_grad_dual(x, preshuffle=True)
+    # the pre-shuffled copies are byte permutations of the plain ones, in the shapes the reference's shape function states
+    g_plain = m4._quantize_grad_dual(x, use_rht=False)
+    g_pre = m4._quantize_grad_dual(x, preshuffle=True, use_rht=False)       # gradients: scales shuffled, codes not
+    assert torch.equal(g_pre[0].view(torch.uint8), g_plain[0].view(torch.uint8))
+    assert torch.equal(g_pre[2].view(torch.uint8), g_plain[2].view(torch.uint8))
+    assert tuple(g_pre[1].shape) == (256, 8) and tuple(g_pre[3].shape) == (256, 8)
+    assert np.array_equal(g_pre[1].view(torch.uint8).cpu().numpy(), o.shuffle_e8m0(g_plain[1].view(torch.uint8).cpu().numpy()))
+    assert np.array_equal(g_pre[3].view(torch.uint8).cpu().numpy(), o.shuffle_e8m0(g_plain[3].view(torch.uint8).cpu().numpy()))
+    w_pre = m4._quantize_weight_dual(w, preshuffle=True)                    # weights: everything shuffled
+    for got, plain in ((w_pre[0], wr), (w_pre[2], wc)):
+        assert np.array_equal(got.view(torch.uint8).cpu().numpy(), o.shuffle_codes_16x16(plain.view(torch.uint8).cpu().numpy()))
+    for got, plain in ((w_pre[1], wrs), (w_pre[3], wcs)):
+        assert np.array_equal(got.view(torch.uint8).cpu().numpy(), o.shuffle_e8m0(plain.view(torch.uint8).cpu().numpy()))
     # stochastic rounding keeps shapes and scales (the codes are checked in test_gpu_fp4_options.py)
     sr = m4._quantize_grad_dual(x, use_sr=True)
     assert torch.equal(sr[1].view(torch.uint8), row_s.view(torch.uint8)) and sr[0].shape == row.shape
@@ -321,7 +332,7 @@ def test_mxfp4_linear_function_snr_against_bf16(mg, gpu):
     x = torch.randn(128, 256, device=gpu).bfloat16().requires_grad_()
     w = (torch.randn(512, 256, device=gpu) * 0.05).bfloat16().requires_grad_()
     dy = torch.randn(128, 512, device=gpu).bfloat16()
-    y = MXFP4LinearFunction.apply(x, w)
+    y = MXFP4LinearFunction.apply(x, w, False, False, None, 0, 0, False)[0]
     y.backward(dy)
     xr, wr = x.detach().float().requires_grad_(), w.detach().float().requires_grad_()
     yr = xr @ wr.T
@@ -331,6 +342,56 @@ def test_mxfp4_linear_function_snr_against_bf16(mg, gpu):
         assert _snr_db(a.detach(), b.detach()) > 10.0, (name, _snr_db(a.detach(), b.detach()))
     # and the forward equals the oracle's MXFP4 linear
     _close(y, o.linear_fwd_ref(x.detach().cpu(), w.detach().cpu(), o.FMT_E2M1, o.FMT_E2M1), 3e-2)
+
+
+def test_mxfp4_linear_function_preshuffled_is_bit_identical(mg, gpu):
+    """With the pre-shuffle switch on, the bytes between the quantiser and the GEMM travel in the shuffled order and
+    every result is the same bit for bit."""
+    from primus_amd.megatron.extensions.primus_turbo_mxfp4_local import MXFP4LinearFunction, mxfp4_linear
+
+    torch.manual_seed(11)
+    res = []
+    for pre in (False, True):
+        x = torch.randn(3, 100, 256, device=gpu).bfloat16().requires_grad_()
+        w = (torch.randn(192, 256, device=gpu) * 0.05).bfloat16().requires_grad_()
+        if res:
+            x.data.copy_(res[0][3]), w.data.copy_(res[0][4])
+        out = MXFP4LinearFunction.apply(x, w, pre, False, None, 0, 0, False)
+        assert len(out) == 5 and all(t.dtype == torch.uint8 for t in out[1:])
+        assert tuple(out[2].shape) == ((256, 16) if pre else (256, 12))          # X^T scales: 256 features x 384/32 blocks
+        dy = torch.ones_like(out[0]) * 0.5 + out[0].detach() * 0.01
+        out[0].backward(dy)
+        res.append((out[0].detach(), x.grad, w.grad, x.detach().clone(), w.detach().clone()))
+    for a, b in zip(res[0][:3], res[1][:3]):
+        assert torch.equal(a, b)
+    assert torch.equal(mxfp4_linear(res[0][3], res[0][4], preshuffle=True), res[0][0])
+
+
+def test_mxfp4_linear_function_fp8_backward(mg, gpu):
+    """The hybrid mode: MXFP4 forward, backward on the saved bf16 tensors re-quantised to E5M2 with one scale per
+    tensor; checked against the oracle's tensor-wise quantiser and GEMM."""
+    from primus_amd.megatron.extensions.primus_turbo_mxfp4_local import MXFP4LinearFunction
+    from primus_amd.pytorch.core.low_precision import ScalingGranularity, float8_e5m2
+
+    torch.manual_seed(12)
+    x = torch.randn(128, 256, device=gpu).bfloat16().requires_grad_()
+    w = (torch.randn(192, 256, device=gpu) * 0.05).bfloat16().requires_grad_()
+    dy = torch.randn(128, 192, device=gpu).bfloat16()
+    out = MXFP4LinearFunction.apply(x, w, False, True, float8_e5m2, ScalingGranularity.TENSORWISE.value, 0, False)
+    assert len(out) == 3
+    y = out[0]
+    y.backward(dy)
+    plain = MXFP4LinearFunction.apply(x.detach(), w.detach(), False, False, None, 0, 0, False)[0]
+    assert torch.equal(y.detach(), plain)                                           # the forward is the same
+    qd, sd = o.quantize_tensorwise(dy.cpu(), o.FMT_E5M2)
+    qx, sx = o.quantize_tensorwise(x.detach().cpu(), o.FMT_E5M2)
+    qw, sw = o.quantize_tensorwise(w.detach().cpu(), o.FMT_E5M2)
+    want_dx = o.tensorwise_gemm_nt_ref(qd, sd, np.ascontiguousarray(qw.T), sw, o.FMT_E5M2, o.FMT_E5M2)
+    want_dw = o.tensorwise_gemm_nt_ref(np.ascontiguousarray(qd.T), sd, np.ascontiguousarray(qx.T), sx, o.FMT_E5M2, o.FMT_E5M2)
+    _close(x.grad, want_dx, 1e-2)
+    _close(w.grad, want_dw, 1e-2)
+    with pytest.raises(ValueError, match="tensor-wise"):
+        MXFP4LinearFunction.apply(x, w, False, True, float8_e5m2, ScalingGranularity.MX_BLOCKWISE.value, 0, False)
 
 
 def test_qdq_mxfp4_is_the_forward_weight_grid(mg, gpu):

@@ -55,7 +55,7 @@ WORKLOADS = {
 # elementwise kernel: 2.000 and 1.000).  The counter summary is committed as
 # profiles/bench_mixtral_mxfp8_hbm_traffic.txt.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "mixtral_8x7b_moe_mxfp8": (3257550.1 * 2.000 + 826636.6 * 1.000) * 1024,
+    "mixtral_8x7b_moe_mxfp8": (3244218.8 * 2.000 + 827147.6 * 1.000) * 1024,
 }
 
 
@@ -203,8 +203,9 @@ def gemm_calibration(fp4_weights, dev):
     """What this board's matrix cores deliver, measured in the same process, to read the GEMM figures against
     (the published peak assumes the 2.4 GHz boost clock; under load the board sits at its power limit):
     the library's register-only loop of the GEMM's own scaled MFMA (no memory traffic: the ceiling of any GEMM here),
-    and torch's vendor-library GEMMs on a dense problem of the benchmark's size (M 32768, N 28672, K 4096): FP8 with one
-    scale per tensor (no block scales) and, where torch supports it, MXFP8 with E8M0 block scales.  About 2 s."""
+    then one dense problem of the benchmark's size (M 32768, N 28672, K 4096) through this library's MX GEMM and through
+    torch's vendor-library GEMMs: FP8 with one scale per tensor (no block scales) and, where torch supports it, MXFP8
+    with E8M0 block scales.  About 4 s."""
     import torch
 
     from primus_amd import _lib
@@ -238,12 +239,22 @@ def gemm_calibration(fp4_weights, dev):
             _lib.check(lib.mxl_calibrate_mfma(fa, fb, iters, st), "mxl_calibrate_mfma")
         out["mfma_only_loop_%s_TFLOP/s" % name] = rate(loop, flops)
     out["mfma_only_loop"] = "mxl_calibrate_mfma: 256 workgroups x 4 waves, 16 scaled MFMAs 32x32x64 per K step on register operands, no memory traffic"
+    M, N, Kd = 32768, 28672, 4096
+    out["dense_gemm_shape_mnk"] = [M, N, Kd]
+    # this library's MX GEMM on the same dense problem (one group), for a like-for-like figure beside torch's
+    from primus_amd.pytorch import kernels as K
+    x = torch.randn(M, Kd, device=dev).bfloat16()
+    w = (torch.randn(N, Kd, device=dev) * 0.02).bfloat16()
+    lay = K.pick_layout(1, N, Kd, M, fp8=True)
+    xq, xs, _, _ = K.quantize_mx_impl(x, _lib.FMT_E4M3, rowwise=True, colwise=False, pad_to=K.GEMM_K_ALIGN, kchunk=lay)
+    wq, ws, _, _ = K.quantize_mx_weight_2d_impl(w, _lib.FMT_E4M3, rowwise=True, colwise=False, pad_to=K.GEMM_K_ALIGN, kchunk=lay)
+    del x, w
+    out["this_library_mxfp8_block_scales_TFLOP/s"] = rate(lambda: K.gemm_mx_nt_impl(xq, xs, wq, ws, kchunk=lay), 2.0 * M * N * Kd)
+    del xq, xs, wq, ws
     try:
-        M, N, Kd = 32768, 28672, 4096
         a8 = (torch.randn(M, Kd, device=dev) * 100).to(torch.float8_e4m3fn)
         b8 = (torch.randn(N, Kd, device=dev) * 100).to(torch.float8_e4m3fn)
         one = torch.ones((), device=dev)
-        out["vendor_gemm_shape_mnk"] = [M, N, Kd]
         out["torch_scaled_mm_fp8_per_tensor_scale_TFLOP/s"] = rate(
             lambda: torch._scaled_mm(a8, b8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 2.0 * M * N * Kd)
         try:
@@ -314,6 +325,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm-calibration", action="store_true",
                     help="skip the matrix-core calibration (register-only MFMA loop, torch's vendor GEMMs)")
+    ap.add_argument("--calibration-only", action="store_true",
+                    help="run the matrix-core calibration alone and print its JSON (the command of the hardware-counter "
+                         "comparison between torch's FP8 GEMM and this library's on one dense problem)")
     ap.add_argument("--no-wgrad-overlap", action="store_true",
                     help="keep wgrad on the launch stream behind dgrad (per-kernel durations are then undisturbed)")
     ap.add_argument("--board-seconds", type=float, default=2.0,
@@ -337,6 +351,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     spec = WORKLOADS[args.workload]
+    if args.calibration_only:
+        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev)}))
+        return
     lens = route(spec)
     G, M = spec["G"], sum(lens)
     grouped = spec["routing"] != "dense"

@@ -96,6 +96,16 @@ __device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_off, uint32_t voff,
                  : "memory");
 }
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// The same load with the LDS address formed in M0 by one scalar add (base register + constant) and the scalar
+// offset taken as it is: the ring kernel keeps a round's row offset in the per-lane offset instead of adding it to
+// the scalar one, which leaves two scalar instructions per request.
+template <int LDS_IMM>
+__device__ __forceinline__ void dma16_at(v4i rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
+                 :
+                 : "s"(lds_base), "n"(LDS_IMM), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "scc");
+}
 
 // Output stores are marked non-temporal: the kernel never reads its output back, and keeping it
 // out of the way leaves L2 to the operand tiles that neighbouring workgroups share.
@@ -601,6 +611,14 @@ constexpr int ring_lds_bytes() {
     return RING_SLOTS * RING_STAGE + RING_PANEL_BUFS * 2 * RING_PANEL + RING_TBL * 4 + RING_TBL * 8 + RING_TBL * 4 + RING_TBL * 4;
 }
 
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 template <int AFMT, int BFMT, int MODE, bool ALPHA>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     static_assert(AFMT != kFmtE2M1, "the row operand is FP8");
@@ -703,6 +721,14 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     // second group of 8 rows so that the 16-byte fragment reads of 16 consecutive rows cover all banks
     const uint32_t ld_voff_b = B4 ? (uint32_t)((t >> 1) * B_ROW + 16 * ((t & 1) ^ ((t >> 4) & 1))) : ld_voff;
     const uint32_t s_voff = (uint32_t)(t * 16);     // scale panel: row t of the tile, 16 bytes
+    // per-lane offsets of the load rounds: round e of an operand starts e * 64 rows = e * 4 KiB further on
+    const uint32_t wave_base = smem_base + (uint32_t)(w * 1024);    // ring slot 0, this wave's 1 KiB of a round
+    uint32_t va[4], vb[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        va[e] = ld_voff + (uint32_t)(e * 64 * BK);
+        vb[e] = ld_voff_b + (uint32_t)(e * 4096);
+    }
 
     struct Tile {
         v4i ra, rb, rsa, rsb;
@@ -800,10 +826,12 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         cgb = gb;
     };
     // round e (0 .. 7) of the group in flight into ring slot `slot` (0 .. 3, run time)
-    auto issue_e = [&](int e, uint32_t slot_base) __attribute__((always_inline)) {
-        if (e < 4) dma16(lra, slot_base + (uint32_t)((e * 4 + w) * 1024), ld_voff, ga + (uint32_t)(e * 64 * BK));
-        else if (e >= 6) dma16(crb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff_b, cgb + (uint32_t)((e - 4) * 4096));
-        else dma16(lrb, slot_base + (uint32_t)(A_BYTES + ((e - 4) * 4 + w) * 1024), ld_voff_b, gb + (uint32_t)((e - 4) * 4096));
+    // (slot_base already holds the wave's 1 KiB share, w * 1024; the round's 4 KiB come in as a constant)
+    auto issue_e = [&](auto e_tag, uint32_t slot_base) __attribute__((always_inline)) {
+        constexpr int e = decltype(e_tag)::value;
+        if constexpr (e < 4) dma16_at<e * 4096>(lra, slot_base, va[e], ga);
+        else if constexpr (e >= 6) dma16_at<A_BYTES + (e - 4) * 4096>(crb, slot_base, vb[e - 4], cgb);
+        else dma16_at<A_BYTES + (e - 4) * 4096>(lrb, slot_base, vb[e - 4], gb);
     };
     // scale panel pn of tile d (its K steps 8 pn .. 8 pn + 7) into panel buffer `buf`: 4 KiB per operand
     auto issue_s = [&](const Tile& d, int pn, int buf) __attribute__((always_inline)) {
@@ -897,11 +925,12 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     stream_enter(d);
     issue_s(d, 0, 0);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < 3; ++s) {
         group_begin();
-#pragma unroll
-        for (int e = 0; e < (s < 3 ? ROUNDS : 6); ++e) issue_e(e, smem_base + (uint32_t)(s * STAGE));
+        static_for<0, ROUNDS>([&](auto e) { issue_e(e, wave_base + (uint32_t)(s * STAGE)); });
     }
+    group_begin();
+    static_for<0, 6>([&](auto e) { issue_e(e, wave_base + (uint32_t)(3 * STAGE)); });
     wait_vm<2 * ROUNDS + 6>();       // everything up to K step 0 has landed
     __syncthreads();
 
@@ -927,15 +956,19 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // One K step s (local number, parity PAR) of 16 MFMAs.  MF: multiply (false for the padding steps of a
         // tile whose contraction range is shorter than four steps).  LAST: the tile's last step; the six rounds
         // that would go into the slot the epilogue is about to use are issued after the epilogue instead.
+        using E0 = std::integral_constant<int, 0>; using E1 = std::integral_constant<int, 1>;
+        using E2 = std::integral_constant<int, 2>; using E3 = std::integral_constant<int, 3>;
+        using E4 = std::integral_constant<int, 4>; using E5 = std::integral_constant<int, 5>;
+        using E6 = std::integral_constant<int, 6>; using E7 = std::integral_constant<int, 7>;
         auto kstep = [&](auto par_tag, auto mf_tag, auto last_tag, int s, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
             constexpr int PAR = decltype(par_tag)::value;
             constexpr bool MF = decltype(mf_tag)::value;
             constexpr bool LAST = decltype(last_tag)::value;
-            const uint32_t slot_prev = smem_base + (uint32_t)(((gs + 3) & 3) * STAGE);   // group of step gs + 3
-            const uint32_t slot_new = smem_base + (uint32_t)((gs & 3) * STAGE);          // group of step gs + 4
-            MXL_MFMA(cur, 0, 0); if (ROUNDS == 8) issue_e(6, slot_prev); MXL_PIN;
+            const uint32_t slot_prev = wave_base + (uint32_t)(((gs + 3) & 3) * STAGE);   // group of step gs + 3
+            const uint32_t slot_new = wave_base + (uint32_t)((gs & 3) * STAGE);          // group of step gs + 4
+            MXL_MFMA(cur, 0, 0); if (ROUNDS == 8) issue_e(E6{}, slot_prev); MXL_PIN;
             MXL_MFMA(cur, 1, 0); MXL_PIN;
-            MXL_MFMA(cur, 2, 0); if (ROUNDS == 8) issue_e(7, slot_prev); MXL_PIN;
+            MXL_MFMA(cur, 2, 0); if (ROUNDS == 8) issue_e(E7{}, slot_prev); MXL_PIN;
             MXL_MFMA(cur, 3, 0); MXL_PIN;
             wait_vm<2 * ROUNDS>();       // the group of step gs + 1 has landed (two younger groups may be in flight)
             __syncthreads();
@@ -950,17 +983,17 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             const uint8_t* sn = smem + ((gs + 1) & 3) * STAGE;
             const int psh = 8 * (s1 & 7);
             MXL_PIN;
-            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(0, slot_new); MXL_PIN;
+            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(E0{}, slot_new); MXL_PIN;
             MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1);  MXL_PIN;
-            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1);  if (!LAST) issue_e(1, slot_new); MXL_PIN;
+            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1);  if (!LAST) issue_e(E1{}, slot_new); MXL_PIN;
             MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1);  MXL_PIN;
-            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2);  if (!LAST) issue_e(2, slot_new); MXL_PIN;
+            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2);  if (!LAST) issue_e(E2{}, slot_new); MXL_PIN;
             MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2);  MXL_SC_B(nxt, 0); MXL_PIN;
-            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(3, slot_new); MXL_SC_A(nxt, 0); MXL_PIN;
+            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(E3{}, slot_new); MXL_SC_A(nxt, 0); MXL_PIN;
             MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2);  MXL_SC_A(nxt, 1); MXL_PIN;
-            MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(4, slot_new); MXL_SC_A(nxt, 2); MXL_PIN;
+            MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(E4{}, slot_new); MXL_SC_A(nxt, 2); MXL_PIN;
             MXL_MFMA(cur, 1, 3); MXL_SC_A(nxt, 3); MXL_SC_B(nxt, 1); MXL_PIN;
-            MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(5, slot_new); MXL_SC_B(nxt, 2); MXL_PIN;
+            MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(E5{}, slot_new); MXL_SC_B(nxt, 2); MXL_PIN;
             MXL_MFMA(cur, 3, 3); MXL_SC_B(nxt, 3); MXL_PIN;
             ++gs;
         };
@@ -1053,9 +1086,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // (the stream entered the next tile four steps ago; the group of its step 3 begins here)
         group_begin();
         {
-            const uint32_t slot_new = smem_base + (uint32_t)(((gs + 3) & 3) * STAGE);
-#pragma unroll
-            for (int e = 0; e < 6; ++e) issue_e(e, slot_new);
+            const uint32_t slot_new = wave_base + (uint32_t)(((gs + 3) & 3) * STAGE);
+            static_for<0, 6>([&](auto e) { issue_e(e, slot_new); });
         }
         d = dn;
         tile = tile_n;

@@ -270,6 +270,55 @@ def gemm_calibration(fp4_weights, dev):
     return out
 
 
+def quantizer_twin(dev):
+    """The dual MXFP8 quantiser's traffic without its arithmetic (mxl_calibrate_tile_copy: the same tiles in the same
+    order, 2 bytes read and 1 + 1 written per element, streaming loads and stores) against the quantiser itself on
+    the same tensor: how much of the distance to the stream calibration is the access pattern (a transposed copy
+    written in 128-byte pieces a row pitch apart) and how much the kernel."""
+    import torch
+
+    from primus_amd import _lib
+    from primus_amd.pytorch import kernels as K
+
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    res = {"kernel": "mxl_calibrate_tile_copy: 128x128 bf16 tiles read, 1 byte/element to a row-major and 1 to a transposed array"}
+    for rows, cols in ((32768, 4096), (32768, 28672)):
+        x = torch.randn(rows, cols, device=dev, dtype=torch.bfloat16)
+        o1 = torch.empty(rows, cols, dtype=torch.uint8, device=dev)
+        o2 = torch.empty(cols, rows, dtype=torch.uint8, device=dev)
+
+        def timed(fn, nbytes):
+            for _ in range(3):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return round(10 * nbytes / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1)
+
+        def twin(a, b):
+            return lambda: _lib.check(lib.mxl_calibrate_tile_copy(x.data_ptr(), rows, cols, a, b, st), "mxl_calibrate_tile_copy")
+
+        n = rows * cols
+        entry = {
+            "read+row+transposed_GB/s": timed(twin(o1.data_ptr(), o2.data_ptr()), 4.0 * n),
+            "read+row_GB/s": timed(twin(o1.data_ptr(), None), 3.0 * n),
+            "read+transposed_GB/s": timed(twin(None, o2.data_ptr()), 3.0 * n),
+            "read_only_GB/s": timed(twin(None, None), 2.0 * n),
+        }
+        del o1, o2
+        lay = K.pick_layout(1, 4096, cols, rows, fp8=True)
+        entry["quantizer_GB/s"] = timed(
+            lambda: K.quantize_mx_impl(x, _lib.FMT_E4M3, rowwise=True, colwise=True, pad_to=K.GEMM_K_ALIGN, kchunk=lay),
+            (4.0 + 2.0 / 32) * n)
+        res["%dx%d" % (rows, cols)] = entry
+        del x
+    return res
+
+
 def board_sample(run_step, seconds):
     """Socket power and shader clocks (``amd-smi metric --power --clock``) sampled while ``run_step`` loops for
     ``seconds``: says how far below the 2.4 GHz that the MFMA peak is quoted at the chip clocks under this load.
@@ -352,7 +401,7 @@ def main():
     torch.cuda.set_device(dev)
     spec = WORKLOADS[args.workload]
     if args.calibration_only:
-        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev)}))
+        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev), "quantizer_traffic_twin": quantizer_twin(dev)}))
         return
     lens = route(spec)
     G, M = spec["G"], sum(lens)
@@ -534,6 +583,8 @@ def main():
     for name in ("quantize", "quantize_weight_2d"):
         if name in kernels and "GB/s" in kernels[name]:
             kernels[name]["frac_of_stream_calibration"] = round(kernels[name]["GB/s"] / stream_gbs, 4)
+    if not args.no_gemm_calibration:
+        out["hbm_stream_calibration"]["quantizer_traffic_twin"] = quantizer_twin(dev)
     if not args.no_gemm_calibration:
         out["mfma_calibration"] = cal = gemm_calibration(spec["fp4"], dev)
         ceiling = cal.get("mfma_only_loop_fp8_x_fp4_TFLOP/s" if spec["fp4"] else "mfma_only_loop_fp8_x_fp8_TFLOP/s")

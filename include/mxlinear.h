@@ -415,6 +415,11 @@ int mxl_shuffle_scales(const void* src, int64_t rows, int64_t cols, void* dst, i
  * traffic at all: its rate is what the matrix cores of the board sustain under its power limit, the ceiling for any
  * GEMM on it.  mxl_calibrate_mfma_flops(iters) = the floating-point operations of one such launch. */
 int mxl_calibrate_mfma(int a_fmt, int b_fmt, int64_t iters, void* stream);
+/* mxl_calibrate_tile_copy moves the bytes of the dual MXFP8 quantiser without its arithmetic: x [rows, cols] bf16 read
+ * in 128 x 128 tiles, one byte per element written to out_row [rows, cols] and one to out_colT [cols, rows] (either may
+ * be null: read + one output, or read only), tiles in the quantiser's order; rows and cols multiples of 128.  Its rate
+ * is what that access pattern reaches on the board. */
+int mxl_calibrate_tile_copy(const void* in_bf16, int64_t rows, int64_t cols, void* out_row, void* out_colT, void* stream);
 int64_t mxl_calibrate_mfma_flops(int64_t iters);
 
 #ifdef __cplusplus

@@ -72,6 +72,7 @@ EXPORTS = (
     "mxl_shuffle_scales",
     "mxl_calibrate_mfma",
     "mxl_calibrate_mfma_flops",
+    "mxl_calibrate_tile_copy",
 )
 
 
@@ -175,6 +176,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_shuffle_scales.argtypes = [vp, i64, i64, vp, i32, vp]
         lib.mxl_calibrate_mfma.restype = i32
         lib.mxl_calibrate_mfma.argtypes = [i32, i32, i64, vp]
+        lib.mxl_calibrate_tile_copy.restype = i32
+        lib.mxl_calibrate_tile_copy.argtypes = [vp, i64, i64, vp, vp, vp]
         lib.mxl_calibrate_mfma_flops.restype = i64
         lib.mxl_calibrate_mfma_flops.argtypes = [i64]
         lib.mxl_gemm_nt_blockwise.restype = i32

@@ -58,9 +58,78 @@ __global__ __launch_bounds__(256) void mfma_only_kernel(int iters) {
     if (s == 12345.678f) calibrate_sink[threadIdx.x & 63] = s;   // keeps the loop alive; practically never taken
 }
 
+// The traffic of the dual quantiser without its arithmetic: every workgroup reads a 128 x 128 bf16 tile (16 bytes per
+// lane, rows adjacent) and writes one byte per element at the tile's place in a row-major array and one byte per
+// element at its place in the transposed array (16-byte stores; the bytes are XORs of the input, nothing is
+// transposed or converted), streaming loads and stores, tiles walked in the quantiser's order (8 x 8 supertiles, one
+// XCD each).  What this moves per second is what the quantiser's access pattern allows on the board.
+typedef uint32_t cu32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t cu32x2 __attribute__((ext_vector_type(2)));
+template <bool ROW, bool COL>
+__global__ __launch_bounds__(256) void tile_copy_kernel(const uint16_t* in, uint8_t* o_row, uint8_t* o_col, int64_t cols,
+                                                        int64_t w_ld, int tiles_r, int tiles_c, int super_c, int n_super) {
+    constexpr int TR = 128, TC = 128;
+    const int L = blockIdx.x, xcd = L & 7, k = L >> 3;
+    const int sup = (k / 64) * 8 + xcd;
+    if (sup >= n_super) return;
+    const int within = k % 64;
+    const int pt = (sup / super_c) * 8 + within / 8, ct = (sup % super_c) * 8 + within % 8;
+    if (pt >= tiles_r || ct >= tiles_c) return;
+    const int t = threadIdx.x;
+    constexpr int LPR = TC * 2 / 16, RPI = 256 / LPR, NIT = TR / RPI;   // 16 lanes a row, 16 rows a pass, 8 passes
+    cu32x4 d[NIT];
+    const int64_t r0 = (int64_t)pt * TR, c0 = (int64_t)ct * TC;
+#pragma unroll
+    for (int i = 0; i < NIT; ++i) {
+        const int r = i * RPI + t / LPR, c = (t % LPR) * 8;
+        d[i] = __builtin_nontemporal_load((const cu32x4*)(in + (r0 + r) * cols + c0 + c));
+    }
+    cu32x4 acc = d[0];
+#pragma unroll
+    for (int i = 1; i < NIT; ++i) acc ^= d[i];
+    if (ROW) {
+#pragma unroll
+        for (int i = 0; i < NIT; ++i) {
+            const int r = i * RPI + t / LPR, c = (t % LPR) * 8;
+            const cu32x2 v = {d[i].x ^ d[i].y, d[i].z ^ d[i].w};
+            __builtin_nontemporal_store(v, (cu32x2*)(o_row + (r0 + r) * cols + c0 + c));
+        }
+    }
+    if (COL) {
+        constexpr int LPR2 = TR / 16, RPI2 = 256 / LPR2;                // 8 lanes a transposed row, 32 rows a pass
+#pragma unroll
+        for (int i = 0; i < TC / RPI2; ++i) {
+            const int c = i * RPI2 + t / LPR2, ch = t % LPR2;
+            __builtin_nontemporal_store(acc ^ d[i % NIT], (cu32x4*)(o_col + (c0 + c) * w_ld + r0 + ch * 16));
+        }
+    }
+    if (!ROW && !COL && acc.x == 0x12345u && acc.y == 0x54321u) calibrate_sink[t & 63] = 1.f;   // keeps the loads alive
+}
+
 }  // namespace mxl
 
 using namespace mxl;
+
+extern "C" int mxl_calibrate_tile_copy(const void* in_bf16, int64_t rows, int64_t cols, void* out_row, void* out_colT,
+                                       void* stream) {
+    if (rows <= 0 || cols <= 0 || rows % 128 || cols % 128 || rows > (int64_t(1) << 30) || cols > (int64_t(1) << 30) || !in_bf16)
+        return MXL_EINVAL;
+    if ((((uintptr_t)in_bf16 | (uintptr_t)out_row | (uintptr_t)out_colT) & 15) != 0) return MXL_EINVAL;
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    const int tiles_r = (int)(rows / 128), tiles_c = (int)(cols / 128);
+    const int super_r = (tiles_r + 7) / 8, super_c = (tiles_c + 7) / 8, n_super = super_r * super_c;
+    const int64_t wgs = (int64_t)(n_super + 7) / 8 * 8 * 64;
+    if (wgs > 0x7FFFFFFF) return MXL_EINVAL;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)wgs), block(256);
+    const uint16_t* in = (const uint16_t*)in_bf16;
+    uint8_t *o1 = (uint8_t*)out_row, *o2 = (uint8_t*)out_colT;
+    if (o1 && o2) hipLaunchKernelGGL((tile_copy_kernel<true, true>), grid, block, 0, st, in, o1, o2, cols, rows, tiles_r, tiles_c, super_c, n_super);
+    else if (o1) hipLaunchKernelGGL((tile_copy_kernel<true, false>), grid, block, 0, st, in, o1, o2, cols, rows, tiles_r, tiles_c, super_c, n_super);
+    else if (o2) hipLaunchKernelGGL((tile_copy_kernel<false, true>), grid, block, 0, st, in, o1, o2, cols, rows, tiles_r, tiles_c, super_c, n_super);
+    else hipLaunchKernelGGL((tile_copy_kernel<false, false>), grid, block, 0, st, in, o1, o2, cols, rows, tiles_r, tiles_c, super_c, n_super);
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
 
 extern "C" int64_t mxl_calibrate_mfma_flops(int64_t iters) {
     // 256 workgroups x 4 waves x iters x 16 MFMAs of 32 x 32 x 64

@@ -49,6 +49,8 @@ def test_host_only_entry_points(lib):
     assert lib.mxl_calibrate_mfma_flops(-1) == -1
     assert lib.mxl_calibrate_mfma(_lib.FMT_E4M3, _lib.FMT_E4M3, 0, None) == -1      # no iterations
     assert lib.mxl_calibrate_mfma(7, _lib.FMT_E4M3, 16, None) == -1                 # unknown format
+    assert lib.mxl_calibrate_tile_copy(None, 128, 128, None, None, None) == -1      # no input
+    assert lib.mxl_calibrate_tile_copy(ctypes.c_void_p(4096), 100, 128, None, None, None) == -1   # rows % 128
 
 
 def test_constants_match_the_header():

@@ -412,3 +412,26 @@ def test_calibration_loop_runs_for_every_operand_mix():
         for fb in (_lib.FMT_E4M3, _lib.FMT_E2M1):
             assert lib.mxl_calibrate_mfma(fa, fb, 8, st) == 0
     torch.cuda.synchronize()
+
+
+def test_quantizer_traffic_twin_runs_in_every_mode():
+    """The tile-copy kernel of the benchmark's calibration: each output it is given receives one byte per element
+    (every byte of both arrays is written), the input is untouched."""
+    from primus_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    x = torch.randn(256, 384, device=dev).bfloat16()
+    keep = x.clone()
+    for want_row, want_col in ((True, True), (True, False), (False, True), (False, False)):
+        o1 = torch.full((256, 384), 0xA5, dtype=torch.uint8, device=dev)
+        o2 = torch.full((384, 256), 0xA5, dtype=torch.uint8, device=dev)
+        rc = lib.mxl_calibrate_tile_copy(x.data_ptr(), 256, 384, o1.data_ptr() if want_row else None,
+                                         o2.data_ptr() if want_col else None, st)
+        assert rc == 0
+        torch.cuda.synchronize()
+        # XORs of random bf16 halves: practically never all 0xA5 in a written array, exactly 0xA5 in an untouched one
+        assert bool((o1 != 0xA5).any()) == want_row and bool((o2 != 0xA5).any()) == want_col
+    assert torch.equal(x, keep)
+    assert lib.mxl_calibrate_tile_copy(x.data_ptr(), 256, 100, None, None, st) == -1

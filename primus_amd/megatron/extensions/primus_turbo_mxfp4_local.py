@@ -183,9 +183,52 @@ def _quantize_grad_dual(grad_2d, preshuffle: bool = False, use_sr: bool = False,
     return _dual(grad_2d, False, use_sr, use_rht, (preshuffle, False, preshuffle, False))
 
 
-def _gemm_nt(a, a_scale, b, b_scale, out_dtype, preshuffle=False):
+# The GEMMs of the function are custom ops too (the reference's gemm_fp4_impl / gemm_fp8_impl are ops of its C++
+# extension): torch.compile then traces MXFP4LinearFunction without a graph break, which the reference tests
+# (tests/unit_tests/backends/megatron/test_primus_turbo_mxfp4_local.py:202-287).
+def _gemm_fp4_nt_impl(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor,
+                      out_dtype: torch.dtype, preshuffled: bool) -> torch.Tensor:
     return K.gemm_fp4_impl(a, a_scale, False, b, b_scale, True, out_dtype, False, granularity=_GRAN_VALUE,
-                           default_backend=None, preshuffled=preshuffle)
+                           default_backend=None, preshuffled=preshuffled)
+
+
+_gemm_fp4_nt_op = torch.library.custom_op("primus_amd::mxfp4_gemm_nt", _gemm_fp4_nt_impl, mutates_args=(), device_types="cuda")
+_gemm_fp4_nt_op.register_fake(lambda a, a_scale, b, b_scale, out_dtype, preshuffled:
+                              torch.empty((a.shape[0], b.shape[0]), dtype=out_dtype, device=a.device))
+
+
+def _gemm_nt(a, a_scale, b, b_scale, out_dtype, preshuffle=False):
+    return _gemm_fp4_nt_op(a, a_scale, b, b_scale, out_dtype, preshuffle)
+
+
+def _fp8_tw_backward_op_impl(grad_2d: torch.Tensor, input_2d: torch.Tensor, weight: torch.Tensor,
+                             fmt: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    dx, dw = _fp8_tw_backward(grad_2d, input_2d, weight, fmt)
+    return dx.contiguous(), dw.contiguous()
+
+
+_fp8_tw_backward_op = torch.library.custom_op("primus_amd::mxfp4_fp8_backward", _fp8_tw_backward_op_impl, mutates_args=(),
+                                              device_types="cuda")
+_fp8_tw_backward_op.register_fake(lambda grad_2d, input_2d, weight, fmt: (
+    torch.empty((grad_2d.shape[0], weight.shape[1]), dtype=torch.bfloat16, device=grad_2d.device),
+    torch.empty(tuple(weight.shape), dtype=torch.bfloat16, device=grad_2d.device)))
+
+
+def _enable_preshuffle() -> bool:
+    """The reference turns the pre-shuffled layouts on when its FP4 GEMM backend is pinned to AITER and autotuning is
+    off (:61-74).  This library has one backend, which reads both layouts; the same environment switches are honoured
+    so that a launch script written for the reference behaves the same way."""
+    import os
+
+    pinned = "FP4:AITER" in os.environ.get("PRIMUS_TURBO_GEMM_BACKEND", "").upper().replace(" ", "")
+    return pinned and not os.environ.get("PRIMUS_TURBO_AUTO_TUNE")
+
+
+def _assert_preshuffle_contract(config, preshuffle: bool) -> None:
+    """The reference refuses MXFP4 without its pre-shuffle fast path, because its other backends would misread
+    shuffled bytes or pay extra shuffle passes (:77-105).  Neither can happen here (the flag travels with every
+    call and the GEMM converts what it is told is shuffled), so there is nothing to refuse."""
+    return None
 
 
 def _fp8_tw_backward(grad_2d, input_2d, weight, fmt):
@@ -264,7 +307,8 @@ class MXFP4LinearFunction(torch.autograd.Function):
             grad_2d = grad_2d.to(torch.bfloat16)
         if ctx.backward_is_fp8:
             input_2d, weight = ctx.saved_tensors
-            grad_input, grad_weight = _fp8_tw_backward(grad_2d, input_2d.detach(), weight.detach(), ctx.fp8_fmt)
+            grad_input, grad_weight = _fp8_tw_backward_op(grad_2d, input_2d.detach().contiguous(), weight.detach().contiguous(),
+                                                          ctx.fp8_fmt)
             return (grad_input.reshape(ctx.orig_shape), grad_weight) + (None,) * 6
         a_t, a_t_s, b_t, b_t_s = ctx.saved_tensors
         a_t, b_t = a_t.view(_FP4_DTYPE), b_t.view(_FP4_DTYPE)

@@ -394,6 +394,35 @@ def test_mxfp4_linear_function_fp8_backward(mg, gpu):
         MXFP4LinearFunction.apply(x, w, False, True, float8_e5m2, ScalingGranularity.MX_BLOCKWISE.value, 0, False)
 
 
+def test_mxfp4_linear_function_traces_without_graph_breaks(mg, gpu):
+    """What the reference's own tests ask of the function (test_primus_turbo_mxfp4_local.py:202-287): torch.compile
+    traces it without a graph break in both modes, and the traced forward and backward equal the eager ones."""
+    from primus_amd.megatron.extensions.primus_turbo_mxfp4_local import MXFP4LinearFunction
+    from primus_amd.pytorch.core.low_precision import ScalingGranularity, float8_e5m2
+
+    torch.manual_seed(42)
+    x = torch.randn(128, 256, dtype=torch.bfloat16, device=gpu)
+    w = torch.randn(512, 256, dtype=torch.bfloat16, device=gpu)
+    modes = ((False, False, None, 0, 0, False), (True, False, None, 0, 0, False),
+             (False, True, float8_e5m2, ScalingGranularity.TENSORWISE.value, 0, False))
+    for args in modes:
+        torch._dynamo.reset()
+        explanation = torch._dynamo.explain(MXFP4LinearFunction.apply)(x, w, *args)
+        assert explanation.graph_break_count == 0, explanation.break_reasons
+    torch._dynamo.reset()
+    for args in modes:
+        xe, we = x.clone().requires_grad_(), w.clone().requires_grad_()
+        xc, wc = x.clone().requires_grad_(), w.clone().requires_grad_()
+        eager = MXFP4LinearFunction.apply(xe, we, *args)[0]
+        compiled = torch.compile(MXFP4LinearFunction.apply, backend="aot_eager")(xc, wc, *args)[0]
+        assert torch.equal(eager, compiled)
+        dy = torch.randn_like(eager)
+        eager.backward(dy)
+        compiled.backward(dy)
+        assert torch.equal(xe.grad, xc.grad) and torch.equal(we.grad, wc.grad)
+    torch._dynamo.reset()
+
+
 def test_qdq_mxfp4_is_the_forward_weight_grid(mg, gpu):
     from primus_amd.megatron.optimizer.weight_deosc import qdq_mxfp4, qdq_mxfp4_local_shard
 

@@ -723,6 +723,25 @@ def test_dual_quantize_recipes_per_operand(monkeypatch):
     assert calls[3] == (fp4, pad, False, False, False, False, False, True, True, False, True, True)
 
 
+def test_preshuffle_switch_follows_the_reference_environment(monkeypatch):
+    """_enable_preshuffle (primus_turbo_mxfp4_local.py:61-74): on when the FP4 GEMM backend is pinned to AITER and
+    autotuning is off; the contract check never refuses here."""
+    monkeypatch.delenv("PRIMUS_TURBO_GEMM_BACKEND", raising=False)
+    monkeypatch.delenv("PRIMUS_TURBO_AUTO_TUNE", raising=False)
+    assert mxfp4_local._enable_preshuffle() is False
+    monkeypatch.setenv("PRIMUS_TURBO_GEMM_BACKEND", "FP4:AITER")
+    assert mxfp4_local._enable_preshuffle() is True
+    monkeypatch.setenv("PRIMUS_TURBO_GEMM_BACKEND", "fp8:hipblaslt, fp4:aiter")
+    assert mxfp4_local._enable_preshuffle() is True
+    monkeypatch.setenv("PRIMUS_TURBO_AUTO_TUNE", "1")
+    assert mxfp4_local._enable_preshuffle() is False
+    monkeypatch.setenv("PRIMUS_TURBO_GEMM_BACKEND", "FP4:HIPBLASLT")
+    monkeypatch.delenv("PRIMUS_TURBO_AUTO_TUNE")
+    assert mxfp4_local._enable_preshuffle() is False
+    import types
+    assert mxfp4_local._assert_preshuffle_contract(types.SimpleNamespace(fp4="mxfp4"), False) is None
+
+
 # --------------------------------------------------------------------------- a13
 def test_local_shard_qdq_keeps_tile_coordinates(monkeypatch):
     calls = []

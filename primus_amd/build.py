@@ -38,15 +38,37 @@ def hipcc_path() -> str:
 
 
 def build(verbose: bool = False) -> str:
-    """Compile every HIP source into primus_amd/lib/libmxlinear.so; returns its path."""
+    """Compile every HIP source (one hipcc process per file, side by side) and link primus_amd/lib/libmxlinear.so;
+    returns its path."""
+    from concurrent.futures import ThreadPoolExecutor
+
     os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH]
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    hipcc = hipcc_path()
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+
+    def compile_one(src: str):
+        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc, *compile_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        return obj, subprocess.run(cmd, capture_output=True, text=True)
+
+    workers = max(1, min(len(SOURCES), os.cpu_count() or 1, 8))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        results = list(pool.map(compile_one, SOURCES))
+    for obj, res in results:
+        if res.returncode != 0:
+            sys.stderr.write(res.stdout + res.stderr)
+            raise RuntimeError("hipcc failed compiling %s" % os.path.basename(obj))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[obj for obj, _ in results], "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("hipcc failed building libmxlinear.so")
+        raise RuntimeError("hipcc failed linking libmxlinear.so")
     return LIB_PATH
 
 

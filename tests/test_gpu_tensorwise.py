@@ -189,6 +189,60 @@ def test_scaled_gemm_is_exact_on_exact_operands(gpu, afmt):
     assert np.array_equal(_f(y), o.bf16_bits_to_f32(o.f32_to_bf16_bits(want)))
 
 
+@pytest.mark.parametrize("kchunk", [False, True])
+def test_e5m2_times_e5m2_is_exact_on_exact_operands(gpu, kchunk):
+    """Both operands in the gradient format (the FP8 backward of the MXFP4 linear re-quantises dY, X and W to E5M2):
+    forward-shaped and wgrad-shaped GEMMs on integer codes, bit for bit; the K-step-major layout is refused."""
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator().manual_seed(17)
+    lens = [130, 0, 62, 192]
+    rows, n, k = sum(lens), 160, 256
+    a_int = torch.randint(-3, 4, (rows, k), generator=g).float()
+    d_int = torch.randint(-3, 4, (rows, n), generator=g).float()
+    w_int = torch.randint(-3, 4, (len(lens), n, k), generator=g).float()
+    # first the GEMM alone on codes written here (small integers are exact in E5M2, the factors are powers of two)
+    def codes(t):
+        return torch.from_numpy(o.cast_e5m2(t.numpy().astype(np.float32))).view(torch.float8_e5m2)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    one = torch.ones(1, device=gpu)
+    half = torch.full((1,), 0.5, device=gpu)
+    unit = lambda r, c: torch.full((r, c // 32), 127, dtype=torch.uint8, device=gpu).view(torch.float8_e8m0fnu)  # noqa: E731
+    if not kchunk:
+        y = K.gemm_tw_nt_impl(codes(a_int).to(gpu), unit(rows, k), one, codes(w_int).to(gpu), unit(len(lens) * n, k).view(len(lens), n, -1),
+                              half, gl)
+        want = torch.cat([a @ w_int[e].T for e, a in enumerate(torch.split(a_int, lens))]) * 0.5
+        assert torch.equal(y.float().cpu(), want.bfloat16().float())
+    # through the quantisers (tensor-wise, E5M2 for every operand), both 2-slot layouts, against the oracle
+    x = (a_int * 0.37).bfloat16(); dy = (d_int * 1.3).bfloat16(); w = (w_int * 0.011).bfloat16()
+    da = K.quantize_tensorwise_impl(dy.to(gpu), 2, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kchunk)
+    xa = K.quantize_tensorwise_impl(x.to(gpu), 2, rowwise=False, colwise=True, group_lens=gl, kchunk=kchunk)
+    wq = K.quantize_weight_tensorwise_impl(w.to(gpu), 2, rowwise=False, colwise=True, pad_to=128, kchunk=kchunk)
+    dx = K.gemm_tw_nt_impl(da[0], da[1], da[4], wq[2], wq[3], wq[4], gl, kchunk=kchunk)[:, :k]
+    dw = K.gemm_tw_wgrad_impl(da[2], da[3], da[4], xa[2], xa[3], xa[4], gl, rows, kchunk=kchunk)
+    dc, dsi = o.quantize_tensorwise(dy, 2)
+    xc, xsi = o.quantize_tensorwise(x, 2)
+    wc, wsi = o.quantize_tensorwise(w.reshape(-1, k), 2)
+    wc = wc.reshape(-1, n, k)
+    pos = 0
+    for e, ln in enumerate(lens):
+        if ln:
+            want_dx = o.bf16_bits_to_f32(o.tensorwise_gemm_nt_ref(dc[pos:pos + ln], dsi, np.ascontiguousarray(wc[e].T), wsi, 2, 2))
+            assert np.abs(_f(dx)[pos:pos + ln] - want_dx).max() <= TOL * max(np.abs(want_dx).max(), 1e-30)
+            want_dw = o.bf16_bits_to_f32(o.tensorwise_gemm_nt_ref(np.ascontiguousarray(dc[pos:pos + ln].T), dsi,
+                                                                  np.ascontiguousarray(xc[pos:pos + ln].T), xsi, 2, 2))
+            assert np.abs(_f(dw)[e] - want_dw).max() <= TOL * max(np.abs(want_dw).max(), 1e-30)
+        else:
+            assert not _f(dw)[e].any()
+        pos += ln
+    if kchunk:
+        from primus_amd._lib import MXLinearError
+        d2 = K.quantize_tensorwise_impl(dy.to(gpu), 2, rowwise=True, colwise=False, pad_to=128, kchunk=2)
+        w2 = K.quantize_weight_tensorwise_impl(w.to(gpu), 2, rowwise=False, colwise=True, pad_to=128, kchunk=2)
+        with pytest.raises(MXLinearError):
+            K.gemm_tw_nt_impl(d2[0], d2[1], d2[4], w2[2], w2[3], w2[4], gl, kchunk=2)
+
+
 def _tw_cfg(hybrid):
     from primus_amd.pytorch.core import Float8QuantConfig, Format, ScalingGranularity
 

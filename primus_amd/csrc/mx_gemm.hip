@@ -327,6 +327,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     };
     // scale panel pn (K slots 4pn .. 4pn+3) into panel buffer pn & 1
     auto issue_s = [&](const Tile& d, int pn) __attribute__((always_inline)) {
+        if (ALPHA) return;   // per-tensor factors: the block scales are the unit byte by contract and are not read
         const uint32_t base = smem_base + NSLOT * STAGE + (pn & 1) * 2 * PANEL;
         dma16(d.rsa, base + w * 1024, s_voff, d.ks0 + 16 * pn);
         dma16(d.rsb, base + PANEL + w * 1024, s_voff, d.ks0 + 16 * pn);
@@ -346,10 +347,10 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // read one fragment (+ its scale byte) of the K step described by (sn, pan, ks_n)
 #define MXL_RD_A(F, I) \
     do { if ((I) < NA) { F.a[I] = read_frag<AFMT>(sn, wm * 128 + (I) * 32 + lr, ks_n, g); \
-                         F.sa[I] = pan[16 * (wm * 128 + (I) * 32 + lr)]; } } while (0)
+                         F.sa[I] = ALPHA ? 127 : pan[16 * (wm * 128 + (I) * 32 + lr)]; } } while (0)
 #define MXL_RD_B(F, J) \
     do { if (NA > 0) { F.b[J] = read_frag<BFMT>(sn + A_BYTES, wn * 128 + (J) * 32 + lr, ks_n, g); \
-                       F.sb[J] = pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]; } } while (0)
+                       F.sb[J] = ALPHA ? 127 : pan[PANEL + 16 * (wn * 128 + (J) * 32 + lr)]; } } while (0)
 
     int tile = vwg;
     if (tile >= total_tiles) return;
@@ -835,6 +836,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     };
     // scale panel pn of tile d (its K steps 8 pn .. 8 pn + 7) into panel buffer `buf`: 4 KiB per operand
     auto issue_s = [&](const Tile& d, int pn, int buf) __attribute__((always_inline)) {
+        if (ALPHA) return;   // per-tensor factors: the block scales are the unit byte by contract and are not read
         const uint32_t base = smem_base + (uint32_t)(RING_SLOTS * STAGE + buf * 2 * PANEL);
         dma16(d.rsa, base + w * 1024, s_voff, d.pa0 + (uint32_t)pn * a_pstride);
         dma16(d.rsb, base + PANEL + w * 1024, s_voff, d.pb0 + (uint32_t)pn * b_pstride);
@@ -863,8 +865,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
          } } while (0)
     // the scale byte of step `psh / 8` of the panel, for fragment I of A / J of B (one shift each; they are spread
     // over the second half of a step's MFMAs so that the panel reads have long landed)
-#define MXL_SC_A(F, I) do { F.sa[I] = (int)(uint32_t)(psa[I] >> psh); } while (0)
-#define MXL_SC_B(F, J) do { F.sb[J] = (int)(uint32_t)(psb[J] >> psh); } while (0)
+#define MXL_SC_A(F, I) do { F.sa[I] = ALPHA ? 127 : (int)(uint32_t)(psa[I] >> psh); } while (0)
+#define MXL_SC_B(F, J) do { F.sb[J] = ALPHA ? 127 : (int)(uint32_t)(psb[J] >> psh); } while (0)
     // per-lane constants of the fragment reads: 64-byte rows, piece index XOR (row / 4) % 4
     const int sw = (lr >> 2) & 3;
     const int a_frag = (wm * 128 + lr) * BK, b_frag = (wn * 128 + lr) * B_ROW;
@@ -876,7 +878,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     const int a_sc = (wm * 128 + lr) * 16 + 8 * g, b_sc = (wn * 128 + lr) * 16 + 8 * g;
     uint64_t psa[4], psb[4];
 #define MXL_RD_PANEL(PAN) \
-    do { _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) { \
+    do { if (!ALPHA) _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) { \
              psa[i_] = *(const uint64_t*)((PAN) + a_sc + i_ * (32 * 16)); \
              psb[i_] = *(const uint64_t*)((PAN) + PANEL + b_sc + i_ * (32 * 16)); } } while (0)
 
@@ -1275,7 +1277,8 @@ static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt,
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;
     if (num_groups > 1 && !group_lens) return MXL_EINVAL;
     if (total_m == 0) return MXL_OK;   // no rows: nothing to read or write (the row operands may be null)
-    if (!a_codes || !a_scales || !b_codes || !b_scales || !c_bf16) return MXL_EINVAL;
+    if (!a_codes || !b_codes || !c_bf16) return MXL_EINVAL;
+    if (alpha_a == nullptr && (!a_scales || !b_scales)) return MXL_EINVAL;   // block scales are read unless per-tensor factors are given
     GemmArgs a;
     a.a = (const uint8_t*)a_codes;
     a.sa = (const uint8_t*)a_scales;
@@ -1355,7 +1358,8 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
                            words);
         return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
     }
-    if (!a_codes || !a_scales || !b_codes || !b_scales) return MXL_EINVAL;
+    if (!a_codes || !b_codes) return MXL_EINVAL;
+    if (alpha_a == nullptr && (!a_scales || !b_scales)) return MXL_EINVAL;   // block scales are read unless per-tensor factors are given
     GemmArgs a;
     a.a = (const uint8_t*)a_codes;
     a.sa = (const uint8_t*)a_scales;

@@ -34,6 +34,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 FP8_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+FP4_PEAK_TFLOPS = 10100.0  # MI355X dense FP4 MFMA
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 WORKLOADS = {
@@ -42,6 +43,8 @@ WORKLOADS = {
     "deepseek_v3_shard_mxfp8": dict(G=32, topk=8, tokens=8192, hidden=7168, fc1_out=4096, fc2_in=2048, routing="zipf", seed=1004, fp4=False),
     "gpt_oss_120b_mxfp4": dict(G=128, topk=4, tokens=16384, hidden=2880, fc1_out=5760, fc2_in=2880, routing="uniform", seed=1005, fp4=True, wgrad=False),
     "llama3_8b_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False),
+    # the pure MXFP4 recipe (E2M1 activations, weights and gradients) on the headline shapes
+    "mixtral_8x7b_moe_mxfp4": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=True, act_fp4=True),
     # the non-MX "current scaling" recipe on the headline shapes (HYBRID: E4M3 forward, E5M2 gradients)
     "mixtral_8x7b_moe_fp8_tensorwise": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, tensorwise=True),
     # the same MLP with the RMSNorm that precedes fc1 in the layer (LayerNormColumnParallelLinear), folded into fc1's quantiser
@@ -142,6 +145,7 @@ def cpu_baseline(spec, lens, sample_div=16):
     threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
     torch.set_num_threads(threads)
     fmt_w = o.FMT_E2M1 if spec["fp4"] else o.FMT_E4M3
+    fmt_a = o.FMT_E2M1 if spec.get("act_fp4") else o.FMT_E4M3
     G = spec["G"]
     slens = [max(1, ln // sample_div) if ln else 0 for ln in lens]
     m = sum(slens)
@@ -152,15 +156,15 @@ def cpu_baseline(spec, lens, sample_div=16):
         x = o.to_bf16_bits(torch.randn(m, k, generator=g).bfloat16())
         dy = o.to_bf16_bits(torch.randn(m, n, generator=g).bfloat16())
         w = o.to_bf16_bits((torch.randn(G, n, k, generator=g) * 0.02).bfloat16())
-        xq, xs = C.quantize_rowwise(x, o.FMT_E4M3)
-        xt, xts = C.quantize_colwise_segmented(x, slens, o.FMT_E4M3)
-        dq, ds = C.quantize_rowwise(dy, o.FMT_E4M3)
-        dt, dts = C.quantize_colwise_segmented(dy, slens, o.FMT_E4M3)
+        xq, xs = C.quantize_rowwise(x, fmt_a)
+        xt, xts = C.quantize_colwise_segmented(x, slens, fmt_a)
+        dq, ds = C.quantize_rowwise(dy, fmt_a)
+        dt, dts = C.quantize_colwise_segmented(dy, slens, fmt_a)
         wq, ws, wqt, wst = C.quantize_2d(w, fmt_w)
-        xf = torch.from_numpy(C.dequantize(xq, xs, o.FMT_E4M3))
-        df = torch.from_numpy(C.dequantize(dq, ds, o.FMT_E4M3))
-        xtf = torch.from_numpy(C.dequantize(xt, xts, o.FMT_E4M3))
-        dtf = torch.from_numpy(C.dequantize(dt, dts, o.FMT_E4M3))
+        xf = torch.from_numpy(C.dequantize(xq, xs, fmt_a))
+        df = torch.from_numpy(C.dequantize(dq, ds, fmt_a))
+        xtf = torch.from_numpy(C.dequantize(xt, xts, fmt_a))
+        dtf = torch.from_numpy(C.dequantize(dt, dts, fmt_a))
         offs = np.concatenate([[0], np.cumsum(slens)])
         _, poffs = o.segment_layout(slens)
         for e in range(G):
@@ -199,7 +203,7 @@ def cpu_baseline(spec, lens, sample_div=16):
     }
 
 
-def gemm_calibration(fp4_weights, dev):
+def gemm_calibration(fp4_weights, dev, fp4_acts=False):
     """What this board's matrix cores deliver, measured in the same process, to read the GEMM figures against
     (the published peak assumes the 2.4 GHz boost clock; under load the board sits at its power limit):
     the library's register-only loop of the GEMM's own scaled MFMA (no memory traffic: the ceiling of any GEMM here),
@@ -234,7 +238,8 @@ def gemm_calibration(fp4_weights, dev):
 
     iters = 4096
     flops = float(lib.mxl_calibrate_mfma_flops(iters))
-    for name, (fa, fb) in (("fp8_x_fp8", (_lib.FMT_E4M3, _lib.FMT_E4M3)),) + ((("fp8_x_fp4", (_lib.FMT_E4M3, _lib.FMT_E2M1)),) if fp4_weights else ()):
+    for name, (fa, fb) in (("fp8_x_fp8", (_lib.FMT_E4M3, _lib.FMT_E4M3)),) + ((("fp8_x_fp4", (_lib.FMT_E4M3, _lib.FMT_E2M1)),) if fp4_weights and not fp4_acts else ()) \
+            + ((("fp4_x_fp4", (_lib.FMT_E2M1, _lib.FMT_E2M1)),) if fp4_acts else ()):
         def loop(fa=fa, fb=fb):
             _lib.check(lib.mxl_calibrate_mfma(fa, fb, iters, st), "mxl_calibrate_mfma")
         out["mfma_only_loop_%s_TFLOP/s" % name] = rate(loop, flops)
@@ -401,13 +406,13 @@ def main():
     torch.cuda.set_device(dev)
     spec = WORKLOADS[args.workload]
     if args.calibration_only:
-        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev), "quantizer_traffic_twin": quantizer_twin(dev)}))
+        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev, bool(spec.get("act_fp4"))), "quantizer_traffic_twin": quantizer_twin(dev)}))
         return
     lens = route(spec)
     G, M = spec["G"], sum(lens)
     grouped = spec["routing"] != "dense"
     if spec["fp4"]:
-        cfg = Float4QuantConfig(activation_format=Format.E4M3)
+        cfg = Float4QuantConfig(activation_format=Format.E2M1_X2 if spec.get("act_fp4") else Format.E4M3)
         op = pt.ops.grouped_gemm_fp4
     elif spec.get("tensorwise"):
         cfg = Float8QuantConfig(format=Format.HYBRID, granularity=ScalingGranularity.TENSORWISE)
@@ -505,16 +510,20 @@ def main():
     fwd_name = "grouped_gemm_nt" if grouped else "gemm_nt"
     gk = acc[fwd_name]
     gemm_tflops = gk["flops"] / gk["sec"] / 1e12
+    act_fp4 = bool(spec.get("act_fp4"))
+    # the MFMA peak of the slower operand format: FP8 rate unless both operands are E2M1
+    peak = FP4_PEAK_TFLOPS if act_fp4 else FP8_PEAK_TFLOPS
     roofline = {
-        # FP8 x FP8 operands (MX or tensor-wise scaled) run on the 4-slot ring kernel, FP4 operands on the 2-slot kernel
-        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_kernel" if spec["fp4"] else "mx_gemm_ring_kernel",
-                                                   "e4m3|e5m2" if spec.get("tensorwise") else "e4m3", "e2m1" if spec["fp4"] else "e4m3",
+        # FP8 x FP8 (MX or tensor-wise scaled) and E2M1 x E2M1 run on the 4-slot ring kernel, FP8 x E2M1 on the 2-slot kernel
+        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_kernel" if spec["fp4"] and not act_fp4 else "mx_gemm_ring_kernel",
+                                                   "e4m3|e5m2" if spec.get("tensorwise") else "e2m1" if act_fp4 else "e4m3",
+                                                   "e2m1" if spec["fp4"] else "e4m3",
                                                    ",alpha" if spec.get("tensorwise") else "", fwd_name),
         "bound": "mfma",
         "achieved": round(gemm_tflops, 2),
-        "peak": FP8_PEAK_TFLOPS,
+        "peak": peak,
         "unit": "TFLOP/s",
-        "frac": round(gemm_tflops / FP8_PEAK_TFLOPS, 4),
+        "frac": round(gemm_tflops / peak, 4),
         "avg_launch_ms": round(gk["sec"] / gk["n"] * 1e3, 4),
         "flops_per_launch": gk["flops"] / gk["n"],
         "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
@@ -524,7 +533,7 @@ def main():
         ent = {"launches_per_step": a["n"] // kernel_steps, "ms_per_step": round(a["sec"] * 1e3 / kernel_steps, 4)}
         if a["flops"]:
             ent["TFLOP/s"] = round(a["flops"] / a["sec"] / 1e12, 2)
-            ent["frac_fp8_mfma_peak"] = round(a["flops"] / a["sec"] / 1e12 / FP8_PEAK_TFLOPS, 4)
+            ent["frac_fp4_mfma_peak" if act_fp4 else "frac_fp8_mfma_peak"] = round(a["flops"] / a["sec"] / 1e12 / peak, 4)
         else:
             ent["GB/s"] = round(a["bytes"] / a["sec"] / 1e9, 1)
             ent["frac_hbm_peak"] = round(a["bytes"] / a["sec"] / 1e9 / HBM_PEAK_GBS, 4)
@@ -534,7 +543,7 @@ def main():
 
     out = {
         "metric": "%s grouped-GEMM TFLOPS (%s, quantisers inside the timed step)"
-                  % ("FP8 tensor-wise" if spec.get("tensorwise") else "MXFP8", "fwd+dgrad+wgrad" if spec.get("wgrad", True) else "fwd+dgrad"),
+                  % ("FP8 tensor-wise" if spec.get("tensorwise") else "MXFP4" if spec.get("act_fp4") else "MXFP8", "fwd+dgrad+wgrad" if spec.get("wgrad", True) else "fwd+dgrad"),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -544,7 +553,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"]
+        "dtype": "mxfp4_e2m1 (E8M0 block scales) for every operand, fp32 accumulate" if spec.get("act_fp4")
+                 else "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"]
                  else "fp8 e4m3 forward / e5m2 gradients, one fp32 scale per tensor, fp32 accumulate" if spec.get("tensorwise")
                  else "mxfp8_e4m3 (E8M0 block scales), fp32 accumulate",
         "data": "synthetic (seeded, generated on the GPU; random-init weights N(0,0.02))",
@@ -556,9 +566,9 @@ def main():
             "gemms_nk": [[n, k] for (_, _, _, k, n) in layers],
             "flops_per_step": flops_step,
         },
-        "frac_fp8_mfma_peak_whole_step": round(value / FP8_PEAK_TFLOPS, 4),
+        ("frac_fp4_mfma_peak_whole_step" if act_fp4 else "frac_fp8_mfma_peak_whole_step"): round(value / peak, 4),
         "gemm_only_TFLOP/s": round(gemm_flops / gemm_sec / 1e12, 2),
-        "gemm_only_frac_fp8_mfma_peak": round(gemm_flops / gemm_sec / 1e12 / FP8_PEAK_TFLOPS, 4),
+        ("gemm_only_frac_fp4_mfma_peak" if act_fp4 else "gemm_only_frac_fp8_mfma_peak"): round(gemm_flops / gemm_sec / 1e12 / peak, 4),
         "wgrad_overlaps_dgrad": not args.no_wgrad_overlap,
         "kernels_note": "per-kernel figures: separate pass of %d steps after the timed region, wgrad serialised behind dgrad" % kernel_steps,
         "kernels": kernels,
@@ -586,8 +596,9 @@ def main():
     if not args.no_gemm_calibration:
         out["hbm_stream_calibration"]["quantizer_traffic_twin"] = quantizer_twin(dev)
     if not args.no_gemm_calibration:
-        out["mfma_calibration"] = cal = gemm_calibration(spec["fp4"], dev)
-        ceiling = cal.get("mfma_only_loop_fp8_x_fp4_TFLOP/s" if spec["fp4"] else "mfma_only_loop_fp8_x_fp8_TFLOP/s")
+        out["mfma_calibration"] = cal = gemm_calibration(spec["fp4"], dev, act_fp4)
+        ceiling = cal.get("mfma_only_loop_fp4_x_fp4_TFLOP/s" if act_fp4 else
+                          "mfma_only_loop_fp8_x_fp4_TFLOP/s" if spec["fp4"] else "mfma_only_loop_fp8_x_fp8_TFLOP/s")
         for name, entry in kernels.items():
             if "gemm" in name and "TFLOP/s" in entry and ceiling:
                 entry["frac_of_mfma_only_loop"] = round(entry["TFLOP/s"] / ceiling, 4)

@@ -103,13 +103,18 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
  *                  row-major layout.  The GEMM entry points take such operands with MXL_GF_KCHUNK.  This is
  *                  the role the reference's pre-shuffled layouts play for its kernels (use_preshuffle,
  *                  primus_turbo_mxfp4_local.py:184-198); the arrangement itself is this library's own.
- *   MXL_QF_KSTEP   K-step-major layout of codes AND scales for both copies (FP8 formats only; excludes
+ *   MXL_QF_KSTEP   K-step-major layout of codes AND scales for both copies (excludes
  *                  MXL_QF_KCHUNK): codes [ld / 64][rows][64] -- the 64 elements one MFMA K step consumes --
  *                  and scales [ceil(ld / 512)][rows][16], i.e. the 16 scale bytes (8 K steps) of a row stay
  *                  together and consecutive rows follow each other.  Every request of the ring GEMM kernel
  *                  (MXL_GF_KSTEP) then reads whole consecutive cache lines: 64 rows of a K step are 4 KiB,
  *                  the scales of 256 rows for 8 K steps are 4 KiB.  Needs row_ld % 128 == 0; a scale array
  *                  holds ceil(ld / 512) * rows * 16 bytes (bytes past ld / 32 of a row are not written).
+ *                  E2M1 codes: an activation copy is written in steps of 128 elements, [ld / 128][rows][64 bytes]
+ *                  (the byte geometry of an FP8 copy; the operand format of the FP4 x FP4 ring GEMM), scales as
+ *                  above.  A weight (mxl_quantize_weight_2d_ex) is written in steps of 64 elements,
+ *                  [ld / 64][rows][32 bytes], the partner of FP8 activations, unless MXL_QF_KSTEP128 is set too:
+ *                  then in steps of 128 elements like the activations, the partner of E2M1 activations.
  *
  * and, for fmt = MXL_FMT_E2M1 only, the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
  * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288):
@@ -136,6 +141,7 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
 #define MXL_QF_RHT_COL 2u
 #define MXL_QF_KCHUNK 4u
 #define MXL_QF_KSTEP 8u
+#define MXL_QF_KSTEP128 16u
 int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                     const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                     void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);
@@ -203,8 +209,9 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * token width in wgrad).  Scales stay row-major.  Same results bit for bit; an operand must stay below 4 GiB. */
 #define MXL_GF_KCHUNK 1u
 /* MXL_GF_KSTEP (instead of MXL_GF_KCHUNK): codes and scales of both operands are K-step-major, as written by the
- * quantisers with MXL_QF_KSTEP.  FP8-format operands, at most 128 groups, bf16 output (no MXL_GF_ACCUM_F32);
- * anything else returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
+ * quantisers with MXL_QF_KSTEP.  FP8-format operands, FP8 rows against E2M1 weights in 64-element steps (forward /
+ * dgrad), or E2M1 against E2M1 in 128-element steps (MXL_QF_KSTEP128 weights); at most 128 groups, bf16 output (no
+ * MXL_GF_ACCUM_F32); anything else returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
  * With either layout flag the kernels request whole 256-row tiles of a K chunk: a code or scale array whose row count
  * is not a multiple of 256 must be followed by 32 KiB of readable memory (the values read there are never used). */
 #define MXL_GF_KSTEP 4u

@@ -622,15 +622,21 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 template <int AFMT, int BFMT, int MODE, bool ALPHA>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
-    static_assert(AFMT != kFmtE2M1, "the row operand is FP8");
-    static_assert(BFMT != kFmtE2M1 || (MODE == MODE_FWD && !ALPHA), "an E2M1 weight operand: forward / dgrad of the MX recipe");
-    constexpr bool B4 = BFMT == kFmtE2M1;             // the weight operand is FP4: 32 bytes per row and K step
+    // F44: both operands FP4, stored like FP8 operands byte for byte -- 64-byte rows per K step, which then hold 128
+    // elements: a step is two MFMA K steps (the low and the high half of every fragment register group), scale panels
+    // cover 4 steps instead of 8, and a contraction range may be an odd number of steps.
+    constexpr bool F44 = AFMT == kFmtE2M1 && BFMT == kFmtE2M1;
+    static_assert(AFMT != kFmtE2M1 || (F44 && !ALPHA), "an FP4 row operand needs an FP4 weight operand (MX recipe)");
+    static_assert(BFMT != kFmtE2M1 || F44 || (MODE == MODE_FWD && !ALPHA), "an E2M1 weight operand against FP8 rows: forward / dgrad of the MX recipe");
+    constexpr bool B4 = BFMT == kFmtE2M1 && !F44;     // FP4 weights against FP8 rows: 32 bytes per row and K step
+    constexpr int KS = F44 ? 2 * BK : BK;             // elements of the contraction per step
+    constexpr int PSTEPS = 512 / KS;                  // steps per scale panel
     constexpr int B_ROW = B4 ? BK / 2 : BK;           // bytes of a row of b in a K step
     constexpr int ROUNDS = B4 ? 6 : 8;                // load rounds of 4 KiB per K step: 4 of a, 2 or 4 of b
     constexpr int A_BYTES = 256 * BK;                 // 16 KiB
     constexpr int STAGE = RING_STAGE;
     constexpr int PANEL = RING_PANEL;
-    constexpr int CB = B4 ? 4 : BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE5M2 ? 1 : 0;
+    constexpr int CB = BFMT == kFmtE2M1 ? 4 : BFMT == kFmtE5M2 ? 1 : 0, BL = F44 ? 4 : AFMT == kFmtE5M2 ? 1 : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* panels = smem + RING_SLOTS * STAGE;
     int* pre_tiles = (int*)(panels + RING_PANEL_BUFS * 2 * PANEL);
@@ -736,7 +742,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         uint32_t ca0, cb0;         // byte offset of the first K step of each operand
         uint32_t pa0, pb0;         // byte offset of the scale panel of the first K step
         uint32_t cal, cbl;         // byte offset of the LAST K step of the contraction range (requests never pass it)
-        int nst, nst_real;         // K steps of 64 to run (>= 4, even) and how many of them multiply (2 or nst)
+        int nst, nst_real;         // K steps to run (>= 4, even) and how many of them multiply (the first nst_real)
         int m_valid, n_valid;
         int64_t c_off;
     };
@@ -784,15 +790,16 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         const int64_t n0 = (int64_t)pid_n * BN;
         d.n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
         d.c_off = c_row0 * p.n + n0;
-        const int nreal = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BK));   // even: the range is a multiple of 128
+        // the range is a multiple of 128 elements: an even number of steps, except with FP4 rows (one step each)
+        const int nreal = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / KS));
         d.nst_real = nreal;
-        d.nst = nreal < 4 ? 4 : nreal;
+        d.nst = nreal < 4 ? 4 : nreal + (nreal & 1);
         // descriptors anchored at the tile's first row inside K step 0 / panel 0; readable up to the operand's end
-        d.ra = make_rsrc(p.a + a_row0 * BK, a_rows_total * p.k - a_row0 * BK);
-        d.rb = make_rsrc(p.b + b_row0 * B_ROW, b_rows_total * (p.k / BK) * B_ROW - b_row0 * B_ROW);
+        d.ra = make_rsrc(p.a + a_row0 * BK, a_rows_total * (p.k / KS) * BK - a_row0 * BK);
+        d.rb = make_rsrc(p.b + b_row0 * B_ROW, b_rows_total * (p.k / KS) * B_ROW - b_row0 * B_ROW);
         d.rsa = make_rsrc(p.sa + a_row0 * 16, a_rows_total * n_panels * 16 - a_row0 * 16);
         d.rsb = make_rsrc(p.sb + b_row0 * 16, b_rows_total * n_panels * 16 - b_row0 * 16);
-        const uint32_t st0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(k0 / BK));
+        const uint32_t st0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(k0 / KS));
         d.ca0 = st0 * a_cstride;
         d.cb0 = st0 * b_cstride;
         d.cal = d.ca0 + (uint32_t)(nreal - 1) * a_cstride;
@@ -844,7 +851,11 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     auto next3 = [](int b) { return b == 2 ? 0 : b + 1; };
 
 #define MXL_MFMA(F, I, J) \
-    do { if (MF) acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I]); } while (0)
+    do { if (MF) { \
+             acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I]); \
+             if (F44) acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4( \
+                 __builtin_shufflevector(F.b[J], F.b[J], 4, 5, 6, 7, 4, 5, 6, 7), __builtin_shufflevector(F.a[I], F.a[I], 4, 5, 6, 7, 4, 5, 6, 7), \
+                 acc[I][J], CB, BL, 1, F.sb[J], 1, F.sa[I]); } } while (0)
 #define MXL_PIN __builtin_amdgcn_sched_barrier(0)
     // fragment (+ scale byte) reads of the K step in ring slot at `sn`, panel bytes at `pan`
 #define MXL_RD_A(F, I) \
@@ -977,13 +988,13 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             MXL_PIN;
             // bookkeeping between the barrier and the first read: panel of the next step, stream hand-over
             const int s1 = s + 1;
-            if ((s1 & 7) == 0 && s1 < nst) {
+            if ((s1 & (PSTEPS - 1)) == 0 && s1 < nst) {
                 pb_rd = next3(pb_rd);
                 MXL_RD_PANEL(panels + pb_rd * 2 * PANEL);
             }
             if (!LAST) group_begin();
             const uint8_t* sn = smem + ((gs + 1) & 3) * STAGE;
-            const int psh = 8 * (s1 & 7);
+            const int psh = (64 / PSTEPS) * (s1 & (PSTEPS - 1));   // FP4 rows: a step owns two bytes, the MFMAs pick with op_sel
             MXL_PIN;
             MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(E0{}, slot_new); MXL_PIN;
             MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1);  MXL_PIN;
@@ -1003,30 +1014,32 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         using P1 = std::integral_constant<int, 1>;
         using Yes = std::integral_constant<bool, true>;
         using No = std::integral_constant<bool, false>;
-        if (nst_real >= 4) {
+        if (nst_real >= 3) {
             for (int s = 0; s < nst - 2; s += 2) {
                 if (s == nst - 4) {
                     // the request stream moves on to the workgroup's next tile: its scale panel 0 first
                     pb_is = next3(pb_is);
                     issue_s(dn, 0, pb_is);
                     stream_enter(dn);
-                } else if ((s & 7) == 4 && s + 4 < nst) {
+                } else if ((s & (PSTEPS - 1)) == PSTEPS - 4 && s + 4 < nst) {
                     // this tile's next scale panel (K steps s + 4 ...): first read three barriers from here
                     pb_is = next3(pb_is);
-                    issue_s(d, (s >> 3) + 1, pb_is);
+                    issue_s(d, (s + 4) / PSTEPS, pb_is);
                 }
                 kstep(P0{}, Yes{}, No{}, s, f0, f1);
                 kstep(P1{}, Yes{}, No{}, s + 1, f1, f0);
             }
             kstep(P0{}, Yes{}, No{}, nst - 2, f0, f1);
-            kstep(P1{}, Yes{}, Yes{}, nst - 1, f1, f0);
+            if (!F44 || nst_real == nst) kstep(P1{}, Yes{}, Yes{}, nst - 1, f1, f0);
+            else kstep(P1{}, No{}, Yes{}, nst - 1, f1, f0);          // an odd range: the padding step does not multiply
         } else {
-            // a contraction range of two steps: four steps run, the last two without multiplying
+            // a contraction range of one or two steps: four steps run, the others without multiplying
             pb_is = next3(pb_is);
             issue_s(dn, 0, pb_is);
             stream_enter(dn);
             kstep(P0{}, Yes{}, No{}, 0, f0, f1);
-            kstep(P1{}, Yes{}, No{}, 1, f1, f0);
+            if (!F44 || nst_real == 2) kstep(P1{}, Yes{}, No{}, 1, f1, f0);
+            else kstep(P1{}, No{}, No{}, 1, f1, f0);
             kstep(P0{}, No{}, No{}, 2, f0, f1);
             kstep(P1{}, No{}, Yes{}, 3, f1, f0);
         }
@@ -1175,7 +1188,8 @@ template <int MODE>
 static bool ring_serves(int afmt, int bfmt, const GemmArgs& a) {
     if (a.num_groups > RING_MAX_GROUPS) return false;
     if (a.alpha_a != nullptr) return bfmt == MXL_FMT_E4M3 && (afmt == MXL_FMT_E4M3 || afmt == MXL_FMT_E5M2);
-    // MX: E4M3 x E4M3, and in the forward / dgrad GEMM E4M3 activations against E2M1 weights
+    // MX: E4M3 x E4M3, in the forward / dgrad GEMM E4M3 activations against E2M1 weights, and E2M1 x E2M1
+    if (afmt == MXL_FMT_E2M1) return bfmt == MXL_FMT_E2M1;
     return afmt == MXL_FMT_E4M3 && (bfmt == MXL_FMT_E4M3 || (bfmt == MXL_FMT_E2M1 && MODE == MODE_FWD));
 }
 template <int MODE>
@@ -1184,6 +1198,7 @@ static int dispatch_gemm_ring(int afmt, int bfmt, const GemmArgs& a, int64_t max
         if (afmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
         return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
     }
+    if (afmt == MXL_FMT_E2M1) return launch_gemm_ring<MXL_FMT_E2M1, MXL_FMT_E2M1, MODE, false>(a, max_tiles, st);
     if constexpr (MODE == MODE_FWD) {
         if (bfmt == MXL_FMT_E2M1) return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E2M1, MODE_FWD, false>(a, max_tiles, st);
     }

@@ -475,7 +475,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         const int64_t nb = (a.row_ld - col0) / 32;  // valid blocks in this tile row
         uint8_t* dst = a.s_row + (src_row0 + t) * sld + col0 / 32;
         const uint32_t v = srow_tile[t];
-        if (a.kchunk == 2) {
+        if (a.kchunk >= 2) {
             store_panel_scales(a.s_row + ((int64_t)(ct >> 2) * a.chunk_rows_row + src_row0 + t) * 16, ct & 3, v);
         } else if (nb >= 4 && (sld & 3) == 0) {
             *(uint32_t*)dst = v;
@@ -490,7 +490,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             uint8_t* dst = a.s_colT + (out_rows_base + col0 + t) * (a.W / 32) + m0 / 32;
             const uint32_t v = scol_tile[t];
             const int64_t nb = (a.W - m0) / 32;
-            if (a.kchunk == 2) {
+            if (a.kchunk >= 2) {
                 const int64_t mt = seg_tile >= 0 ? (int64_t)seg_tile : m0 / QT;
                 store_panel_scales(a.s_colT + ((seg_pan0 + mt / 4) * a.chunk_rows_col + out_rows_base + col0 + t) * 16, (int)(mt & 3), v);
             } else if (nb >= 4 && ((a.W / 32) & 3) == 0) {
@@ -688,10 +688,12 @@ extern "C" int64_t mxl_padded_width(int64_t total_rows, int num_groups) {
     return (total_rows + (int64_t)(MXL_SEG_ALIGN - 1) * num_groups) / MXL_SEG_ALIGN * MXL_SEG_ALIGN;
 }
 
-// code layout selected by the flags: 0 row-major, 1 K-chunk-major, 2 K-step-major, -1 both requested
+// code layout selected by the flags: 0 row-major, 1 K-chunk-major, 2 K-step-major, 3 K-step-major with steps of 128
+// elements (E2M1 only: 64-byte rows, i.e. K-chunk-major codes with K-step-major scale panels), -1 contradictory flags
 static int qf_layout(uint32_t flags) {
     if ((flags & MXL_QF_KCHUNK) && (flags & MXL_QF_KSTEP)) return -1;
-    return (flags & MXL_QF_KSTEP) ? 2 : (flags & MXL_QF_KCHUNK) ? 1 : 0;
+    if ((flags & MXL_QF_KSTEP128) && !(flags & MXL_QF_KSTEP)) return -1;
+    return (flags & MXL_QF_KSTEP128) ? 3 : (flags & MXL_QF_KSTEP) ? 2 : (flags & MXL_QF_KCHUNK) ? 1 : 0;
 }
 
 static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
@@ -701,7 +703,9 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
                        int kchunk = 0, const void* norm_w = nullptr, const void* tensor_amax = nullptr,
                        void* scale_inv_out = nullptr) {
     if (row_ld == 0) row_ld = cols;
-    if (kchunk < 0 || (kchunk == 2 && fmt == MXL_FMT_E2M1)) return MXL_EINVAL;   // both layout flags; activations: K-step-major is FP8 only
+    if (kchunk < 0) return MXL_EINVAL;                  // contradictory layout flags
+    if (kchunk == 2 && fmt == MXL_FMT_E2M1) kchunk = 3;  // E2M1 activations: the K step is 128 elements (64-byte rows)
+    if (kchunk == 3 && fmt != MXL_FMT_E2M1) return MXL_EINVAL;
     if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
     if ((sr || rht) && (fmt != MXL_FMT_E2M1 || act >= 0)) return MXL_EINVAL;
     if (rht && !q_colT) return MXL_EINVAL;   // the transform belongs to the transposed copy
@@ -761,7 +765,7 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
 extern "C" int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                                const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                                void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream) {
-    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT,
                        s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, (flags & MXL_QF_SR) != 0, sr_seed,
                        (flags & MXL_QF_RHT_COL) != 0, rht_signs, qf_layout(flags));
@@ -774,7 +778,7 @@ extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int
     if (act != MXL_ACT_SILU && act != MXL_ACT_GELU) return MXL_EINVAL;
     if (probs_dtype != MXL_PROBS_F32 && probs_dtype != MXL_PROBS_BF16) return MXL_EINVAL;
     if (rows > 0 && !probs) return MXL_EINVAL;
-    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, f, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT, act,
                        probs, probs_dtype, row_mask, stream, false, 0, false, 0, qf_layout(flags));
 }
@@ -783,7 +787,7 @@ extern "C" int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, cons
                                     int64_t row_ld, int fmt, int scale_mode, const int64_t* group_lens, int num_groups,
                                     void* q_row, void* s_row, void* q_colT, void* s_colT, uint32_t flags, void* stream) {
     if (!w_bf16 || (rows > 0 && !rstd_f32)) return MXL_EINVAL;
-    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, k, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
                        PRO_RMSNORM, rstd_f32, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
                        qf_layout(flags), w_bf16);
@@ -794,7 +798,7 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
                               void* stream, const void* tensor_amax = nullptr, void* scale_inv_out = nullptr) {
     if (k_ld == 0) k_ld = k;
     if (n_ld == 0) n_ld = n;
-    if (kchunk < 0) return MXL_EINVAL;
+    if (kchunk < 0 || (kchunk == 3 && fmt != MXL_FMT_E2M1)) return MXL_EINVAL;
     if (kchunk && ((q_row && k_ld % QT != 0) || (q_colT && n_ld % QT != 0))) return MXL_EINVAL;   // whole chunks
     if (k_ld < k || n_ld < n || k_ld % MXL_BLOCK != 0 || n_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if (n_ld > (n + QT - 1) / QT * QT) return MXL_EINVAL;  // padding of the transposed copy stays inside the last tile
@@ -840,7 +844,7 @@ extern "C" int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t
 extern "C" int mxl_quantize_weight_2d_ex(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
                                          int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT,
                                          void* s_colT, uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_weight_2d(w_bf16, batch, n, k, k_ld, n_ld, fmt, scale_mode, q_row, s_row, q_colT, s_colT,
                               qf_layout(flags), stream);
 }

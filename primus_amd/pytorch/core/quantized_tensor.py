@@ -23,6 +23,7 @@ from .. import kernels as K
 from .low_precision import (
     Float4QuantConfig,
     Float8QuantConfig,
+    Format,
     MXScalingRecipe,
     ScaleMode,
     ScalingGranularity,
@@ -68,7 +69,7 @@ class QuantizedTensor(torch.Tensor):
         # tensor-wise scaled payload: float32 reciprocal scale of the whole tensor (one element, on the device);
         # ``scales`` then holds unit E8M0 bytes, which only make the codes acceptable to the GEMM kernels
         self._tensor_scale_inv = tensor_scale_inv
-        self._kchunk = 2 if (kchunk == 2 and kchunk is not True) else int(bool(kchunk))
+        self._kchunk = K._layout(kchunk)
         self._codes = codes
         self._scales = scales
         self._axis = axis
@@ -112,11 +113,12 @@ class QuantizedTensor(torch.Tensor):
 
     def rowmajor_scales(self) -> torch.Tensor:
         """The scales as ``[..., rows, ld / 32]`` whatever layout they are stored in (a copy if K-step-major)."""
-        if self._kchunk != 2:
+        if self._kchunk < K.LAYOUT_KSTEP:
             return self._scales
         if self._segment_lens is not None:
             raise NotImplementedError("row-major scales of a K-step-major copy that is split into groups")
-        blocks = self._codes.shape[0] * self._codes.shape[2] // _lib.BLOCK
+        per = 2 if self.fmt == _lib.FMT_E2M1 else 1   # elements per code byte
+        blocks = self._codes.shape[0] * self._codes.shape[2] * per // _lib.BLOCK
         flat = K.unpanel(self._scales.view(torch.uint8), blocks).view(self._scales.dtype)
         return flat.view(tuple(self.shape[:-1]) + (blocks,))
 
@@ -293,7 +295,8 @@ def create_quantized_weight(
         return row, col
     if kchunk is None:
         kchunk = K.pick_layout(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1, w.shape[-2], w.shape[-1],
-                               fp8=fmt != _lib.FMT_E2M1)
+                               fp8=fmt != _lib.FMT_E2M1,
+                               fp4=fmt == _lib.FMT_E2M1 and getattr(quant_config, "activation_format", None) == Format.E2M1_X2)
     q_row, s_row, q_col, s_col = K.quantize_mx_weight_2d_impl(
         w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN,
         kchunk=kchunk,

@@ -89,23 +89,36 @@ PANEL = 512
 #   2          K-step-major codes [ld / 64, rows, 64] and scales [panels, rows, 16] (FP8 formats only): what the
 #              ring GEMM kernel reads; a transposed copy that is split into groups has its scale panels restart
 #              at every group (ceil(ld / 512) + groups + 1 panels are allocated)
-LAYOUT_ROWMAJOR, LAYOUT_KCHUNK, LAYOUT_KSTEP = 0, 1, 2
+#   3          the K-step-major layout of E2M1 operands that meet E2M1 operands: steps of 128 elements, i.e. codes
+#              [ld / 128, rows, 64 bytes] (the bytes of layout 1) with the scale panels of layout 2
+LAYOUT_ROWMAJOR, LAYOUT_KCHUNK, LAYOUT_KSTEP, LAYOUT_KSTEP128 = 0, 1, 2, 3
 RING_MAX_GROUPS = 128   # the ring GEMM kernel keeps its group tables for at most this many groups
 
 
 def _layout(kchunk) -> int:
-    return LAYOUT_KSTEP if (kchunk == 2 and kchunk is not True) else (LAYOUT_KCHUNK if kchunk else LAYOUT_ROWMAJOR)
+    if kchunk is True or kchunk is False or kchunk is None:
+        return LAYOUT_KCHUNK if kchunk else LAYOUT_ROWMAJOR
+    if int(kchunk) not in (0, 1, 2, 3):
+        raise ValueError(f"unknown operand layout {kchunk!r}")
+    return int(kchunk)
+
+
+def _paneled(kchunk) -> bool:
+    """Whether the layout keeps its scales in K-step-major panels."""
+    return _layout(kchunk) >= LAYOUT_KSTEP
 
 
 def _code_shape(rows: int, ld: int, per: int, kchunk):
     lay = _layout(kchunk)
+    if lay == LAYOUT_KSTEP128 and per != 2:
+        raise ValueError("the 128-element K-step layout holds E2M1 codes only")
     if lay == LAYOUT_KSTEP:
         return (ld // KSTEP, rows, KSTEP // per)
     return (ld // KCHUNK, rows, KCHUNK // per) if lay else (rows, ld // per)
 
 
 def _scale_shape(rows: int, ld: int, kchunk, groups: int = 0):
-    if _layout(kchunk) == LAYOUT_KSTEP:
+    if _paneled(kchunk):
         return ((ld + PANEL - 1) // PANEL + (groups + 1 if groups else 0), rows, 16)
     return (rows, ld // BLOCK)
 
@@ -126,21 +139,23 @@ def _empty_tail(shape, dtype, device):
 
 
 def _qflag(kchunk) -> int:
-    return (0, _lib.QF_KCHUNK, _lib.QF_KSTEP)[_layout(kchunk)]
+    return (0, _lib.QF_KCHUNK, _lib.QF_KSTEP, _lib.QF_KSTEP | _lib.QF_KSTEP128)[_layout(kchunk)]
 
 
 def _gflag(kchunk) -> int:
-    return (0, _lib.GF_KCHUNK, _lib.GF_KSTEP)[_layout(kchunk)]
+    return (0, _lib.GF_KCHUNK, _lib.GF_KSTEP, _lib.GF_KSTEP)[_layout(kchunk)]
 
 
-def pick_layout(groups: int, n: int, k: int, rows: int = 0, fp8: bool = True, accum: bool = False) -> int:
+def pick_layout(groups: int, n: int, k: int, rows: int = 0, fp8: bool = True, accum: bool = False,
+                fp4: bool = False) -> int:
     """Layout the differentiable operators store their quantised operands in: K-step-major when every operand
-    is FP8, the groups fit the ring kernel and the weight gradient is not accumulated in the GEMM; otherwise
-    K-chunk-major; row-major when the layouts are switched off or an operand reaches 4 GiB."""
+    is FP8 (``fp8``; steps of 64 elements) or every operand is E2M1 (``fp4``; steps of 128 elements), the groups
+    fit the ring kernel and the weight gradient is not accumulated in the GEMM; otherwise K-chunk-major;
+    row-major when the layouts are switched off or an operand reaches 4 GiB."""
     if not (kchunk_default() and kchunk_fits(groups, n, k, rows)):
         return LAYOUT_ROWMAJOR
-    if fp8 and groups <= RING_MAX_GROUPS and not accum and _kstep_default:
-        return LAYOUT_KSTEP
+    if (fp8 or fp4) and groups <= RING_MAX_GROUPS and not accum and _kstep_default:
+        return LAYOUT_KSTEP if fp8 else LAYOUT_KSTEP128
     return LAYOUT_KCHUNK
 
 
@@ -372,12 +387,12 @@ def quantize_mx_weight_2d_impl(
     if rowwise:
         shape = _code_shape(batch * n, k_ld, per, kchunk) if kchunk else lead + (n, k_ld // per)
         q_row = _empty_tail(shape, dtype=torch.uint8, device=dev)
-        sshape = _scale_shape(batch * n, k_ld, kchunk) if _layout(kchunk) == LAYOUT_KSTEP else lead + (n, k_ld // BLOCK)
+        sshape = _scale_shape(batch * n, k_ld, kchunk) if _paneled(kchunk) else lead + (n, k_ld // BLOCK)
         s_row = _empty_tail(sshape, dtype=torch.uint8, device=dev)
     if colwise:
         shape = _code_shape(batch * k, n_ld, per, kchunk) if kchunk else lead + (k, n_ld // per)
         q_col = _empty_tail(shape, dtype=torch.uint8, device=dev)
-        sshape = _scale_shape(batch * k, n_ld, kchunk) if _layout(kchunk) == LAYOUT_KSTEP else lead + (k, n_ld // BLOCK)
+        sshape = _scale_shape(batch * k, n_ld, kchunk) if _paneled(kchunk) else lead + (k, n_ld // BLOCK)
         s_col = _empty_tail(sshape, dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_2d_ex(
@@ -438,14 +453,14 @@ def _check_out_dtype(out_dtype) -> None:
 
 def _chunked_dims(codes: torch.Tensor, fmt: int, kchunk=True):
     """(rows, k) of K-chunk-major codes [k / 128, rows, 128] or K-step-major codes [k / 64, rows, 64]."""
-    step = KSTEP if _layout(kchunk) == LAYOUT_KSTEP else KCHUNK
+    step = KSTEP if _layout(kchunk) == LAYOUT_KSTEP else KCHUNK   # layout 3: 128-element steps
     if codes.dim() != 3 or codes.shape[2] * _per_byte(fmt) != step or not codes.is_contiguous():
         raise ValueError(f"chunked codes must be a contiguous [k / {step}, rows, {step}-element] tensor")
     return codes.shape[1], codes.shape[0] * step
 
 
 def _check_scales(scales: torch.Tensor, rows: int, k: int, kchunk, what: str) -> None:
-    if _layout(kchunk) == LAYOUT_KSTEP:
+    if _paneled(kchunk):
         ok = scales.dim() == 3 and scales.shape[1] == rows and scales.shape[2] == 16 and scales.shape[0] * PANEL >= k
     else:
         ok = scales.numel() == rows * (k // BLOCK) and scales.shape[-1] == k // BLOCK
@@ -459,7 +474,7 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=Fal
     _require_cuda(a, a_scale, b, b_scale)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
     if kchunk:
-        return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _layout(kchunk) == LAYOUT_KSTEP else b_scale.unsqueeze(0),
+        return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _paneled(kchunk) else b_scale.unsqueeze(0),
                                        None, kchunk=kchunk)
     _check_contraction(a.shape[-1] * _per_byte(a_fmt), b.shape[-1] * _per_byte(b_fmt))
     a, a_scale, k = _pad_k(a, a_scale, a_fmt)
@@ -486,7 +501,7 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
         total_m, k = _chunked_dims(a, a_fmt, kchunk)
         b_rows, kb = _chunked_dims(b, b_fmt, kchunk)
         groups = max(G, 1)
-        if _layout(kchunk) == LAYOUT_KSTEP:
+        if _paneled(kchunk):
             if b_rows % groups:
                 raise ValueError("the rows of b do not split into num_groups weights")
             n = b_rows // groups
@@ -552,7 +567,7 @@ def grouped_gemm_mx_wgrad_impl(a_t, a_t_scale, b_t, b_t_scale, group_lens, total
         n, k = a_t.shape[0], b_t.shape[0]
         if a_t.shape[1] * _per_byte(a_fmt) != W or b_t.shape[1] * _per_byte(b_fmt) != W:
             raise ValueError(f"transposed operands must have padded width {W}")
-    if _layout(kchunk) == LAYOUT_KSTEP:
+    if _paneled(kchunk):
         for sc, r in ((a_t_scale, n), (b_t_scale, k)):
             if tuple(sc.shape) != _scale_shape(r, W, kchunk, G) or not sc.is_contiguous():
                 raise ValueError("K-step-major scales of the transposed operands must be [panels, rows, 16]")
@@ -749,7 +764,7 @@ def quantize_weight_tensorwise_impl(w, fmt: int, *, rowwise: bool = True, colwis
     scale_inv = torch.empty((1,), dtype=torch.float32, device=dev)
     k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     q_row = s_row = q_col = s_col = None
-    kstep = _layout(kchunk) == LAYOUT_KSTEP
+    kstep = _paneled(kchunk)
     if rowwise:
         q_row = _empty_tail(_code_shape(batch * n, k_ld, 1, kchunk) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
         s_row = _empty_tail(_scale_shape(batch * n, k_ld, kchunk) if kstep else lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
@@ -783,7 +798,7 @@ def gemm_tw_nt_impl(a, a_unit, a_scale_inv, b, b_unit, b_scale_inv, group_lens=N
     G = _check_group_lens(group_lens, a.device)
     groups = max(G, 1)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
-    kstep = _layout(kchunk) == LAYOUT_KSTEP
+    kstep = _paneled(kchunk)
     if kchunk:
         total_m, k = _chunked_dims(a, a_fmt, kchunk)
         b_rows, kb = _chunked_dims(b, b_fmt, kchunk)
@@ -823,7 +838,7 @@ def gemm_tw_wgrad_impl(a_t, a_t_unit, a_scale_inv, b_t, b_t_unit, b_scale_inv, g
     G = _check_group_lens(group_lens, a_t.device)
     a_fmt, b_fmt = fmt_of(a_t), fmt_of(b_t)
     W = padded_width(total_m, G)
-    kstep = _layout(kchunk) == LAYOUT_KSTEP
+    kstep = _paneled(kchunk)
     if kchunk:
         (n, wa), (k, wb) = _chunked_dims(a_t, a_fmt, kchunk), _chunked_dims(b_t, b_fmt, kchunk)
     else:

@@ -120,19 +120,23 @@ def _fusable(target) -> bool:
 def _cached_codes(q: QuantizedTensor, kchunk) -> torch.Tensor:
     """Codes of a cached weight copy in the layout this call's GEMMs use.  A chunked cache is
     rearranged (one pass over the weight) only when this call cannot use that layout."""
-    return q.codes if int(q.kchunk) == int(kchunk) else q.rowmajor_codes()
+    if int(q.kchunk) == int(kchunk) or (int(q.kchunk) == K.LAYOUT_KSTEP128 and int(kchunk) == K.LAYOUT_KCHUNK):
+        return q.codes          # the 128-element step layout stores its codes K-chunk-major
+    return q.rowmajor_codes()
 
 
 def _cached_scales(q: QuantizedTensor, kchunk) -> torch.Tensor:
     return q.scales if int(q.kchunk) == int(kchunk) else q.rowmajor_scales()
 
 
-def _cache_layout(b: QuantizedTensor, b_t, kc: int, fp8: bool, groups: int) -> int:
+def _cache_layout(b: QuantizedTensor, b_t, kc: int, fp8: bool, groups: int, fp4: bool = False) -> int:
     """Layout of a call on cached weight copies: the cache's own, row-major when the pair disagrees or
     this call cannot read that layout."""
     lay = int(b.kchunk) if (b_t is None or int(b_t.kchunk) == int(b.kchunk)) else 0
     if lay == K.LAYOUT_KSTEP and not (fp8 and groups <= K.RING_MAX_GROUPS):
         lay = 0
+    if lay == K.LAYOUT_KSTEP128 and not (fp4 and groups <= K.RING_MAX_GROUPS):
+        lay = K.LAYOUT_KCHUNK   # same codes; the scales are rearranged (1/16 of the bytes of the codes)
     return lay if kc else 0
 
 
@@ -154,13 +158,16 @@ class _MXLinearFunction(torch.autograd.Function):
         # Every operand of the three GEMMs is stored in one layout, K-chunk-major unless an operand is
         # too large for it (or the layout is switched off): same codes, same results, faster loads.
         groups = b.shape[0] if grouped else 1
-        # K-step-major operands (the ring kernel) for FP8 x FP8 only.  The ring kernel also takes FP8 activations against
+        # K-step-major operands (the ring kernel) for FP8 x FP8 and E2M1 x E2M1.  The ring kernel also takes FP8 activations against
         # FP4 weights, but at the shapes that recipe is used on (GPT-OSS: K = 2880, 46 K steps per tile, ragged row
         # tiles) the 2-slot kernel with its live-fragment variants is the faster one (2.04 against 1.89 PFLOP/s)
         fp8 = act_fmt != _lib.FMT_E2M1 and w_fmt != _lib.FMT_E2M1
-        kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, accum=accum is not None and _fusable(accum[0]))
+        # E2M1 x E2M1 runs on the ring kernel too, in steps of 128 elements (two MFMAs per step)
+        fp4 = act_fmt == _lib.FMT_E2M1 and w_fmt == _lib.FMT_E2M1
+        kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, fp4=fp4,
+                           accum=accum is not None and _fusable(accum[0]))
         if isinstance(b, QuantizedTensor):   # cached copies decide: the call uses the layout they are stored in
-            kc = _cache_layout(b, b_t, kc, fp8, groups)
+            kc = _cache_layout(b, b_t, kc, fp8, groups, fp4)
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
         # (row-wise copies are padded to the GEMM's K granularity, like the reference pads its
         # MXFP4 operands to 128: primus_turbo_mxfp4_local.py:119-124)

@@ -51,6 +51,39 @@ def test_weight_quantiser_kchunk_is_a_rearrangement(gpu, fmt, shape):
     assert _same(K.unchunk(b[2]), a[2].reshape(-1, a[2].shape[-1])) and _same(b[3], a[3])
 
 
+def test_quantisers_write_the_128_element_step_layout_of_e2m1(gpu):
+    """Layout 3 holds the codes of the K-chunk-major layout and the scale panels of the K-step-major one."""
+    from primus_amd.pytorch import kernels as K
+
+    lens, cols = [33, 0, 130, 1, 92, 600], 672
+    rows = sum(lens)
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(rows, cols, generator=g) * torch.logspace(-2, 2, cols)[None, :]).bfloat16().to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    a = K.quantize_mx_impl(x, 1, rowwise=True, colwise=True, group_lens=gl, kchunk=True)
+    b = K.quantize_mx_impl(x, 1, rowwise=True, colwise=True, group_lens=gl, kchunk=3)
+    assert _same(b[0], a[0]) and _same(b[2], a[2])
+    assert _same(K.unpanel(b[1].view(torch.uint8), a[1].shape[1]), a[1].view(torch.uint8))
+    # the transposed copy's panels restart at every group: compare group by group
+    W, off, pan = a[3].shape[1] * 32, 0, 0
+    s_col = b[3].view(torch.uint8)
+    for ln in lens:
+        seg = (ln + 127) // 128 * 128
+        npan = (seg // 128 + 3) // 4
+        if seg:
+            got = K.unpanel(s_col[pan:pan + npan], seg // 32)
+            assert torch.equal(got, a[3].view(torch.uint8)[:, off // 32:(off + seg) // 32])
+        off, pan = off + seg, pan + npan
+    w = (torch.randn(2, 416, 288, generator=g) * 0.05).bfloat16().to(gpu)
+    wa = K.quantize_mx_weight_2d_impl(w, 1, rowwise=True, colwise=True, kchunk=True)
+    wb = K.quantize_mx_weight_2d_impl(w, 1, rowwise=True, colwise=True, kchunk=3)
+    assert _same(wb[0], wa[0]) and _same(wb[2], wa[2])
+    assert _same(K.unpanel(wb[1].view(torch.uint8), wa[1].shape[-1]), wa[1].reshape(-1, wa[1].shape[-1]).view(torch.uint8))
+    assert _same(K.unpanel(wb[3].view(torch.uint8), wa[3].shape[-1]), wa[3].reshape(-1, wa[3].shape[-1]).view(torch.uint8))
+    with pytest.raises(ValueError):
+        K.quantize_mx_impl(x, 0, rowwise=True, colwise=False, kchunk=3)
+
+
 @pytest.mark.parametrize("activation", ["silu", "gelu"])
 def test_fused_activation_quantiser_kchunk(gpu, activation):
     from primus_amd.pytorch import kernels as K
@@ -82,13 +115,14 @@ def test_gemms_give_identical_results_on_either_layout(gpu, afmt, wfmt, lens, n,
     w = (torch.randn(G, n, k, generator=g) * 0.05).bfloat16().to(gpu)
     gl = None if lens is None else torch.tensor(lens, dtype=torch.int64, device=gpu)
     res = []
-    # 2: K-step-major codes and scales (the 4-slot ring kernel): FP8 activations against FP8 or FP4 weights
-    for kc in (False, True) + ((2,) if afmt == 0 else ()):
+    # 2: K-step-major codes and scales (the 4-slot ring kernel): FP8 activations against FP8 or FP4 weights;
+    # 3: the same with steps of 128 elements: E2M1 against E2M1 (1, 2, 3, 5, 8 and 16 steps per tile in these cases)
+    for kc in (False, True) + ((2,) if afmt == 0 else ()) + ((3,) if afmt == 1 and wfmt == 1 else ()):
         xq = K.quantize_mx_impl(x, afmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kc)
         dq = K.quantize_mx_impl(dy, afmt, rowwise=True, colwise=True, group_lens=gl, pad_to=128, kchunk=kc)
         wq = K.quantize_mx_weight_2d_impl(w, wfmt, rowwise=True, colwise=True, pad_to=128, kchunk=kc)
         if lens is None:
-            ws_row, ws_col = (wq[1], wq[3]) if kc == 2 else (wq[1][0], wq[3][0])
+            ws_row, ws_col = (wq[1], wq[3]) if kc in (2, 3) else (wq[1][0], wq[3][0])
             w_row = wq[0] if kc else wq[0][0]
             w_col = wq[2] if kc else wq[2][0]
             y = K.gemm_mx_nt_impl(xq[0], xq[1], w_row, ws_row, kchunk=kc)

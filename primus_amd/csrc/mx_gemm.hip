@@ -468,25 +468,32 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         // reading it; then the next tile's first requests go out and overlap with the epilogue.
         wait_vm<0>();
         __syncthreads();
-        const int m_valid = d.m_valid, n_valid = d.n_valid;
-        uint16_t* ctile = p.c + d.c_off;
+        // The tile's facts are uniform: moved to scalar registers they stay out of the vector registers' spills.  The
+        // lane number is taken afresh from the hardware, and every offset of the epilogue is rebuilt from it: computed in
+        // front of the tile loop those offsets would have to live through the main loop, where every register is taken,
+        // and would come back from scratch memory one dependent load after the other.
+        const int m_valid = __builtin_amdgcn_readfirstlane(d.m_valid), n_valid = __builtin_amdgcn_readfirstlane(d.n_valid);
+        const int64_t c_off = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(d.c_off >> 32)) << 32) |
+                                        (uint32_t)__builtin_amdgcn_readfirstlane((int)d.c_off));
+        auto lane_now = [] { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); };
+        uint16_t* ctile = p.c + c_off;
         // ACCUM: the old float32 values of the first 32-row block are requested before the next tile's operand
         // requests go out (memory returns in order per wave: behind them they would wait for 64 KiB of loads)
-        float* ctile32 = (float*)p.c + d.c_off;
+        float* ctile32 = (float*)p.c + c_off;
         const bool full_tile = (m_valid == BM) && (n_valid == BN);
         v4f old[ACCUM ? 2 : 1][ACCUM ? 16 : 1];
-        auto fetch_old = [&](int i, v4f* dst) {
+        auto fetch_old = [&](int i, v4f* dst, int el) {
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
-                    const int row = wm * 128 + i * 32 + 4 * u + (l >> 4), col = wn * 128 + (l & 15) * 4 + jj * 64;
+                    const int row = wm * 128 + i * 32 + 4 * u + (el >> 4), col = wn * 128 + (el & 15) * 4 + jj * 64;
                     dst[jj * 8 + u] = v4f{0.f, 0.f, 0.f, 0.f};
                     if (full_tile || (row < m_valid && col < n_valid))
                         dst[jj * 8 + u] = *(const v4f*)(ctile32 + (int64_t)row * p.n + col);
                 }
         };
-        if (ACCUM) fetch_old(0, old[0]);
+        if (ACCUM) fetch_old(0, old[0], lane_now());
         tile += nwg;
         // (past the last tile the requests are still sent, for the last tile again: nobody reads them)
         d = decode(tile < total_tiles ? tile : total_tiles - 1);
@@ -503,11 +510,13 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             // already writing
             constexpr int SP = (4 * 32 * 272 <= STAGE) ? 272 : 256;
             static_assert(4 * 32 * SP <= STAGE, "the epilogue patches must stay inside ring slot 1");
+            const int el = lane_now();     // taken behind the requests above: no register is held across them
+            const int elr = el & 31, eg = el >> 5;
             uint8_t* stg = smem + STAGE + w * (32 * SP);
-            uint8_t* wr = stg + lr * SP + 8 * g;                   // this lane's row while writing
-            const uint8_t* rd = stg + (l >> 4) * SP + (l & 15) * 16;  // this lane's 16 bytes while reading
-            const int rr = l >> 4, cc = wn * 128 + (l & 15) * 8;
-            const uint32_t lane_off = (uint32_t)((rr * (int)p.n + (l & 15) * 8) * 2);
+            uint8_t* wr = stg + elr * SP + 8 * eg;                   // this lane's row while writing
+            const uint8_t* rd = stg + (el >> 4) * SP + (el & 15) * 16;  // this lane's 16 bytes while reading
+            const int rr = el >> 4, cc = wn * 128 + (el & 15) * 8;
+            const uint32_t lane_off = (uint32_t)((rr * (int)p.n + (el & 15) * 8) * 2);
             const bool full = (m_valid == BM) && (n_valid == BN);
             float alpha = 1.f;
             if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
@@ -516,11 +525,11 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
                 // the same patch: a memory instruction covers 4 rows x 256 contiguous bytes.  The old values of
                 // a 32-row block (16 x 16 bytes per lane) are requested one block ahead, so their latency is
                 // covered by the staging and the stores of the block before.
-                uint8_t* wr32 = stg + lr * SP + 16 * g;
-                const int colq = wn * 128 + (l & 15) * 4;
+                uint8_t* wr32 = stg + elr * SP + 16 * eg;
+                const int colq = wn * 128 + (el & 15) * 4;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (i + 1 < 4) fetch_old(i + 1, old[(i + 1) & 1]);
+                    if (i + 1 < 4) fetch_old(i + 1, old[(i + 1) & 1], el);
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
@@ -774,22 +783,28 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             const int64_t g_row0 = pre_rows[grp], g_rows = pre_rows[grp + 1] - g_row0;
             const int64_t r = (int64_t)(pid_m - pre_tiles[grp]) * BM;
             a_row0 = g_row0 + r;
-            d.m_valid = (g_rows - r) < BM ? (int)(g_rows - r) : BM;
+            d.m_valid = __builtin_amdgcn_readfirstlane((g_rows - r) < BM ? (int)(g_rows - r) : BM);
             b_row0 = (int64_t)grp * p.n + (int64_t)pid_n * BN;
             c_row0 = a_row0;
             k0 = 0;
             k1 = p.k;
         } else {
             a_row0 = (int64_t)pid_m * BM;
-            d.m_valid = (p.m - a_row0) < BM ? (int)(p.m - a_row0) : BM;
+            d.m_valid = __builtin_amdgcn_readfirstlane((p.m - a_row0) < BM ? (int)(p.m - a_row0) : BM);
             b_row0 = (int64_t)pid_n * BN;
             c_row0 = (int64_t)grp * p.m + a_row0;
             k0 = pre_rows[grp];
             k1 = pre_rows[grp + 1];
         }
         const int64_t n0 = (int64_t)pid_n * BN;
-        d.n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
-        d.c_off = c_row0 * p.n + n0;
+        // the epilogue's tile facts are uniform: kept in scalar registers they survive the main loop without
+        // taking part in the vector register spills
+        d.n_valid = __builtin_amdgcn_readfirstlane((p.n - n0) < BN ? (int)(p.n - n0) : BN);
+        {
+            const int64_t off = c_row0 * p.n + n0;
+            d.c_off = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(off >> 32)) << 32) |
+                                (uint32_t)__builtin_amdgcn_readfirstlane((int)off));
+        }
         // the range is a multiple of 128 elements: an even number of steps, except with FP4 rows (one step each)
         const int nreal = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / KS));
         d.nst_real = nreal;
@@ -1053,48 +1068,63 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // contiguous bytes per instruction.  The patch is not padded (the four patches fill half a slot);
         // 16-byte pieces are XOR-swizzled by (row / 2) % 8 and the 8-byte halves swapped in rows 16-31:
         // conflict-free for the 8-byte writes (a lane owns a row) and the 16-byte reads (8 lanes per row).
+        // The lane's offsets into the patch and into the output tile are rebuilt here from the lane number, taken afresh
+        // from the hardware: computed once in front of the tile loop they would have to live through the main loop, where
+        // every register is taken, and would come back from scratch memory one dependent load after the other, each of
+        // them waiting for all operand requests in flight (measured: 5 of the epilogue's 6.5 us).
         {
+            const int lo = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            const int elr = lo & 31, eg = lo >> 5;
             const int m_valid = d.m_valid, n_valid = d.n_valid;
             uint16_t* ctile = p.c + d.c_off;
             uint8_t* stg = smem + ((gs + 3) & 3) * STAGE + w * (32 * 128);
-            uint8_t* wr = stg + lr * 128 + 8 * (g ^ (lr >> 4));
-            const int wsw = (lr >> 1) & 7;
-            const int rrow = l >> 3, rch = l & 7;
+            uint8_t* wr = stg + elr * 128 + 8 * (eg ^ (elr >> 4));
+            const int wsw = (elr >> 1) & 7;
+            const int rrow = lo >> 3, rch = lo & 7;
             // rows 8u + rrow: (row / 2) % 8 = (4 (u & 1) + rrow / 2) % 8
             const uint8_t* rd0 = stg + rrow * 128 + 16 * (rch ^ (rrow >> 1));
             const uint8_t* rd1 = stg + rrow * 128 + 16 * (rch ^ (4 + (rrow >> 1)));
             const bool full = (m_valid == BM) && (n_valid == BN);
             float alpha = 1.f;
             if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
+            // the loop exists twice, for whole tiles and for tiles at an edge: a whole tile's reads and stores are not
+            // predicated, so the compiler can send the four reads of a patch together and overlap them with the next
+            // patch's conversions
+            auto write_out = [&](auto full_tag) __attribute__((always_inline)) {
+                constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < 4; ++i) {
 #pragma unroll
-                for (int jh = 0; jh < 2; ++jh) {
+                    for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
-                    for (int jl = 0; jl < 2; ++jl)
+                        for (int jl = 0; jl < 2; ++jl)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const int j = 2 * jh + jl;
-                            if (ALPHA) {
+                            for (int q = 0; q < 4; ++q) {
+                                const int j = 2 * jh + jl;
+                                if (ALPHA) {
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] *= alpha;
+                                    for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] *= alpha;
+                                }
+                                v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
+                                          (__bf16)acc[i][j][4 * q + 3]};
+                                *(v4bf*)(wr + 16 * ((4 * jl + q) ^ wsw)) = o;
                             }
-                            v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
-                                      (__bf16)acc[i][j][4 * q + 3]};
-                            *(v4bf*)(wr + 16 * ((4 * jl + q) ^ wsw)) = o;
-                        }
-                    uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32 + rrow) * p.n + wn * 128 + jh * 64 + rch * 8);
-                    const int cc = wn * 128 + jh * 64 + rch * 8;
+                        uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32 + rrow) * p.n + wn * 128 + jh * 64 + rch * 8);
+                        const int cc = wn * 128 + jh * 64 + rch * 8;
+                        uint4 v[4];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        uint4 v = *(const uint4*)(((u & 1) ? rd1 : rd0) + u * (8 * 128));
-                        if (u >= 2) v = make_uint4(v.z, v.w, v.x, v.y);
-                        if (full || (wm * 128 + i * 32 + 8 * u + rrow < m_valid && cc < n_valid))
-                            store16_streaming(rowbase + (int64_t)(8 * u) * p.n * 2, v);
+                        for (int u = 0; u < 4; ++u) v[u] = *(const uint4*)(((u & 1) ? rd1 : rd0) + u * (8 * 128));
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            if (FULL || (wm * 128 + i * 32 + 8 * u + rrow < m_valid && cc < n_valid))
+                                store16_streaming(rowbase + (int64_t)(8 * u) * p.n * 2,
+                                                  u >= 2 ? make_uint4(v[u].z, v[u].w, v[u].x, v[u].y) : v[u]);
                     }
+                    MXL_PIN;
                 }
-                MXL_PIN;
-            }
+            };
+            if (full) write_out(std::true_type{});
+            else write_out(std::false_type{});
         }
         if (tile_n >= total_tiles) break;
         __syncthreads();      // every wave has left the patch: its slot takes K step 3 of the next tile

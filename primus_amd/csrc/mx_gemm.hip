@@ -475,7 +475,13 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         const int m_valid = __builtin_amdgcn_readfirstlane(d.m_valid), n_valid = __builtin_amdgcn_readfirstlane(d.n_valid);
         const int64_t c_off = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(d.c_off >> 32)) << 32) |
                                         (uint32_t)__builtin_amdgcn_readfirstlane((int)d.c_off));
-        auto lane_now = [] { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); };
+        // (the count starts from a zero the optimiser cannot see through: a plain lane count is loop-invariant to it, and
+        // would again be computed in front of the tile loop and spilled)
+        auto lane_now = [] {
+            uint32_t z = 0;
+            asm volatile("" : "+v"(z));
+            return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z));
+        };
         uint16_t* ctile = p.c + c_off;
         // ACCUM: the old float32 values of the first 32-row block are requested before the next tile's operand
         // requests go out (memory returns in order per wave: behind them they would wait for 64 KiB of loads)
@@ -1073,7 +1079,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // every register is taken, and would come back from scratch memory one dependent load after the other, each of
         // them waiting for all operand requests in flight (measured: 5 of the epilogue's 6.5 us).
         {
-            const int lo = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            uint32_t z = 0;    // a zero the optimiser cannot see through: the count must not be hoisted out of the tile loop
+            asm volatile("" : "+v"(z));
+            const int lo = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z));
             const int elr = lo & 31, eg = lo >> 5;
             const int m_valid = d.m_valid, n_valid = d.n_valid;
             uint16_t* ctile = p.c + d.c_off;
@@ -1087,15 +1095,18 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             const bool full = (m_valid == BM) && (n_valid == BN);
             float alpha = 1.f;
             if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
-            // the loop exists twice, for whole tiles and for tiles at an edge: a whole tile's reads and stores are not
-            // predicated, so the compiler can send the four reads of a patch together and overlap them with the next
-            // patch's conversions
+            // Eight patches (32 rows x 64 columns each) go through the staging area one after the other.  The LDS runs
+            // a wave's accesses in order, so patch n + 1 may be written as soon as the reads of patch n have been ISSUED:
+            // the stores of patch n, which wait for those reads, come behind the conversions and writes of patch n + 1
+            // and find their data there.  The loop exists twice, for whole tiles (nothing predicated) and for tiles at
+            // an edge.
             auto write_out = [&](auto full_tag) __attribute__((always_inline)) {
                 constexpr bool FULL = decltype(full_tag)::value;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-#pragma unroll
-                    for (int jh = 0; jh < 2; ++jh) {
+                uint4 v[4];
+                static_for<0, 9>([&](auto it_tag) {
+                    constexpr int it = decltype(it_tag)::value;
+                    if constexpr (it < 8) {
+                        constexpr int i = it >> 1, jh = it & 1;
 #pragma unroll
                         for (int jl = 0; jl < 2; ++jl)
 #pragma unroll
@@ -1109,19 +1120,23 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                                           (__bf16)acc[i][j][4 * q + 3]};
                                 *(v4bf*)(wr + 16 * ((4 * jl + q) ^ wsw)) = o;
                             }
+                    }
+                    if constexpr (it > 0) {
+                        constexpr int i = (it - 1) >> 1, jh = (it - 1) & 1;
                         uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32 + rrow) * p.n + wn * 128 + jh * 64 + rch * 8);
                         const int cc = wn * 128 + jh * 64 + rch * 8;
-                        uint4 v[4];
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) v[u] = *(const uint4*)(((u & 1) ? rd1 : rd0) + u * (8 * 128));
 #pragma unroll
                         for (int u = 0; u < 4; ++u)
                             if (FULL || (wm * 128 + i * 32 + 8 * u + rrow < m_valid && cc < n_valid))
                                 store16_streaming(rowbase + (int64_t)(8 * u) * p.n * 2,
                                                   u >= 2 ? make_uint4(v[u].z, v[u].w, v[u].x, v[u].y) : v[u]);
                     }
+                    if constexpr (it < 8) {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] = *(const uint4*)(((u & 1) ? rd1 : rd0) + u * (8 * 128));
+                    }
                     MXL_PIN;
-                }
+                });
             };
             if (full) write_out(std::true_type{});
             else write_out(std::false_type{});

@@ -147,6 +147,15 @@ struct Frags {
     int sa[4], sb[4];
 };
 
+// compile-time loop: f(integral_constant<int, I>) for I .. N - 1
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 // LAYOUT 0: operand codes row-major [rows, K].  LAYOUT 1: K-chunk-major [K / 128][rows][128 elements] (what the
 // quantisers write with MXL_QF_KCHUNK): the rows of a tile's K slot are one contiguous block, so a load round
 // fetches 4 KiB in a row instead of 16..64 row pieces; scales are row-major in both.
@@ -558,39 +567,48 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
                     MXL_PIN;
                 }
             } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                // lane (lr, g) holds row lr of this 32-row block: columns j*32 + 8q + 4g .. +3
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if (ALPHA) {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] *= alpha;
-                        }
-                        v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
-                                  (__bf16)acc[i][j][4 * q + 3]};
-                        *(v4bf*)(wr + (j * 32 + 8 * q) * 2) = o;
-                    }
+                // Four patches of 32 rows x 128 columns go through the staging area one after the other.  The LDS runs a
+                // wave's accesses in order, so patch n + 1 may be written once the reads of patch n have been ISSUED: the
+                // stores of patch n, which wait for those reads, come behind the conversions and writes of patch n + 1.
+                // lane (lr, g) holds row lr of a 32-row block: columns j*32 + 8q + 4g .. +3;
                 // 16 lanes per row, 4 rows per store instruction; the row base is uniform
-                uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32) * p.n + wn * 128);
-                if (full) {
+                auto write_out = [&](auto full_tag) __attribute__((always_inline)) {
+                    constexpr bool FULL = decltype(full_tag)::value;
+                    uint4 v[8];
+                    static_for<0, 5>([&](auto it_tag) {
+                        constexpr int it = decltype(it_tag)::value;
+                        if constexpr (it < 4) {
+                            constexpr int i = it;
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        const uint4 v = *(const uint4*)(rd + 4 * u * SP);
-                        store16_streaming(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off, v);
-                    }
-                } else {
+                            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        const uint4 v = *(const uint4*)(rd + 4 * u * SP);
-                        if (wm * 128 + i * 32 + 4 * u + rr < m_valid && cc < n_valid)
-                            store16_streaming(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off, v);
-                    }
-                }
-                MXL_PIN;  // one 32-row block at a time: 64 accumulators live, not 256
-            }
+                                for (int q = 0; q < 4; ++q) {
+                                    if (ALPHA) {
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] *= alpha;
+                                    }
+                                    v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
+                                              (__bf16)acc[i][j][4 * q + 3]};
+                                    *(v4bf*)(wr + (j * 32 + 8 * q) * 2) = o;
+                                }
+                        }
+                        if constexpr (it > 0) {
+                            constexpr int i = it - 1;
+                            uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32) * p.n + wn * 128);
+#pragma unroll
+                            for (int u = 0; u < 8; ++u)
+                                if (FULL || (wm * 128 + i * 32 + 4 * u + rr < m_valid && cc < n_valid))
+                                    store16_streaming(rowbase + (int64_t)(4 * u) * p.n * 2 + lane_off, v[u]);
+                        }
+                        if constexpr (it < 4) {
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) v[u] = *(const uint4*)(rd + 4 * u * SP);
+                        }
+                        MXL_PIN;  // one 32-row block at a time: 64 accumulators live, not 256
+                    });
+                };
+                if (full) write_out(std::true_type{});
+                else write_out(std::false_type{});
             }
         }
     }
@@ -627,13 +645,6 @@ constexpr int ring_lds_bytes() {
     return RING_SLOTS * RING_STAGE + RING_PANEL_BUFS * 2 * RING_PANEL + RING_TBL * 4 + RING_TBL * 8 + RING_TBL * 4 + RING_TBL * 4;
 }
 
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
 
 template <int AFMT, int BFMT, int MODE, bool ALPHA>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {

@@ -514,8 +514,8 @@ def main():
     # the MFMA peak of the slower operand format: FP8 rate unless both operands are E2M1
     peak = FP4_PEAK_TFLOPS if act_fp4 else FP8_PEAK_TFLOPS
     roofline = {
-        # FP8 x FP8 (MX or tensor-wise scaled) and E2M1 x E2M1 run on the 4-slot ring kernel, FP8 x E2M1 on the 2-slot kernel
-        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_kernel" if spec["fp4"] and not act_fp4 else "mx_gemm_ring_kernel",
+        # every benchmark workload runs on the 4-slot ring kernel
+        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_ring_kernel",
                                                    "e4m3|e5m2" if spec.get("tensorwise") else "e2m1" if act_fp4 else "e4m3",
                                                    "e2m1" if spec["fp4"] else "e4m3",
                                                    ",alpha" if spec.get("tensorwise") else "", fwd_name),

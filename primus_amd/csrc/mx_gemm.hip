@@ -770,7 +770,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         uint32_t cal, cbl;         // byte offset of the LAST K step of the contraction range (requests never pass it)
         int nst, nst_real;         // K steps to run (>= 4, even) and how many of them multiply (the first nst_real)
         int m_valid, n_valid;
-        int64_t c_off;
+        int c_row0, c_col0;        // first output row and column of the tile
     };
     auto decode = [&](int tile) __attribute__((always_inline)) {
         Tile d;
@@ -817,11 +817,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // the epilogue's tile facts are uniform: kept in scalar registers they survive the main loop without
         // taking part in the vector register spills
         d.n_valid = __builtin_amdgcn_readfirstlane((p.n - n0) < BN ? (int)(p.n - n0) : BN);
-        {
-            const int64_t off = c_row0 * p.n + n0;
-            d.c_off = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(off >> 32)) << 32) |
-                                (uint32_t)__builtin_amdgcn_readfirstlane((int)off));
-        }
+        d.c_row0 = __builtin_amdgcn_readfirstlane((int)c_row0);
+        d.c_col0 = __builtin_amdgcn_readfirstlane((int)n0);
         // the range is a multiple of 128 elements: an even number of steps, except with FP4 rows (one step each)
         const int nreal = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / KS));
         d.nst_real = nreal;
@@ -883,7 +880,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     auto next3 = [](int b) { return b == 2 ? 0 : b + 1; };
 
 #define MXL_MFMA(F, I, J) \
-    do { if (MF) { \
+    do { if (MF && (I) < LIVE) { \
              acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(F.b[J], F.a[I], acc[I][J], CB, BL, 0, F.sb[J], 0, F.sa[I]); \
              if (F44) acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4( \
                  __builtin_shufflevector(F.b[J], F.b[J], 4, 5, 6, 7, 4, 5, 6, 7), __builtin_shufflevector(F.a[I], F.a[I], 4, 5, 6, 7, 4, 5, 6, 7), \
@@ -891,10 +888,10 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
 #define MXL_PIN __builtin_amdgcn_sched_barrier(0)
     // fragment (+ scale byte) reads of the K step in ring slot at `sn`, panel bytes at `pan`
 #define MXL_RD_A(F, I) \
-    do { const uint8_t* r_ = sn + a_frag + (I) * (32 * BK); \
+    do { if ((I) < LIVE) { const uint8_t* r_ = sn + a_frag + (I) * (32 * BK); \
          const uint4 lo_ = *(const uint4*)(r_ + a_lo), hi_ = *(const uint4*)(r_ + a_hi); \
          F.a[I][0] = lo_.x; F.a[I][1] = lo_.y; F.a[I][2] = lo_.z; F.a[I][3] = lo_.w; \
-         F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; } while (0)
+         F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; } } while (0)
 #define MXL_RD_B(F, J) \
     do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * B_ROW); \
          if (B4) { \
@@ -989,91 +986,103 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
         Frags f0, f1;
         const int nst = d.nst, nst_real = d.nst_real;
-        {   // fragments of K step 0
-            const uint8_t* sn = smem + (gs & 3) * STAGE;
-            MXL_RD_PANEL(panels + pb_rd * 2 * PANEL);
-            const int psh = 0;
-            MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
-            MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
-            MXL_SC_B(f0, 0); MXL_SC_B(f0, 1); MXL_SC_B(f0, 2); MXL_SC_B(f0, 3);
-            MXL_SC_A(f0, 0); MXL_SC_A(f0, 1); MXL_SC_A(f0, 2); MXL_SC_A(f0, 3);
-        }
-        // One K step s (local number, parity PAR) of 16 MFMAs.  MF: multiply (false for the padding steps of a
-        // tile whose contraction range is shorter than four steps).  LAST: the tile's last step; the six rounds
-        // that would go into the slot the epilogue is about to use are issued after the epilogue instead.
-        using E0 = std::integral_constant<int, 0>; using E1 = std::integral_constant<int, 1>;
-        using E2 = std::integral_constant<int, 2>; using E3 = std::integral_constant<int, 3>;
-        using E4 = std::integral_constant<int, 4>; using E5 = std::integral_constant<int, 5>;
-        using E6 = std::integral_constant<int, 6>; using E7 = std::integral_constant<int, 7>;
-        auto kstep = [&](auto par_tag, auto mf_tag, auto last_tag, int s, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
-            constexpr int PAR = decltype(par_tag)::value;
-            constexpr bool MF = decltype(mf_tag)::value;
-            constexpr bool LAST = decltype(last_tag)::value;
-            const uint32_t slot_prev = wave_base + (uint32_t)(((gs + 3) & 3) * STAGE);   // group of step gs + 3
-            const uint32_t slot_new = wave_base + (uint32_t)((gs & 3) * STAGE);          // group of step gs + 4
-            MXL_MFMA(cur, 0, 0); if (ROUNDS == 8) issue_e(E6{}, slot_prev); MXL_PIN;
-            MXL_MFMA(cur, 1, 0); MXL_PIN;
-            MXL_MFMA(cur, 2, 0); if (ROUNDS == 8) issue_e(E7{}, slot_prev); MXL_PIN;
-            MXL_MFMA(cur, 3, 0); MXL_PIN;
-            wait_vm<2 * ROUNDS>();       // the group of step gs + 1 has landed (two younger groups may be in flight)
-            __syncthreads();
-            MXL_PIN;
-            // bookkeeping between the barrier and the first read: panel of the next step, stream hand-over
-            const int s1 = s + 1;
-            if ((s1 & (PSTEPS - 1)) == 0 && s1 < nst) {
-                pb_rd = next3(pb_rd);
+        // LIVE: how many of the wave's four 32-row fragments hold rows of the tile (4, 2 or 0).  A tile at the ragged end of
+        // a group has fewer than 256 rows; fragments beyond them are neither read nor multiplied (loads, barriers and the
+        // request stream are the same for every wave).
+        auto run_tile = [&](auto live_tag) __attribute__((always_inline)) {
+            constexpr int LIVE = decltype(live_tag)::value;
+            {   // fragments of K step 0
+                const uint8_t* sn = smem + (gs & 3) * STAGE;
                 MXL_RD_PANEL(panels + pb_rd * 2 * PANEL);
+                const int psh = 0;
+                MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
+                MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
+                MXL_SC_B(f0, 0); MXL_SC_B(f0, 1); MXL_SC_B(f0, 2); MXL_SC_B(f0, 3);
+                MXL_SC_A(f0, 0); MXL_SC_A(f0, 1); MXL_SC_A(f0, 2); MXL_SC_A(f0, 3);
             }
-            if (!LAST) group_begin();
-            const uint8_t* sn = smem + ((gs + 1) & 3) * STAGE;
-            const int psh = (64 / PSTEPS) * (s1 & (PSTEPS - 1));   // FP4 rows: a step owns two bytes, the MFMAs pick with op_sel
-            MXL_PIN;
-            MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(E0{}, slot_new); MXL_PIN;
-            MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1);  MXL_PIN;
-            MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1);  if (!LAST) issue_e(E1{}, slot_new); MXL_PIN;
-            MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1);  MXL_PIN;
-            MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2);  if (!LAST) issue_e(E2{}, slot_new); MXL_PIN;
-            MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2);  MXL_SC_B(nxt, 0); MXL_PIN;
-            MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(E3{}, slot_new); MXL_SC_A(nxt, 0); MXL_PIN;
-            MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2);  MXL_SC_A(nxt, 1); MXL_PIN;
-            MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(E4{}, slot_new); MXL_SC_A(nxt, 2); MXL_PIN;
-            MXL_MFMA(cur, 1, 3); MXL_SC_A(nxt, 3); MXL_SC_B(nxt, 1); MXL_PIN;
-            MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(E5{}, slot_new); MXL_SC_B(nxt, 2); MXL_PIN;
-            MXL_MFMA(cur, 3, 3); MXL_SC_B(nxt, 3); MXL_PIN;
-            ++gs;
-        };
-        using P0 = std::integral_constant<int, 0>;
-        using P1 = std::integral_constant<int, 1>;
-        using Yes = std::integral_constant<bool, true>;
-        using No = std::integral_constant<bool, false>;
-        if (nst_real >= 3) {
-            for (int s = 0; s < nst - 2; s += 2) {
-                if (s == nst - 4) {
-                    // the request stream moves on to the workgroup's next tile: its scale panel 0 first
-                    pb_is = next3(pb_is);
-                    issue_s(dn, 0, pb_is);
-                    stream_enter(dn);
-                } else if ((s & (PSTEPS - 1)) == PSTEPS - 4 && s + 4 < nst) {
-                    // this tile's next scale panel (K steps s + 4 ...): first read three barriers from here
-                    pb_is = next3(pb_is);
-                    issue_s(d, (s + 4) / PSTEPS, pb_is);
+            // One K step s (local number, parity PAR) of 16 MFMAs.  MF: multiply (false for the padding steps of a
+            // tile whose contraction range is shorter than four steps).  LAST: the tile's last step; the six rounds
+            // that would go into the slot the epilogue is about to use are issued after the epilogue instead.
+            using E0 = std::integral_constant<int, 0>; using E1 = std::integral_constant<int, 1>;
+            using E2 = std::integral_constant<int, 2>; using E3 = std::integral_constant<int, 3>;
+            using E4 = std::integral_constant<int, 4>; using E5 = std::integral_constant<int, 5>;
+            using E6 = std::integral_constant<int, 6>; using E7 = std::integral_constant<int, 7>;
+            auto kstep = [&](auto par_tag, auto mf_tag, auto last_tag, int s, Frags& cur, Frags& nxt) __attribute__((always_inline)) {
+                constexpr int PAR = decltype(par_tag)::value;
+                constexpr bool MF = decltype(mf_tag)::value;
+                constexpr bool LAST = decltype(last_tag)::value;
+                const uint32_t slot_prev = wave_base + (uint32_t)(((gs + 3) & 3) * STAGE);   // group of step gs + 3
+                const uint32_t slot_new = wave_base + (uint32_t)((gs & 3) * STAGE);          // group of step gs + 4
+                MXL_MFMA(cur, 0, 0); if (ROUNDS == 8) issue_e(E6{}, slot_prev); MXL_PIN;
+                MXL_MFMA(cur, 1, 0); MXL_PIN;
+                MXL_MFMA(cur, 2, 0); if (ROUNDS == 8) issue_e(E7{}, slot_prev); MXL_PIN;
+                MXL_MFMA(cur, 3, 0); MXL_PIN;
+                wait_vm<2 * ROUNDS>();       // the group of step gs + 1 has landed (two younger groups may be in flight)
+                __syncthreads();
+                MXL_PIN;
+                // bookkeeping between the barrier and the first read: panel of the next step, stream hand-over
+                const int s1 = s + 1;
+                if ((s1 & (PSTEPS - 1)) == 0 && s1 < nst) {
+                    pb_rd = next3(pb_rd);
+                    MXL_RD_PANEL(panels + pb_rd * 2 * PANEL);
                 }
-                kstep(P0{}, Yes{}, No{}, s, f0, f1);
-                kstep(P1{}, Yes{}, No{}, s + 1, f1, f0);
+                if (!LAST) group_begin();
+                const uint8_t* sn = smem + ((gs + 1) & 3) * STAGE;
+                const int psh = (64 / PSTEPS) * (s1 & (PSTEPS - 1));   // FP4 rows: a step owns two bytes, the MFMAs pick with op_sel
+                MXL_PIN;
+                MXL_RD_B(nxt, 0); MXL_MFMA(cur, 0, 1);  if (!LAST) issue_e(E0{}, slot_new); MXL_PIN;
+                MXL_RD_A(nxt, 0); MXL_MFMA(cur, 1, 1);  MXL_PIN;
+                MXL_RD_A(nxt, 1); MXL_MFMA(cur, 2, 1);  if (!LAST) issue_e(E1{}, slot_new); MXL_PIN;
+                MXL_RD_A(nxt, 2); MXL_MFMA(cur, 3, 1);  MXL_PIN;
+                MXL_RD_A(nxt, 3); MXL_MFMA(cur, 0, 2);  if (!LAST) issue_e(E2{}, slot_new); MXL_PIN;
+                MXL_RD_B(nxt, 1); MXL_MFMA(cur, 1, 2);  MXL_SC_B(nxt, 0); MXL_PIN;
+                MXL_RD_B(nxt, 2); MXL_MFMA(cur, 2, 2);  if (!LAST) issue_e(E3{}, slot_new); MXL_SC_A(nxt, 0); MXL_PIN;
+                MXL_RD_B(nxt, 3); MXL_MFMA(cur, 3, 2);  MXL_SC_A(nxt, 1); MXL_PIN;
+                MXL_MFMA(cur, 0, 3); if (!LAST) issue_e(E4{}, slot_new); MXL_SC_A(nxt, 2); MXL_PIN;
+                MXL_MFMA(cur, 1, 3); MXL_SC_A(nxt, 3); MXL_SC_B(nxt, 1); MXL_PIN;
+                MXL_MFMA(cur, 2, 3); if (!LAST) issue_e(E5{}, slot_new); MXL_SC_B(nxt, 2); MXL_PIN;
+                MXL_MFMA(cur, 3, 3); MXL_SC_B(nxt, 3); MXL_PIN;
+                ++gs;
+            };
+            using P0 = std::integral_constant<int, 0>;
+            using P1 = std::integral_constant<int, 1>;
+            using Yes = std::integral_constant<bool, true>;
+            using No = std::integral_constant<bool, false>;
+            if (nst_real >= 3) {
+                for (int s = 0; s < nst - 2; s += 2) {
+                    if (s == nst - 4) {
+                        // the request stream moves on to the workgroup's next tile: its scale panel 0 first
+                        pb_is = next3(pb_is);
+                        issue_s(dn, 0, pb_is);
+                        stream_enter(dn);
+                    } else if ((s & (PSTEPS - 1)) == PSTEPS - 4 && s + 4 < nst) {
+                        // this tile's next scale panel (K steps s + 4 ...): first read three barriers from here
+                        pb_is = next3(pb_is);
+                        issue_s(d, (s + 4) / PSTEPS, pb_is);
+                    }
+                    kstep(P0{}, Yes{}, No{}, s, f0, f1);
+                    kstep(P1{}, Yes{}, No{}, s + 1, f1, f0);
+                }
+                kstep(P0{}, Yes{}, No{}, nst - 2, f0, f1);
+                if (!F44 || nst_real == nst) kstep(P1{}, Yes{}, Yes{}, nst - 1, f1, f0);
+                else kstep(P1{}, No{}, Yes{}, nst - 1, f1, f0);          // an odd range: the padding step does not multiply
+            } else {
+                // a contraction range of one or two steps: four steps run, the others without multiplying
+                pb_is = next3(pb_is);
+                issue_s(dn, 0, pb_is);
+                stream_enter(dn);
+                kstep(P0{}, Yes{}, No{}, 0, f0, f1);
+                if (!F44 || nst_real == 2) kstep(P1{}, Yes{}, No{}, 1, f1, f0);
+                else kstep(P1{}, No{}, No{}, 1, f1, f0);
+                kstep(P0{}, No{}, No{}, 2, f0, f1);
+                kstep(P1{}, No{}, Yes{}, 3, f1, f0);
             }
-            kstep(P0{}, Yes{}, No{}, nst - 2, f0, f1);
-            if (!F44 || nst_real == nst) kstep(P1{}, Yes{}, Yes{}, nst - 1, f1, f0);
-            else kstep(P1{}, No{}, Yes{}, nst - 1, f1, f0);          // an odd range: the padding step does not multiply
-        } else {
-            // a contraction range of one or two steps: four steps run, the others without multiplying
-            pb_is = next3(pb_is);
-            issue_s(dn, 0, pb_is);
-            stream_enter(dn);
-            kstep(P0{}, Yes{}, No{}, 0, f0, f1);
-            if (!F44 || nst_real == 2) kstep(P1{}, Yes{}, No{}, 1, f1, f0);
-            else kstep(P1{}, No{}, No{}, 1, f1, f0);
-            kstep(P0{}, No{}, No{}, 2, f0, f1);
-            kstep(P1{}, No{}, Yes{}, 3, f1, f0);
+        };
+        {
+            const int live = (MODE == MODE_FWD) ? d.m_valid - wm * 128 : 128;
+            if (MODE != MODE_FWD || live > 64) run_tile(std::integral_constant<int, 4>{});
+            else if (live > 0) run_tile(std::integral_constant<int, 2>{});
+            else run_tile(std::integral_constant<int, 0>{});
         }
         // K step 0 of the next tile (and its scale panel) has landed; every wave is done reading the ring
         wait_vm<2 * ROUNDS>();
@@ -1095,7 +1104,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             const int lo = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z));
             const int elr = lo & 31, eg = lo >> 5;
             const int m_valid = d.m_valid, n_valid = d.n_valid;
-            uint16_t* ctile = p.c + d.c_off;
+            uint16_t* ctile = p.c + ((int64_t)d.c_row0 * p.n + d.c_col0);
             uint8_t* stg = smem + ((gs + 3) & 3) * STAGE + w * (32 * 128);
             uint8_t* wr = stg + elr * 128 + 8 * (eg ^ (elr >> 4));
             const int wsw = (elr >> 1) & 7;
@@ -1103,6 +1112,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
             // rows 8u + rrow: (row / 2) % 8 = (4 (u & 1) + rrow / 2) % 8
             const uint8_t* rd0 = stg + rrow * 128 + 16 * (rch ^ (rrow >> 1));
             const uint8_t* rd1 = stg + rrow * 128 + 16 * (rch ^ (4 + (rrow >> 1)));
+            const uint32_t lane_off = (uint32_t)((rrow * (int)p.n + rch * 8) * 2);   // bytes from the row base
             const bool full = (m_valid == BM) && (n_valid == BN);
             float alpha = 1.f;
             if (ALPHA) alpha = *p.alpha_a * *p.alpha_b;
@@ -1134,12 +1144,13 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                     }
                     if constexpr (it > 0) {
                         constexpr int i = (it - 1) >> 1, jh = (it - 1) & 1;
-                        uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32 + rrow) * p.n + wn * 128 + jh * 64 + rch * 8);
+                        // uniform base of the patch's rows; the lane adds a 32-bit offset
+                        uint8_t* rowbase = (uint8_t*)(ctile + (int64_t)(wm * 128 + i * 32) * p.n + wn * 128 + jh * 64);
                         const int cc = wn * 128 + jh * 64 + rch * 8;
 #pragma unroll
                         for (int u = 0; u < 4; ++u)
                             if (FULL || (wm * 128 + i * 32 + 8 * u + rrow < m_valid && cc < n_valid))
-                                store16_streaming(rowbase + (int64_t)(8 * u) * p.n * 2,
+                                store16_streaming(rowbase + (int64_t)(8 * u) * p.n * 2 + lane_off,
                                                   u >= 2 ? make_uint4(v[u].z, v[u].w, v[u].x, v[u].y) : v[u]);
                     }
                     if constexpr (it < 8) {
@@ -1309,6 +1320,8 @@ static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tile
         if (accum || !ring_serves<MODE>(afmt, bfmt, a)) return MXL_EINVAL;
         // offsets inside an operand are 32-bit
         if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
+        // the kernel keeps a tile's first output row in 32 bits
+        if ((MODE == MODE_WGRAD ? (int64_t)a.num_groups * a.m : a.total_m) >= ((int64_t)1 << 31)) return MXL_EINVAL;
         return dispatch_gemm_ring<MODE>(afmt, bfmt, a, max_tiles, st);
     }
     if (accum) {

@@ -295,7 +295,7 @@ def create_quantized_weight(
         return row, col
     if kchunk is None:
         kchunk = K.pick_layout(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1, w.shape[-2], w.shape[-1],
-                               fp8=fmt != _lib.FMT_E2M1,
+                               fp8=fmt != _lib.FMT_E2M1 or getattr(quant_config, "activation_format", None) == Format.E4M3,
                                fp4=fmt == _lib.FMT_E2M1 and getattr(quant_config, "activation_format", None) == Format.E2M1_X2)
     q_row, s_row, q_col, s_col = K.quantize_mx_weight_2d_impl(
         w.contiguous(), fmt, mode.value, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN,

@@ -158,10 +158,9 @@ class _MXLinearFunction(torch.autograd.Function):
         # Every operand of the three GEMMs is stored in one layout, K-chunk-major unless an operand is
         # too large for it (or the layout is switched off): same codes, same results, faster loads.
         groups = b.shape[0] if grouped else 1
-        # K-step-major operands (the ring kernel) for FP8 x FP8 and E2M1 x E2M1.  The ring kernel also takes FP8 activations against
-        # FP4 weights, but at the shapes that recipe is used on (GPT-OSS: K = 2880, 46 K steps per tile, ragged row
-        # tiles) the 2-slot kernel with its live-fragment variants is the faster one (2.04 against 1.89 PFLOP/s)
-        fp8 = act_fmt != _lib.FMT_E2M1 and w_fmt != _lib.FMT_E2M1
+        # K-step-major operands (the ring kernel) whenever the activations are FP8: against FP8 weights in all three
+        # GEMMs, against E2M1 weights in forward and dgrad (wgrad is FP8 x FP8 then)
+        fp8 = act_fmt != _lib.FMT_E2M1
         # E2M1 x E2M1 runs on the ring kernel too, in steps of 128 elements (two MFMAs per step)
         fp4 = act_fmt == _lib.FMT_E2M1 and w_fmt == _lib.FMT_E2M1
         kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, fp4=fp4,

@@ -321,3 +321,49 @@ def test_full_size_mixtral_chunked_scaled_and_accumulating_bit_exact(gpu):
     for g in range(G):
         a, b = int(offs[g]), int(offs[g + 1])
         assert torch.equal(buf[g], before[g] + dyf[a:b].T @ xf[a:b]), g
+
+
+@pytest.mark.parametrize("fmt,layout", [(0, 2), (1, 3)])
+def test_full_size_mixtral_ring_kernel_bit_exact(gpu, fmt, layout):
+    """The full-size Mixtral fc1 through the quantisers and the 4-slot ring kernel (K-step-major operands: MXFP8 in
+    64-element steps, MXFP4 x MXFP4 in 128-element steps): forward, dgrad and a 512-column slice of the weight gradient,
+    EVERY output element.  The inputs are small integers (|v| <= 4) times a power of two per tensor: whatever a block's
+    largest magnitude is, its E8M0 scale leaves every element on an E4M3 / E2M1 code, so quantisation is exact, every
+    partial sum is an integer below 2^24, and the fp32 matrix product of the bf16 inputs is the exact result in any
+    summation order."""
+    from primus_amd.pytorch import kernels as K
+
+    spec = bench.WORKLOADS["mixtral_8x7b_moe_mxfp8"]
+    lens = bench.route(spec)
+    G, M, k, n = spec["G"], sum(lens), spec["hidden"], spec["fc1_out"]
+    gen = torch.Generator(device=gpu).manual_seed(79 + fmt)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+
+    def ints(rows, cols, factor):
+        return (torch.randint(-4, 5, (rows, cols), generator=gen, device=gpu).float() * factor).bfloat16()
+
+    x = ints(M, k, 0.5)
+    w = ints(G * n, k, 0.25).view(G, n, k)
+    xq = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=True, group_lens=gl, kchunk=layout)
+    wq = K.quantize_mx_weight_2d_impl(w, fmt, rowwise=True, colwise=True, kchunk=layout)
+    y = K.grouped_gemm_mx_nt_impl(xq[0], xq[1], wq[0], wq[1], gl, kchunk=layout)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        assert torch.equal(y[a:b], (x[a:b].float() @ w[g].float().T).bfloat16()), ("fwd", g)
+    del y
+    # dgrad: dX = dY . W_g (contraction over n = 28672)
+    dy = ints(M, n, 2.0)
+    dq = K.quantize_mx_impl(dy, fmt, rowwise=True, colwise=False, group_lens=gl, kchunk=layout)
+    dx = K.grouped_gemm_mx_nt_impl(dq[0], dq[1], wq[2], wq[3], gl, kchunk=layout)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        assert torch.equal(dx[a:b], (dy[a:b].float() @ w[g].float()).bfloat16()), ("dgrad", g)
+    del dx, dq, wq
+    # wgrad on a 512-column slice of dY: dW_g = dY_g^T . X_g over the group's (padded) token segment
+    dys = dy[:, :512].contiguous()
+    dqs = K.quantize_mx_impl(dys, fmt, rowwise=False, colwise=True, group_lens=gl, kchunk=layout)
+    dw = K.grouped_gemm_mx_wgrad_impl(dqs[2], dqs[3], xq[2], xq[3], gl, M, kchunk=layout)
+    for g in range(G):
+        a, b = int(offs[g]), int(offs[g + 1])
+        assert torch.equal(dw[g], (dys[a:b].float().T @ x[a:b].float()).bfloat16()), ("wgrad", g)

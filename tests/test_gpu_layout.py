@@ -272,3 +272,32 @@ def test_operators_same_on_both_layouts_random_shapes(gpu, seed):
         for i, (r, o) in enumerate(zip(ref, out)):
             assert r.shape == o.shape and _same(r, o), (i, fp4, lens, n, k, cached, glu)
         done += 1
+
+
+@pytest.mark.parametrize("act_fp4", [False, True])
+def test_fp4_weight_cache_layout_follows_the_activation_format(gpu, act_fp4):
+    """A cached E2M1 weight pair is stored for the GEMM it will meet: 64-element K steps when the config's activations
+    are FP8, 128-element steps when they are E2M1.  Either cache dequantises to the same values as a row-major one and
+    gives the same forward and input gradient bit for bit."""
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch import kernels as K
+    from primus_amd.pytorch.core import (Float4QuantConfig, Format, QuantizedTensorPair, create_quantized_weight,
+                                         float4_e2m1fn_x2)
+
+    cfg = Float4QuantConfig(activation_format=Format.E2M1_X2 if act_fp4 else Format.E4M3)
+    g = torch.Generator().manual_seed(11)
+    lens = [70, 0, 300, 58]
+    x = torch.randn(sum(lens), 160, generator=g).bfloat16().to(gpu).requires_grad_()
+    w = (torch.randn(4, 96, 160, generator=g) * 0.05).bfloat16().to(gpu)
+    dy = torch.randn(sum(lens), 96, generator=g).bfloat16().to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    auto = QuantizedTensorPair(*create_quantized_weight(w, float4_e2m1fn_x2, cfg))
+    flat = QuantizedTensorPair(*create_quantized_weight(w, float4_e2m1fn_x2, cfg, kchunk=False))
+    assert auto.data.kchunk == (K.LAYOUT_KSTEP128 if act_fp4 else K.LAYOUT_KSTEP) and flat.data.kchunk == 0
+    assert _same(auto.data.dequantize(), flat.data.dequantize()) and _same(auto.data_t.dequantize(), flat.data_t.dequantize())
+    res = []
+    for pair in (flat, auto):
+        y = turbo.ops.grouped_gemm_fp4(x, pair, gl, config=cfg)
+        (dx,) = torch.autograd.grad(y, [x], dy)
+        res.append((y, dx))
+    assert _same(res[0][0], res[1][0]) and _same(res[0][1], res[1][1])

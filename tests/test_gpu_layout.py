@@ -295,9 +295,14 @@ def test_fp4_weight_cache_layout_follows_the_activation_format(gpu, act_fp4):
     flat = QuantizedTensorPair(*create_quantized_weight(w, float4_e2m1fn_x2, cfg, kchunk=False))
     assert auto.data.kchunk == (K.LAYOUT_KSTEP128 if act_fp4 else K.LAYOUT_KSTEP) and flat.data.kchunk == 0
     assert _same(auto.data.dequantize(), flat.data.dequantize()) and _same(auto.data_t.dequantize(), flat.data_t.dequantize())
+    # a cache made for the other activation format still serves this call (its scales are rearranged on the way)
+    other_cfg = Float4QuantConfig(activation_format=Format.E4M3 if act_fp4 else Format.E2M1_X2)
+    other = QuantizedTensorPair(*create_quantized_weight(w, float4_e2m1fn_x2, other_cfg))
+    assert other.data.kchunk != auto.data.kchunk
     res = []
-    for pair in (flat, auto):
+    for pair in (flat, auto, other):
         y = turbo.ops.grouped_gemm_fp4(x, pair, gl, config=cfg)
         (dx,) = torch.autograd.grad(y, [x], dy)
         res.append((y, dx))
-    assert _same(res[0][0], res[1][0]) and _same(res[0][1], res[1][1])
+    for y, dx in res[1:]:
+        assert _same(res[0][0], y) and _same(res[0][1], dx)

@@ -978,12 +978,6 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
 
     while (true) {
         v16f acc[4][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
         Frags f0, f1;
         const int nst = d.nst, nst_real = d.nst_real;
         // LIVE: how many of the wave's four 32-row fragments hold rows of the tile (4, 2 or 0).  A tile at the ragged end of
@@ -997,6 +991,15 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                 const int psh = 0;
                 MXL_RD_B(f0, 0); MXL_RD_B(f0, 1); MXL_RD_B(f0, 2); MXL_RD_B(f0, 3);
                 MXL_RD_A(f0, 0); MXL_RD_A(f0, 1); MXL_RD_A(f0, 2); MXL_RD_A(f0, 3);
+                MXL_PIN;
+                // the accumulators are cleared while those reads are on their way
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+                MXL_PIN;
                 MXL_SC_B(f0, 0); MXL_SC_B(f0, 1); MXL_SC_B(f0, 2); MXL_SC_B(f0, 3);
                 MXL_SC_A(f0, 0); MXL_SC_A(f0, 1); MXL_SC_A(f0, 2); MXL_SC_A(f0, 3);
             }

@@ -148,10 +148,10 @@ def _gflag(kchunk) -> int:
 
 def pick_layout(groups: int, n: int, k: int, rows: int = 0, fp8: bool = True, accum: bool = False,
                 fp4: bool = False) -> int:
-    """Layout the differentiable operators store their quantised operands in: K-step-major when every operand
-    is FP8 (``fp8``; steps of 64 elements) or every operand is E2M1 (``fp4``; steps of 128 elements), the groups
-    fit the ring kernel and the weight gradient is not accumulated in the GEMM; otherwise K-chunk-major;
-    row-major when the layouts are switched off or an operand reaches 4 GiB."""
+    """Layout the differentiable operators store their quantised operands in: K-step-major when the activations and
+    gradients are FP8 (``fp8``; steps of 64 elements, the weights FP8 or E2M1) or every operand is E2M1 (``fp4``; steps
+    of 128 elements), the groups fit the ring kernel and the weight gradient is not accumulated in the GEMM; otherwise
+    K-chunk-major; row-major when the layouts are switched off or an operand reaches 4 GiB."""
     if not (kchunk_default() and kchunk_fits(groups, n, k, rows)):
         return LAYOUT_ROWMAJOR
     if (fp8 or fp4) and groups <= RING_MAX_GROUPS and not accum and _kstep_default:

@@ -282,7 +282,7 @@ def create_quantized_weight(
     mode = quant_config.scale_mode
     if quant_config.granularity == ScalingGranularity.TENSORWISE:
         if kchunk is None:
-            kchunk = K.kchunk_default() and K.kchunk_fits(w.numel() // (w.shape[-1] * w.shape[-2]), w.shape[-2], w.shape[-1])
+            kchunk = K.pick_layout(w.numel() // (w.shape[-1] * w.shape[-2]) if w.dim() > 2 else 1, w.shape[-2], w.shape[-1], fp8=True)
         q_row, s_row, q_col, s_col, si = K.quantize_weight_tensorwise_impl(
             w.contiguous(), fmt, rowwise=True, colwise=need_weight_transpose_cache, pad_to=K.GEMM_K_ALIGN, kchunk=kchunk)
         row = QuantizedTensor(q_row, s_row, logical_shape=w.shape, orig_dtype=w.dtype, axis=-1, kchunk=kchunk,

@@ -296,7 +296,14 @@ def _transposed_cache(q: QuantizedTensor, kchunk: bool):
     out[..., :n] = t.view(torch.uint8)
     unit = torch.full(tuple(t.shape[:-1]) + (n_ld // _lib.BLOCK,), 127, dtype=torch.uint8, device=codes.device)
     if kchunk:
-        out = out.reshape(-1, n_ld // K.KCHUNK, K.KCHUNK).permute(1, 0, 2).contiguous()
+        # K-chunk-major or K-step-major: [n_ld / step][rows][step]; such operands carry a readable tail behind them
+        step = K.KSTEP if int(kchunk) == K.LAYOUT_KSTEP else K.KCHUNK
+        rows = out.numel() // n_ld
+        laid = K._empty_tail((n_ld // step, rows, step), dtype=torch.uint8, device=codes.device)
+        laid.copy_(out.reshape(rows, n_ld // step, step).permute(1, 0, 2))
+        out = laid
+        if int(kchunk) == K.LAYOUT_KSTEP:
+            unit = K._empty_tail(K._scale_shape(rows, n_ld, kchunk), dtype=torch.uint8, device=codes.device).fill_(127)
     return out.view(codes.dtype), unit.view(q.scales.dtype)
 
 
@@ -314,9 +321,14 @@ class _TWLinearFunction(torch.autograd.Function):
         grouped = group_lens is not None
         groups = b.shape[0] if grouped else 1
         if isinstance(b, QuantizedTensor):
-            # cached copies are stored row-major or K-chunk-major
-            kc = K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])
-            kc = int(bool(kc and b.kchunk and (b_t is None or b_t.kchunk)))
+            # cached copies decide: the call uses the layout they are stored in, row-major when it cannot
+            kc = int(b.kchunk) if (b_t is None or int(b_t.kchunk) == int(b.kchunk)) else 0
+            if not (K.kchunk_default() and K.kchunk_fits(groups, b.shape[-2], b.shape[-1], a.shape[0])):
+                kc = 0
+            if kc == K.LAYOUT_KSTEP and (groups > K.RING_MAX_GROUPS or (accum is not None and _fusable(accum[0]))):
+                kc = 0          # the ring kernel neither accumulates into float32 nor takes more groups
+            if kc == K.LAYOUT_KSTEP128:
+                kc = 0
         else:
             kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=True,
                                accum=accum is not None and _fusable(accum[0]))
@@ -325,11 +337,11 @@ class _TWLinearFunction(torch.autograd.Function):
         if isinstance(b, QuantizedTensor):
             if b.axis != -1 or b.tensor_scale_inv is None:
                 raise ValueError("the forward weight copy must be a tensor-wise scaled copy quantised along axis=-1")
-            w_row, w_ru, w_si = _cached_codes(b, kc), b.scales, b.tensor_scale_inv
+            w_row, w_ru, w_si = _cached_codes(b, kc), _cached_scales(b, kc), b.tensor_scale_inv
             w_col = w_cu = None
             if need_dgrad:
                 if b_t is not None:
-                    w_col, w_cu = _cached_codes(b_t, kc), b_t.scales
+                    w_col, w_cu = _cached_codes(b_t, kc), _cached_scales(b_t, kc)
                 else:
                     w_col, w_cu = _transposed_cache(b, kc)
         else:

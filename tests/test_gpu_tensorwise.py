@@ -311,9 +311,17 @@ def test_cached_weights_give_the_same_results(gpu, hybrid, transpose_cache):
     (dx0,) = torch.autograd.grad(y0, [x], dy)
     pair = QuantizedTensorPair(*create_quantized_weight(w, float8_e4m3, cfg, need_weight_transpose_cache=transpose_cache))
     assert (pair.data_t is None) is (not transpose_cache) and pair.data.tensor_scale_inv is not None
+    assert pair.data.kchunk == 2          # stored for the ring kernel, like the operands of a call on bf16 weights
     y1 = turbo.ops.grouped_gemm_fp8(x, pair, gl, config=cfg)
     (dx1,) = torch.autograd.grad(y1, [x], dy)
     assert torch.equal(y0, y1) and torch.equal(dx0, dx1)
+    # caches in the other layouts serve the call as well
+    for lay in (0, 1):
+        other = QuantizedTensorPair(*create_quantized_weight(w, float8_e4m3, cfg, need_weight_transpose_cache=transpose_cache,
+                                                             kchunk=lay))
+        y2 = turbo.ops.grouped_gemm_fp8(x, other, gl, config=cfg)
+        (dx2,) = torch.autograd.grad(y2, [x], dy)
+        assert torch.equal(y0, y2) and torch.equal(dx0, dx2), lay
     deq = pair.data.dequantize()
     assert deq.shape == w.shape and (deq.float() - w.float()).abs().max() <= 0.07 * w.float().abs().max()
 

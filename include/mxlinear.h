@@ -284,7 +284,7 @@ int mxl_quantize_weight_tensorwise(const void* w_bf16, int64_t batch, int64_t n,
  * factors read on the device (the scale_inv outputs above), applied in fp32 before the rounding to bf16.  The operands
  * are what the two quantisers above write: their block scales are the unit byte by construction, so the scale arrays
  * are NOT read (they may be null); an operand with other block scales belongs to mxl_grouped_gemm_nt / _wgrad.
- * Operand formats: E4M3 x E4M3, E5M2 (a) x E4M3 (b), and E5M2 x E5M2 on row-major or K-chunk-major operands. */
+ * Operand formats: E4M3 x E4M3, E5M2 (a) x E4M3 (b), and E5M2 x E5M2, in every layout. */
 int mxl_grouped_gemm_nt_scaled(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                                const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                                int num_groups, int64_t total_m, int64_t n, int64_t k, const float* alpha_a,

@@ -1257,7 +1257,8 @@ static int launch_gemm_ring(const GemmArgs& a, int64_t max_tiles, hipStream_t st
 template <int MODE>
 static bool ring_serves(int afmt, int bfmt, const GemmArgs& a) {
     if (a.num_groups > RING_MAX_GROUPS) return false;
-    if (a.alpha_a != nullptr) return bfmt == MXL_FMT_E4M3 && (afmt == MXL_FMT_E4M3 || afmt == MXL_FMT_E5M2);
+    if (a.alpha_a != nullptr)    // per-tensor factors: E4M3 or E5M2 rows against E4M3, and E5M2 against E5M2
+        return (bfmt == MXL_FMT_E4M3 && (afmt == MXL_FMT_E4M3 || afmt == MXL_FMT_E5M2)) || (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E5M2);
     // MX: E4M3 x E4M3, in the forward / dgrad GEMM E4M3 activations against E2M1 weights, and E2M1 x E2M1
     if (afmt == MXL_FMT_E2M1) return bfmt == MXL_FMT_E2M1;
     return afmt == MXL_FMT_E4M3 && (bfmt == MXL_FMT_E4M3 || (bfmt == MXL_FMT_E2M1 && MODE == MODE_FWD));
@@ -1265,6 +1266,7 @@ static bool ring_serves(int afmt, int bfmt, const GemmArgs& a) {
 template <int MODE>
 static int dispatch_gemm_ring(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     if (a.alpha_a != nullptr) {
+        if (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E5M2, MODE, true>(a, max_tiles, st);
         if (afmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
         return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE, true>(a, max_tiles, st);
     }

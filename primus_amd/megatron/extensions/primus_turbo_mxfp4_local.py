@@ -238,8 +238,7 @@ def _fp8_tw_backward(grad_2d, input_2d, weight, fmt):
     if n % K.BLOCK or k % K.BLOCK:
         raise ValueError(f"the FP8 backward needs weight dims that are multiples of {K.BLOCK} (got {n} x {k})")
     m = grad_2d.shape[0]
-    # E5M2 x E5M2 runs on the 2-slot GEMM kernel: row-major or K-chunk-major operands
-    kc = int(bool(K.kchunk_default() and K.kchunk_fits(1, n, k, m)))
+    kc = K.pick_layout(1, n, k, m, fp8=True)
     d_row, d_ru, d_col, d_cu, d_si = K.quantize_tensorwise_impl(grad_2d, fmt, rowwise=True, colwise=True,
                                                                pad_to=K.GEMM_K_ALIGN, kchunk=kc)
     _, _, x_col, x_cu, x_si = K.quantize_tensorwise_impl(input_2d.contiguous(), fmt, rowwise=False, colwise=True,

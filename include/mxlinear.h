@@ -116,6 +116,10 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
  *                  [ld / 64][rows][32 bytes], the partner of FP8 activations, unless MXL_QF_KSTEP128 is set too:
  *                  then in steps of 128 elements like the activations, the partner of E2M1 activations.
  *
+ *   MXL_QF_COL_KCHUNK  (with MXL_QF_KSTEP, activation quantisers only) the transposed copy alone is written K-chunk-major
+ *                  with row-major scales, as MXL_QF_KCHUNK would: forward and dgrad then run on the ring kernel while the
+ *                  weight-gradient GEMM that accumulates into a float32 buffer (MXL_GF_ACCUM_F32) reads its layout.
+ *
  * and, for fmt = MXL_FMT_E2M1 only, the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
  * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288):
  *
@@ -142,6 +146,7 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
 #define MXL_QF_KCHUNK 4u
 #define MXL_QF_KSTEP 8u
 #define MXL_QF_KSTEP128 16u
+#define MXL_QF_COL_KCHUNK 32u
 int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                     const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                     void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);

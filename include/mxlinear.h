@@ -116,10 +116,6 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
  *                  [ld / 64][rows][32 bytes], the partner of FP8 activations, unless MXL_QF_KSTEP128 is set too:
  *                  then in steps of 128 elements like the activations, the partner of E2M1 activations.
  *
- *   MXL_QF_COL_KCHUNK  (with MXL_QF_KSTEP, activation quantisers only) the transposed copy alone is written K-chunk-major
- *                  with row-major scales, as MXL_QF_KCHUNK would: forward and dgrad then run on the ring kernel while the
- *                  weight-gradient GEMM that accumulates into a float32 buffer (MXL_GF_ACCUM_F32) reads its layout.
- *
  * and, for fmt = MXL_FMT_E2M1 only, the options of the MXFP4 recipe's dual quantiser, quantize_mxfp4_dual
  * (primus_turbo_mxfp4_local.py:133-161; per-operand settings :234-288):
  *
@@ -146,7 +142,6 @@ int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld,
 #define MXL_QF_KCHUNK 4u
 #define MXL_QF_KSTEP 8u
 #define MXL_QF_KSTEP128 16u
-#define MXL_QF_COL_KCHUNK 32u
 int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                     const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                     void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream);
@@ -215,12 +210,13 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
 #define MXL_GF_KCHUNK 1u
 /* MXL_GF_KSTEP (instead of MXL_GF_KCHUNK): codes and scales of both operands are K-step-major, as written by the
  * quantisers with MXL_QF_KSTEP.  FP8-format operands, FP8 rows against E2M1 weights in 64-element steps (forward /
- * dgrad), or E2M1 against E2M1 in 128-element steps (MXL_QF_KSTEP128 weights); at most 128 groups, bf16 output (no
- * MXL_GF_ACCUM_F32); anything else returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
+ * dgrad), or E2M1 against E2M1 in 128-element steps (MXL_QF_KSTEP128 weights); at most 128 groups; anything else
+ * returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
  * With either layout flag the kernels request whole 256-row tiles of a K chunk: a code or scale array whose row count
  * is not a multiple of 256 must be followed by 32 KiB of readable memory (the values read there are never used). */
 #define MXL_GF_KSTEP 4u
-/* mxl_grouped_gemm_wgrad_ex / _scaled only, together with MXL_GF_KCHUNK: c_bf16 points to FLOAT32 [g, n, k] and the
+/* mxl_grouped_gemm_wgrad_ex / _scaled only, together with MXL_GF_KCHUNK or MXL_GF_KSTEP (the latter: E4M3 x E4M3,
+ * E2M1 x E2M1 and, scaled, E4M3 | E5M2 x E4M3): c_bf16 points to FLOAT32 [g, n, k] and the
  * result is ADDED to it in fp32 (no rounding to bf16).  This is the gradient-accumulation fusion of the reference
  * (fuse_bgrad_accum_pattern = "megatron": the GEMM's beta = 1 epilogue adds into weight.main_grad,
  * primus_turbo.py:166-240, 243-275) -- available here for the MX recipes too.  With no tokens nothing is added. */

@@ -27,7 +27,7 @@ GEMM_K_ALIGN = 128  # the GEMM kernels take the contraction dim in multiples of 
 MAX_GROUPS = 1024
 ACT_SILU, ACT_GELU = 0, 1
 PROBS_F32, PROBS_BF16 = 0, 1
-QF_SR, QF_RHT_COL, QF_KCHUNK, QF_KSTEP, QF_KSTEP128, QF_COL_KCHUNK = 1, 2, 4, 8, 16, 32   # flags of mxl_quantize_ex
+QF_SR, QF_RHT_COL, QF_KCHUNK, QF_KSTEP, QF_KSTEP128 = 1, 2, 4, 8, 16   # flags of mxl_quantize_ex
 GF_KCHUNK = 1                               # flag of the GEMM _ex entry points: operands are K-chunk-major
 GF_KSTEP = 4                                # ... K-step-major codes and scales (ring kernel)
 GF_ACCUM_F32 = 2                            # wgrad: the output is float32 and the result is added to it

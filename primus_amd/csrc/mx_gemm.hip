@@ -646,8 +646,11 @@ constexpr int ring_lds_bytes() {
 }
 
 
-template <int AFMT, int BFMT, int MODE, bool ALPHA>
+template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
+    // ACCUM (wgrad): p.c is a float32 buffer the result is ADDED to (one workgroup per output tile: no race, and the
+    // sum does not depend on any order)
+    static_assert(!ACCUM || MODE == MODE_WGRAD, "the accumulating epilogue belongs to the weight-gradient GEMM");
     // F44: both operands FP4, stored like FP8 operands byte for byte -- 64-byte rows per K step, which then hold 128
     // elements: a step is two MFMA K steps (the low and the high half of every fragment register group), scale panels
     // cover 4 steps instead of 8, and a contraction range may be an odd number of steps.
@@ -942,11 +945,13 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                 const int first = (rem / width) * GROUP_M;
                 const int gsz = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
                 const int64_t row0 = (int64_t)(first + (rem % width) % gsz) * BM, col0 = (int64_t)((rem % width) / gsz) * BN;
-                uint16_t* ct = p.c + ((int64_t)grp * p.m + row0) * p.n + col0;
-                const int mv = (p.m - row0) < BM ? (int)(p.m - row0) : BM, nv = (p.n - col0) < BN ? (int)(p.n - col0) : BN;
-                for (int r = t >> 5; r < mv; r += GTHREADS / 32) {
-                    const int c = (t & 31) * 8;
-                    if (c < nv) store16_streaming((uint8_t*)(ct + (int64_t)r * p.n + c), make_uint4(0u, 0u, 0u, 0u));
+                if (!ACCUM) {    // (nothing to add for a group without tokens)
+                    uint16_t* ct = p.c + ((int64_t)grp * p.m + row0) * p.n + col0;
+                    const int mv = (p.m - row0) < BM ? (int)(p.m - row0) : BM, nv = (p.n - col0) < BN ? (int)(p.n - col0) : BN;
+                    for (int r = t >> 5; r < mv; r += GTHREADS / 32) {
+                        const int c = (t & 31) * 8;
+                        if (c < nv) store16_streaming((uint8_t*)(ct + (int64_t)r * p.n + c), make_uint4(0u, 0u, 0u, 0u));
+                    }
                 }
                 tl = tile_at(++round);
             }
@@ -1163,8 +1168,55 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
                     MXL_PIN;
                 });
             };
-            if (full) write_out(std::true_type{});
-            else write_out(std::false_type{});
+            // ACCUM: the same staging with float32 patches of 32 rows x 32 columns (sixteen per wave; 16-byte pieces
+            // XOR-swizzled by (row / 2) % 8), read back one word per lane -- two whole output rows of the patch per
+            // instruction -- and added to the buffer with float atomics that return nothing: the L2 does the
+            // read-modify-write, the wave waits for no old value.  Every output element belongs to one workgroup and gets
+            // exactly one add per launch.
+            auto add_out = [&](auto full_tag) __attribute__((always_inline)) {
+                constexpr bool FULL = decltype(full_tag)::value;
+                float* ctile32 = (float*)p.c + ((int64_t)d.c_row0 * p.n + d.c_col0);
+                uint8_t* wr32 = stg + elr * 128;
+                const int wsw32 = (elr >> 1) & 7;
+                const int rw = lo & 31, rr2 = lo >> 5;                         // word of the row, row parity while reading
+                const uint8_t* rd32 = stg + rr2 * 128 + 4 * (rw & 3);
+                const uint32_t lane_off32 = (uint32_t)(rr2 * (int)p.n + rw);  // elements from a patch's first one
+                float val[16];
+                static_for<0, 17>([&](auto it_tag) {
+                    constexpr int it = decltype(it_tag)::value;
+                    if constexpr (it < 16) {
+                        constexpr int i = it >> 2, j = it & 3;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            v4f o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                            if (ALPHA) o *= alpha;
+                            *(v4f*)(wr32 + 16 * ((2 * q + eg) ^ wsw32)) = o;
+                        }
+                    }
+                    if constexpr (it > 0) {
+                        constexpr int i = (it - 1) >> 2, j = (it - 1) & 3;
+                        float* base = ctile32 + (int64_t)(wm * 128 + i * 32) * p.n + wn * 128 + j * 32;   // uniform
+                        const bool col_ok = FULL || wn * 128 + j * 32 + rw < n_valid;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (FULL || (col_ok && wm * 128 + i * 32 + 2 * v + rr2 < m_valid))
+                                unsafeAtomicAdd(base + (int64_t)(2 * v) * p.n + lane_off32, val[v]);
+                    }
+                    if constexpr (it < 16) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)    // row 2 v + rr2: its swizzle is v % 8
+                            val[v] = *(const float*)(rd32 + v * 256 + 16 * ((rw >> 2) ^ (v & 7)));
+                    }
+                    MXL_PIN;
+                });
+            };
+            if constexpr (ACCUM) {
+                if (full) add_out(std::true_type{});
+                else add_out(std::false_type{});
+            } else {
+                if (full) write_out(std::true_type{});
+                else write_out(std::false_type{});
+            }
         }
         if (tile_n >= total_tiles) break;
         __syncthreads();      // every wave has left the patch: its slot takes K step 3 of the next tile
@@ -1233,13 +1285,13 @@ static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
-template <int AFMT, int BFMT, int MODE, bool ALPHA>
+template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false>
 static int launch_gemm_ring(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = ring_lds_bytes();
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set[64];
     const int slot = current_device_slot();
-    auto kern = mx_gemm_ring_kernel<AFMT, BFMT, MODE, ALPHA>;
+    auto kern = mx_gemm_ring_kernel<AFMT, BFMT, MODE, ALPHA, ACCUM>;
     if (!attr_set[slot].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
@@ -1315,6 +1367,19 @@ static int dispatch_wgrad_accum(int afmt, int bfmt, const GemmArgs& a, int64_t m
     return MXL_EINVAL;
 }
 
+// the weight-gradient GEMM that adds into a float32 buffer, on K-step-major operands
+static int dispatch_wgrad_accum_ring(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    constexpr int W = MODE_WGRAD;
+    if (a.alpha_a != nullptr) {
+        if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, W, true, true>(a, max_tiles, st);
+        if (afmt == MXL_FMT_E5M2 && bfmt == MXL_FMT_E4M3) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, W, true, true>(a, max_tiles, st);
+        return MXL_EINVAL;
+    }
+    if (afmt == MXL_FMT_E4M3 && bfmt == MXL_FMT_E4M3) return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, W, false, true>(a, max_tiles, st);
+    if (afmt == MXL_FMT_E2M1 && bfmt == MXL_FMT_E2M1) return launch_gemm_ring<MXL_FMT_E2M1, MXL_FMT_E2M1, W, false, true>(a, max_tiles, st);
+    return MXL_EINVAL;
+}
+
 // a_rows / b_rows: rows of the whole operands (for the 4 GiB bound of the chunk-major layout)
 // layout: 0 row-major codes, 1 K-chunk-major codes, 2 K-step-major codes and scales
 template <int MODE>
@@ -1322,11 +1387,12 @@ static int dispatch_gemm(int afmt, int bfmt, const GemmArgs& a, int64_t max_tile
                          hipStream_t st, bool accum = false) {
     const bool kchunk = layout == 1;
     if (layout == 2) {
-        if (accum || !ring_serves<MODE>(afmt, bfmt, a)) return MXL_EINVAL;
+        if ((accum && MODE != MODE_WGRAD) || !ring_serves<MODE>(afmt, bfmt, a)) return MXL_EINVAL;
         // offsets inside an operand are 32-bit
         if (a_rows * a.k >= ((int64_t)1 << 32) || b_rows * a.k >= ((int64_t)1 << 32)) return MXL_EINVAL;
         // the kernel keeps a tile's first output row in 32 bits
         if ((MODE == MODE_WGRAD ? (int64_t)a.num_groups * a.m : a.total_m) >= ((int64_t)1 << 31)) return MXL_EINVAL;
+        if (accum) return dispatch_wgrad_accum_ring(afmt, bfmt, a, max_tiles, st);
         return dispatch_gemm_ring<MODE>(afmt, bfmt, a, max_tiles, st);
     }
     if (accum) {
@@ -1423,7 +1489,7 @@ static int grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_f
     if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP | MXL_GF_ACCUM_F32)) return MXL_EINVAL;
     if ((flags & MXL_GF_KCHUNK) && (flags & MXL_GF_KSTEP)) return MXL_EINVAL;
     const bool accum = (flags & MXL_GF_ACCUM_F32) != 0;
-    if (accum && !(flags & MXL_GF_KCHUNK)) return MXL_EINVAL;
+    if (accum && !(flags & (MXL_GF_KCHUNK | MXL_GF_KSTEP))) return MXL_EINVAL;
     if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
     if (num_groups < 0 || num_groups > MXL_MAX_GROUPS) return MXL_EINVAL;

@@ -77,8 +77,7 @@ struct QuantArgs {
     // each other, so a GEMM tile's slot is one contiguous block and this kernel writes 128 x 128-element
     // pieces contiguously.  chunk_rows_row / chunk_rows_col: rows of the whole row-wise / transposed operand.
     // 2: K-step-major (FP8 only): codes [ld / 64][rows][64], scales [ceil(ld / 512)][rows][16].
-    int kchunk;        // layout of the row-wise copy (0 row-major, 1 K-chunk-major, 2 / 3 K-step-major)
-    int kchunk_col;    // layout of the transposed copy: the same, or 1 beside a K-step-major row-wise copy
+    int kchunk;
     int64_t chunk_rows_row, chunk_rows_col;
     uint64_t sr_seed;       // SR kernels: seed of the stochastic rounding
     uint32_t rht_signs;     // RHT kernels: sign bit i flips row i of every 16-row group before the transform
@@ -491,7 +490,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             uint8_t* dst = a.s_colT + (out_rows_base + col0 + t) * (a.W / 32) + m0 / 32;
             const uint32_t v = scol_tile[t];
             const int64_t nb = (a.W - m0) / 32;
-            if (a.kchunk_col >= 2) {
+            if (a.kchunk >= 2) {
                 const int64_t mt = seg_tile >= 0 ? (int64_t)seg_tile : m0 / QT;
                 store_panel_scales(a.s_colT + ((seg_pan0 + mt / 4) * a.chunk_rows_col + out_rows_base + col0 + t) * 16, (int)(mt & 3), v);
             } else if (nb >= 4 && ((a.W / 32) & 3) == 0) {
@@ -511,11 +510,11 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             const int ch = t % LPR;
             if (col0 + c < a.cols && 16 * ch < avail) {
                 const uint4 v = *(const uint4*)(t_tile + c * TPITCH + 16 * ch);
-                const int64_t at = (FP4 && a.kchunk_col == 2)
+                const int64_t at = (FP4 && a.kchunk == 2)
                                        ? ((2 * (m0 / QT) + (ch >> 1)) * a.chunk_rows_col + out_rows_base + col0 + c) * (QT / 4) + 16 * (ch & 1)
-                                   : a.kchunk_col == 2
+                                   : a.kchunk == 2
                                        ? ((2 * (m0 / QT) + (ch >> 2)) * a.chunk_rows_col + out_rows_base + col0 + c) * (QT / 2) + 16 * (ch & 3)
-                                   : a.kchunk_col ? ((m0 / QT) * a.chunk_rows_col + out_rows_base + col0 + c) * ROWB + 16 * ch
+                                   : a.kchunk ? ((m0 / QT) * a.chunk_rows_col + out_rows_base + col0 + c) * ROWB + 16 * ch
                                               : (out_rows_base + col0 + c) * wbytes + m0b + 16 * ch;
                 store16_streaming(a.q_colT + at, v);
             }
@@ -702,10 +701,9 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
                        int act, const void* probs, int probs_dtype, const uint8_t* row_mask, void* stream,
                        bool sr = false, uint64_t sr_seed = 0, bool rht = false, uint32_t rht_signs = 0,
                        int kchunk = 0, const void* norm_w = nullptr, const void* tensor_amax = nullptr,
-                       void* scale_inv_out = nullptr, bool col_kchunk = false) {
+                       void* scale_inv_out = nullptr) {
     if (row_ld == 0) row_ld = cols;
     if (kchunk < 0) return MXL_EINVAL;                  // contradictory layout flags
-    if (col_kchunk && kchunk < 2) return MXL_EINVAL;     // the option belongs to a K-step-major row-wise copy
     if (kchunk == 2 && fmt == MXL_FMT_E2M1) kchunk = 3;  // E2M1 activations: the K step is 128 elements (64-byte rows)
     if (kchunk == 3 && fmt != MXL_FMT_E2M1) return MXL_EINVAL;
     if (kchunk && q_row && row_ld % QT != 0) return MXL_EINVAL;   // whole 128-element chunks
@@ -738,7 +736,6 @@ static int quantize_1d(const void* x_bf16, int64_t rows, int64_t cols, int64_t r
     a.sr_seed = sr_seed;
     a.rht_signs = rht_signs & 0xFFFFu;
     a.kchunk = kchunk;
-    a.kchunk_col = col_kchunk ? 1 : kchunk;
     a.chunk_rows_row = rows;
     a.chunk_rows_col = cols;
     const int64_t gx = q_colT ? a.W / QT : (rows + QT - 1) / QT;
@@ -768,11 +765,10 @@ extern "C" int mxl_quantize(const void* x_bf16, int64_t rows, int64_t cols, int6
 extern "C" int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_ld, int fmt, int scale_mode,
                                const int64_t* group_lens, int num_groups, void* q_row, void* s_row, void* q_colT,
                                void* s_colT, uint32_t flags, uint64_t sr_seed, uint32_t rht_signs, void* stream) {
-    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128 | MXL_QF_COL_KCHUNK)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_SR | MXL_QF_RHT_COL | MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, cols, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT,
                        s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, (flags & MXL_QF_SR) != 0, sr_seed,
-                       (flags & MXL_QF_RHT_COL) != 0, rht_signs, qf_layout(flags), nullptr, nullptr, nullptr,
-                       (flags & MXL_QF_COL_KCHUNK) != 0);
+                       (flags & MXL_QF_RHT_COL) != 0, rht_signs, qf_layout(flags));
 }
 
 extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int probs_dtype, const uint8_t* row_mask,
@@ -782,20 +778,19 @@ extern "C" int mxl_glu_probs_quantize(const void* x_bf16, const void* probs, int
     if (act != MXL_ACT_SILU && act != MXL_ACT_GELU) return MXL_EINVAL;
     if (probs_dtype != MXL_PROBS_F32 && probs_dtype != MXL_PROBS_BF16) return MXL_EINVAL;
     if (rows > 0 && !probs) return MXL_EINVAL;
-    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128 | MXL_QF_COL_KCHUNK)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, f, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT, act,
-                       probs, probs_dtype, row_mask, stream, false, 0, false, 0, qf_layout(flags), nullptr, nullptr, nullptr,
-                       (flags & MXL_QF_COL_KCHUNK) != 0);
+                       probs, probs_dtype, row_mask, stream, false, 0, false, 0, qf_layout(flags));
 }
 
 extern "C" int mxl_rmsnorm_quantize(const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows, int64_t k,
                                     int64_t row_ld, int fmt, int scale_mode, const int64_t* group_lens, int num_groups,
                                     void* q_row, void* s_row, void* q_colT, void* s_colT, uint32_t flags, void* stream) {
     if (!w_bf16 || (rows > 0 && !rstd_f32)) return MXL_EINVAL;
-    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128 | MXL_QF_COL_KCHUNK)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_KSTEP128)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, k, row_ld, fmt, scale_mode, group_lens, num_groups, q_row, s_row, q_colT, s_colT,
                        PRO_RMSNORM, rstd_f32, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
-                       qf_layout(flags), w_bf16, nullptr, nullptr, (flags & MXL_QF_COL_KCHUNK) != 0);
+                       qf_layout(flags), w_bf16);
 }
 
 static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld, int64_t n_ld, int fmt,
@@ -832,7 +827,6 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
     a.sr_seed = 0;
     a.rht_signs = 0;
     a.kchunk = kchunk;
-    a.kchunk_col = kchunk;
     a.chunk_rows_row = batch * n;   // the batch is one operand of batch * n rows (resp. batch * k for the transposed copy)
     a.chunk_rows_col = batch * k;
     const int64_t gx = batch * ((n + QT - 1) / QT);
@@ -860,10 +854,10 @@ extern "C" int mxl_quantize_tensorwise(const void* x_bf16, int64_t rows, int64_t
                                        void* s_row, void* q_colT, void* s_colT, void* scale_inv_f32, uint32_t flags,
                                        void* stream) {
     if (!amax_f32 || (fmt != MXL_FMT_E4M3 && fmt != MXL_FMT_E5M2)) return MXL_EINVAL;
-    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP | MXL_QF_COL_KCHUNK)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_QF_KCHUNK | MXL_QF_KSTEP)) return MXL_EINVAL;
     return quantize_1d(x_bf16, rows, cols, row_ld, fmt, MXL_SCALE_OCP_FLOOR, group_lens, num_groups, q_row, s_row, q_colT,
                        s_colT, -1, nullptr, MXL_PROBS_F32, nullptr, stream, false, 0, false, 0,
-                       qf_layout(flags), nullptr, amax_f32, scale_inv_f32, (flags & MXL_QF_COL_KCHUNK) != 0);
+                       qf_layout(flags), nullptr, amax_f32, scale_inv_f32);
 }
 
 extern "C" int mxl_quantize_weight_tensorwise(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,

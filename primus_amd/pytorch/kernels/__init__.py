@@ -142,16 +142,6 @@ def _qflag(kchunk) -> int:
     return (0, _lib.QF_KCHUNK, _lib.QF_KSTEP, _lib.QF_KSTEP | _lib.QF_KSTEP128)[_layout(kchunk)]
 
 
-def _col_layout(kchunk, col_kchunk: bool):
-    """Layout of the transposed copy: the row-wise copy's, or K-chunk-major beside a K-step-major row-wise copy when the
-    weight-gradient GEMM is the one that accumulates into a float32 buffer (it reads that layout)."""
-    return LAYOUT_KCHUNK if (col_kchunk and _paneled(kchunk)) else kchunk
-
-
-def _qflag2(kchunk, col_kchunk: bool) -> int:
-    return _qflag(kchunk) | (_lib.QF_COL_KCHUNK if (col_kchunk and _paneled(kchunk)) else 0)
-
-
 def _gflag(kchunk) -> int:
     return (0, _lib.GF_KCHUNK, _lib.GF_KSTEP, _lib.GF_KSTEP)[_layout(kchunk)]
 
@@ -299,12 +289,8 @@ def quantize_mx_impl(
     sr_seed: Optional[int] = None,
     rht_signs: Optional[int] = None,
     kchunk=False,
-    col_kchunk: bool = False,
 ):
     """MX-quantise bf16 ``x[rows, cols]``.
-
-    ``col_kchunk`` (beside a K-step-major ``kchunk``): the transposed copy alone comes back K-chunk-major with
-    row-major scales.
 
     ``kchunk`` stores the codes K-chunk-major, the layout the GEMMs load fastest: the code tensors come
     back 3-D, ``[ld / 128, rows, 128]`` (``64`` bytes in the last dim for FP4) instead of ``[rows, ld]``
@@ -348,9 +334,8 @@ def quantize_mx_impl(
         s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        kcol = _col_layout(kchunk, col_kchunk)
-        q_col = _empty_tail(_code_shape(cols, W, per, kcol), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(cols, W, kcol, G), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
         row_ok = rows > 0
@@ -361,7 +346,7 @@ def quantize_mx_impl(
                 rc = _lib.load().mxl_quantize(*args, _stream())
             else:
                 flags = ((_lib.QF_SR if sr_seed is not None else 0) | (_lib.QF_RHT_COL if rht_signs is not None else 0)
-                         | _qflag2(kchunk, col_kchunk))
+                         | _qflag(kchunk))
                 rc = _lib.load().mxl_quantize_ex(
                     *args, flags, int(sr_seed or 0) & 0xFFFFFFFFFFFFFFFF, int(rht_signs or 0) & 0xFFFF, _stream())
         _lib.check(rc, "mxl_quantize")
@@ -555,8 +540,8 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
 
 def _accum_target(accum_into, shape, kchunk, device):
     """Checks the float32 buffer a wgrad GEMM is to add its result to."""
-    if _layout(kchunk) != LAYOUT_KCHUNK:
-        raise ValueError("accumulating wgrad needs K-chunk-major operands")
+    if _layout(kchunk) == LAYOUT_ROWMAJOR:
+        raise ValueError("accumulating wgrad needs K-chunk-major or K-step-major operands")
     if (accum_into.dtype != torch.float32 or tuple(accum_into.shape) != tuple(shape) or not accum_into.is_contiguous()
             or accum_into.device != device):
         raise ValueError(f"accum_into must be a contiguous float32 tensor of shape {tuple(shape)} on the operands' device")
@@ -659,7 +644,7 @@ def glu_with_probs_bwd_impl(dy, x, probs, row_mask, activation: str):
 
 def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *,
                                  colwise: bool = False, group_lens: Optional[torch.Tensor] = None, pad_to: int = 1,
-                                 kchunk=False, col_kchunk: bool = False):
+                                 kchunk=False):
     """``quantize_mx_impl(glu_with_probs_fwd_impl(x, ...))`` in one pass over ``x [tokens, 2F]``, the
     activated tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
     act, pd, row_mask = _glu_args(x, probs, row_mask, activation)
@@ -679,16 +664,15 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, G)
-        kcol = _col_layout(kchunk, col_kchunk)
-        q_col = _empty_tail(_code_shape(f, W, per, kcol), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(f, W, kcol, G), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(f, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         row_ok = rows > 0
         with _hooked("glu_probs_quantize", rows=rows, cols=f, fmt=fmt, rowwise=True, colwise=colwise):
             rc = _lib.load().mxl_glu_probs_quantize(
                 _ptr(x) if row_ok else None, _ptr(probs), pd, _ptr(row_mask), rows, f, row_ld, act, fmt, scale_mode,
                 _ptr(group_lens), G, _ptr(q_row) if row_ok else None, _ptr(s_row) if row_ok else None, _ptr(q_col),
-                _ptr(s_col), _qflag2(kchunk, col_kchunk), _stream(),
+                _ptr(s_col), _qflag(kchunk), _stream(),
             )
         _lib.check(rc, "mxl_glu_probs_quantize")
     cd = _code_dtype(fmt)
@@ -717,7 +701,7 @@ def amax_impl(x: torch.Tensor) -> torch.Tensor:
 
 def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool = False,
                              group_lens: Optional[torch.Tensor] = None, pad_to: int = 1, kchunk: bool = False,
-                             amax: Optional[torch.Tensor] = None, col_kchunk: bool = False):
+                             amax: Optional[torch.Tensor] = None):
     """``(q_row, s_row, q_colT, s_colT, scale_inv)`` for a 2-D bfloat16 ``x``: codes in the layouts of
     ``quantize_mx_impl`` but scaled by ``fp8_max / max(amax, 1e-12)`` for the whole tensor; the ``s_*`` arrays
     hold the unit E8M0 byte (they only make the codes acceptable to the GEMMs), ``scale_inv`` is the float32
@@ -744,9 +728,8 @@ def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool
         s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        kcol = _col_layout(kchunk, col_kchunk)
-        q_col = _empty_tail(_code_shape(cols, W, 1, kcol), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(cols, W, kcol, G), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows == 0 and not (colwise and q_col.numel()):
         scale_inv.fill_(1e-12 / (448.0 if fmt == _lib.FMT_E4M3 else 57344.0))
     else:
@@ -754,7 +737,7 @@ def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool
             rc = _lib.load().mxl_quantize_tensorwise(
                 _ptr(x) if rows else None, rows, cols, row_ld if rowwise else 0, fmt, _ptr(amax),
                 _ptr(group_lens) if colwise else None, G, _ptr(q_row) if rows else None, _ptr(s_row) if rows else None,
-                _ptr(q_col), _ptr(s_col), _ptr(scale_inv), _qflag2(kchunk, col_kchunk), _stream(),
+                _ptr(q_col), _ptr(s_col), _ptr(scale_inv), _qflag(kchunk), _stream(),
             )
         _lib.check(rc, "mxl_quantize_tensorwise")
     cd = _code_dtype(fmt)
@@ -863,8 +846,6 @@ def gemm_tw_wgrad_impl(a_t, a_t_unit, a_scale_inv, b_t, b_t_unit, b_scale_inv, g
     if wa != W or wb != W:
         raise ValueError(f"transposed operands must have padded width {W}")
     if kstep:
-        if accum_into is not None:
-            raise ValueError("the accumulating wgrad epilogue takes K-chunk-major operands")
         for sc, r, what in ((a_t_unit, n, "a_t_unit"), (b_t_unit, k, "b_t_unit")):
             if tuple(sc.shape) != _scale_shape(r, W, kchunk, G) or not sc.is_contiguous():
                 raise ValueError(f"{what} must be the K-step-major scale array of its operand")
@@ -938,7 +919,7 @@ def rmsnorm_bwd_impl(dy, x, weight, rstd):
 
 
 def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCALE_OCP_FLOOR, *, colwise: bool = False,
-                          pad_to: int = 1, kchunk=False, col_kchunk: bool = False):
+                          pad_to: int = 1, kchunk=False):
     """``quantize_mx_impl(rmsnorm_fwd_impl(x, weight, eps)[0])`` in one pass over ``x`` given ``rstd``, the
     normalised tensor never reaching memory; same return tuple (the row-wise copy is always produced)."""
     _norm_args(x, weight)
@@ -958,13 +939,12 @@ def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCAL
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, 0)
-        kcol = _col_layout(kchunk, col_kchunk)
-        q_col = _empty_tail(_code_shape(k, W, per, kcol), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(k, W, kcol), dtype=torch.uint8, device=dev)
+        q_col = _empty_tail(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = _empty_tail(_scale_shape(k, W, kchunk), dtype=torch.uint8, device=dev)
     with _hooked("rmsnorm_quantize", rows=rows, cols=k, fmt=fmt, rowwise=True, colwise=colwise):
         rc = _lib.load().mxl_rmsnorm_quantize(
             _ptr(x), _ptr(weight), _ptr(rstd), rows, k, row_ld, fmt, scale_mode, None, 0, _ptr(q_row), _ptr(s_row),
-            _ptr(q_col), _ptr(s_col), _qflag2(kchunk, col_kchunk), _stream(),
+            _ptr(q_col), _ptr(s_col), _qflag(kchunk), _stream(),
         )
     _lib.check(rc, "mxl_rmsnorm_quantize")
     cd = _code_dtype(fmt)

@@ -166,28 +166,25 @@ class _MXLinearFunction(torch.autograd.Function):
         kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=fp8, fp4=fp4)
         if isinstance(b, QuantizedTensor):   # cached copies decide: the call uses the layout they are stored in
             kc = _cache_layout(b, b_t, kc, fp8, groups, fp4)
-        # A weight gradient that is added to a float32 buffer inside the GEMM reads K-chunk-major copies: beside
-        # K-step-major row-wise copies (forward and dgrad on the ring kernel) the transposed ones are written that way
-        ckc = bool(accum is not None and _fusable(accum[0]) and kc >= K.LAYOUT_KSTEP)
+        # (a weight gradient that is added to a float32 buffer inside the GEMM runs on either chunked layout)
         # activations: row-wise for the forward GEMM, transposed col-wise kept for wgrad
         # (row-wise copies are padded to the GEMM's K granularity, like the reference pads its
         # MXFP4 operands to 128: primus_turbo_mxfp4_local.py:119-124)
         if glu:
             a_row, a_rs, a_col, a_cs = K.glu_with_probs_quantize_impl(
                 a, probs, row_mask, activation, act_fmt, scale_mode, colwise=need_wgrad, group_lens=group_lens,
-                pad_to=K.GEMM_K_ALIGN, kchunk=kc, col_kchunk=ckc,
+                pad_to=K.GEMM_K_ALIGN, kchunk=kc,
             )
         elif norm:
             # X = rmsnorm(a) is formed inside the quantiser from a, the norm weight and the row statistics
             _, rstd = K.rmsnorm_fwd_impl(a, norm_weight.detach(), norm_eps, want_y=False)
             a_row, a_rs, a_col, a_cs = K.rmsnorm_quantize_impl(
                 a, norm_weight.detach(), rstd, act_fmt, scale_mode, colwise=need_wgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
-                col_kchunk=ckc,
             )
         else:
             a_row, a_rs, a_col, a_cs = K.quantize_mx_impl(
                 a, act_fmt, scale_mode, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
-                rht_signs=rht_signs if need_wgrad else None, kchunk=kc, col_kchunk=ckc,
+                rht_signs=rht_signs if need_wgrad else None, kchunk=kc,
             )
         if isinstance(b, QuantizedTensor):
             # cached weight copies (primus_turbo.py:1105-1115): nothing to quantise here
@@ -222,7 +219,6 @@ class _MXLinearFunction(torch.autograd.Function):
         ctx.grad_sr = bool(grad_sr) and act_fmt == _lib.FMT_E2M1
         ctx.rht_signs = rht_signs
         ctx.kchunk = kc
-        ctx.col_kchunk = ckc
         ctx.norm = norm
         ctx.accum = accum      # (float32 buffer the weight gradient is added to, object that gets the flag) or None
         return y
@@ -240,10 +236,9 @@ class _MXLinearFunction(torch.autograd.Function):
             dy, act_fmt, scale_mode, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN,
             sr_seed=K.next_sr_seed() if ctx.grad_sr else None,
             rht_signs=ctx.rht_signs if need_wgrad else None,   # same signs as the saved activation copy
-            kchunk=ctx.kchunk, col_kchunk=ctx.col_kchunk,
+            kchunk=ctx.kchunk,
         )
         kc = ctx.kchunk
-        kw = K.LAYOUT_KCHUNK if ctx.col_kchunk else kc          # layout of the transposed copies the wgrad GEMM reads
         grad_a = grad_b = None
         overlap = _wgrad_overlap and need_dgrad and need_wgrad
         if overlap:
@@ -257,10 +252,10 @@ class _MXLinearFunction(torch.autograd.Function):
                 grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
-            fused = _fusable(target) and kw == K.LAYOUT_KCHUNK   # the GEMM's epilogue adds into the float32 buffer
+            fused = _fusable(target) and kc != K.LAYOUT_ROWMAJOR   # the GEMM's epilogue adds into the float32 buffer
 
             def wgrad():
-                return K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kw,
+                return K.grouped_gemm_mx_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, total_m, kchunk=kc,
                                                     accum_into=target if fused else None)
 
             if overlap:
@@ -336,11 +331,8 @@ class _TWLinearFunction(torch.autograd.Function):
                 kc = 0
         else:
             kc = K.pick_layout(groups, b.shape[-2], b.shape[-1], a.shape[0], fp8=True)
-        # (the accumulating wgrad GEMM reads K-chunk-major transposed copies, as in the MX function)
-        ckc = bool(accum is not None and _fusable(accum[0]) and kc >= K.LAYOUT_KSTEP)
         a_row, a_ru, a_col, a_cu, a_si = K.quantize_tensorwise_impl(
-            a, fwd_fmt, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
-            col_kchunk=ckc)
+            a, fwd_fmt, rowwise=True, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
         if isinstance(b, QuantizedTensor):
             if b.axis != -1 or b.tensor_scale_inv is None:
                 raise ValueError("the forward weight copy must be a tensor-wise scaled copy quantised along axis=-1")
@@ -356,21 +348,19 @@ class _TWLinearFunction(torch.autograd.Function):
                 b.detach(), fwd_fmt, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
         y = K.gemm_tw_nt_impl(a_row, a_ru, a_si, w_row, w_ru, w_si, group_lens, kchunk=kc)
         ctx.save_for_backward(a_col, a_cu, a_si, w_col, w_cu, w_si, group_lens)
-        ctx.cfg = (bwd_fmt, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape), kc, ckc)
+        ctx.cfg = (bwd_fmt, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape), kc)
         ctx.accum = accum
         return y
 
     @staticmethod
     def backward(ctx, dy):
         a_col, a_cu, a_si, w_col, w_cu, w_si, group_lens = ctx.saved_tensors
-        bwd_fmt, total_m, need_dgrad, need_wgrad, w_shape, kc, ckc = ctx.cfg
-        kw = K.LAYOUT_KCHUNK if ckc else kc
+        bwd_fmt, total_m, need_dgrad, need_wgrad, w_shape, kc = ctx.cfg
         dy = dy.contiguous()
         if dy.dtype != torch.bfloat16:
             dy = dy.to(torch.bfloat16)
         d_row, d_ru, d_col, d_cu, d_si = K.quantize_tensorwise_impl(
-            dy, bwd_fmt, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
-            col_kchunk=ckc)
+            dy, bwd_fmt, rowwise=need_dgrad, colwise=need_wgrad, group_lens=group_lens, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
         grad_a = grad_b = None
         overlap = _wgrad_overlap and need_dgrad and need_wgrad
         if overlap:
@@ -381,10 +371,10 @@ class _TWLinearFunction(torch.autograd.Function):
             grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
-            fused = _fusable(target) and kw == K.LAYOUT_KCHUNK
+            fused = _fusable(target) and kc != K.LAYOUT_ROWMAJOR
 
             def wgrad():
-                return K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kw,
+                return K.gemm_tw_wgrad_impl(d_col, d_cu, d_si, a_col, a_cu, a_si, group_lens, total_m, kchunk=kc,
                                             accum_into=target if fused else None)
 
             if overlap:

@@ -307,46 +307,3 @@ def test_fp4_weight_cache_layout_follows_the_activation_format(gpu, act_fp4):
     for y, dx in res[1:]:
         assert _same(res[0][0], y) and _same(res[0][1], dx)
 
-
-@pytest.mark.parametrize("fmt", [0, 1])
-def test_quantisers_can_write_the_transposed_copy_alone_k_chunk_major(gpu, fmt):
-    """Beside a K-step-major row-wise copy the transposed copy may be asked for K-chunk-major with row-major scales (what
-    the weight-gradient GEMM that accumulates into a float32 buffer reads): each copy equals the one a single-layout call
-    writes, for the plain, the tensor-wise, the fused-activation and the fused-norm quantiser."""
-    from primus_amd.pytorch import kernels as K
-
-    lens, cols = [33, 0, 130, 1, 92, 600], 672
-    rows = sum(lens)
-    g = torch.Generator().manual_seed(5)
-    x = (torch.randn(rows, cols, generator=g) * torch.logspace(-2, 2, cols)[None, :]).bfloat16().to(gpu)
-    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
-    step = 3 if fmt == 1 else 2
-    a = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=True, group_lens=gl, kchunk=step)
-    b = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=True, group_lens=gl, kchunk=1)
-    c = K.quantize_mx_impl(x, fmt, rowwise=True, colwise=True, group_lens=gl, kchunk=step, col_kchunk=True)
-    nb = a[0].shape[0] * a[0].shape[2] * (2 if fmt == 1 else 1) // 32      # scale blocks of a row (panel bytes behind them are not written)
-
-    def same_panels(p, q):
-        return torch.equal(K.unpanel(p.view(torch.uint8), nb), K.unpanel(q.view(torch.uint8), nb))
-
-    assert _same(c[0], a[0]) and same_panels(c[1], a[1]) and _same(c[2], b[2]) and _same(c[3], b[3])
-    if fmt == 0:
-        ta = K.quantize_tensorwise_impl(x, 0, rowwise=True, colwise=True, group_lens=gl, kchunk=2)
-        tb = K.quantize_tensorwise_impl(x, 0, rowwise=True, colwise=True, group_lens=gl, kchunk=1)
-        tc = K.quantize_tensorwise_impl(x, 0, rowwise=True, colwise=True, group_lens=gl, kchunk=2, col_kchunk=True)
-        assert _same(tc[0], ta[0]) and _same(tc[2], tb[2]) and _same(tc[3], tb[3]) and torch.equal(tc[4], ta[4])
-    p = torch.rand(rows, generator=g).to(gpu)
-    x2 = torch.cat([x, x.flip(1)], dim=1).contiguous()
-    ga = K.glu_with_probs_quantize_impl(x2, p, None, "silu", fmt, colwise=True, group_lens=gl, kchunk=step)
-    gb = K.glu_with_probs_quantize_impl(x2, p, None, "silu", fmt, colwise=True, group_lens=gl, kchunk=1)
-    gc = K.glu_with_probs_quantize_impl(x2, p, None, "silu", fmt, colwise=True, group_lens=gl, kchunk=step, col_kchunk=True)
-    assert _same(gc[0], ga[0]) and same_panels(gc[1], ga[1]) and _same(gc[2], gb[2]) and _same(gc[3], gb[3])
-    nw = torch.rand(cols, generator=g).bfloat16().to(gpu)
-    _, rstd = K.rmsnorm_fwd_impl(x, nw, 1e-5, want_y=False)
-    na = K.rmsnorm_quantize_impl(x, nw, rstd, fmt, colwise=True, kchunk=step)
-    nb_ = K.rmsnorm_quantize_impl(x, nw, rstd, fmt, colwise=True, kchunk=1)
-    nc = K.rmsnorm_quantize_impl(x, nw, rstd, fmt, colwise=True, kchunk=step, col_kchunk=True)
-    assert _same(nc[0], na[0]) and same_panels(nc[1], na[1]) and _same(nc[2], nb_[2]) and _same(nc[3], nb_[3])
-    with pytest.raises(Exception):
-        K._lib.check(K._lib.load().mxl_quantize_ex(x.data_ptr(), rows, cols, 768, fmt, 0, None, 0, c[0].data_ptr(), c[1].data_ptr(),
-                                                   None, None, K._lib.QF_KCHUNK | K._lib.QF_COL_KCHUNK, 0, 0, 0), "mxl_quantize_ex")

@@ -27,8 +27,12 @@ def _cfg(kind):
     return Float8QuantConfig(format=Format.HYBRID if kind == "hybrid" else Format.E4M3, granularity=ScalingGranularity.TENSORWISE)
 
 
-@pytest.mark.parametrize("lens,n,k", [(None, 96, 160), ([33, 0, 130, 1, 92], 160, 96), ([300, 212], 384, 256), ([0, 0], 64, 64)])
-def test_kernel_adds_exactly(gpu, lens, n, k):
+@pytest.mark.parametrize("lens,n,k", [(None, 96, 160), ([33, 0, 130, 1, 92], 160, 96), ([300, 212], 384, 256), ([0, 0], 64, 64),
+                                      ([700, 0, 1300], 544, 320)])
+@pytest.mark.parametrize("fmt,layout", [(0, 1), (0, 2), (1, 1), (1, 3)])
+def test_kernel_adds_exactly(gpu, lens, n, k, fmt, layout):
+    """K-chunk-major operands: the 2-slot kernel loads the old values and stores the sums; K-step-major operands: the ring
+    kernel adds with float atomics.  Either way every element receives exactly one float32 add per call."""
     from primus_amd.pytorch import kernels as K
 
     rng = np.random.default_rng(n + k)
@@ -40,9 +44,9 @@ def test_kernel_adds_exactly(gpu, lens, n, k):
     shape = (n, k) if lens is None else (G, n, k)
     before = torch.from_numpy(rng.integers(-1000, 1000, size=shape).astype(np.float32)).to(gpu)
     buf = before.clone()
-    _, _, dq, ds = K.quantize_mx_impl(dy, 0, rowwise=False, colwise=True, group_lens=gl, kchunk=True)
-    _, _, xq, xs = K.quantize_mx_impl(x, 0, rowwise=False, colwise=True, group_lens=gl, kchunk=True)
-    out = K.grouped_gemm_mx_wgrad_impl(dq, ds, xq, xs, gl, rows, kchunk=True, accum_into=buf)
+    _, _, dq, ds = K.quantize_mx_impl(dy, fmt, rowwise=False, colwise=True, group_lens=gl, kchunk=layout)
+    _, _, xq, xs = K.quantize_mx_impl(x, fmt, rowwise=False, colwise=True, group_lens=gl, kchunk=layout)
+    out = K.grouped_gemm_mx_wgrad_impl(dq, ds, xq, xs, gl, rows, kchunk=layout, accum_into=buf)
     assert out.data_ptr() == buf.data_ptr()
     want = before.cpu().numpy().reshape(G, n, k).copy()
     pos = 0
@@ -51,13 +55,13 @@ def test_kernel_adds_exactly(gpu, lens, n, k):
         pos += ln
     assert np.array_equal(buf.cpu().numpy().reshape(G, n, k), want)
     # a second call adds again
-    K.grouped_gemm_mx_wgrad_impl(dq, ds, xq, xs, gl, rows, kchunk=True, accum_into=buf)
+    K.grouped_gemm_mx_wgrad_impl(dq, ds, xq, xs, gl, rows, kchunk=layout, accum_into=buf)
     assert np.array_equal(buf.cpu().numpy().reshape(G, n, k), 2 * want - before.cpu().numpy().reshape(G, n, k))
     with pytest.raises(ValueError):
-        K.grouped_gemm_mx_wgrad_impl(dq, ds, xq, xs, gl, rows, kchunk=True, accum_into=buf.bfloat16())
+        K.grouped_gemm_mx_wgrad_impl(dq, ds, xq, xs, gl, rows, kchunk=layout, accum_into=buf.bfloat16())
     with pytest.raises(ValueError):
-        a = K.quantize_mx_impl(dy, 0, rowwise=False, colwise=True, group_lens=gl)
-        b = K.quantize_mx_impl(x, 0, rowwise=False, colwise=True, group_lens=gl)
+        a = K.quantize_mx_impl(dy, fmt, rowwise=False, colwise=True, group_lens=gl)
+        b = K.quantize_mx_impl(x, fmt, rowwise=False, colwise=True, group_lens=gl)
         K.grouped_gemm_mx_wgrad_impl(a[2], a[3], b[2], b[3], gl, rows, accum_into=buf)   # row-major operands
 
 

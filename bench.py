@@ -11,8 +11,9 @@ grouped GEMM, the dgrad grouped GEMM and the variable-K wgrad grouped GEMM.
 Default workload: the Mixtral-8x7B-shape MoE layer (8 experts, top-2, 16384
 tokens -> 32768 routed rows, hidden 4096, ffn 14336, gate+up fused 28672),
 routing from softmax of Gaussian logits plus a per-expert bias (skewed, ragged
-tokens-per-expert).  Inputs are generated on the GPU from fixed seeds and are
-resident in HBM before the timed region.
+tokens-per-expert).  Inputs are generated with the CPU generator from fixed
+seeds (fp32, cast to bf16), uploaded, and resident in HBM before the timed
+region; the CPU baseline runs on a row sample of the same tensors.
 
 Prints ONE JSON line:  metric = grouped-GEMM algorithmic TFLOP/s of the whole
 step (2*M*N*K per GEMM over all six GEMMs, divided by the wall time of the
@@ -42,13 +43,17 @@ WORKLOADS = {
     "mixtral_8x7b_moe_mxfp8": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False),
     "deepseek_v3_shard_mxfp8": dict(G=32, topk=8, tokens=8192, hidden=7168, fc1_out=4096, fc2_in=2048, routing="zipf", seed=1004, fp4=False),
     "gpt_oss_120b_mxfp4": dict(G=128, topk=4, tokens=16384, hidden=2880, fc1_out=5760, fc2_in=2880, routing="uniform", seed=1005, fp4=True, wgrad=False),
-    "llama3_8b_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False),
+    # the same shapes under the Mixtral workload's routing recipe (Gaussian logits plus a per-expert bias): 16 experts
+    # without tokens, 49 with fewer than 16, 11 with more than four times the mean
+    "gpt_oss_120b_mxfp4_skewed": dict(G=128, topk=4, tokens=16384, hidden=2880, fc1_out=5760, fc2_in=2880, routing="gauss_bias", seed=1005, fp4=True, wgrad=False),
+    # activations with 0.1 % of the entries multiplied by 50 (what moves E8M0 scales and saturates codes)
+    "llama3_8b_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, outliers=True),
     # the pure MXFP4 recipe (E2M1 activations, weights and gradients) on the headline shapes
     "mixtral_8x7b_moe_mxfp4": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=True, act_fp4=True),
     # the non-MX "current scaling" recipe on the headline shapes (HYBRID: E4M3 forward, E5M2 gradients)
     "mixtral_8x7b_moe_fp8_tensorwise": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, tensorwise=True),
     # the same MLP with the RMSNorm that precedes fc1 in the layer (LayerNormColumnParallelLinear), folded into fc1's quantiser
-    "llama3_8b_norm_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, norm=True),
+    "llama3_8b_norm_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, norm=True, outliers=True),
 }
 
 
@@ -79,6 +84,38 @@ def route(spec):
     probs = torch.softmax(logits, dim=-1)
     idx = probs.topk(topk, dim=-1).indices.reshape(-1)
     return torch.bincount(idx, minlength=G).tolist()
+
+
+def synth(shape, gen, device, scale=1.0, outliers=False, chunk=1 << 26):
+    """Seeded synthetic bf16 tensor ~ N(0, scale^2) on ``device``: drawn in fp32 from ``gen`` (a CPU generator in the
+    benchmark; tests may pass a device generator) in pieces of ``chunk`` elements of the flattened tensor, cast to
+    bf16 and uploaded.  ``outliers``: 0.1 % of the entries, chosen by a uniform draw from the same generator right
+    after each piece, are multiplied by 50 before the cast."""
+    import torch
+
+    n = 1
+    for d in shape:
+        n *= int(d)
+    out = torch.empty(n, dtype=torch.bfloat16, device=device)
+    for i in range(0, n, chunk):
+        c = torch.randn(min(chunk, n - i), generator=gen, device=gen.device)
+        if scale != 1.0:
+            c *= scale
+        if outliers:
+            hit = torch.rand(c.numel(), generator=gen, device=gen.device) < 1e-3
+            c = torch.where(hit, c * 50.0, c)
+        out[i:i + c.numel()] = c.bfloat16().to(device)
+    return out.view(*shape)
+
+
+def synth_layer(spec, layer, rows, gen, device):
+    """(x, w, dy, k, n) of linear ``layer`` (0: fc1, 1: fc2) of a workload, without autograd flags."""
+    k, n = ((spec["hidden"], spec["fc1_out"]), (spec["fc2_in"], spec["hidden"]))[layer]
+    grouped = spec["routing"] != "dense"
+    x = synth((rows, k), gen, device, outliers=bool(spec.get("outliers")))
+    w = synth((spec["G"], n, k) if grouped else (n, k), gen, device, scale=0.02)
+    dy = synth((rows, n), gen, device)
+    return x, w, dy, k, n
 
 
 class LaunchTimer:
@@ -130,10 +167,10 @@ def quant_bytes(info):
     return el * (2.0 + copies * (code + 1.0 / 32.0))
 
 
-def cpu_baseline(spec, lens, sample_div=16):
-    """The oracle's C restatement on the host cores, on 1/sample_div of the rows
-    (same experts and weights shapes): quantise -> dequantise -> fp32 matmul
-    (torch CPU) -> bf16, forward + dgrad + wgrad of both linears."""
+def cpu_baseline(spec, lens, layers, sample_div=16):
+    """The oracle's C restatement on the host cores, on 1/sample_div of the rows of the SAME tensors the GPU leg
+    ran on (the first rows of every expert, the full-size weights): quantise -> dequantise -> fp32 matmul
+    (torch CPU) -> bf16, forward + dgrad + wgrad of both linears.  ``layers``: (x, w, dy, k, n) device tensors."""
     import numpy as np
     import torch
 
@@ -149,13 +186,18 @@ def cpu_baseline(spec, lens, sample_div=16):
     G = spec["G"]
     slens = [max(1, ln // sample_div) if ln else 0 for ln in lens]
     m = sum(slens)
-    g = torch.Generator().manual_seed(spec["seed"])
+    starts = np.concatenate([[0], np.cumsum(lens)])[:-1]
+    pick = torch.from_numpy(np.concatenate([np.arange(s0, s0 + ln) for s0, ln in zip(starts, slens)]).astype(np.int64))
+    host = []
+    for (x, w, dy, k, n) in layers:     # device -> host copies are outside the timed region
+        idx = pick.to(x.device)
+        host.append((x.detach()[idx].cpu(), w.detach().reshape(G, n, k).cpu(), dy.detach()[idx].cpu(), k, n))
     flops = 0.0
     t0 = time.perf_counter()
-    for (k, n) in ((spec["hidden"], spec["fc1_out"]), (spec["fc2_in"], spec["hidden"])):
-        x = o.to_bf16_bits(torch.randn(m, k, generator=g).bfloat16())
-        dy = o.to_bf16_bits(torch.randn(m, n, generator=g).bfloat16())
-        w = o.to_bf16_bits((torch.randn(G, n, k, generator=g) * 0.02).bfloat16())
+    for (xs_, ws_, dys_, k, n) in host:
+        x = o.to_bf16_bits(xs_)
+        dy = o.to_bf16_bits(dys_)
+        w = o.to_bf16_bits(ws_)
         xq, xs = C.quantize_rowwise(x, fmt_a)
         xt, xts = C.quantize_colwise_segmented(x, slens, fmt_a)
         dq, ds = C.quantize_rowwise(dy, fmt_a)
@@ -198,7 +240,7 @@ def cpu_baseline(spec, lens, sample_div=16):
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"same workload with tokens-per-expert divided by {sample_div} ({m} routed rows), full-size weights; "
+        "sample": f"the GPU leg's own tensors: the first 1/{sample_div} of every expert's rows ({m} routed rows), full-size weights; "
         f"C oracle quantise/dequantise + torch CPU fp32 matmul; {dt_s:.1f} s",
     }
 
@@ -421,15 +463,24 @@ def main():
         cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0, block_size=32)
         op = pt.ops.grouped_gemm_fp8 if grouped else None
 
-    gen = torch.Generator(device=dev).manual_seed(spec["seed"])
-    shapes = ((spec["hidden"], spec["fc1_out"]), (spec["fc2_in"], spec["hidden"]))
-    layers = []
-    for (k, n) in shapes:
-        x = torch.randn(M, k, generator=gen, device=dev).bfloat16().requires_grad_()
-        wshape = (G, n, k) if grouped else (n, k)
-        w = (torch.randn(*wshape, generator=gen, device=dev) * 0.02).bfloat16().requires_grad_(spec.get("wgrad", True))
-        dy = torch.randn(M, n, generator=gen, device=dev).bfloat16()
-        layers.append((x, w, dy, k, n))
+    # inputs from the CPU generator (fp32 -> bf16 -> upload), one seed per workload; `raw` keeps the plain tensors
+    # for the CPU baseline
+    gen = torch.Generator().manual_seed(spec["seed"])
+    raw = [synth_layer(spec, i, M, gen, dev) for i in range(2)]
+
+    def with_grad(layer, copy):
+        x, w, dy, k, n = layer
+        if copy:
+            x, w, dy = x.clone(), w.clone(), dy.clone()
+        return (x.requires_grad_(), w.requires_grad_(spec.get("wgrad", True)), dy, k, n)
+
+    # Rotating buffer sets: a workload whose tensors would sit in the 256 MiB memory-side cache from one step to the
+    # next runs over enough distinct copies to exceed 2 GB (the reference's own GEMM benchmark does the same,
+    # primus/tools/benchmark/gemm_bench.py:60-123); the Mixtral workload's single set is 12 GB already.
+    set_bytes = sum(t.numel() * 2 for (x, w, dy, _, _) in raw for t in (x, w, dy))
+    n_sets = max(1, min(8, -(-(2 << 30) // set_bytes)))
+    sets = [[with_grad(layer, i > 0) for layer in raw] for i in range(n_sets)]
+    layers = sets[0]
     gl = torch.tensor(lens, dtype=torch.int64, device=dev)
     norm_w = torch.ones(spec["hidden"], device=dev).bfloat16().requires_grad_() if spec.get("norm") else None
     if not spec.get("wgrad", True):
@@ -439,13 +490,19 @@ def main():
         from primus_amd.pytorch.core import QuantizedTensorPair, create_quantized_weight, float4_e2m1fn_x2, float8_e4m3
 
         dest = float4_e2m1fn_x2 if spec["fp4"] else float8_e4m3
-        layers = [(x, QuantizedTensorPair(*create_quantized_weight(w, dest, cfg)), dy, k, n) for (x, w, dy, k, n) in layers]
+        sets = [[(x, QuantizedTensorPair(*create_quantized_weight(w, dest, cfg)), dy, k, n) for (x, w, dy, k, n) in layer_set]
+                for layer_set in sets]
+        layers = sets[0]
     # forward + dgrad (+ wgrad unless the workload is defined without it): 2 M N K flops each
     passes = 3.0 if spec.get("wgrad", True) else 2.0
     flops_step = sum(2.0 * passes * M * n * k for (_, _, _, k, n) in layers)
 
+    step_no = [0]
+
     def step():
-        for i, (x, w, dy, k, n) in enumerate(layers):
+        cur = sets[step_no[0] % n_sets]
+        step_no[0] += 1
+        for i, (x, w, dy, k, n) in enumerate(cur):
             if grouped:
                 y = op(x, w, gl, trans_b=True, config=cfg)
             elif norm_w is not None and i == 0:
@@ -557,7 +614,8 @@ def main():
                  else "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"]
                  else "fp8 e4m3 forward / e5m2 gradients, one fp32 scale per tensor, fp32 accumulate" if spec.get("tensorwise")
                  else "mxfp8_e4m3 (E8M0 block scales), fp32 accumulate",
-        "data": "synthetic (seeded, generated on the GPU; random-init weights N(0,0.02))",
+        "data": "synthetic (seeded CPU generator, fp32 -> bf16, uploaded; activations and gradients N(0,1)%s, random-init weights N(0,0.02)); %d rotating buffer set%s"
+                % (" with 0.1 % of the activation entries x50" if spec.get("outliers") else "", n_sets, "" if n_sets == 1 else "s"),
         "config": {
             "workload": args.workload,
             "experts": G,
@@ -606,7 +664,7 @@ def main():
         pt.ops.set_wgrad_overlap(not args.no_wgrad_overlap)
         out["board"] = board_sample(step, args.board_seconds)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(spec, lens)
+        out["cpu_baseline"] = cpu_baseline(spec, lens, raw)
     print(json.dumps(out))
 
 

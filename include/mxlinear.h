@@ -33,6 +33,7 @@ extern "C" {
 #define MXL_ELAUNCH (-2) /* HIP reported an error at launch */
 #define MXL_ENODEV (-3)  /* current device is not gfx950 */
 #define MXL_ESCRATCH (-4) /* the problem needs more scratch memory than an allocation-free entry point owns */
+#define MXL_ESTREAM (-5)  /* an allocation-free entry point was called on a stream it is not bound to */
 
 #define MXL_FMT_E4M3 0
 #define MXL_FMT_E2M1 1
@@ -212,8 +213,9 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * quantisers with MXL_QF_KSTEP.  FP8-format operands, FP8 rows against E2M1 weights in 64-element steps (forward /
  * dgrad), or E2M1 against E2M1 in 128-element steps (MXL_QF_KSTEP128 weights); at most 128 groups; anything else
  * returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
- * With either layout flag the kernels request whole 256-row tiles of a K chunk: a code or scale array whose row count
- * is not a multiple of 256 must be followed by 32 KiB of readable memory (the values read there are never used). */
+ * In every layout the kernels request whole 256-row tiles, also where a group or the operand ends earlier; a request for
+ * a row behind the operand's last row is dropped by the buffer descriptor's range check (the row offset of every request
+ * sits where that check sees it), so operands need no readable memory behind them. */
 #define MXL_GF_KSTEP 4u
 /* mxl_grouped_gemm_wgrad_ex / _scaled only, together with MXL_GF_KCHUNK or MXL_GF_KSTEP (the latter: E4M3 x E4M3,
  * E2M1 x E2M1 and, scaled, E4M3 | E5M2 x E4M3): c_bf16 points to FLOAT32 [g, n, k] and the
@@ -318,10 +320,16 @@ int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const void* w_bf16,
  * mxl_rmsnorm_bwd_noalloc_max_bytes() = 8 MiB that every GPU the library runs on holds until the process ends.
  * A problem with mxl_rmsnorm_bwd_workspace_bytes(rows, k) above that returns MXL_ESCRATCH (e.g. k = 4096 with
  * more than 512 rows; k <= 1024 always fits).  Calls no hipMalloc / hipFree or other allocating routine.  All
- * calls on one GPU share the array: calls that overlap on a GPU (two streams, two threads) race; calls on one
- * stream are ordered.  Nothing in the array has to be cleared between calls (every word read was written by
- * the same call). */
+ * calls on one GPU share the array, so two calls in flight at once would corrupt each other: per device the entry
+ * point is BOUND TO ONE STREAM (calls on one stream are ordered) and returns MXL_ESTREAM, launching nothing, for any
+ * other.  mxl_rmsnorm_bwd_noalloc_bind(stream) binds the current device's array to `stream` (and looks its address up,
+ * once per device); the first call on an unbound device binds its own stream.  Rebinding is the caller's statement
+ * that the work of the previous stream is finished or ordered in front of the new stream's.  A call on an unbound
+ * device while `stream` is being captured returns MXL_ESTREAM: bind before the capture begins (a captured call
+ * replays on whatever stream launches the graph; ordering replays against other users of the array is the caller's).
+ * Nothing in the array has to be cleared between calls (every word read was written by the same call). */
 int64_t mxl_rmsnorm_bwd_noalloc_max_bytes(void);
+int mxl_rmsnorm_bwd_noalloc_bind(void* stream);
 int mxl_rmsnorm_bwd_noalloc(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32, int64_t rows,
                             int64_t k, void* dx_bf16, void* dw_bf16, void* stream);
 
@@ -431,6 +439,15 @@ int mxl_calibrate_mfma(int a_fmt, int b_fmt, int64_t iters, void* stream);
  * is what that access pattern reaches on the board. */
 int mxl_calibrate_tile_copy(const void* in_bf16, int64_t rows, int64_t cols, void* out_row, void* out_colT, void* stream);
 int64_t mxl_calibrate_mfma_flops(int64_t iters);
+/* mxl_calibrate_range_check makes the hardware rule observable on which the GEMM kernels' operand requests rely (a
+ * request for rows past the end of an operand must read nothing): for each of num_cases triples of uint32
+ * {voffset, soffset, num_records} (device array `cases`) one LDS-direct 16-byte buffer load goes through a raw
+ * descriptor over `buf` with that num_records, per-lane offset and scalar offset, and out[4 i .. 4 i + 3] (uint32,
+ * device) receives the four dwords that arrived -- zeros where the range check dropped them.  max_offset_host = the
+ * largest voffset + soffset of the cases as the caller states it; the call is refused unless that plus 16 fits
+ * buf_bytes, so no case can leave `buf` whatever the hardware decides. */
+int mxl_calibrate_range_check(const void* buf, int64_t buf_bytes, const void* cases, int num_cases, void* out,
+                              int64_t max_offset_host, void* stream);
 
 #ifdef __cplusplus
 }

@@ -54,6 +54,7 @@ EXPORTS = (
     "mxl_rmsnorm_bwd_workspace_bytes",
     "mxl_rmsnorm_bwd_noalloc",
     "mxl_rmsnorm_bwd_noalloc_max_bytes",
+    "mxl_rmsnorm_bwd_noalloc_bind",
     "mxl_rmsnorm_quantize",
     "mxl_amax",
     "mxl_quantize_tensorwise",
@@ -73,6 +74,7 @@ EXPORTS = (
     "mxl_calibrate_mfma",
     "mxl_calibrate_mfma_flops",
     "mxl_calibrate_tile_copy",
+    "mxl_calibrate_range_check",
 )
 
 
@@ -144,6 +146,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_rmsnorm_bwd_noalloc.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp]
         lib.mxl_rmsnorm_bwd_noalloc_max_bytes.restype = i64
         lib.mxl_rmsnorm_bwd_noalloc_max_bytes.argtypes = []
+        lib.mxl_rmsnorm_bwd_noalloc_bind.restype = i32
+        lib.mxl_rmsnorm_bwd_noalloc_bind.argtypes = [vp]
         lib.mxl_rmsnorm_quantize.restype = i32
         lib.mxl_rmsnorm_quantize.argtypes = [vp, vp, vp, i64, i64, i64, i32, i32, vp, i32, vp, vp, vp, vp, u32, vp]
         lib.mxl_amax.restype = i32
@@ -178,6 +182,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_calibrate_mfma.argtypes = [i32, i32, i64, vp]
         lib.mxl_calibrate_tile_copy.restype = i32
         lib.mxl_calibrate_tile_copy.argtypes = [vp, i64, i64, vp, vp, vp]
+        lib.mxl_calibrate_range_check.restype = i32
+        lib.mxl_calibrate_range_check.argtypes = [vp, i64, vp, i32, vp, i64, vp]
         lib.mxl_calibrate_mfma_flops.restype = i64
         lib.mxl_calibrate_mfma_flops.argtypes = [i64]
         lib.mxl_gemm_nt_blockwise.restype = i32

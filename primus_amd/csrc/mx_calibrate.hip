@@ -106,6 +106,35 @@ __global__ __launch_bounds__(256) void tile_copy_kernel(const uint16_t* in, uint
     if (!ROW && !COL && acc.x == 0x12345u && acc.y == 0x54321u) calibrate_sink[t & 63] = 1.f;   // keeps the loads alive
 }
 
+
+// The rule the GEMM kernels' operand requests rely on, made observable: one LDS-direct 16-byte buffer load per case
+// through a raw descriptor over `buf` with num_records = cases[i].records, per-lane offset .voff and scalar offset
+// .soff; out[4 i .. 4 i + 3] = the four dwords that arrived in LDS (zeros where the range check dropped them).
+struct RangeCase { uint32_t voff, soff, records; };
+__global__ __launch_bounds__(64) void range_check_kernel(const uint8_t* buf, const RangeCase* cases, int n, uint32_t* out) {
+    __shared__ __attribute__((aligned(16))) uint32_t lds[64 * 4];
+    const uint64_t p = (uint64_t)buf;
+    for (int i = 0; i < n; ++i) {
+        const RangeCase cs = cases[i];
+        v4i r;
+        r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+        r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32) & 0xFFFF);
+        r[2] = __builtin_amdgcn_readfirstlane((int)cs.records);
+        r[3] = 0x00020000;
+        const uint32_t voff = cs.voff, soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)cs.soff);
+        for (int j = threadIdx.x; j < 256; j += 64) lds[j] = 0xDEADBEEFu;
+        __syncthreads();
+        const uint32_t lbase = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds\n\ts_waitcnt vmcnt(0)"
+                     :
+                     : "s"(lbase), "v"(voff), "s"(r), "s"(soff)
+                     : "memory");
+        __syncthreads();
+        if (threadIdx.x < 4) out[4 * i + threadIdx.x] = lds[threadIdx.x];
+        __syncthreads();
+    }
+}
+
 }  // namespace mxl
 
 using namespace mxl;
@@ -147,5 +176,18 @@ extern "C" int mxl_calibrate_mfma(int a_fmt, int b_fmt, int64_t iters, void* str
     else if (a4) hipLaunchKernelGGL((mfma_only_kernel<4, 0>), grid, block, 0, st, (int)iters);
     else if (b4) hipLaunchKernelGGL((mfma_only_kernel<0, 4>), grid, block, 0, st, (int)iters);
     else hipLaunchKernelGGL((mfma_only_kernel<0, 0>), grid, block, 0, st, (int)iters);
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
+
+extern "C" int mxl_calibrate_range_check(const void* buf, int64_t buf_bytes, const void* cases, int num_cases, void* out,
+                                         int64_t max_offset_host, void* stream) {
+    // max_offset_host: the largest voff + soff among the cases, stated by the caller: every case must stay inside
+    // `buf` whatever the hardware decides, so that the probe can never touch memory it does not own
+    if (!buf || !cases || !out || num_cases < 0 || max_offset_host < 0 || max_offset_host + 16 > buf_bytes) return MXL_EINVAL;
+    if (((uintptr_t)buf & 15) != 0) return MXL_EINVAL;
+    if (num_cases == 0) return MXL_OK;
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    hipLaunchKernelGGL(range_check_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (const uint8_t*)buf,
+                       (const RangeCase*)cases, num_cases, (uint32_t*)out);
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }

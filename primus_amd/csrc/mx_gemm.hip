@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "mx_device.h"
+#include "mx_gemm_addr.h"
 
 namespace mxl {
 
@@ -239,14 +240,15 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     const int64_t a_rows_total = (MODE == MODE_FWD) ? p.total_m : p.m;
     const int64_t b_rows_total = (MODE == MODE_FWD) ? (int64_t)G * p.n : p.n;
 
-    // per-thread constants of the global -> LDS mapping
-    const int a_row = t / Op<AFMT>::cpr, b_row = t / Op<BFMT>::cpr;
-    const uint32_t a_voff = (uint32_t)(a_row * (LAYOUT ? Op<AFMT>::kb : (int)lda) + 16 * ((t % Op<AFMT>::cpr) ^ Op<AFMT>::swz(a_row)));
-    const uint32_t b_voff = (uint32_t)(b_row * (LAYOUT ? Op<BFMT>::kb : (int)ldb) + 16 * ((t % Op<BFMT>::cpr) ^ Op<BFMT>::swz(b_row)));
+    // per-thread constants of the global -> LDS mapping (mx_gemm_addr.h holds the arithmetic and the rule it follows:
+    // descriptors end with the operand, and the range check covers the per-lane and the scalar offset)
+    const uint32_t a_voff = addr::slot2_code_lane(LAYOUT, t, Op<AFMT>::cpr, Op<AFMT>::swz(t / Op<AFMT>::cpr), lda, Op<AFMT>::kb);
+    const uint32_t b_voff = addr::slot2_code_lane(LAYOUT, t, Op<BFMT>::cpr, Op<BFMT>::swz(t / Op<BFMT>::cpr), ldb, Op<BFMT>::kb);
     // LAYOUT 1: bytes from one K chunk of an operand to the next (the host has checked that an operand stays below 4 GiB)
     const uint32_t a_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * Op<AFMT>::kb));
     const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * Op<BFMT>::kb));
-    const uint32_t s_voff = (uint32_t)(t * (int)ld_s);
+
+    const uint32_t s_voff = addr::slot2_scale_off(t, ld_s, 0u, 0);
 
     // Everything a tile needs, decoded from its index on the device.
     struct Tile {
@@ -301,18 +303,18 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
         d.n_valid = (p.n - n0) < BN ? (int)(p.n - n0) : BN;
         d.c_off = c_row0 * p.n + n0;
         d.np = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / BKP));
-        // Rows past the end of the operand read as zero; rows of a neighbouring group are read
-        // but never stored.
-        if (LAYOUT) {
-            // anchored at the tile's first row inside chunk 0; everything up to the end of the operand is readable
-            d.ra = make_rsrc(p.a + a_row0 * Op<AFMT>::kb, a_rows_total * lda - a_row0 * Op<AFMT>::kb);
-            d.rb = make_rsrc(p.b + b_row0 * Op<BFMT>::kb, b_rows_total * ldb - b_row0 * Op<BFMT>::kb);
-        } else {
-            d.ra = make_rsrc(p.a + a_row0 * lda, (a_rows_total - a_row0) * lda);
-            d.rb = make_rsrc(p.b + b_row0 * ldb, (b_rows_total - b_row0) * ldb);
+        // Descriptors start at the tile's first row and end with the operand: whatever lies past the operand's last
+        // byte is dropped by the range check and reads as zero; rows of a neighbouring group are read but never stored.
+        {
+            const addr::Desc da = addr::slot2_code_desc(LAYOUT, a_rows_total, a_row0, lda, Op<AFMT>::kb);
+            const addr::Desc db = addr::slot2_code_desc(LAYOUT, b_rows_total, b_row0, ldb, Op<BFMT>::kb);
+            const addr::Desc dsa = addr::slot2_scale_desc(a_rows_total, a_row0, ld_s);
+            const addr::Desc dsb = addr::slot2_scale_desc(b_rows_total, b_row0, ld_s);
+            d.ra = make_rsrc(p.a + da.base, da.records);
+            d.rb = make_rsrc(p.b + db.base, db.records);
+            d.rsa = make_rsrc(p.sa + dsa.base, dsa.records);
+            d.rsb = make_rsrc(p.sb + dsb.base, dsb.records);
         }
-        d.rsa = make_rsrc(p.sa + a_row0 * ld_s, (a_rows_total - a_row0) * ld_s);
-        d.rsb = make_rsrc(p.sb + b_row0 * ld_s, (b_rows_total - b_row0) * ld_s);
         // first byte of the contraction range inside a row (LAYOUT 0) or its first K chunk (LAYOUT 1)
         d.ka0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(LAYOUT ? k0 / BKP : (Op<AFMT>::fp4 ? k0 / 2 : k0)));
         d.kb0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(LAYOUT ? k0 / BKP : (Op<BFMT>::fp4 ? k0 / 2 : k0)));
@@ -324,22 +326,23 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // the N-side operand for LPA <= r < LPT; a round past the end is a no-op.
     auto issue_1 = [&](const Tile& d, int kp, int slot, int r) __attribute__((always_inline)) {
         if (r < LPA) {
-            const uint32_t soff = LAYOUT ? (d.ka0 + (uint32_t)kp) * a_cstride + (uint32_t)(r * Op<AFMT>::rows_per_ld * Op<AFMT>::kb)
-                                         : d.ka0 + kp * Op<AFMT>::kb + (uint32_t)(r * Op<AFMT>::rows_per_ld) * (uint32_t)lda;
-            dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff, soff);
+            const uint32_t off = addr::slot2_code_k(LAYOUT, d.ka0, kp, Op<AFMT>::kb, a_cstride) +
+                                 addr::slot2_code_round(LAYOUT, r, Op<AFMT>::rows_per_ld, lda, Op<AFMT>::kb);
+            dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff, off);
         } else if (r < LPT) {
             const int i = r - LPA;
-            const uint32_t soff = LAYOUT ? (d.kb0 + (uint32_t)kp) * b_cstride + (uint32_t)(i * Op<BFMT>::rows_per_ld * Op<BFMT>::kb)
-                                         : d.kb0 + kp * Op<BFMT>::kb + (uint32_t)(i * Op<BFMT>::rows_per_ld) * (uint32_t)ldb;
-            dma16(d.rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff, soff);
+            const uint32_t off = addr::slot2_code_k(LAYOUT, d.kb0, kp, Op<BFMT>::kb, b_cstride) +
+                                 addr::slot2_code_round(LAYOUT, i, Op<BFMT>::rows_per_ld, ldb, Op<BFMT>::kb);
+            dma16(d.rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff, off);
         }
     };
     // scale panel pn (K slots 4pn .. 4pn+3) into panel buffer pn & 1
     auto issue_s = [&](const Tile& d, int pn) __attribute__((always_inline)) {
         if (ALPHA) return;   // per-tensor factors: the block scales are the unit byte by contract and are not read
         const uint32_t base = smem_base + NSLOT * STAGE + (pn & 1) * 2 * PANEL;
-        dma16(d.rsa, base + w * 1024, s_voff, d.ks0 + 16 * pn);
-        dma16(d.rsb, base + PANEL + w * 1024, s_voff, d.ks0 + 16 * pn);
+        const uint32_t koff = addr::slot2_scale_off(0, ld_s, d.ks0, pn);
+        dma16(d.rsa, base + w * 1024, s_voff, koff);
+        dma16(d.rsb, base + PANEL + w * 1024, s_voff, koff);
     };
     // first requests of a tile: scale panel 0 and all of K slot 0
     auto issue_head = [&](const Tile& d) __attribute__((always_inline)) {
@@ -747,23 +750,20 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * B_ROW));
     const uint32_t a_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * 16));
     const uint32_t b_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * 16));
-    // panels in a scale array: a contraction that is split into groups restarts its panels at every group
-    const int64_t n_panels = (p.k + 511) / 512 + ((MODE == MODE_WGRAD && p.group_lens) ? G + 1 : 0);
     // a load round covers 64 consecutive rows = 4 KiB: thread -> (row t / 4, 16-byte piece t % 4); the XOR swizzle of
     // the piece index is applied on the global side so that the LDS image (64-byte rows) reads without bank conflicts
-    const int ld_row = t >> 2;
-    const uint32_t ld_voff = (uint32_t)(ld_row * BK + 16 * ((t & 3) ^ ((ld_row >> 2) & 3)));
+    // panels in a scale array: a contraction that is split into groups restarts its panels at every group
+    const int64_t n_panels = (p.k + 511) / 512 + ((MODE == MODE_WGRAD && p.group_lens) ? G + 1 : 0);
     // FP4 rows are 32 bytes: a round covers 128 rows, thread -> (row t / 2, piece t % 2), pieces swapped in every
     // second group of 8 rows so that the 16-byte fragment reads of 16 consecutive rows cover all banks
-    const uint32_t ld_voff_b = B4 ? (uint32_t)((t >> 1) * B_ROW + 16 * ((t & 1) ^ ((t >> 4) & 1))) : ld_voff;
-    const uint32_t s_voff = (uint32_t)(t * 16);     // scale panel: row t of the tile, 16 bytes
+    const uint32_t s_voff = addr::ring_panel_lane(t);     // scale panel: row t of the tile, 16 bytes
     // per-lane offsets of the load rounds: round e of an operand starts e * 64 rows = e * 4 KiB further on
     const uint32_t wave_base = smem_base + (uint32_t)(w * 1024);    // ring slot 0, this wave's 1 KiB of a round
     uint32_t va[4], vb[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        va[e] = ld_voff + (uint32_t)(e * 64 * BK);
-        vb[e] = ld_voff_b + (uint32_t)(e * 4096);
+        va[e] = addr::ring_code_lane(t, e, false);
+        vb[e] = addr::ring_code_lane(t, e, B4);
     }
 
     struct Tile {
@@ -826,11 +826,17 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         const int nreal = __builtin_amdgcn_readfirstlane((int)((k1 - k0) / KS));
         d.nst_real = nreal;
         d.nst = nreal < 4 ? 4 : nreal + (nreal & 1);
-        // descriptors anchored at the tile's first row inside K step 0 / panel 0; readable up to the operand's end
-        d.ra = make_rsrc(p.a + a_row0 * BK, a_rows_total * (p.k / KS) * BK - a_row0 * BK);
-        d.rb = make_rsrc(p.b + b_row0 * B_ROW, b_rows_total * (p.k / KS) * B_ROW - b_row0 * B_ROW);
-        d.rsa = make_rsrc(p.sa + a_row0 * 16, a_rows_total * n_panels * 16 - a_row0 * 16);
-        d.rsb = make_rsrc(p.sb + b_row0 * 16, b_rows_total * n_panels * 16 - b_row0 * 16);
+        // Descriptors start at the tile's first row inside K step 0 / panel 0 and end with the operand: the range
+        // check covers the per-lane offset (row, load round) and the scalar offset (K step / panel) together, so a
+        // row past the operand's last one is dropped in the last plane and reads a later plane's rows in the others.
+        {
+            const addr::Desc da = addr::ring_code_desc(a_rows_total, p.k / KS, a_row0, BK), db = addr::ring_code_desc(b_rows_total, p.k / KS, b_row0, B_ROW);
+            const addr::Desc dsa = addr::ring_panel_desc(a_rows_total, n_panels, a_row0), dsb = addr::ring_panel_desc(b_rows_total, n_panels, b_row0);
+            d.ra = make_rsrc(p.a + da.base, da.records);
+            d.rb = make_rsrc(p.b + db.base, db.records);
+            d.rsa = make_rsrc(p.sa + dsa.base, dsa.records);
+            d.rsb = make_rsrc(p.sb + dsb.base, dsb.records);
+        }
         const uint32_t st0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(k0 / KS));
         d.ca0 = st0 * a_cstride;
         d.cb0 = st0 * b_cstride;
@@ -1567,6 +1573,7 @@ extern "C" const char* mxl_error_string(int code) {
         case MXL_ELAUNCH: return "HIP launch error";
         case MXL_ENODEV: return "device is not gfx950";
         case MXL_ESCRATCH: return "the problem needs more scratch memory than this allocation-free entry point owns";
+        case MXL_ESTREAM: return "the allocation-free entry point is bound to another stream on this device (or unbound while capturing)";
         default: return "unknown error";
     }
 }

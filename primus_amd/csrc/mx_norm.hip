@@ -255,15 +255,21 @@ extern "C" int mxl_rmsnorm_bwd(const void* dy_bf16, const void* x_bf16, const vo
 constexpr int64_t NORM_SCRATCH_BYTES = (int64_t)8 << 20;
 static __device__ __align__(256) unsigned char scratch[NORM_SCRATCH_BYTES];
 
-static int norm_scratch_ptr(void** out) {
-    constexpr int MAXDEV = 64;
-    static std::atomic<void*> ptrs[MAXDEV];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return MXL_ELAUNCH;
-    void* ptr = (dev >= 0 && dev < MAXDEV) ? ptrs[dev].load(std::memory_order_acquire) : nullptr;
+// Per device: the array's address and the stream the entry point is bound to.  All calls on a GPU share the one
+// array, so two calls in flight at once would mix their partial sums: the entry point serves ONE stream per device
+// (calls on a stream are ordered) and refuses any other with MXL_ESTREAM until the caller rebinds it.
+constexpr int NORM_MAXDEV = 1024;
+static std::atomic<void*> norm_scratch_ptrs[NORM_MAXDEV];
+static std::atomic<uintptr_t> norm_scratch_owner[NORM_MAXDEV];      // 0 = unbound, else the stream handle | 1
+static uintptr_t stream_key(void* stream) { return (uintptr_t)stream | 1u; }
+
+// the current device's copy of the array; asked for once per device (never while a stream is capturing: the
+// query is not a stream operation, but it may initialise the module on the device)
+static int norm_scratch_resolve(int dev, void** out) {
+    void* ptr = norm_scratch_ptrs[dev].load(std::memory_order_acquire);
     if (!ptr) {
         if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MXL_ELAUNCH;
-        if (dev >= 0 && dev < MAXDEV) ptrs[dev].store(ptr, std::memory_order_release);
+        norm_scratch_ptrs[dev].store(ptr, std::memory_order_release);
     }
     *out = ptr;
     return MXL_OK;
@@ -271,15 +277,37 @@ static int norm_scratch_ptr(void** out) {
 
 extern "C" int64_t mxl_rmsnorm_bwd_noalloc_max_bytes(void) { return NORM_SCRATCH_BYTES; }
 
+extern "C" int mxl_rmsnorm_bwd_noalloc_bind(void* stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NORM_MAXDEV) return MXL_ENODEV;
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    void* ptr = nullptr;
+    const int rc = norm_scratch_resolve(dev, &ptr);
+    if (rc != MXL_OK) return rc;
+    norm_scratch_owner[dev].store(stream_key(stream), std::memory_order_release);
+    return MXL_OK;
+}
+
 extern "C" int mxl_rmsnorm_bwd_noalloc(const void* dy_bf16, const void* x_bf16, const void* w_bf16, const void* rstd_f32,
                                        int64_t rows, int64_t k, void* dx_bf16, void* dw_bf16, void* stream) {
     if (!norm_shape_ok(rows, k) || !dw_bf16) return MXL_EINVAL;
     // same partial-sum geometry as mxl_rmsnorm_bwd (hence the same bits); a problem whose partial sums do not
     // fit the static array is refused
     if ((int64_t)norm_bwd_blocks(rows, k) * k * 4 > NORM_SCRATCH_BYTES) return MXL_ESCRATCH;
-    if (!device_is_gfx950()) return MXL_ENODEV;
-    void* ptr = nullptr;
-    const int rc = norm_scratch_ptr(&ptr);
-    if (rc != MXL_OK) return rc;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NORM_MAXDEV) return MXL_ENODEV;
+    uintptr_t owner = norm_scratch_owner[dev].load(std::memory_order_acquire);
+    if (owner == 0) {
+        // first use on this device without a bind: this call binds its stream, unless that stream is being
+        // captured (set-up does not belong into a capture: the caller binds beforehand)
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing((hipStream_t)stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return MXL_ESTREAM;
+        const int rc = mxl_rmsnorm_bwd_noalloc_bind(stream);
+        if (rc != MXL_OK) return rc;
+        owner = stream_key(stream);
+    }
+    if (owner != stream_key(stream)) return MXL_ESTREAM;
+    void* ptr = norm_scratch_ptrs[dev].load(std::memory_order_acquire);
+    if (!ptr) return MXL_ELAUNCH;
     return rmsnorm_bwd(dy_bf16, x_bf16, w_bf16, rstd_f32, rows, k, dx_bf16, dw_bf16, ptr, NORM_SCRATCH_BYTES, stream);
 }

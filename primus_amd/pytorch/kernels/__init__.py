@@ -123,21 +123,6 @@ def _scale_shape(rows: int, ld: int, kchunk, groups: int = 0):
     return (rows, ld // BLOCK)
 
 
-OPERAND_TAIL = 32 * 1024
-
-
-def _empty_tail(shape, dtype, device):
-    """A code or scale buffer followed by ``OPERAND_TAIL`` bytes the GEMMs may read (never use).  In the chunked
-    layouts the GEMMs request whole 256-row tiles of a K chunk; for an operand whose row count is not a multiple of
-    256 the last tile's requests in the last chunk reach up to 32 KiB past the last code (the values land in tile
-    rows that are never stored).  The tail keeps those reads inside the allocation."""
-    n = 1
-    for d in shape:
-        n *= int(d)
-    flat = torch.empty((n + OPERAND_TAIL,), dtype=dtype, device=device)
-    return flat[:n].view(shape)
-
-
 def _qflag(kchunk) -> int:
     return (0, _lib.QF_KCHUNK, _lib.QF_KSTEP, _lib.QF_KSTEP | _lib.QF_KSTEP128)[_layout(kchunk)]
 
@@ -146,15 +131,15 @@ def _gflag(kchunk) -> int:
     return (0, _lib.GF_KCHUNK, _lib.GF_KSTEP, _lib.GF_KSTEP)[_layout(kchunk)]
 
 
-def pick_layout(groups: int, n: int, k: int, rows: int = 0, fp8: bool = True, accum: bool = False,
-                fp4: bool = False) -> int:
+def pick_layout(groups: int, n: int, k: int, rows: int = 0, fp8: bool = True, fp4: bool = False) -> int:
     """Layout the differentiable operators store their quantised operands in: K-step-major when the activations and
     gradients are FP8 (``fp8``; steps of 64 elements, the weights FP8 or E2M1) or every operand is E2M1 (``fp4``; steps
-    of 128 elements), the groups fit the ring kernel and the weight gradient is not accumulated in the GEMM; otherwise
-    K-chunk-major; row-major when the layouts are switched off or an operand reaches 4 GiB."""
+    of 128 elements) and the groups fit the ring kernel -- also when the weight gradient is accumulated into float32
+    inside the GEMM, which the ring kernel's wgrad instantiations do; otherwise K-chunk-major; row-major when the
+    layouts are switched off or an operand reaches 4 GiB."""
     if not (kchunk_default() and kchunk_fits(groups, n, k, rows)):
         return LAYOUT_ROWMAJOR
-    if (fp8 or fp4) and groups <= RING_MAX_GROUPS and not accum and _kstep_default:
+    if (fp8 or fp4) and groups <= RING_MAX_GROUPS and _kstep_default:
         return LAYOUT_KSTEP if fp8 else LAYOUT_KSTEP128
     return LAYOUT_KCHUNK
 
@@ -330,12 +315,12 @@ def quantize_mx_impl(
     q_row = s_row = q_col = s_col = None
     row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
-        q_row = _empty_tail(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-        s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+        q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        q_col = _empty_tail(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(cols, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         # with no tokens only the padding of the transposed copy is left to write
         row_ok = rows > 0
@@ -386,14 +371,14 @@ def quantize_mx_weight_2d_impl(
     k_ld, n_ld = _round_up(k, KCHUNK if kchunk else pad_to), _round_up(n, KCHUNK if kchunk else pad_to)
     if rowwise:
         shape = _code_shape(batch * n, k_ld, per, kchunk) if kchunk else lead + (n, k_ld // per)
-        q_row = _empty_tail(shape, dtype=torch.uint8, device=dev)
+        q_row = torch.empty(shape, dtype=torch.uint8, device=dev)
         sshape = _scale_shape(batch * n, k_ld, kchunk) if _paneled(kchunk) else lead + (n, k_ld // BLOCK)
-        s_row = _empty_tail(sshape, dtype=torch.uint8, device=dev)
+        s_row = torch.empty(sshape, dtype=torch.uint8, device=dev)
     if colwise:
         shape = _code_shape(batch * k, n_ld, per, kchunk) if kchunk else lead + (k, n_ld // per)
-        q_col = _empty_tail(shape, dtype=torch.uint8, device=dev)
+        q_col = torch.empty(shape, dtype=torch.uint8, device=dev)
         sshape = _scale_shape(batch * k, n_ld, kchunk) if _paneled(kchunk) else lead + (k, n_ld // BLOCK)
-        s_col = _empty_tail(sshape, dtype=torch.uint8, device=dev)
+        s_col = torch.empty(sshape, dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_2d_ex(
             _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
@@ -659,13 +644,13 @@ def glu_with_probs_quantize_impl(x, probs, row_mask, activation: str, fmt: int, 
     per = _per_byte(fmt)
     dev = x.device
     row_ld = _round_up(f, KCHUNK if kchunk else pad_to)
-    q_row = _empty_tail(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-    s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+    q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+    s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, G)
-        q_col = _empty_tail(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(f, W, kchunk, G), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(f, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(f, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows > 0 or (q_col is not None and q_col.numel() > 0):
         row_ok = rows > 0
         with _hooked("glu_probs_quantize", rows=rows, cols=f, fmt=fmt, rowwise=True, colwise=colwise):
@@ -724,12 +709,12 @@ def quantize_tensorwise_impl(x, fmt: int, *, rowwise: bool = True, colwise: bool
     q_row = s_row = q_col = s_col = None
     row_ld = _round_up(cols, KCHUNK if kchunk else pad_to)
     if rowwise:
-        q_row = _empty_tail(_code_shape(rows, row_ld, 1, kchunk), dtype=torch.uint8, device=dev)
-        s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+        q_row = torch.empty(_code_shape(rows, row_ld, 1, kchunk), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     if colwise:
         W = padded_width(rows, G)
-        q_col = _empty_tail(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(cols, W, 1, kchunk), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(cols, W, kchunk, G), dtype=torch.uint8, device=dev)
     if rows == 0 and not (colwise and q_col.numel()):
         scale_inv.fill_(1e-12 / (448.0 if fmt == _lib.FMT_E4M3 else 57344.0))
     else:
@@ -766,11 +751,11 @@ def quantize_weight_tensorwise_impl(w, fmt: int, *, rowwise: bool = True, colwis
     q_row = s_row = q_col = s_col = None
     kstep = _paneled(kchunk)
     if rowwise:
-        q_row = _empty_tail(_code_shape(batch * n, k_ld, 1, kchunk) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
-        s_row = _empty_tail(_scale_shape(batch * n, k_ld, kchunk) if kstep else lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
+        q_row = torch.empty(_code_shape(batch * n, k_ld, 1, kchunk) if kchunk else lead + (n, k_ld), dtype=torch.uint8, device=dev)
+        s_row = torch.empty(_scale_shape(batch * n, k_ld, kchunk) if kstep else lead + (n, k_ld // BLOCK), dtype=torch.uint8, device=dev)
     if colwise:
-        q_col = _empty_tail(_code_shape(batch * k, n_ld, 1, kchunk) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(batch * k, n_ld, kchunk) if kstep else lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(batch * k, n_ld, 1, kchunk) if kchunk else lead + (k, n_ld), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(batch * k, n_ld, kchunk) if kstep else lead + (k, n_ld // BLOCK), dtype=torch.uint8, device=dev)
     with _hooked("quantize_weight_tensorwise", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
         rc = _lib.load().mxl_quantize_weight_tensorwise(
             _ptr(w), batch, n, k, k_ld, n_ld, fmt, _ptr(amax), _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
@@ -934,13 +919,13 @@ def rmsnorm_quantize_impl(x, weight, rstd, fmt: int, scale_mode: int = _lib.SCAL
     per = _per_byte(fmt)
     dev = x.device
     row_ld = _round_up(k, KCHUNK if kchunk else pad_to)
-    q_row = _empty_tail(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
-    s_row = _empty_tail(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
+    q_row = torch.empty(_code_shape(rows, row_ld, per, kchunk), dtype=torch.uint8, device=dev)
+    s_row = torch.empty(_scale_shape(rows, row_ld, kchunk), dtype=torch.uint8, device=dev)
     q_col = s_col = None
     if colwise:
         W = padded_width(rows, 0)
-        q_col = _empty_tail(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
-        s_col = _empty_tail(_scale_shape(k, W, kchunk), dtype=torch.uint8, device=dev)
+        q_col = torch.empty(_code_shape(k, W, per, kchunk), dtype=torch.uint8, device=dev)
+        s_col = torch.empty(_scale_shape(k, W, kchunk), dtype=torch.uint8, device=dev)
     with _hooked("rmsnorm_quantize", rows=rows, cols=k, fmt=fmt, rowwise=True, colwise=colwise):
         rc = _lib.load().mxl_rmsnorm_quantize(
             _ptr(x), _ptr(weight), _ptr(rstd), rows, k, row_ld, fmt, scale_mode, None, 0, _ptr(q_row), _ptr(s_row),

@@ -296,14 +296,14 @@ def _transposed_cache(q: QuantizedTensor, kchunk: bool):
     out[..., :n] = t.view(torch.uint8)
     unit = torch.full(tuple(t.shape[:-1]) + (n_ld // _lib.BLOCK,), 127, dtype=torch.uint8, device=codes.device)
     if kchunk:
-        # K-chunk-major or K-step-major: [n_ld / step][rows][step]; such operands carry a readable tail behind them
+        # K-chunk-major or K-step-major: [n_ld / step][rows][step]
         step = K.KSTEP if int(kchunk) == K.LAYOUT_KSTEP else K.KCHUNK
         rows = out.numel() // n_ld
-        laid = K._empty_tail((n_ld // step, rows, step), dtype=torch.uint8, device=codes.device)
+        laid = torch.empty((n_ld // step, rows, step), dtype=torch.uint8, device=codes.device)
         laid.copy_(out.reshape(rows, n_ld // step, step).permute(1, 0, 2))
         out = laid
         if int(kchunk) == K.LAYOUT_KSTEP:
-            unit = K._empty_tail(K._scale_shape(rows, n_ld, kchunk), dtype=torch.uint8, device=codes.device).fill_(127)
+            unit = torch.empty(K._scale_shape(rows, n_ld, kchunk), dtype=torch.uint8, device=codes.device).fill_(127)
     return out.view(codes.dtype), unit.view(q.scales.dtype)
 
 

@@ -1,6 +1,7 @@
-"""The benchmark configurations at their FULL shapes (Llama-3-8B MLP, Mixtral-8x7B,
-DeepSeek-V3 expert shard, GPT-OSS-120B with MXFP4 weights): same seeded routing and
-tensor shapes as bench.py.
+"""The benchmark configurations at their FULL shapes (Llama-3-8B MLP with outlier-injected
+activations, Mixtral-8x7B, DeepSeek-V3 expert shard, GPT-OSS-120B with MXFP4 weights under
+uniform and under skewed routing): same seeded routing, tensor shapes and per-tensor
+distributions as bench.py.
 
 A full CPU oracle run at these sizes would take hours, so each case checks
  (1) quantised bytes and scales BIT-EXACT against the oracle on sampled bands (the
@@ -69,6 +70,7 @@ CASES = [
     ("mixtral_8x7b_moe_mxfp8", 0),
     ("deepseek_v3_shard_mxfp8", 0),
     ("gpt_oss_120b_mxfp4", 0),
+    ("gpt_oss_120b_mxfp4_skewed", 0),     # 16 experts without tokens, 11 with more than four times the mean
 ]
 
 
@@ -92,10 +94,13 @@ def test_full_size_linear(gpu, workload, layer):
         cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE,
                                 scale_dtype=ScaleDtype.E8M0, block_size=32)
     rng = np.random.default_rng(spec["seed"] + layer)
+    # the benchmark's own recipe per tensor (for the Llama MLP: activations with 0.1 % of the entries times 50), drawn
+    # from a device generator here: a CPU draw of these sizes would take most of the suite's time
     gen = torch.Generator(device=gpu).manual_seed(spec["seed"] + 17 * layer)
-    x = torch.randn(M, k, generator=gen, device=gpu).bfloat16()
-    w = (torch.randn(*((n, k) if dense else (G, n, k)), generator=gen, device=gpu) * 0.02).bfloat16()
-    dy = torch.randn(M, n, generator=gen, device=gpu).bfloat16()
+    x, w, dy, _, _ = bench.synth_layer(spec, layer, M, gen, gpu)
+    if spec.get("outliers"):
+        big = (x.float().abs() > 8).float().mean().item()
+        assert 5e-4 < big < 1.5e-3, big          # N(0, 1) alone puts nothing there
     gl = None if dense else torch.tensor(lens, dtype=torch.int64, device=gpu)
     glens = [M] if dense else lens
 

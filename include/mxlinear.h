@@ -230,6 +230,25 @@ int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_f
                               const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                               int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);
 
+/* Grouped GEMM on UNQUANTISED bf16 operands, tokens-per-expert consumed on the device: ops.grouped_gemm, which the
+ * reference's grouped linear calls when no low-precision recipe is active
+ * (primus/backends/megatron/core/extensions/primus_turbo.py:2210-2216; the first / last layers of an FP4 run:
+ * primus/backends/megatron/core/fp4_utils.py:155-165).  fp32 accumulation, one rounding to bf16.
+ *   mxl_grouped_gemm_bf16: c[total_m, n] (bf16): the rows of a[total_m, k] are split by group_lens and group g is
+ *     multiplied by b[g] = [n, k] (c = a . b_g^T: forward of an NT linear) or, with MXL_BF_B_KN, by b[g] = [k, n]
+ *     (c = a . b_g: the dgrad of an NT linear with a = dy, k = its n; or the forward of trans_b = False).
+ *     Requires k % 32 == 0, n % 8 == 0, 16-byte aligned pointers.
+ *   mxl_grouped_gemm_bf16_wgrad: c[num_groups, m_out, n_out] = sum over the tokens t of group g of
+ *     p[t, m_out] * q[t, n_out]  (p = dy, q = x gives the [n, k] weight gradient); a group without tokens yields zeros.
+ *     bf16 output, or with MXL_BF_ACCUM_F32 c is float32 and the result is ADDED to it (the main_grad fusion).
+ *     Requires m_out % 8 == 0, n_out % 8 == 0; an operand stays below 4 GiB. */
+#define MXL_BF_B_KN 1u
+#define MXL_BF_ACCUM_F32 2u
+int mxl_grouped_gemm_bf16(const void* a_bf16, const void* b_bf16, void* c_bf16, const int64_t* group_lens, int num_groups,
+                          int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);
+int mxl_grouped_gemm_bf16_wgrad(const void* p_bf16, const void* q_bf16, void* c, const int64_t* group_lens, int num_groups,
+                                int64_t total_m, int64_t m_out, int64_t n_out, uint32_t flags, void* stream);
+
 /* Gated activation of the expert MLP fused with the router probability and the row mask
  * (swiglu_with_probs / geglu_with_probs behind fused_bias_act_with_probs, primus_turbo.py:1954-1980;
  * the unfused arithmetic is experts.py:100-118):

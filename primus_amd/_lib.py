@@ -31,6 +31,7 @@ QF_SR, QF_RHT_COL, QF_KCHUNK, QF_KSTEP, QF_KSTEP128 = 1, 2, 4, 8, 16   # flags o
 GF_KCHUNK = 1                               # flag of the GEMM _ex entry points: operands are K-chunk-major
 GF_KSTEP = 4                                # ... K-step-major codes and scales (ring kernel)
 GF_ACCUM_F32 = 2                            # wgrad: the output is float32 and the result is added to it
+BF_B_KN, BF_ACCUM_F32 = 1, 2                # flags of the bf16 grouped GEMMs
 
 EXPORTS = (
     "mxl_version",
@@ -46,6 +47,8 @@ EXPORTS = (
     "mxl_grouped_gemm_wgrad",
     "mxl_grouped_gemm_nt_ex",
     "mxl_grouped_gemm_wgrad_ex",
+    "mxl_grouped_gemm_bf16",
+    "mxl_grouped_gemm_bf16_wgrad",
     "mxl_glu_probs_fwd",
     "mxl_glu_probs_bwd",
     "mxl_glu_probs_quantize",
@@ -129,6 +132,10 @@ def load() -> ctypes.CDLL:
         lib.mxl_grouped_gemm_nt.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
         lib.mxl_grouped_gemm_wgrad.restype = i32
         lib.mxl_grouped_gemm_wgrad.argtypes = [vp, vp, i32, vp, vp, i32, vp, vp, i32, i64, i64, i64, vp]
+        lib.mxl_grouped_gemm_bf16.restype = i32
+        lib.mxl_grouped_gemm_bf16.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, u32, vp]
+        lib.mxl_grouped_gemm_bf16_wgrad.restype = i32
+        lib.mxl_grouped_gemm_bf16_wgrad.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, u32, vp]
         lib.mxl_glu_probs_fwd.restype = i32
         lib.mxl_glu_probs_fwd.argtypes = [vp, vp, i32, vp, i64, i64, i32, vp, vp]
         lib.mxl_glu_probs_bwd.restype = i32

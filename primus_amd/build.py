@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmxlinear.so")
-SOURCES = ["mx_quantize.hip", "mx_gemm.hip", "mx_activation.hip", "mx_norm.hip", "mx_pad.hip", "mx_blockwise.hip", "mx_calibrate.hip", "mx_shuffle.hip"]
+SOURCES = ["mx_quantize.hip", "mx_gemm.hip", "mx_gemm_bf16.hip", "mx_activation.hip", "mx_norm.hip", "mx_pad.hip", "mx_blockwise.hip", "mx_calibrate.hip", "mx_shuffle.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

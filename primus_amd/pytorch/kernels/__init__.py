@@ -600,6 +600,58 @@ def _glu_args(x, probs, row_mask, activation):
     return _ACTS[activation], pd, row_mask
 
 
+def grouped_gemm_bf16_impl(a: torch.Tensor, b: torch.Tensor, group_lens: Optional[torch.Tensor], b_kn: bool = False) -> torch.Tensor:
+    """Grouped GEMM on unquantised bf16 operands: the rows of ``a [total_m, k]`` are split by ``group_lens`` (device,
+    never read back) and group g is multiplied by ``b[g]^T`` with ``b [G, n, k]``, or by ``b[g]`` with ``b [G, k, n]``
+    when ``b_kn``.  ``group_lens`` None: one group (``b`` 2-D or with a leading 1)."""
+    _require_cuda(a, b, group_lens)
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.dim() != 2:
+        raise ValueError("the bf16 grouped GEMM takes a 2-D bf16 activation and a bf16 weight")
+    G = _check_group_lens(group_lens, a.device) or 1
+    b3 = b.reshape(1, *b.shape) if b.dim() == 2 else b
+    if b3.dim() != 3 or b3.shape[0] != G:
+        raise ValueError("b must be [G, n, k] (or [G, k, n]) with one matrix per group")
+    total_m, k = a.shape
+    kk, n = (b3.shape[1], b3.shape[2]) if b_kn else (b3.shape[2], b3.shape[1])
+    if kk != k:
+        raise ValueError("contraction lengths of a and b differ")
+    if k % 32 != 0 or n % 8 != 0:
+        raise ValueError("the bf16 grouped GEMM needs the contraction length in multiples of 32 and n in multiples of 8")
+    out = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+    lib = _lib.load()
+    with _hooked("grouped_gemm_bf16", m=total_m, n=n, k=k):
+        rc = lib.mxl_grouped_gemm_bf16(_ptr(a), _ptr(b3), _ptr(out), _ptr(group_lens), G, total_m, n, k,
+                                       _lib.BF_B_KN if b_kn else 0, _stream())
+    _lib.check(rc, "mxl_grouped_gemm_bf16")
+    return out
+
+
+def grouped_gemm_bf16_wgrad_impl(p: torch.Tensor, q: torch.Tensor, group_lens: Optional[torch.Tensor],
+                                 accum_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``c[g] = p[rows of g]^T . q[rows of g]`` for bf16 ``p [total_m, m_out]``, ``q [total_m, n_out]``: ``[G, m_out,
+    n_out]`` bf16, zeros for a group without tokens; or added to the float32 ``accum_into`` of that shape."""
+    _require_cuda(p, q, group_lens, accum_into)
+    if p.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or p.dim() != 2 or q.dim() != 2 or p.shape[0] != q.shape[0]:
+        raise ValueError("the bf16 weight-gradient GEMM takes two 2-D bf16 tensors with the same number of rows")
+    G = _check_group_lens(group_lens, p.device) or 1
+    total_m, m_out = p.shape
+    n_out = q.shape[1]
+    if m_out % 8 != 0 or n_out % 8 != 0:
+        raise ValueError("the bf16 weight-gradient GEMM needs both output dims in multiples of 8")
+    if accum_into is not None:
+        if accum_into.dtype != torch.float32 or accum_into.numel() != G * m_out * n_out:
+            raise ValueError("accum_into must be a contiguous float32 buffer of the weight's size")
+        out = accum_into
+    else:
+        out = torch.empty((G, m_out, n_out), dtype=torch.bfloat16, device=p.device)
+    lib = _lib.load()
+    with _hooked("grouped_gemm_bf16_wgrad", m=total_m, n=m_out, k=n_out):
+        rc = lib.mxl_grouped_gemm_bf16_wgrad(_ptr(p), _ptr(q), _ptr(out), _ptr(group_lens), G, total_m, m_out, n_out,
+                                             _lib.BF_ACCUM_F32 if accum_into is not None else 0, _stream())
+    _lib.check(rc, "mxl_grouped_gemm_bf16_wgrad")
+    return out
+
+
 def glu_with_probs_fwd_impl(x, probs, row_mask, activation: str) -> torch.Tensor:
     """``act(x[:, :F]) * x[:, F:] * probs[:, None]`` in fp32, one rounding to bf16; masked rows give 0."""
     act, pd, row_mask = _glu_args(x, probs, row_mask, activation)

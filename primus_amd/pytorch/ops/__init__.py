@@ -643,36 +643,56 @@ def glu_grouped_gemm_fp4(x, probs, b, group_lens: torch.Tensor, activation: str 
 
 # ---------------------------------------------------------------------------
 # Unquantised operators.  The reference's modules fall back to them outside a
-# low-precision autocast (primus_turbo.py:1180-1188, :2210-2216).  They are not
-# part of the MX path and have no kernels of their own here: the dense one is
-# the library GEMM behind ``torch.matmul``, the grouped one a loop of those
-# (which reads ``group_lens`` back to the host).
+# low-precision autocast (primus_turbo.py:1180-1188, :2210-2216).  The grouped
+# one has its own kernels (csrc/mx_gemm_bf16.hip): tokens per expert stay on
+# the device, as in the quantised operators.  The dense one is the library GEMM
+# behind ``torch.matmul``.
 # ---------------------------------------------------------------------------
 class _PlainLinearAccum(torch.autograd.Function):
-    """Unquantised ``a . b^T`` (dense or per expert) whose weight gradient is added to ``b.main_grad``."""
+    """Unquantised dense ``a . b^T`` whose weight gradient is added to ``b.main_grad``."""
 
     @staticmethod
-    def forward(ctx, a, b, lens, accum):
+    def forward(ctx, a, b, accum):
         ctx.save_for_backward(a, b)
-        ctx.lens, ctx.accum = lens, accum
-        if lens is None:
-            return torch.matmul(a, b.transpose(-2, -1))
-        return torch.cat([torch.matmul(rows, b[g].transpose(-2, -1)) for g, rows in enumerate(torch.split(a, lens, dim=0))], dim=0)
+        ctx.accum = accum
+        return torch.matmul(a, b.transpose(-2, -1))
 
     @staticmethod
     def backward(ctx, dy):
         a, b = ctx.saved_tensors
         target, _ = ctx.accum
-        if ctx.lens is None:
-            grad_a = torch.matmul(dy, b)
-            target.add_(torch.matmul(dy.transpose(-2, -1), a))
-        else:
-            parts = []
-            for g, (d, rows) in enumerate(zip(torch.split(dy, ctx.lens, dim=0), torch.split(a, ctx.lens, dim=0))):
-                parts.append(torch.matmul(d, b[g]))
-                target[g].add_(torch.matmul(d.transpose(-2, -1), rows))
-            grad_a = torch.cat(parts, dim=0)
-        return grad_a, _finish_wgrad(None, ctx.accum, True, tuple(b.shape)), None, None
+        grad_a = torch.matmul(dy, b)
+        target.add_(torch.matmul(dy.transpose(-2, -1), a))
+        return grad_a, _finish_wgrad(None, ctx.accum, True, tuple(b.shape)), None
+
+
+class _GroupedLinearBf16(torch.autograd.Function):
+    """``a[rows of g] . b[g]^T`` (``trans_b``) or ``a[rows of g] . b[g]`` on bf16 operands through the grouped bf16
+    kernels; ``group_lens`` is a device tensor and is never read on the host.  With ``accum`` the weight gradient is
+    added to the float32 ``main_grad`` inside the wgrad GEMM."""
+
+    @staticmethod
+    def forward(ctx, a, b, group_lens, trans_b, accum):
+        ctx.save_for_backward(a, b, group_lens)
+        ctx.trans_b, ctx.accum = trans_b, accum
+        return K.grouped_gemm_bf16_impl(a, b, group_lens, b_kn=not trans_b)
+
+    @staticmethod
+    def backward(ctx, dy):
+        a, b, group_lens = ctx.saved_tensors
+        dy = dy.contiguous()
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        grad_a = grad_b = None
+        if ctx.needs_input_grad[0]:
+            # b [G, n, k]: dx = dy . b_g contracts over n, which is b's slow dim; b [G, k, n]: dx = dy . b_g^T
+            grad_a = K.grouped_gemm_bf16_impl(dy, b, group_lens, b_kn=ctx.trans_b)
+        if ctx.needs_input_grad[1]:
+            p, q = (dy, a) if ctx.trans_b else (a, dy)      # dW [n, k] = dy^T x;  dW [k, n] = x^T dy
+            fused = ctx.accum is not None and _fusable(ctx.accum[0])
+            gb = K.grouped_gemm_bf16_wgrad_impl(p, q, group_lens, accum_into=ctx.accum[0] if fused else None)
+            grad_b = _finish_wgrad(None if fused else gb, ctx.accum, fused, tuple(b.shape))
+        return grad_a, grad_b, None, None, None
 
 
 def gemm(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[torch.dtype] = None,
@@ -681,7 +701,7 @@ def gemm(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[
     if accum is not None:
         if trans_a or not trans_b or a.dim() != 2:
             raise ValueError("fuse_bgrad_accum_pattern is defined for the NT linear on 2-D activations")
-        out = _PlainLinearAccum.apply(a, b, None, accum)
+        out = _PlainLinearAccum.apply(a, b, accum)
         return out if out_dtype is None else out.to(out_dtype)
     a2 = a.transpose(-2, -1) if trans_a else a
     b2 = b.transpose(-2, -1) if trans_b else b
@@ -689,21 +709,48 @@ def gemm(a, b, trans_a: bool = False, trans_b: bool = True, out_dtype: Optional[
     return out if out_dtype is None else out.to(out_dtype)
 
 
+class _GroupedLinearLibrary(torch.autograd.Function):
+    """The same operator for operands the bf16 kernels do not take -- float32 / float16, or tensors in host memory, as
+    the host-side module tests use them: a loop of the library GEMM behind ``torch.matmul`` per expert, which reads
+    the counts on the host.  bf16 operands on the GPU never come here."""
+
+    @staticmethod
+    def forward(ctx, a, b, lens, trans_b, accum):
+        ctx.save_for_backward(a, b)
+        ctx.lens, ctx.trans_b, ctx.accum = lens, trans_b, accum
+        parts = [torch.matmul(rows, b[g].transpose(-2, -1) if trans_b else b[g]) for g, rows in enumerate(torch.split(a, lens, dim=0))]
+        return torch.cat(parts, dim=0)
+
+    @staticmethod
+    def backward(ctx, dy):
+        a, b = ctx.saved_tensors
+        parts, grads = [], []
+        for g, (d, rows) in enumerate(zip(torch.split(dy, ctx.lens, dim=0), torch.split(a, ctx.lens, dim=0))):
+            parts.append(torch.matmul(d, b[g] if ctx.trans_b else b[g].transpose(-2, -1)))
+            grads.append(torch.matmul(d.transpose(-2, -1), rows) if ctx.trans_b else torch.matmul(rows.transpose(-2, -1), d))
+        grad_b = torch.stack(grads, dim=0).to(b.dtype)
+        return torch.cat(parts, dim=0), _finish_wgrad(grad_b, ctx.accum, False, tuple(b.shape)), None, None, None
+
+
 def grouped_gemm(a, b, group_lens: torch.Tensor, trans_b: bool = True,
                  fuse_bgrad_accum_pattern: Optional[str] = None):
+    """Per expert g: ``a[rows of g] @ b[g]^T`` (``trans_b``; ``b [G, n, k]``) or ``a[rows of g] @ b[g]`` (``b [G, k, n]``)
+    (primus/backends/megatron/core/extensions/primus_turbo.py:2210-2216).  bf16 operands on the GPU -- what the
+    reference's modules pass -- run on the grouped bf16 kernels: ``group_lens`` (int64, on the device) is consumed by
+    the kernels, no host read, so the call can be captured in a graph; rows of ``a`` the counts do not cover are left
+    unwritten; contraction length and output width in multiples of 32 (anything else raises: there is no second path
+    for bf16).  Other dtypes, and tensors in host memory, go through a per-expert loop of the library GEMM."""
+    accum = _accum_from(b, fuse_bgrad_accum_pattern)
+    if accum is not None and not trans_b:
+        raise ValueError("fuse_bgrad_accum_pattern is defined for the NT linear")
+    if a.is_cuda and a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16:
+        if a.shape[-1] % 32 != 0 or b.shape[-1] % 32 != 0 or b.shape[-2] % 32 != 0:
+            raise ValueError("the bf16 grouped GEMM needs k and n in multiples of 32 (forward and dgrad contract over them)")
+        return _GroupedLinearBf16.apply(a.contiguous(), b.contiguous(), _lens(group_lens), bool(trans_b), accum)
     lens = [int(v) for v in _lens(group_lens).tolist()]
     if sum(lens) != a.shape[0]:
         raise ValueError("group_lens must sum to the number of rows of a")
-    accum = _accum_from(b, fuse_bgrad_accum_pattern)
-    if accum is not None:
-        if not trans_b:
-            raise ValueError("fuse_bgrad_accum_pattern is defined for the NT linear")
-        return _PlainLinearAccum.apply(a, b, lens, accum)
-    outs = []
-    for g, rows in enumerate(torch.split(a, lens, dim=0)):
-        w = b[g].transpose(-2, -1) if trans_b else b[g]
-        outs.append(torch.matmul(rows, w))
-    return torch.cat(outs, dim=0)
+    return _GroupedLinearLibrary.apply(a, b, lens, bool(trans_b), accum)
 
 
 # ---------------------------------------------------------------------------

@@ -156,7 +156,9 @@ int mxl_quantize_ex(const void* x_bf16, int64_t rows, int64_t cols, int64_t row_
  * k_ld / n_ld are the padded pitches of the two copies (>= k / >= n, multiples
  * of 32, n_ld at most n rounded up to 128; 0 means no padding): codes
  * [batch, n, k_ld] and [batch, k, n_ld], padding = zero codes, scale byte 0.
- * Requires n % 32 == 0 and k % 32 == 0. */
+ * Requires n % 32 == 0 and k % 32 == 0.  q_colT may be NULL while s_colT is not (and q_row is given): then only the
+ * SCALES of the transposed copy are written -- with 2-D blocks its codes are the row-wise codes transposed, which
+ * the GEMM can read as they lie (MXL_GF_B_TRANSPOSED). */
 int mxl_quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int64_t k, int64_t k_ld,
                            int64_t n_ld, int fmt, int scale_mode, void* q_row, void* s_row, void* q_colT, void* s_colT,
                            void* stream);
@@ -223,6 +225,15 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * (fuse_bgrad_accum_pattern = "megatron": the GEMM's beta = 1 epilogue adds into weight.main_grad,
  * primus_turbo.py:166-240, 243-275) -- available here for the MX recipes too.  With no tokens nothing is added. */
 #define MXL_GF_ACCUM_F32 2u
+/* mxl_grouped_gemm_nt_ex / _scaled only, together with MXL_GF_KSTEP: b_codes are the K-step-major codes of the TRANSPOSED
+ * matrices -- of [num_groups, k, n] quantised along n, i.e. [n_ld / 64][num_groups * k][64 bytes] with n_ld = n rounded up
+ * to 128 -- while b_scales stay the scales of [num_groups, n, k / 32].  This is the dgrad GEMM reading the ROW-WISE copy
+ * of the weight, so that no transposed copy of the weight's codes has to be written or cached (the reference keeps a
+ * second quantised copy for it, _maybe_create_quantized_weight_buffers, primus_turbo.py:278-358).  Meaningful where a
+ * transposed copy is the same codes transposed: 2-D 32 x 32 block scales (mxl_quantize_weight_2d_ex writes the transposed
+ * copy's scales alone when q_colT is NULL and s_colT is not) or tensor-wise scaling.  E4M3 weights, E4M3 (or, scaled,
+ * E5M2) rows, at most 128 groups; k % 128 == 0.  Bit-identical to the GEMM on the transposed copy. */
+#define MXL_GF_B_TRANSPOSED 8u
 int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                            const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                            int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);

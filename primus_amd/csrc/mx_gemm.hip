@@ -649,8 +649,18 @@ constexpr int ring_lds_bytes() {
 }
 
 
-template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false>
+// BT (forward / dgrad of FP8-format operands): b_codes hold the codes of the TRANSPOSED matrices -- [G, k, n] instead of
+// [G, n, k], K-step-major along n: [n_ld / 64][G * k][64] -- i.e. the row-wise copy of a weight serves its dgrad GEMM
+// and no transposed copy of the codes is ever written.  Valid where transposing the codes is all a transposed copy
+// amounts to: 2-D 32 x 32 block scales (the quantiser's transposed SCALES are still passed as b_scales, they are
+// 1/32 of the bytes) or one scale per tensor.  A K step of b is then 64 rows (contraction) x 256 columns: four pieces
+// of 64 rows x 64 bytes, one per 64-column plane, each a contiguous 4 KiB; the fragments come out of LDS through the
+// transposing read ds_read_b64_tr_b8, which hands a lane 8 consecutive contraction bytes of its own column.  Measured
+// lane mapping of that read: inside a block of 16 lanes, lane 8 a + e receives byte e of the 8-byte pieces
+// addressed by lanes a, a + 2, ..., a + 14 (in this order).
+template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false, bool BT = false>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
+    static_assert(!BT || (MODE == MODE_FWD && AFMT != kFmtE2M1 && BFMT != kFmtE2M1), "transposed weight codes: forward / dgrad, FP8 formats");
     // ACCUM (wgrad): p.c is a float32 buffer the result is ADDED to (one workgroup per output tile: no race, and the
     // sum does not depend on any order)
     static_assert(!ACCUM || MODE == MODE_WGRAD, "the accumulating epilogue belongs to the weight-gradient GEMM");
@@ -747,7 +757,10 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     const int64_t b_rows_total = (MODE == MODE_FWD) ? (int64_t)G * p.n : p.n;
     // K-step-major codes: [k / 64][rows][64]; scales: [ceil(k / 512)][rows][16] (16 bytes = 8 K steps of a row)
     const uint32_t a_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * BK));
-    const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * B_ROW));
+    // BT: the rows of b's code array are the contraction index (G * k of them); a K step moves on by 64 rows inside
+    // a plane, and the four load rounds of a step are one plane apart
+    const int64_t bt_rows = (int64_t)G * p.k;
+    const uint32_t b_cstride = BT ? (uint32_t)(64 * BK) : (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * B_ROW));
     const uint32_t a_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * 16));
     const uint32_t b_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * 16));
     // a load round covers 64 consecutive rows = 4 KiB: thread -> (row t / 4, 16-byte piece t % 4); the XOR swizzle of
@@ -763,7 +776,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         va[e] = addr::ring_code_lane(t, e, false);
-        vb[e] = addr::ring_code_lane(t, e, B4);
+        vb[e] = BT ? addr::ring_bt_lane(t, e, bt_rows) : addr::ring_code_lane(t, e, B4);
     }
 
     struct Tile {
@@ -830,7 +843,9 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // check covers the per-lane offset (row, load round) and the scalar offset (K step / panel) together, so a
         // row past the operand's last one is dropped in the last plane and reads a later plane's rows in the others.
         {
-            const addr::Desc da = addr::ring_code_desc(a_rows_total, p.k / KS, a_row0, BK), db = addr::ring_code_desc(b_rows_total, p.k / KS, b_row0, B_ROW);
+            const addr::Desc da = addr::ring_code_desc(a_rows_total, p.k / KS, a_row0, BK);
+            const addr::Desc db = BT ? addr::ring_bt_desc(bt_rows, (p.n + 127) / 128 * 2, (int64_t)grp * p.k, (int64_t)pid_n * (BN / 64))
+                                     : addr::ring_code_desc(b_rows_total, p.k / KS, b_row0, B_ROW);
             const addr::Desc dsa = addr::ring_panel_desc(a_rows_total, n_panels, a_row0), dsb = addr::ring_panel_desc(b_rows_total, n_panels, b_row0);
             d.ra = make_rsrc(p.a + da.base, da.records);
             d.rb = make_rsrc(p.b + db.base, db.records);
@@ -903,7 +918,13 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
          F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; } } while (0)
 #define MXL_RD_B(F, J) \
     do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * B_ROW); \
-         if (B4) { \
+         if (BT) { \
+             uint8_t* t_ = (uint8_t*)sn + A_BYTES + (2 * wn + ((J) >> 1)) * 4096; \
+             _Pragma("unroll") for (int q_ = 0; q_ < 2; ++q_) _Pragma("unroll") for (int h_ = 0; h_ < 2; ++h_) { \
+                 const v2i v_ = __builtin_amdgcn_ds_read_tr8_b64_v2i32( \
+                     (__attribute__((address_space(3))) v2i*)(t_ + 2048 * q_ + bt_off[h_][(J) & 1])); \
+                 F.b[J][4 * q_ + 2 * h_] = v_[0]; F.b[J][4 * q_ + 2 * h_ + 1] = v_[1]; } \
+         } else if (B4) { \
              const uint4 lo_ = *(const uint4*)(r_ + b4_lo); \
              F.b[J][0] = lo_.x; F.b[J][1] = lo_.y; F.b[J][2] = lo_.z; F.b[J][3] = lo_.w; \
              F.b[J][4] = 0; F.b[J][5] = 0; F.b[J][6] = 0; F.b[J][7] = 0; \
@@ -920,6 +941,20 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     const int sw = (lr >> 2) & 3;
     const int a_frag = (wm * 128 + lr) * BK, b_frag = (wn * 128 + lr) * B_ROW;
     const int b4_lo = 16 * (g ^ ((lr >> 3) & 1));      // FP4: lane (row, g) holds elements 32 g .. 32 g + 31 of the K step
+    // BT: this lane ADDRESSES contraction row 16 g + 8 h + tj (+ 32 for the second half of the step) and the 8-byte
+    // piece of its 16-lane block's 16 columns: bt_off[h][J & 1] inside a plane's 64 rows x 64 bytes (same swizzle
+    // as the loads: 16-byte piece XOR (row / 4) % 4)
+    int bt_off[2][2];
+    if (BT) {
+        const int tj = (l & 15) >> 1, ta = l & 1, tblk = (l >> 4) & 1;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int row = 16 * g + 8 * h + tj, cb = 32 * jj + 16 * tblk + 8 * ta;
+                bt_off[h][jj] = row * 64 + 16 * ((cb >> 4) ^ ((row >> 2) & 3)) + (cb & 15);
+            }
+    }
     const int a_lo = 16 * (g ^ sw), a_hi = 16 * ((2 + g) ^ sw);
     // Scale bytes: a panel row holds [g][K step] = 2 x 8 bytes, so the 8 bytes at (row, g) are the lane's scale
     // bytes of the panel's 8 K steps.  They are read once per panel (8 reads of 8 bytes per wave, 512 consecutive
@@ -1291,13 +1326,13 @@ static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
-template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false>
+template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false, bool BT = false>
 static int launch_gemm_ring(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = ring_lds_bytes();
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set[64];
     const int slot = current_device_slot();
-    auto kern = mx_gemm_ring_kernel<AFMT, BFMT, MODE, ALPHA, ACCUM>;
+    auto kern = mx_gemm_ring_kernel<AFMT, BFMT, MODE, ALPHA, ACCUM, BT>;
     if (!attr_set[slot].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
@@ -1386,6 +1421,18 @@ static int dispatch_wgrad_accum_ring(int afmt, int bfmt, const GemmArgs& a, int6
     return MXL_EINVAL;
 }
 
+// forward / dgrad on the row-wise codes of the transposed weight (MXL_GF_B_TRANSPOSED): E4M3 weights, E4M3 or E5M2 rows
+static int dispatch_gemm_ring_bt(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
+    if (bfmt != MXL_FMT_E4M3 || a.num_groups > RING_MAX_GROUPS) return MXL_EINVAL;
+    if (a.alpha_a != nullptr) {
+        if (afmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE_FWD, true, false, true>(a, max_tiles, st);
+        if (afmt == MXL_FMT_E4M3) return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE_FWD, true, false, true>(a, max_tiles, st);
+        return MXL_EINVAL;
+    }
+    if (afmt != MXL_FMT_E4M3) return MXL_EINVAL;
+    return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE_FWD, false, false, true>(a, max_tiles, st);
+}
+
 // a_rows / b_rows: rows of the whole operands (for the 4 GiB bound of the chunk-major layout)
 // layout: 0 row-major codes, 1 K-chunk-major codes, 2 K-step-major codes and scales
 template <int MODE>
@@ -1430,8 +1477,9 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t w
 static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes, const void* b_scales,
                            int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
                            int64_t k, const float* alpha_a, const float* alpha_b, uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP | MXL_GF_B_TRANSPOSED)) return MXL_EINVAL;
     if ((flags & MXL_GF_KCHUNK) && (flags & MXL_GF_KSTEP)) return MXL_EINVAL;
+    if ((flags & MXL_GF_B_TRANSPOSED) && !(flags & MXL_GF_KSTEP)) return MXL_EINVAL;
     if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
     if (k > MAX_CONTRACTION) return MXL_EINVAL;   // tile-relative byte offsets are 32-bit
@@ -1455,6 +1503,13 @@ static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt,
     a.alpha_a = alpha_a;
     a.alpha_b = alpha_b;
     const int64_t max_tiles = (total_m / BM + num_groups) * ((n + BN - 1) / BN);
+    if (flags & MXL_GF_B_TRANSPOSED) {
+        // offsets inside an operand are 32-bit; the kernel keeps a tile's first output row in 32 bits
+        const int64_t n_ld = (n + 127) / 128 * 128;
+        if (total_m * k >= ((int64_t)1 << 32) || (int64_t)num_groups * k * n_ld >= ((int64_t)1 << 32) || total_m >= ((int64_t)1 << 31))
+            return MXL_EINVAL;
+        return dispatch_gemm_ring_bt(a_fmt, b_fmt, a, max_tiles, (hipStream_t)stream);
+    }
     return dispatch_gemm<MODE_FWD>(a_fmt, b_fmt, a, max_tiles, (flags & MXL_GF_KSTEP) ? 2 : (flags & MXL_GF_KCHUNK) ? 1 : 0, total_m,
                                    (int64_t)num_groups * n, (hipStream_t)stream);
 }

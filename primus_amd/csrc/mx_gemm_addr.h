@@ -70,6 +70,17 @@ MXL_HD uint32_t ring_code_lane(int t, int e, bool half_rows) {
     const int row = t >> 2;
     return (uint32_t)(row * 64 + 16 * ((t & 3) ^ ((row >> 2) & 3)) + e * 4096);
 }
+// The same operand read TRANSPOSED (the ring kernel's BT mode): the code array is [planes][rows_total][64] with
+// rows_total = groups * contraction length; a tile's descriptor starts at plane `plane0` (its first 64 output columns),
+// row `row0` (the group's first contraction row); load round e adds e planes per lane, the K step adds
+// step * 64 rows * 64 bytes as the scalar offset (clamped to the contraction range by the kernel).
+MXL_HD Desc ring_bt_desc(int64_t rows_total, int64_t planes, int64_t row0, int64_t plane0) {
+    const int64_t base = (plane0 * rows_total + row0) * 64;
+    return Desc{base, planes * rows_total * 64 - base};
+}
+MXL_HD uint32_t ring_bt_lane(int t, int e, int64_t rows_total) {
+    return ring_code_lane(t, 0, false) + (uint32_t)e * (uint32_t)(rows_total * 64);
+}
 // Scale panels [panels][rows_total][16]: thread t fetches the 16 bytes of tile row t; the panel is chosen by the
 // scalar offset panel * rows_total * 16.
 MXL_HD Desc ring_panel_desc(int64_t rows_total, int64_t panels, int64_t row0) {

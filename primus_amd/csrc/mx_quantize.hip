@@ -289,6 +289,11 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
         m = max(m, (uint32_t)__shfl_xor((int)m, 16));
         m = max(m, (uint32_t)__shfl_xor((int)m, 32));
         tile_byte = block_byte<FMT, SMODE>(m);
+        // the transposed copy's scales without its codes: the tile's byte for each of the lane's 8 columns
+        if (!COL && a.s_colT != nullptr && rg == 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ((uint8_t*)scol_tile)[(8 * c16 + j) * 4 + w] = (uint8_t)tile_byte;
+        }
     } else if (COL && !RHT) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -483,7 +488,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
             for (int b = 0; b < 4 && b < nb; ++b) dst[b] = (uint8_t)(v >> (8 * b));
         }
     }
-    if (COL) {
+    if (COL || (TWOD && a.s_colT != nullptr)) {
         const int64_t out_rows_base = TWOD ? (batch_off_rows / a.mat_rows) * a.cols : 0;  // TWOD: matrix * k
         const int64_t m0 = TWOD ? (src_row0 - batch_off_rows) : (int64_t)pt * QT;          // position along W
         if (t < QT && col0 + t < a.cols) {
@@ -499,6 +504,7 @@ __global__ __launch_bounds__(QTHREADS) void mx_quant_kernel(QuantArgs a) {
                 for (int b = 0; b < 4 && b < nb; ++b) dst[b] = (uint8_t)(v >> (8 * b));
             }
         }
+        if (!COL) return;                        // (scales only)
         constexpr int ROWB = FP4 ? QT / 2 : QT;  // bytes per transposed tile row
         constexpr int LPR = ROWB / 16;           // lanes per row
         const int64_t wbytes = FP4 ? a.W / 2 : a.W;
@@ -803,7 +809,9 @@ static int quantize_weight_2d(const void* w_bf16, int64_t batch, int64_t n, int6
     if (k_ld < k || n_ld < n || k_ld % MXL_BLOCK != 0 || n_ld % MXL_BLOCK != 0) return MXL_EINVAL;
     if (n_ld > (n + QT - 1) / QT * QT) return MXL_EINVAL;  // padding of the transposed copy stays inside the last tile
     if (!w_bf16 || batch <= 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % MXL_BLOCK != 0) return MXL_EINVAL;
-    if ((q_row == nullptr) != (s_row == nullptr) || (q_colT == nullptr) != (s_colT == nullptr)) return MXL_EINVAL;
+    // (the transposed copy's scales may be asked for without its codes, next to a row-wise copy)
+    if ((q_row == nullptr) != (s_row == nullptr) || (q_colT != nullptr && s_colT == nullptr)) return MXL_EINVAL;
+    if (s_colT != nullptr && q_colT == nullptr && q_row == nullptr) return MXL_EINVAL;
     if (!q_row && !q_colT) return MXL_EINVAL;
     QuantArgs a;
     a.x = (const uint16_t*)w_bf16;

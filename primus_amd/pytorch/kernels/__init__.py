@@ -349,12 +349,16 @@ def quantize_mx_weight_2d_impl(
     colwise: bool = True,
     pad_to: int = 1,
     kchunk=False,
+    col_scales_only: bool = False,
 ):
     """2-D (32x32 tile) MX quantisation of ``w[n, k]`` or ``w[G, n, k]``;
     returns ``(q_row [.., n, k], s_row [.., n, k/32], q_colT [.., k, n],
     s_colT [.., k, n/32])`` with ``None`` for a copy that was not requested.
     ``pad_to`` rounds the last dim of both copies up (zero padding).  With ``kchunk`` the codes come back
-    K-chunk-major over the flattened batch: ``[k_ld / 128, G * n, 128]`` and ``[n_ld / 128, G * k, 128]``."""
+    K-chunk-major over the flattened batch: ``[k_ld / 128, G * n, 128]`` and ``[n_ld / 128, G * k, 128]``.
+    ``col_scales_only`` (with ``rowwise`` and ``colwise``): the transposed copy's SCALES are written, its codes are not
+    (``q_colT`` comes back None): with 2-D blocks they are the row-wise codes transposed, which the forward / dgrad
+    GEMM reads as they lie (``b_transposed``)."""
     if w.dtype != torch.bfloat16 or w.dim() not in (2, 3):
         raise ValueError("weight quantisation expects a 2-D or 3-D bfloat16 tensor")
     _require_cuda(w)
@@ -374,12 +378,15 @@ def quantize_mx_weight_2d_impl(
         q_row = torch.empty(shape, dtype=torch.uint8, device=dev)
         sshape = _scale_shape(batch * n, k_ld, kchunk) if _paneled(kchunk) else lead + (n, k_ld // BLOCK)
         s_row = torch.empty(sshape, dtype=torch.uint8, device=dev)
+    if col_scales_only and not (rowwise and colwise):
+        raise ValueError("col_scales_only asks for the row-wise copy plus the transposed copy's scales")
     if colwise:
-        shape = _code_shape(batch * k, n_ld, per, kchunk) if kchunk else lead + (k, n_ld // per)
-        q_col = torch.empty(shape, dtype=torch.uint8, device=dev)
+        if not col_scales_only:
+            shape = _code_shape(batch * k, n_ld, per, kchunk) if kchunk else lead + (k, n_ld // per)
+            q_col = torch.empty(shape, dtype=torch.uint8, device=dev)
         sshape = _scale_shape(batch * k, n_ld, kchunk) if _paneled(kchunk) else lead + (k, n_ld // BLOCK)
         s_col = torch.empty(sshape, dtype=torch.uint8, device=dev)
-    with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise):
+    with _hooked("quantize_weight_2d", rows=batch * n, cols=k, fmt=fmt, rowwise=rowwise, colwise=colwise and not col_scales_only):
         rc = _lib.load().mxl_quantize_weight_2d_ex(
             _ptr(w), batch, n, k, k_ld, n_ld, fmt, scale_mode, _ptr(q_row), _ptr(s_row), _ptr(q_col), _ptr(s_col),
             _qflag(kchunk), _stream()
@@ -453,14 +460,15 @@ def _check_scales(scales: torch.Tensor, rows: int, k: int, kchunk, what: str) ->
         raise ValueError(f"{what}: scale shape {tuple(scales.shape)} does not match {rows} rows x {k} elements")
 
 
-def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=False) -> torch.Tensor:
-    """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T.  ``kchunk``: both code tensors are K-chunk-major."""
+def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=False, b_transposed: bool = False) -> torch.Tensor:
+    """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T.  ``kchunk``: both code tensors are K-chunk-major.  ``b_transposed``: see
+    ``grouped_gemm_mx_nt_impl``."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
     if kchunk:
         return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _paneled(kchunk) else b_scale.unsqueeze(0),
-                                       None, kchunk=kchunk)
+                                       None, kchunk=kchunk, b_transposed=b_transposed)
     _check_contraction(a.shape[-1] * _per_byte(a_fmt), b.shape[-1] * _per_byte(b_fmt))
     a, a_scale, k = _pad_k(a, a_scale, a_fmt)
     b, b_scale, kb = _pad_k(b, b_scale, b_fmt)
@@ -474,14 +482,41 @@ def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=Fal
     return c
 
 
-def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16, kchunk=False) -> torch.Tensor:
+def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.bfloat16, kchunk=False,
+                            b_transposed: bool = False) -> torch.Tensor:
     """Forward / dgrad grouped GEMM: rows of ``a[total_m, k]`` split by
     ``group_lens``; ``b`` is ``[G, n, k]``.  ``kchunk``: both code tensors are K-chunk-major,
-    ``a [k / 128, total_m, 128]`` and ``b [k / 128, G * n, 128]``; ``b_scale`` is ``[G, n, k / 32]`` as always."""
+    ``a [k / 128, total_m, 128]`` and ``b [k / 128, G * n, 128]``; ``b_scale`` is ``[G, n, k / 32]`` as always.
+    ``b_transposed`` (K-step-major FP8 operands): ``b`` holds the codes of the transposed matrices, ``[n_ld / 64,
+    G * k, 64]`` -- the row-wise copy of a weight ``[G, k, n]`` serving its dgrad GEMM -- and ``b_scale`` the scale
+    panels of ``[G * n, k]`` (the transposed copy's scales)."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale, group_lens)
     G = _check_group_lens(group_lens, a.device)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if b_transposed:
+        if _layout(kchunk) != LAYOUT_KSTEP:
+            raise ValueError("b_transposed needs K-step-major operands")
+        total_m, k = _chunked_dims(a, a_fmt, kchunk)
+        groups = max(G, 1)
+        bt_rows, n_ld = _chunked_dims(b, b_fmt, kchunk)           # rows = groups * k, width = n padded to 128
+        if bt_rows != groups * k:
+            raise ValueError("b_transposed: the rows of b's code array must be num_groups * k")
+        if b_scale.dim() != 3 or b_scale.shape[2] != 16 or b_scale.shape[1] % groups:
+            raise ValueError("b_transposed: b_scale must be the K-step-major scale panels of [num_groups * n, k]")
+        n = b_scale.shape[1] // groups
+        if _round_up(n, KCHUNK) != n_ld:
+            raise ValueError("b_transposed: the code array's width does not match the scales' rows")
+        _check_scales(a_scale, total_m, k, kchunk, "a_scale")
+        _check_scales(b_scale, groups * n, k, kchunk, "b_scale")
+        c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+        with _hooked("grouped_gemm_nt" if G else "gemm_nt", m=total_m, n=n, k=k):
+            rc = _lib.load().mxl_grouped_gemm_nt_ex(
+                _ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), _ptr(group_lens), groups, total_m, n, k,
+                _lib.GF_KSTEP | _lib.GF_B_TRANSPOSED, _stream()
+            )
+        _lib.check(rc, "mxl_grouped_gemm_nt_ex")
+        return c
     if kchunk:
         total_m, k = _chunked_dims(a, a_fmt, kchunk)
         b_rows, kb = _chunked_dims(b, b_fmt, kchunk)

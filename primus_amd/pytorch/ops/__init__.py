@@ -36,6 +36,7 @@ from ..core.low_precision import (
 from ..core.quantized_tensor import QuantizedTensor, QuantizedTensorPair
 
 __all__ = ["gemm", "grouped_gemm", "gemm_fp8", "gemm_fp4", "grouped_gemm_fp8", "grouped_gemm_fp4", "set_wgrad_overlap",
+           "set_dgrad_reads_rowwise_weight",
            "swiglu_with_probs", "geglu_with_probs", "tokens_per_expert_to_mask", "glu_grouped_gemm_fp8",
            "glu_grouped_gemm_fp4", "manual_sr_seed", "set_kchunk_layout", "rmsnorm", "rmsnorm_gemm_fp8", "rmsnorm_gemm_fp4", "pad_groups", "unpad_groups"]
 
@@ -56,6 +57,16 @@ def set_kchunk_layout(enabled: bool) -> None:
     """Store quantised operands K-chunk-major between the quantisers and the GEMMs (default on; the
     row-major layout gives the same results bit for bit and is what operands of 4 GiB or more use)."""
     K.set_kchunk_default(enabled)
+
+
+_dgrad_reads_rowwise = True
+
+
+def set_dgrad_reads_rowwise_weight(enabled: bool) -> None:
+    """Whether the MXFP8 operators let dgrad read the row-wise weight codes transposed instead of writing a
+    transposed copy of the codes in the forward (default on; same results bit for bit)."""
+    global _dgrad_reads_rowwise
+    _dgrad_reads_rowwise = bool(enabled)
 
 
 def set_wgrad_overlap(enabled: bool) -> None:
@@ -201,9 +212,16 @@ class _MXLinearFunction(torch.autograd.Function):
                     raise ValueError("QuantizedTensorPair.data_t must be quantised along axis=-2")
                 w_col, w_cs = _cached_codes(b_t, kc), _cached_scales(b_t, kc)
         else:
+            # FP8 weights on the ring kernel: dgrad reads the ROW-WISE codes transposed (2-D blocks: the transposed
+            # copy is the same codes transposed), so only that copy's scales are written next to the row-wise copy
+            bt = (need_dgrad and _dgrad_reads_rowwise and kc == K.LAYOUT_KSTEP and w_fmt == _lib.FMT_E4M3
+                  and act_fmt == _lib.FMT_E4M3 and b.shape[-2] % K.GEMM_K_ALIGN == 0 and b.shape[-1] % K.GEMM_K_ALIGN == 0)
             w_row, w_rs, w_col, w_cs = K.quantize_mx_weight_2d_impl(
                 b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
+                col_scales_only=bt,
             )
+            if bt:
+                w_col = w_row
         if grouped:
             y = K.grouped_gemm_mx_nt_impl(a_row, a_rs, w_row, w_rs, group_lens, kchunk=kc)
         else:
@@ -219,6 +237,7 @@ class _MXLinearFunction(torch.autograd.Function):
         ctx.grad_sr = bool(grad_sr) and act_fmt == _lib.FMT_E2M1
         ctx.rht_signs = rht_signs
         ctx.kchunk = kc
+        ctx.b_transposed = (not isinstance(b, QuantizedTensor)) and bt
         ctx.norm = norm
         ctx.accum = accum      # (float32 buffer the weight gradient is added to, object that gets the flag) or None
         return y
@@ -247,9 +266,9 @@ class _MXLinearFunction(torch.autograd.Function):
             side.wait_stream(main)   # the quantised operands are ready
         if need_dgrad:
             if grouped:
-                grad_a = K.grouped_gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, group_lens, kchunk=kc)
+                grad_a = K.grouped_gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, group_lens, kchunk=kc, b_transposed=ctx.b_transposed)
             else:
-                grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc)
+                grad_a = K.gemm_mx_nt_impl(d_row, d_rs, w_col, w_cs, kchunk=kc, b_transposed=ctx.b_transposed)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
             fused = _fusable(target) and kc != K.LAYOUT_ROWMAJOR   # the GEMM's epilogue adds into the float32 buffer

@@ -92,7 +92,24 @@ static void check_ring(int row_bytes, int64_t rows_total, int64_t steps, int64_t
             request(dp, ring_panel_lane(t), (uint32_t)(pn * rows_total * 16), pbytes, row0 + t < rows_total && pn < panels, "ring panels");
 }
 
+// the ring kernel reading b transposed: planes of [rows_total][64], descriptor at (plane0, row0), round e = e planes
+// further on per lane, K step = 64 rows further on in the scalar offset
+static void check_ring_bt(int64_t groups, int64_t kc, int64_t planes, int64_t grp, int64_t plane0) {
+    const int64_t rows_total = groups * kc, bytes = planes * rows_total * 64;
+    const Desc d = ring_bt_desc(rows_total, planes, grp * kc, plane0);
+    const int64_t steps = kc / 64;
+    for (int64_t st = 0; st < steps; ++st)           // the kernel clamps the step to the contraction range
+        for (int e = 0; e < 4; ++e)
+            for (int t = 0; t < 256; ++t)
+                request(d, ring_bt_lane(t, e, rows_total), (uint32_t)(st * 64 * 64), bytes, plane0 + e < planes, "ring codes transposed");
+}
+
 int main() {
+    for (int64_t groups : {1, 3})
+        for (int64_t kc : {128, 384})
+            for (int64_t planes : {2, 4, 6, 10})
+                for (int64_t grp = 0; grp < groups; ++grp)
+                    for (int64_t plane0 = 0; plane0 < planes; plane0 += 4) check_ring_bt(groups, kc, planes, grp, plane0);
     for (int64_t rows_total : {1, 31, 37, 255, 256, 257, 300, 511, 513, 1000})
         for (int64_t row0 = 0; row0 < rows_total; row0 += (rows_total > 300 ? 97 : 1) + (row0 % 7 == 0 ? 0 : 12)) {
             for (int64_t k_slots : {1, 2, 5})

@@ -234,6 +234,11 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * copy's scales alone when q_colT is NULL and s_colT is not) or tensor-wise scaling.  E4M3 weights, E4M3 (or, scaled,
  * E5M2) rows, at most 128 groups; k % 128 == 0.  Bit-identical to the GEMM on the transposed copy. */
 #define MXL_GF_B_TRANSPOSED 8u
+/* mxl_grouped_gemm_nt_ex only, alone (row-major operands): b_codes are E2M1 codes in the pre-shuffled byte order of
+ * mxl_shuffle_codes -- what gemm_fp4_impl(..., preshuffled=True) of the reference is handed for its second operand
+ * (primus_turbo_mxfp4_local.py:319-331; the first operand's codes are plain there).  E2M1 x E2M1, block scales in
+ * the plain row-major layout, n % 16 == 0.  Same results bit for bit as on the plain codes. */
+#define MXL_GF_B_SHUFFLED 16u
 int mxl_grouped_gemm_nt_ex(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes,
                            const void* b_scales, int b_fmt, void* c_bf16, const int64_t* group_lens,
                            int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);
@@ -451,8 +456,11 @@ int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, in
  * mxl_shuffle_scales: E8M0 bytes [rows, cols] -> [ceil(rows / 256) * 256, ceil(cols / 8) * 8] with zero bytes in the
  *   padding: every 32 rows x 8 columns become 256 consecutive bytes ([col % 4][row % 16][(col / 4) % 2][(row / 16) % 2]).
  * inverse != 0 converts back (src is the shuffled array, dst [rows, row_bytes] / [rows, cols]).  src and dst must not
- * overlap; code arrays must be 16-byte aligned.  The GEMM entry points read the plain layouts: a caller holding
- * pre-shuffled operands converts them back first (the Python boundary does). */
+ * overlap; code arrays must be 16-byte aligned.  The GEMMs read pre-shuffled weight CODES as they lie
+ * (MXL_GF_B_SHUFFLED); pre-shuffled SCALES (1/16 of the bytes of the codes) are converted back first, which the
+ * Python boundary does.  The byte orders are restated from AITER's published shuffle_weight(layout=(16, 16)) and
+ * e8m0_shuffle; the reference tree holds neither their source nor a fixture, so the orders are parity unpinned
+ * (the array shapes are pinned by primus_turbo_mxfp4_local.py:184-198). */
 int mxl_shuffle_codes(const void* src, int64_t rows, int64_t row_bytes, void* dst, int inverse, void* stream);
 int mxl_shuffle_scales(const void* src, int64_t rows, int64_t cols, void* dst, int inverse, void* stream);
 

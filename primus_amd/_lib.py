@@ -31,6 +31,7 @@ QF_SR, QF_RHT_COL, QF_KCHUNK, QF_KSTEP, QF_KSTEP128 = 1, 2, 4, 8, 16   # flags o
 GF_KCHUNK = 1                               # flag of the GEMM _ex entry points: operands are K-chunk-major
 GF_KSTEP = 4                                # ... K-step-major codes and scales (ring kernel)
 GF_ACCUM_F32 = 2                            # wgrad: the output is float32 and the result is added to it
+GF_B_SHUFFLED = 16                          # forward / dgrad, row-major E2M1: b's codes are in the pre-shuffled byte order
 GF_B_TRANSPOSED = 8                         # forward / dgrad: b's codes are those of the transposed matrices (row-wise weight copy)
 BF_B_KN, BF_ACCUM_F32 = 1, 2                # flags of the bf16 grouped GEMMs
 

@@ -164,8 +164,13 @@ __device__ __forceinline__ void static_for(F&& f) {
 // into the fp32 main_grad buffer that the reference's bridge otherwise adds it to in a separate pass,
 // primus/backends/megatron/core/extensions/primus_turbo.py:166-240); every output tile belongs to one
 // workgroup, so the read-modify-write needs no atomics.
-template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false, bool ACCUM = false>
+// BSHUF (row-major E2M1 operands, forward / dgrad): b's codes are in the pre-shuffled byte order of mxl_shuffle_codes
+// (what gemm_fp4_impl(..., preshuffled=True) is handed, primus_turbo_mxfp4_local.py:319-331).  The order moves whole
+// 16-byte pieces, so the loads fetch each piece from its shuffled place and the LDS image -- hence everything behind
+// the loads -- is that of the plain layout.
+template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false, bool ACCUM = false, bool BSHUF = false>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
+    static_assert(!BSHUF || (BFMT == kFmtE2M1 && LAYOUT == 0 && MODE == MODE_FWD && !ALPHA && !ACCUM), "pre-shuffled codes: row-major E2M1 weights, forward / dgrad");
     constexpr int A_BYTES = Op<AFMT>::tile_bytes, B_BYTES = Op<BFMT>::tile_bytes;
     constexpr int STAGE = A_BYTES + B_BYTES;            // one slot: K = 128 of both operands
     constexpr int LPA = Op<AFMT>::cpr, LPB = Op<BFMT>::cpr;
@@ -243,7 +248,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
     // per-thread constants of the global -> LDS mapping (mx_gemm_addr.h holds the arithmetic and the rule it follows:
     // descriptors end with the operand, and the range check covers the per-lane and the scalar offset)
     const uint32_t a_voff = addr::slot2_code_lane(LAYOUT, t, Op<AFMT>::cpr, Op<AFMT>::swz(t / Op<AFMT>::cpr), lda, Op<AFMT>::kb);
-    const uint32_t b_voff = addr::slot2_code_lane(LAYOUT, t, Op<BFMT>::cpr, Op<BFMT>::swz(t / Op<BFMT>::cpr), ldb, Op<BFMT>::kb);
+    const uint32_t b_voff = BSHUF ? addr::slot2_code_lane_shuffled(t, Op<BFMT>::cpr, Op<BFMT>::swz(t / Op<BFMT>::cpr), ldb)
+                                  : addr::slot2_code_lane(LAYOUT, t, Op<BFMT>::cpr, Op<BFMT>::swz(t / Op<BFMT>::cpr), ldb, Op<BFMT>::kb);
     // LAYOUT 1: bytes from one K chunk of an operand to the next (the host has checked that an operand stays below 4 GiB)
     const uint32_t a_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * Op<AFMT>::kb));
     const uint32_t b_cstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * Op<BFMT>::kb));
@@ -331,7 +337,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
             dma16(d.ra, smem_base + slot * STAGE + (r * 4 + w) * 1024, a_voff, off);
         } else if (r < LPT) {
             const int i = r - LPA;
-            const uint32_t off = addr::slot2_code_k(LAYOUT, d.kb0, kp, Op<BFMT>::kb, b_cstride) +
+            const uint32_t off = (BSHUF ? addr::slot2_code_k_shuffled(kp) : addr::slot2_code_k(LAYOUT, d.kb0, kp, Op<BFMT>::kb, b_cstride)) +
                                  addr::slot2_code_round(LAYOUT, i, Op<BFMT>::rows_per_ld, ldb, Op<BFMT>::kb);
             dma16(d.rb, smem_base + slot * STAGE + A_BYTES + (i * 4 + w) * 1024, b_voff, off);
         }
@@ -1307,13 +1313,13 @@ static int num_cus(int slot) {
     return pr.multiProcessorCount;
 }
 
-template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false, bool ACCUM = false>
+template <int AFMT, int BFMT, int MODE, int LAYOUT, bool ALPHA = false, bool ACCUM = false, bool BSHUF = false>
 static int launch_gemm(const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
     constexpr int lds = gemm_lds_bytes(AFMT, BFMT);
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set[64];   // the attribute belongs to the (kernel, device) pair
     const int slot = current_device_slot();
-    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT, ALPHA, ACCUM>;
+    auto kern = mx_gemm_kernel<AFMT, BFMT, MODE, LAYOUT, ALPHA, ACCUM, BSHUF>;
     if (!attr_set[slot].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return MXL_ELAUNCH;
@@ -1477,8 +1483,11 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* dst, int64_t w
 static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt, const void* b_codes, const void* b_scales,
                            int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m, int64_t n,
                            int64_t k, const float* alpha_a, const float* alpha_b, uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP | MXL_GF_B_TRANSPOSED)) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_GF_KCHUNK | MXL_GF_KSTEP | MXL_GF_B_TRANSPOSED | MXL_GF_B_SHUFFLED)) return MXL_EINVAL;
     if ((flags & MXL_GF_KCHUNK) && (flags & MXL_GF_KSTEP)) return MXL_EINVAL;
+    // pre-shuffled weight codes: row-major E2M1 x E2M1, block scales, whole 16-row blocks per group
+    if ((flags & MXL_GF_B_SHUFFLED) && (flags != MXL_GF_B_SHUFFLED || a_fmt != MXL_FMT_E2M1 || b_fmt != MXL_FMT_E2M1 || alpha_a || n % 16 != 0))
+        return MXL_EINVAL;
     if ((flags & MXL_GF_B_TRANSPOSED) && !(flags & MXL_GF_KSTEP)) return MXL_EINVAL;
     if ((alpha_a == nullptr) != (alpha_b == nullptr)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % MXL_BLOCK != 0 || k % 128 != 0) return MXL_EINVAL;
@@ -1503,6 +1512,7 @@ static int grouped_gemm_nt(const void* a_codes, const void* a_scales, int a_fmt,
     a.alpha_a = alpha_a;
     a.alpha_b = alpha_b;
     const int64_t max_tiles = (total_m / BM + num_groups) * ((n + BN - 1) / BN);
+    if (flags & MXL_GF_B_SHUFFLED) return launch_gemm<MXL_FMT_E2M1, MXL_FMT_E2M1, MODE_FWD, 0, false, false, true>(a, max_tiles, (hipStream_t)stream);
     if (flags & MXL_GF_B_TRANSPOSED) {
         // offsets inside an operand are 32-bit; the kernel keeps a tile's first output row in 32 bits
         const int64_t n_ld = (n + 127) / 128 * 128;

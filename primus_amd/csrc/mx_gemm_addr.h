@@ -49,6 +49,18 @@ MXL_HD uint32_t slot2_code_round(int layout, int r, int rows_per_ld, int64_t ld,
 MXL_HD uint32_t slot2_code_k(int layout, uint32_t k0, int kp, int kb, uint32_t cstride) {
     return layout ? (k0 + (uint32_t)kp) * cstride : k0 + (uint32_t)kp * (uint32_t)kb;
 }
+// Packed FP4 codes in the pre-shuffled byte order (mxl_shuffle_codes): every block of 16 rows x 32 bytes is 512
+// consecutive bytes, [16-byte half][row][16 bytes], blocks row-major.  Byte (row R, column byte c) sits at
+//   ((R / 16) * (ld / 32) + c / 32) * 512 + ((c / 16) % 2) * 256 + (R % 16) * 16 + c % 16.
+// A tile starts at a multiple of 16 rows, so its descriptor is the row-major one (16 rows of ld bytes are 16 * ld bytes
+// in both orders); what changes is the per-lane offset of a 16-byte piece and the advance per K slot of 64 bytes
+// (two 32-byte block columns = 1024 bytes).
+MXL_HD uint32_t slot2_code_lane_shuffled(int t, int cpr, int swz, int64_t ld) {
+    const int row = t / cpr, piece = (t % cpr) ^ swz;
+    return (uint32_t)((int64_t)(row / 16) * (16 * ld) + (piece >> 1) * 512 + (piece & 1) * 256 + (row % 16) * 16);
+}
+MXL_HD uint32_t slot2_code_k_shuffled(int kp) { return (uint32_t)kp * 1024u; }
+
 // Scales are row-major [rows_total, ld_s] bytes; thread t fetches the 16 bytes of panel pn (K slots 4 pn .. 4 pn + 3)
 // of tile row t.  ks0 = first scale byte of the contraction range inside a row.
 MXL_HD Desc slot2_scale_desc(int64_t rows_total, int64_t row0, int64_t ld_s) {

@@ -460,12 +460,26 @@ def _check_scales(scales: torch.Tensor, rows: int, k: int, kchunk, what: str) ->
         raise ValueError(f"{what}: scale shape {tuple(scales.shape)} does not match {rows} rows x {k} elements")
 
 
-def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=False, b_transposed: bool = False) -> torch.Tensor:
+def gemm_mx_nt_impl(a, a_scale, b, b_scale, out_dtype=torch.bfloat16, kchunk=False, b_transposed: bool = False,
+                    b_shuffled: bool = False) -> torch.Tensor:
     """c[m, n] = dq(a)[m, k] . dq(b)[n, k]^T.  ``kchunk``: both code tensors are K-chunk-major.  ``b_transposed``: see
-    ``grouped_gemm_mx_nt_impl``."""
+    ``grouped_gemm_mx_nt_impl``.  ``b_shuffled`` (row-major E2M1 operands, k a multiple of 128): the codes of ``b`` are
+    in the pre-shuffled byte order of ``shuffle_codes_impl``."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if b_shuffled:
+        m, n, k = a.shape[0], b.shape[0], a.shape[-1] * _per_byte(a_fmt)
+        if kchunk or k % GEMM_K_ALIGN or b.shape[-1] * _per_byte(b_fmt) != k:
+            raise ValueError("b_shuffled: row-major operands with the contraction length a multiple of 128")
+        if tuple(a_scale.shape) != (m, k // BLOCK) or tuple(b_scale.shape) != (n, k // BLOCK):
+            raise ValueError("scale shapes must be [rows, k/32]")
+        c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+        with _hooked("gemm_nt", m=m, n=n, k=k):
+            rc = _lib.load().mxl_grouped_gemm_nt_ex(_ptr(a), _ptr(a_scale), a_fmt, _ptr(b), _ptr(b_scale), b_fmt, _ptr(c), None, 1,
+                                                    m, n, k, _lib.GF_B_SHUFFLED, _stream())
+        _lib.check(rc, "mxl_grouped_gemm_nt_ex")
+        return c
     if kchunk:
         return grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale if _paneled(kchunk) else b_scale.unsqueeze(0),
                                        None, kchunk=kchunk, b_transposed=b_transposed)
@@ -1301,14 +1315,19 @@ def unshuffle_scales_impl(shuffled: torch.Tensor, rows: int, blocks: int) -> tor
 def gemm_fp4_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity=None, default_backend=None, preshuffled=False):
     """gemm_fp4_impl of the reference (primus_turbo_mxfp4_local.py:319-331).  ``preshuffled``: the operands are
     what the reference's MXFP4 linear hands over with its pre-shuffle switch on (:234-288): ``a`` plain codes with
-    pre-shuffled scales, ``b`` pre-shuffled codes and scales.  The GEMM kernels read the plain layouts, so the three
-    arrays are converted back first (byte permutations, one pass over half a byte per element)."""
+    pre-shuffled scales, ``b`` pre-shuffled codes and scales.  The GEMM reads the pre-shuffled codes of ``b`` as they
+    lie; the two scale arrays (1/16 of the bytes of the codes) are converted back to the plain order first."""
     if preshuffled:
         _require_mx(granularity)
-        k_blocks = a.shape[-1] * _per_byte(fmt_of(a)) // BLOCK
-        a_scale_inv = unshuffle_scales_impl(a_scale_inv, a.shape[0], k_blocks)
+        if trans_a or not trans_b or trans_c:
+            raise ValueError("MX GEMM supports the NT layout only (trans_a=False, trans_b=True, trans_c=False)")
+        k = a.shape[-1] * _per_byte(fmt_of(a))
+        a_scale_inv = unshuffle_scales_impl(a_scale_inv, a.shape[0], k // BLOCK)
         b_scale_inv = unshuffle_scales_impl(b_scale_inv, b.shape[0], b.shape[-1] * _per_byte(fmt_of(b)) // BLOCK)
-        b = shuffle_codes_impl(b, inverse=True)
+        if fmt_of(a) == _lib.FMT_E2M1 and fmt_of(b) == _lib.FMT_E2M1 and k % GEMM_K_ALIGN == 0 and b.shape[0] % 16 == 0:
+            # the GEMM fetches every 16-byte piece of b from its pre-shuffled place: the codes are not rearranged
+            return gemm_mx_nt_impl(a, a_scale_inv, b, b_scale_inv, out_dtype, b_shuffled=True)
+        b = shuffle_codes_impl(b, inverse=True)     # (a contraction length the GEMM has to pad: plain codes first)
     return gemm_fp8_impl(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out_dtype, trans_c, granularity, default_backend)
 
 

@@ -92,6 +92,21 @@ static void check_ring(int row_bytes, int64_t rows_total, int64_t steps, int64_t
             request(dp, ring_panel_lane(t), (uint32_t)(pn * rows_total * 16), pbytes, row0 + t < rows_total && pn < panels, "ring panels");
 }
 
+// packed FP4 codes in the pre-shuffled order (64-byte K slots, 4 rounds of 64 rows): rows_total a multiple of 16
+static void check_slot2_shuffled(int64_t rows_total, int64_t k_slots, int64_t row0) {
+    const int cpr = 4, rows_per_ld = 64;
+    const int64_t ld = k_slots * 64, bytes = rows_total * ld;
+    const Desc d = slot2_code_desc(0, rows_total, row0, ld, 64);
+    for (int kp = 0; kp < k_slots + 2; ++kp)
+        for (int r = 0; r < 4; ++r)
+            for (int t = 0; t < 256; ++t) {
+                const int row = t / cpr;
+                const uint32_t voff = slot2_code_lane_shuffled(t, cpr, (row >> 2) & 3, ld);
+                const uint32_t soff = slot2_code_round(0, r, rows_per_ld, ld, 64) + slot2_code_k_shuffled(kp);
+                request(d, voff, soff, bytes, row0 + r * rows_per_ld + row < rows_total && kp < k_slots, "slot2 codes pre-shuffled");
+            }
+}
+
 // the ring kernel reading b transposed: planes of [rows_total][64], descriptor at (plane0, row0), round e = e planes
 // further on per lane, K step = 64 rows further on in the scalar offset
 static void check_ring_bt(int64_t groups, int64_t kc, int64_t planes, int64_t grp, int64_t plane0) {
@@ -105,6 +120,9 @@ static void check_ring_bt(int64_t groups, int64_t kc, int64_t planes, int64_t gr
 }
 
 int main() {
+    for (int64_t rows_total : {16, 48, 256, 272, 1008})
+        for (int64_t row0 = 0; row0 < rows_total; row0 += 16)
+            for (int64_t k_slots : {2, 6}) check_slot2_shuffled(rows_total, k_slots, row0);
     for (int64_t groups : {1, 3})
         for (int64_t kc : {128, 384})
             for (int64_t planes : {2, 4, 6, 10})

@@ -74,8 +74,8 @@ def test_shuffle_argument_errors(gpu):
     assert lib.mxl_shuffle_scales(None, 0, 4, None, 1, None) == 0
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 256, 256), (100, 192, 96), (300, 64, 640)])
-def test_gemm_fp4_takes_preshuffled_operands(gpu, m, n, k):
+@pytest.mark.parametrize("m,n,k", [(128, 256, 256), (100, 192, 96), (300, 64, 640), (1000, 2880, 2880), (37, 544, 1152)])
+def test_gemm_fp4_takes_preshuffled_operands(gpu, m, n, k, monkeypatch):
     """a: plain codes with pre-shuffled scales, b: pre-shuffled codes and scales (what the reference's MXFP4 linear
     hands to gemm_fp4_impl with its switch on): the result equals the plain call bit for bit."""
     from primus_amd import _lib
@@ -89,6 +89,16 @@ def test_gemm_fp4_takes_preshuffled_operands(gpu, m, n, k):
     b, b_s, _, _ = K.quantize_mx_weight_2d_impl(w, _lib.FMT_E2M1, rowwise=True, colwise=False, pad_to=128)
     gran = ScalingGranularity.MX_BLOCKWISE.value
     plain = K.gemm_fp4_impl(a, a_s, False, b, b_s, True, torch.bfloat16, False, granularity=gran)
+    shuffled_b = K.shuffle_codes_impl(b)
+
+    def no_unshuffle(*args, **kw):      # the GEMM reads the pre-shuffled codes as they lie
+        raise AssertionError("the weight codes were converted back in front of the GEMM")
+
+    monkeypatch.setattr(K, "shuffle_codes_impl", no_unshuffle)
+    pre = K.gemm_fp4_impl(a, K.shuffle_scales_impl(a_s), False, shuffled_b, K.shuffle_scales_impl(b_s), True,
+                          torch.bfloat16, False, granularity=gran, preshuffled=True)
+    assert torch.equal(plain, pre)
+    monkeypatch.undo()
     pre = K.gemm_fp4_impl(a, K.shuffle_scales_impl(a_s), False, K.shuffle_codes_impl(b), K.shuffle_scales_impl(b_s), True,
                           torch.bfloat16, False, granularity=gran, preshuffled=True)
     assert torch.equal(plain, pre)

@@ -213,7 +213,7 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
 #define MXL_GF_KCHUNK 1u
 /* MXL_GF_KSTEP (instead of MXL_GF_KCHUNK): codes and scales of both operands are K-step-major, as written by the
  * quantisers with MXL_QF_KSTEP.  FP8-format operands, FP8 rows against E2M1 weights in 64-element steps (forward /
- * dgrad), or E2M1 against E2M1 in 128-element steps (MXL_QF_KSTEP128 weights); at most 128 groups; anything else
+ * dgrad), or E2M1 against E2M1 in 128-element steps (MXL_QF_KSTEP128 weights); at most 256 groups; anything else
  * returns MXL_EINVAL.  Served by the 4-slot ring kernel.  Same results bit for bit.
  * In every layout the kernels request whole 256-row tiles, also where a group or the operand ends earlier; a request for
  * a row behind the operand's last row is dropped by the buffer descriptor's range check (the row offset of every request
@@ -232,7 +232,7 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * second quantised copy for it, _maybe_create_quantized_weight_buffers, primus_turbo.py:278-358).  Meaningful where a
  * transposed copy is the same codes transposed: 2-D 32 x 32 block scales (mxl_quantize_weight_2d_ex writes the transposed
  * copy's scales alone when q_colT is NULL and s_colT is not) or tensor-wise scaling.  E4M3 weights, E4M3 (or, scaled,
- * E5M2) rows, at most 128 groups; k % 128 == 0.  Bit-identical to the GEMM on the transposed copy. */
+ * E5M2) rows, at most 256 groups; k % 128 == 0.  Bit-identical to the GEMM on the transposed copy. */
 #define MXL_GF_B_TRANSPOSED 8u
 /* mxl_grouped_gemm_nt_ex only, alone (row-major operands): b_codes are E2M1 codes in the pre-shuffled byte order of
  * mxl_shuffle_codes -- what gemm_fp4_impl(..., preshuffled=True) of the reference is handed for its second operand

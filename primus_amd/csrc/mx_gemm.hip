@@ -645,7 +645,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_kernel(GemmArgs p) {
 // ---------------------------------------------------------------------------------------------------
 constexpr int RING_SLOTS = 4;
 constexpr int RING_STAGE = 2 * 256 * BK;          // both operands, K = 64, FP8: 32 KiB
-constexpr int RING_MAX_GROUPS = 128;
+constexpr int RING_MAX_GROUPS = 256;          // what the group tables may take of the 160 KiB of LDS next to ring and panels
 constexpr int RING_PANEL = 256 * 16;              // scale panel of one operand: 16 bytes per row = 8 K steps
 constexpr int RING_PANEL_BUFS = 3;
 constexpr int RING_TBL = RING_MAX_GROUPS + 2;

@@ -92,7 +92,7 @@ PANEL = 512
 #   3          the K-step-major layout of E2M1 operands that meet E2M1 operands: steps of 128 elements, i.e. codes
 #              [ld / 128, rows, 64 bytes] (the bytes of layout 1) with the scale panels of layout 2
 LAYOUT_ROWMAJOR, LAYOUT_KCHUNK, LAYOUT_KSTEP, LAYOUT_KSTEP128 = 0, 1, 2, 3
-RING_MAX_GROUPS = 128   # the ring GEMM kernel keeps its group tables for at most this many groups
+RING_MAX_GROUPS = 256   # the ring GEMM kernel keeps its group tables for at most this many groups
 
 
 def _layout(kchunk) -> int:

@@ -101,7 +101,9 @@ def test_fused_activation_quantiser_kchunk(gpu, activation):
 
 @pytest.mark.parametrize("afmt,wfmt", [(0, 0), (0, 1), (1, 1), (1, 0)])
 @pytest.mark.parametrize("lens,n,k", [([33, 0, 130, 1, 92], 96, 160), ([300, 212], 544, 512), (None, 320, 384),
-                                      ([1500, 0, 700, 2048, 300, 1024], 2048, 1024)])
+                                      ([1500, 0, 700, 2048, 300, 1024], 2048, 1024),
+                                      # 200 groups: beyond 128, still on the ring kernel (its tables take 256)
+                                      ([(37 * i) % 97 if i % 5 else 0 for i in range(200)], 160, 256)])
 def test_gemms_give_identical_results_on_either_layout(gpu, afmt, wfmt, lens, n, k):
     """Forward, dgrad and wgrad from K-chunk-major operands equal those from row-major operands bit for bit
     (same codes, same scales, same MFMA sequence; only the addresses of the operand loads differ)."""

@@ -36,6 +36,7 @@ if ROOT not in sys.path:
 
 FP8_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
 FP4_PEAK_TFLOPS = 10100.0  # MI355X dense FP4 MFMA
+BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 WORKLOADS = {
@@ -52,6 +53,10 @@ WORKLOADS = {
     "mixtral_8x7b_moe_mxfp4": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=True, act_fp4=True),
     # the non-MX "current scaling" recipe on the headline shapes (HYBRID: E4M3 forward, E5M2 gradients)
     "mixtral_8x7b_moe_fp8_tensorwise": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, tensorwise=True),
+    # the 128-blockwise FP8 recipe (1 x 128 activation blocks, 128 x 128 weight blocks, fp32 scales; HYBRID formats) on the Llama MLP
+    "llama3_8b_mlp_fp8_blockwise": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, blockwise=True, outliers=True),
+    # the unquantised bf16 grouped GEMM (ops.grouped_gemm: what a layer outside the low-precision autocast runs) on the headline shapes
+    "mixtral_8x7b_moe_bf16": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, bf16=True),
     # the same MLP with the RMSNorm that precedes fc1 in the layer (LayerNormColumnParallelLinear), folded into fc1's quantiser
     "llama3_8b_norm_mlp_mxfp8": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, norm=True, outliers=True),
 }
@@ -429,6 +434,8 @@ def main():
     ap.add_argument("--board-seconds", type=float, default=2.0,
                     help="after the timed region, loop the step for this long while sampling socket power and shader "
                          "clocks with amd-smi (0: skip)")
+    ap.add_argument("--no-graph-replay", action="store_true",
+                    help="skip the measurement of the same step captured in a HIP graph and replayed")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="launch one plain 1 GiB-in / 1 GiB-out elementwise kernel first, so that a hardware-counter "
                          "run of this command also reads the counters for a kernel of known HBM traffic")
@@ -459,6 +466,12 @@ def main():
     elif spec.get("tensorwise"):
         cfg = Float8QuantConfig(format=Format.HYBRID, granularity=ScalingGranularity.TENSORWISE)
         op = pt.ops.grouped_gemm_fp8 if grouped else None
+    elif spec.get("blockwise"):
+        cfg = Float8QuantConfig(format=Format.HYBRID, granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+        op = pt.ops.grouped_gemm_fp8 if grouped else None
+    elif spec.get("bf16"):
+        cfg = None
+        op = lambda x, w, gl, trans_b=True, config=None: pt.ops.grouped_gemm(x, w, gl, trans_b=trans_b)  # noqa: E731
     else:
         cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0, block_size=32)
         op = pt.ops.grouped_gemm_fp8 if grouped else None
@@ -564,15 +577,19 @@ def main():
             a["bytes"] += 2.0 * info["n"]
         else:
             a["bytes"] += quant_bytes(info)
-    fwd_name = "grouped_gemm_nt" if grouped else "gemm_nt"
+    fwd_name = ("grouped_gemm_bf16" if spec.get("bf16") else
+                ("grouped_gemm_blockwise_nt" if grouped else "gemm_blockwise_nt") if spec.get("blockwise") else
+                "grouped_gemm_nt" if grouped else "gemm_nt")
     gk = acc[fwd_name]
     gemm_tflops = gk["flops"] / gk["sec"] / 1e12
     act_fp4 = bool(spec.get("act_fp4"))
-    # the MFMA peak of the slower operand format: FP8 rate unless both operands are E2M1
-    peak = FP4_PEAK_TFLOPS if act_fp4 else FP8_PEAK_TFLOPS
+    # the MFMA peak of the slower operand format: FP8 rate unless both operands are E2M1 (or bf16)
+    peak = BF16_PEAK_TFLOPS if spec.get("bf16") else FP4_PEAK_TFLOPS if act_fp4 else FP8_PEAK_TFLOPS
     roofline = {
-        # every benchmark workload runs on the 4-slot ring kernel
-        "kernel": "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_ring_kernel",
+        # the MX and tensor-wise workloads run on the 4-slot ring kernel
+        "kernel": "bf16_gemm_kernel<fwd/dgrad> (grouped_gemm_bf16)" if spec.get("bf16") else
+                  "bw_gemm_kernel<e4m3|e5m2,e4m3> (%s)" % fwd_name if spec.get("blockwise") else
+                  "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_ring_kernel",
                                                    "e4m3|e5m2" if spec.get("tensorwise") else "e2m1" if act_fp4 else "e4m3",
                                                    "e2m1" if spec["fp4"] else "e4m3",
                                                    ",alpha" if spec.get("tensorwise") else "", fwd_name),
@@ -590,7 +607,7 @@ def main():
         ent = {"launches_per_step": a["n"] // kernel_steps, "ms_per_step": round(a["sec"] * 1e3 / kernel_steps, 4)}
         if a["flops"]:
             ent["TFLOP/s"] = round(a["flops"] / a["sec"] / 1e12, 2)
-            ent["frac_fp4_mfma_peak" if act_fp4 else "frac_fp8_mfma_peak"] = round(a["flops"] / a["sec"] / 1e12 / peak, 4)
+            ent["frac_bf16_mfma_peak" if spec.get("bf16") else "frac_fp4_mfma_peak" if act_fp4 else "frac_fp8_mfma_peak"] = round(a["flops"] / a["sec"] / 1e12 / peak, 4)
         else:
             ent["GB/s"] = round(a["bytes"] / a["sec"] / 1e9, 1)
             ent["frac_hbm_peak"] = round(a["bytes"] / a["sec"] / 1e9 / HBM_PEAK_GBS, 4)
@@ -600,7 +617,9 @@ def main():
 
     out = {
         "metric": "%s grouped-GEMM TFLOPS (%s, quantisers inside the timed step)"
-                  % ("FP8 tensor-wise" if spec.get("tensorwise") else "MXFP4" if spec.get("act_fp4") else "MXFP8", "fwd+dgrad+wgrad" if spec.get("wgrad", True) else "fwd+dgrad"),
+                  % ("bf16 (unquantised)" if spec.get("bf16") else "FP8 128-blockwise" if spec.get("blockwise") else
+                     "FP8 tensor-wise" if spec.get("tensorwise") else "MXFP4" if spec.get("act_fp4") else "MXFP8",
+                     "fwd+dgrad+wgrad" if spec.get("wgrad", True) else "fwd+dgrad"),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -610,7 +629,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "mxfp4_e2m1 (E8M0 block scales) for every operand, fp32 accumulate" if spec.get("act_fp4")
+        "dtype": "bf16 operands, fp32 accumulate" if spec.get("bf16")
+                 else "fp8 e4m3 forward / e5m2 gradients, fp32 scales per 1x128 / 128x128 block, fp32 accumulate" if spec.get("blockwise")
+                 else "mxfp4_e2m1 (E8M0 block scales) for every operand, fp32 accumulate" if spec.get("act_fp4")
                  else "mxfp4_e2m1 weights x mxfp8_e4m3 activations, fp32 accumulate" if spec["fp4"]
                  else "fp8 e4m3 forward / e5m2 gradients, one fp32 scale per tensor, fp32 accumulate" if spec.get("tensorwise")
                  else "mxfp8_e4m3 (E8M0 block scales), fp32 accumulate",
@@ -624,9 +645,9 @@ def main():
             "gemms_nk": [[n, k] for (_, _, _, k, n) in layers],
             "flops_per_step": flops_step,
         },
-        ("frac_fp4_mfma_peak_whole_step" if act_fp4 else "frac_fp8_mfma_peak_whole_step"): round(value / peak, 4),
+        ("frac_bf16_mfma_peak_whole_step" if spec.get("bf16") else "frac_fp4_mfma_peak_whole_step" if act_fp4 else "frac_fp8_mfma_peak_whole_step"): round(value / peak, 4),
         "gemm_only_TFLOP/s": round(gemm_flops / gemm_sec / 1e12, 2),
-        ("gemm_only_frac_fp4_mfma_peak" if act_fp4 else "gemm_only_frac_fp8_mfma_peak"): round(gemm_flops / gemm_sec / 1e12 / peak, 4),
+        ("gemm_only_frac_bf16_mfma_peak" if spec.get("bf16") else "gemm_only_frac_fp4_mfma_peak" if act_fp4 else "gemm_only_frac_fp8_mfma_peak"): round(gemm_flops / gemm_sec / 1e12 / peak, 4),
         "wgrad_overlaps_dgrad": not args.no_wgrad_overlap,
         "kernels_note": "per-kernel figures: separate pass of %d steps after the timed region, wgrad serialised behind dgrad" % kernel_steps,
         "kernels": kernels,
@@ -663,6 +684,37 @@ def main():
     if args.board_seconds > 0:
         pt.ops.set_wgrad_overlap(not args.no_wgrad_overlap)
         out["board"] = board_sample(step, args.board_seconds)
+    if not args.no_graph_replay:
+        # The same step captured once in a HIP graph and replayed (nothing on the path allocates behind torch's back,
+        # synchronises or reads tokens-per-expert on the host): what the launch gaps of the eager loop cost.
+        # Reported beside `value`, which stays the eager figure.
+        try:
+            pt.ops.set_wgrad_overlap(not args.no_wgrad_overlap)
+            step_no[0] = 0
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step_no[0] = 0
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            step_no[0] = 0
+            with torch.cuda.graph(graph):
+                step()
+            for _ in range(2):
+                graph.replay()
+            torch.cuda.synchronize()
+            g0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            g_ms = (time.perf_counter() - g0) * 1e3 / args.steps
+            out["graph_replay"] = {"ms_per_step": round(g_ms, 4), "TFLOP/s": round(flops_step / (g_ms * 1e-3) / 1e12, 2),
+                                   "note": "one captured step (buffer set 0) replayed %d times; `value` is the eager loop" % args.steps}
+            del graph
+        except Exception as ex:      # reported, never fatal: the eager figures above stand on their own
+            out["graph_replay"] = {"error": "%s: %s" % (type(ex).__name__, str(ex)[:200])}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(spec, lens, raw)
     print(json.dumps(out))

@@ -484,7 +484,10 @@ def main():
     def with_grad(layer, copy):
         x, w, dy, k, n = layer
         if copy:
-            x, w, dy = x.clone(), w.clone(), dy.clone()
+            # detached copies: a clone of a tensor that already requires grad would be a non-leaf hanging on the first
+            # set's leaves (their gradient-accumulation nodes, made on the default stream, would then outlive every
+            # step, and a captured step would have to wait on that stream)
+            x, w, dy = x.detach().clone(), w.detach().clone(), dy.detach().clone()
         return (x.requires_grad_(), w.requires_grad_(spec.get("wgrad", True)), dy, k, n)
 
     # Rotating buffer sets: a workload whose tensors would sit in the 256 MiB memory-side cache from one step to the
@@ -522,12 +525,9 @@ def main():
                 y = pt.ops.rmsnorm_gemm_fp8(x, norm_w, 1e-5, w, config=cfg)
             else:
                 y = pt.ops.gemm_fp8(x, w, trans_a=False, trans_b=True, out_dtype=None, config=cfg)
-            y.backward(dy)
-            x.grad = None
-            if torch.is_tensor(w):
-                w.grad = None
-            if norm_w is not None:
-                norm_w.grad = None
+            # the gradients are returned and dropped, not accumulated into .grad
+            wanted = [x] + ([w] if torch.is_tensor(w) and w.requires_grad else []) + ([norm_w] if norm_w is not None and i == 0 else [])
+            torch.autograd.grad(y, wanted, dy)
 
     if args.calibrate_traffic:
         src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)   # 1 GiB

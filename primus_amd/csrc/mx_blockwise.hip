@@ -12,8 +12,7 @@
 // reference restates for its tensor-wise quantiser (:194-207) applied per block.  Arbitrary fp32 factors cannot ride on
 // the MFMA's E8M0 scale inputs, so this GEMM keeps two accumulator sets: the MFMAs of one K block of 128 add up in
 // the first (from zero), which is then multiplied into the second with the block's factors.  That takes registers
-// the 256 x 256 kernels do not have: the tile is 128 x 128, 64 x 64 per wave.  Operands go through LDS with plain
-// loads and stores, register-prefetched one K block ahead.
+// the 256 x 256 kernels do not have: the tile is 128 x 256 for 8 waves, 64 x 64 per wave, two waves per SIMD.
 #include "mx_device.h"
 
 namespace mxl {
@@ -53,14 +52,15 @@ struct BwQuantArgs {
 constexpr int BW_MAX_GROUPS = 1024;
 
 // Which group holds tile `y` when every group is cut into tiles of 128 rows (a group's last tile may be ragged):
-// `pre` (LDS, BW_MAX_GROUPS + 1 ints) receives the prefix sum of the groups' tile counts, `red` (LDS, 4 words of 8
-// bytes) is scratch.  Returns the group (or -1 behind the last tile); tile_in_group, the rows in front of the group
+// `pre` (LDS, BW_MAX_GROUPS + 1 ints) receives the prefix sum of the groups' tile counts, `red` (LDS, one word of 8
+// bytes per wave of the workgroup, NT / 64 of them) is scratch.  Returns the group (or -1 behind the last tile); tile_in_group, the rows in front of the group
 // and its length come back through the references.  Negative lens read as 0.  All threads of the workgroup call it.
+template <int NT = 256>
 __device__ __forceinline__ int bw_locate(const int64_t* lens, int groups, int y, int* pre, int64_t* red, int& tile_in_group,
                                          int64_t& rows_before, int64_t& len) {
     const int t = threadIdx.x;
     if (t == 0) pre[0] = 0;
-    for (int j = t; j < groups; j += BW_THREADS) {
+    for (int j = t; j < groups; j += NT) {
         const int64_t l = lens[j] > 0 ? lens[j] : 0;
         pre[j + 1] = (int)((l + BW - 1) / BW);
     }
@@ -96,12 +96,14 @@ __device__ __forceinline__ int bw_locate(const int64_t* lens, int groups, int y,
     }
     tile_in_group = g >= 0 ? y - pre[g] : 0;
     int64_t part = 0;
-    for (int j = t; j < g; j += BW_THREADS) part += lens[j] > 0 ? lens[j] : 0;
+    for (int j = t; j < g; j += NT) part += lens[j] > 0 ? lens[j] : 0;
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) part += __shfl_xor(part, d);
     if ((t & 63) == 0) red[t >> 6] = part;
     __syncthreads();
-    rows_before = red[0] + red[1] + red[2] + red[3];
+    rows_before = 0;
+#pragma unroll
+    for (int i = 0; i < NT / 64; ++i) rows_before += red[i];
     len = g >= 0 ? (lens[g] > 0 ? lens[g] : 0) : 0;
     return g;
 }
@@ -225,8 +227,17 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
 // ------------------------------------------------------------------------------------------------------------
 // GEMM.  c[m, n] (bf16) = sum_kb sa[m, kb] * sb[n >> sb_shift, kb] * (a[m, kb-th 128] . b[n, kb-th 128]),
 // a[m_rows, k], b[n, k] FP8 codes, k % 128 == 0, n % 128 == 0; sb_shift = 0 (a factor per row of b) or 7 (per
-// 128 rows: weights).  Workgroup = 128 x 128 output tile, wave (wm, wn) = 64 x 64 = 2 x 2 MFMA tiles of 32 x 32.
-// LDS: two stages of both operands' 128 x 128 bytes, 16-byte pieces XOR-swizzled by the row, and the factors.
+// 128 rows: weights).
+// Workgroup = 8 waves (two per SIMD) on a 128 x 256 output tile, wave (wm, wn) = 64 x 64 = 2 x 2 MFMA tiles of
+// 32 x 32 with two accumulator sets of 64 registers.  K advances in blocks of 128 through a ring of three LDS stages
+// (128 + 256 rows x 128 bytes = 48 KiB each) filled by LDS-direct loads two blocks ahead: a request has two K blocks
+// of MFMA work (about a microsecond) to land, where a register-staged prefetch of one block left the pipe waiting
+// for memory most of the time (1.1 PFLOP/s on the Llama MLP shapes).  16-byte pieces are XOR-swizzled by the row on the global side, so
+// the fragment reads are conflict-free ds_read_b128.  The two waves of a SIMD cover each other: while one multiplies
+// its block's partial sums into the accumulators (64 FMAs per lane), the other's MFMAs run.  The factors of a block
+// are fetched one block ahead with plain loads and handed round through LDS.  Rows past the end of a group or of
+// the operand are dropped by the buffer descriptor's range check (it covers the per-lane and the scalar offset) and
+// read as zero.
 // ------------------------------------------------------------------------------------------------------------
 struct BwGemmArgs {
     const uint8_t* a;
@@ -245,28 +256,55 @@ struct BwGemmArgs {
     int num_groups;
 };
 
-constexpr int BW_GEMM_LDS = 2 * 2 * BW * BW + 2 * 2 * BW * 4;
+constexpr int BWG_THREADS = 512;
+constexpr int BWG_BM = 128, BWG_BN = 256;
+constexpr int BWG_A = BWG_BM * BW, BWG_B = BWG_BN * BW, BWG_STAGE = BWG_A + BWG_B;      // 16 + 32 KiB
+constexpr int BWG_STAGES = 3;
+constexpr int BWG_FAC = (BWG_BM + BWG_BN) * 4;                                            // factors of one K block
+constexpr int BW_GEMM_LDS = BWG_STAGES * (BWG_STAGE + BWG_FAC);
 
-template <int AFMT, int BFMT>
-__global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
+__device__ __forceinline__ v4i bw_rsrc(const void* base, int64_t bytes) {
+    const uint64_t p = (uint64_t)base;
+    const uint32_t n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)(bytes < 0 ? 0 : bytes);
+    v4i r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32) & 0xFFFF);
+    r[2] = __builtin_amdgcn_readfirstlane((int)n);
+    r[3] = 0x00020000;
+    return r;
+}
+// LDS-direct 16-byte load: lane i's data lands at lds_off + 16 i (M0 holds nothing else in this kernel)
+__device__ __forceinline__ void bw_dma16(v4i rsrc, uint32_t lds_off, uint32_t voff, uint32_t soff) {
+    asm volatile("" : "+s"(soff));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_off), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory");
+}
+
+// SBU: b's factors are per 128 rows (a weight's 128 x 128 blocks), i.e. one value for the wave's 64 columns: the
+// block's factor product is two multiplications per lane instead of 64.
+template <int AFMT, int BFMT, bool SBU>
+__global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
     constexpr int CB = BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE5M2 ? 1 : 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t bw_smem[];
-    uint8_t (*ops)[2][BW * BW] = (uint8_t (*)[2][BW * BW])bw_smem;                     // [stage][operand][row * 128 + swizzled piece]
-    float (*fac)[2][BW] = (float (*)[2][BW])(bw_smem + 2 * 2 * BW * BW);               // [stage][operand][row]
+    float* fac_base = (float*)(bw_smem + BWG_STAGES * BWG_STAGE);        // [stage][a: 128 | b: 256]
     __shared__ int grp_pre[BW_MAX_GROUPS + 1];
-    __shared__ int64_t grp_red[4];
+    __shared__ int64_t grp_red[BWG_THREADS / 64];
     const int t = threadIdx.x;
-    const int w = t >> 6, l = t & 63, lr = l & 31, g = l >> 5, wm = w >> 1, wn = w & 1;
-    int64_t row0 = (int64_t)blockIdx.y * BW;
-    const int64_t col0 = (int64_t)blockIdx.x * BW;
-    const int64_t kb_n = p.k / BW;   // (the argument block itself is only read here and in the copies below)
+    const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l = t & 63, lr = l & 31, g = l >> 5, wm = w >> 2, wn = w & 3;
+    const uint32_t smem_base = (uint32_t)(uintptr_t)bw_smem;
+    int64_t row0 = (int64_t)blockIdx.y * BWG_BM;
+    const int64_t col0 = (int64_t)blockIdx.x * BWG_BN;
+    const int64_t kb_n = p.k / BW;
     int64_t m_end = p.m, b_group = 0, c_group = 0, kb0 = 0, kb1 = kb_n;
     if (p.mode == 1) {
         int tile_in_group;
         int64_t before, len;
-        const int grp = bw_locate(p.group_lens, p.num_groups, (int)blockIdx.y, grp_pre, grp_red, tile_in_group, before, len);
+        const int grp = bw_locate<BWG_THREADS>(p.group_lens, p.num_groups, (int)blockIdx.y, grp_pre, grp_red, tile_in_group, before, len);
         if (grp < 0) return;                     // the grid is sized for the worst case (every group with a ragged tile)
-        row0 = before + (int64_t)tile_in_group * BW;
+        row0 = before + (int64_t)tile_in_group * BWG_BM;
         m_end = before + len < p.m ? before + len : p.m;
         if (row0 >= m_end) return;
         b_group = grp;
@@ -274,61 +312,66 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
         // this group's segment of the contraction: [sum of the padded lens in front, + its own padded len), in blocks
         const int grp = (int)blockIdx.z;
         int64_t part = 0;
-        for (int j = t; j < grp; j += BW_THREADS) part += ((p.group_lens[j] > 0 ? p.group_lens[j] : 0) + BW - 1) / BW;
+        for (int j = t; j < grp; j += BWG_THREADS) part += ((p.group_lens[j] > 0 ? p.group_lens[j] : 0) + BW - 1) / BW;
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) part += __shfl_xor(part, d);
         if ((t & 63) == 0) grp_red[t >> 6] = part;
         __syncthreads();
-        kb0 = grp_red[0] + grp_red[1] + grp_red[2] + grp_red[3];
+        kb0 = 0;
+#pragma unroll
+        for (int i = 0; i < BWG_THREADS / 64; ++i) kb0 += grp_red[i];
         kb1 = kb0 + ((p.group_lens[grp] > 0 ? p.group_lens[grp] : 0) + BW - 1) / BW;
         kb0 = kb0 > kb_n ? kb_n : kb0;           // lens that claim more than the operands hold
         kb1 = kb1 > kb_n ? kb_n : kb1;
         c_group = grp;
     }
-    // loader geometry: piece pc = i * 256 + t of an operand's 1024 pieces: row pc / 8 = 32 i + t / 8, piece t % 8.
-    // Everything the loop needs from the argument block is copied to locals first (and the loader is written as
-    // macros over scalars): a lambda that captures the block or an array by reference puts it on the stack.
     const int64_t pm = m_end, pk = p.k, pn = p.n;
     const int sb_shift = p.sb_shift;
-    const uint8_t* const pa = p.a;
-    const uint8_t* const pb = p.b + b_group * pn * pk;
     const float* const psa = p.sa;
     const float* const psb = p.sb + b_group * (pn >> sb_shift) * kb_n;
     uint16_t* const pc_out = p.c + c_group * p.m * pn;
-    const int lrow = t >> 3, lpc = t & 7;
-    const int lds_off = lrow * BW + 16 * (lpc ^ (lrow & 7));      // rows 32 i + lrow share (row & 7)
-    const uint8_t* ga = pa + (row0 + lrow) * pk + lpc * 16;
-    const uint8_t* gb = pb + (col0 + lrow) * pk + lpc * 16;
-    const bool av0 = row0 + lrow < pm, av1 = row0 + 32 + lrow < pm, av2 = row0 + 64 + lrow < pm, av3 = row0 + 96 + lrow < pm;
-    const float* gsa = psa + (row0 + (t & (BW - 1))) * kb_n;
-    const float* gsb = psb + ((col0 + (t & (BW - 1))) >> sb_shift) * kb_n;
-    const bool fav = t < BW && row0 + t < pm;
-    const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
-    uint4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
-    float fr = 0.f;
-#define MXL_BW_FETCH(KB)                                                                      \
-    do {                                                                                      \
-        const int64_t o_ = (int64_t)(KB) * BW;                                                \
-        ra0 = av0 ? *(const uint4*)(ga + o_) : z4;                                            \
-        ra1 = av1 ? *(const uint4*)(ga + 32 * pk + o_) : z4;                                  \
-        ra2 = av2 ? *(const uint4*)(ga + 64 * pk + o_) : z4;                                  \
-        ra3 = av3 ? *(const uint4*)(ga + 96 * pk + o_) : z4;                                  \
-        rb0 = *(const uint4*)(gb + o_);                                                       \
-        rb1 = *(const uint4*)(gb + 32 * pk + o_);                                             \
-        rb2 = *(const uint4*)(gb + 64 * pk + o_);                                             \
-        rb3 = *(const uint4*)(gb + 96 * pk + o_);                                             \
-        fr = t < BW ? (fav ? gsa[KB] : 0.f) : gsb[KB];                                        \
-    } while (0)
-#define MXL_BW_STASH(ST)                                                                      \
-    do {                                                                                      \
-        uint8_t* oa_ = &ops[ST][0][lds_off];                                                  \
-        uint8_t* ob_ = &ops[ST][1][lds_off];                                                  \
-        *(uint4*)(oa_) = ra0; *(uint4*)(oa_ + 32 * BW) = ra1;                                 \
-        *(uint4*)(oa_ + 64 * BW) = ra2; *(uint4*)(oa_ + 96 * BW) = ra3;                       \
-        *(uint4*)(ob_) = rb0; *(uint4*)(ob_ + 32 * BW) = rb1;                                 \
-        *(uint4*)(ob_ + 64 * BW) = rb2; *(uint4*)(ob_ + 96 * BW) = rb3;                       \
-        fac[ST][t >> 7][t & (BW - 1)] = fr;                                                   \
-    } while (0)
+    // descriptors: from the tile's first row to the last row that may be read (the group's / the operand's end for a,
+    // the end of the group's matrix for b); offsets inside them are 32-bit (the host bounds 256 rows x k)
+    const uint8_t* const b_mat = p.b + b_group * pn * pk;
+    const v4i ra = bw_rsrc(p.a + row0 * pk, (pm - row0) * pk);
+    const v4i rb = bw_rsrc(b_mat + col0 * pk, (pn - col0) * pk);
+    // loader geometry: a round is 512 pieces of 16 bytes = 64 rows x 128 bytes; lane i of wave w lands at chunk
+    // offset 1024 w + 16 i, i.e. row 8 w + i / 8, LDS piece i % 8, and fetches global piece (i % 8) ^ ((row / 2) % 8):
+    // the 16 rows that one cycle of a ds_read_b128 serves (two rows share a 256-byte bank period) then hit 16
+    // different 16-byte bank groups (XOR by row % 8 left rows r and r + 8 on the same one: half of the LDS cycles
+    // were bank conflicts)
+    const int ld_row = t >> 3;
+    const uint32_t ld_voff = (uint32_t)(ld_row * pk + 16 * ((t & 7) ^ ((ld_row >> 1) & 7)));
+    const uint32_t round_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(64 * pk));
+    const uint32_t wave_lds = smem_base + (uint32_t)(w * 1024);
+    auto issue = [&](int kb, int stage) __attribute__((always_inline)) {
+        const uint32_t koff = (uint32_t)__builtin_amdgcn_readfirstlane(kb * BW);
+        const uint32_t base = wave_lds + (uint32_t)(stage * BWG_STAGE);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) bw_dma16(ra, base + e * 8192, ld_voff, koff + e * round_bytes);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bw_dma16(rb, base + BWG_A + e * 8192, ld_voff, koff + e * round_bytes);
+    };
+    // Factors of a K block, one dword per lane straight into LDS (lane i of wave w lands at word 64 w + i): waves 0, 1
+    // fetch a's 128 row factors, waves 2 .. 5 b's 256 (per row of b, or one per 128 rows), waves 6, 7 nothing.  Rows
+    // past the end of the group or of b are dropped by the descriptors and read as zero.
+    const bool f_a = w < 2, f_any = w < 6;
+    const int frow = f_a ? t : t - BWG_BM;
+    const v4i rfac = f_a ? bw_rsrc(psa + row0 * kb_n, (pm - row0) * kb_n * 4)
+                         : bw_rsrc(psb + (col0 >> sb_shift) * kb_n, (((pn - col0) + (1 << sb_shift) - 1) >> sb_shift) * kb_n * 4);
+    const uint32_t fac_voff = (uint32_t)(((f_a ? frow : (frow >> sb_shift)) * kb_n) * 4);
+    const uint32_t fac_lds = smem_base + (uint32_t)(BWG_STAGES * BWG_STAGE + w * 256);
+    auto issue_fac = [&](int kb, int stage) __attribute__((always_inline)) {
+        if (f_any) {
+            uint32_t soff = (uint32_t)__builtin_amdgcn_readfirstlane(kb * 4);
+            const uint32_t lds = fac_lds + (uint32_t)(stage * BWG_FAC);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                         :
+                         : "s"(lds), "v"(fac_voff), "s"(rfac), "s"(soff)
+                         : "memory");
+        }
+    };
+
     bv16f acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -336,14 +379,31 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-    if (kb0 < kb1) {
-        MXL_BW_FETCH(kb0);
-        MXL_BW_STASH(0);
+
+    // pipeline: two blocks ahead.  A wave's requests for a block are its six operand rounds, then (waves 0 .. 5) one
+    // factor request; at the top of block kb everything but the requests of block kb + 1 has landed.
+    const int k0 = (int)kb0, k1 = (int)kb1;      // (block indices: k is below 2^23)
+    if (k0 < k1) {
+        issue(k0, 0);
+        issue_fac(k0, 0);
+        if (k0 + 1 < k1) {
+            issue(k0 + 1, 1);
+            issue_fac(k0 + 1, 1);
+        }
     }
-    __syncthreads();
-    for (int64_t kb = kb0; kb < kb1; ++kb) {
-        const int st = (int)((kb - kb0) & 1);
-        if (kb + 1 < kb1) MXL_BW_FETCH(kb + 1);
+    int st = 0, st2 = 2;                          // stage of block kb, stage of block kb + 2
+    for (int kb = k0; kb < k1; ++kb) {
+        if (kb + 1 >= k1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else if (f_any) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        __syncthreads();       // block kb and its factors are in LDS for every wave; every wave has left block kb - 1
+        if (kb + 2 < k1) {
+            issue(kb + 2, st2);
+            issue_fac(kb + 2, st2);
+        }
+        const float* fac = fac_base + st * (BWG_BM + BWG_BN);
+        const uint8_t* sa_ = bw_smem + st * BWG_STAGE;
+        const uint8_t* sb_ = sa_ + BWG_A;
         bv16f part[2][2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -352,10 +412,10 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
             for (int i = 0; i < 2; ++i) {
                 // lane (lr, g) of a 32-row fragment holds bytes 16 g .. 16 g + 15 and 32 + 16 g .. of the K step
                 const int ra_ = wm * 64 + i * 32 + lr, rb_ = wn * 64 + i * 32 + lr;
-                const uint4 alo = *(const uint4*)(&ops[st][0][ra_ * BW + 16 * ((4 * ks + g) ^ (ra_ & 7))]);
-                const uint4 ahi = *(const uint4*)(&ops[st][0][ra_ * BW + 16 * ((4 * ks + 2 + g) ^ (ra_ & 7))]);
-                const uint4 blo = *(const uint4*)(&ops[st][1][rb_ * BW + 16 * ((4 * ks + g) ^ (rb_ & 7))]);
-                const uint4 bhi = *(const uint4*)(&ops[st][1][rb_ * BW + 16 * ((4 * ks + 2 + g) ^ (rb_ & 7))]);
+                const uint4 alo = *(const uint4*)(sa_ + ra_ * BW + 16 * ((4 * ks + g) ^ ((ra_ >> 1) & 7)));
+                const uint4 ahi = *(const uint4*)(sa_ + ra_ * BW + 16 * ((4 * ks + 2 + g) ^ ((ra_ >> 1) & 7)));
+                const uint4 blo = *(const uint4*)(sb_ + rb_ * BW + 16 * ((4 * ks + g) ^ ((rb_ >> 1) & 7)));
+                const uint4 bhi = *(const uint4*)(sb_ + rb_ * BW + 16 * ((4 * ks + 2 + g) ^ ((rb_ >> 1) & 7)));
                 fa8[i] = bv8i{(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
                 fb8[i] = bv8i{(int)blo.x, (int)blo.y, (int)blo.z, (int)blo.w, (int)bhi.x, (int)bhi.y, (int)bhi.z, (int)bhi.w};
             }
@@ -373,25 +433,30 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
         }
         // acc += part * (sa[row] * sb[col]): lane (lr, g), register e = 4 q + r of tile (i, j) is row i * 32 + lr,
         // column j * 32 + 8 q + 4 g + r of the wave's 64 x 64
+        const float sbu = SBU ? fac[BWG_BM + wn * 64] : 0.f;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const float sa = fac[st][0][wm * 64 + i * 32 + lr];
+            const float sa = fac[wm * 64 + i * 32 + lr];
+            const float sab = sa * sbu;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const float4 sb = *(const float4*)(&fac[st][1][wn * 64 + j * 32 + 8 * q + 4 * g]);
-                    acc[i][j][4 * q + 0] = fmaf(part[i][j][4 * q + 0], sa * sb.x, acc[i][j][4 * q + 0]);
-                    acc[i][j][4 * q + 1] = fmaf(part[i][j][4 * q + 1], sa * sb.y, acc[i][j][4 * q + 1]);
-                    acc[i][j][4 * q + 2] = fmaf(part[i][j][4 * q + 2], sa * sb.z, acc[i][j][4 * q + 2]);
-                    acc[i][j][4 * q + 3] = fmaf(part[i][j][4 * q + 3], sa * sb.w, acc[i][j][4 * q + 3]);
+                    if (SBU) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = fmaf(part[i][j][4 * q + e], sab, acc[i][j][4 * q + e]);
+                    } else {
+                        const float4 sb = *(const float4*)(&fac[BWG_BM + wn * 64 + j * 32 + 8 * q + 4 * g]);
+                        acc[i][j][4 * q + 0] = fmaf(part[i][j][4 * q + 0], sa * sb.x, acc[i][j][4 * q + 0]);
+                        acc[i][j][4 * q + 1] = fmaf(part[i][j][4 * q + 1], sa * sb.y, acc[i][j][4 * q + 1]);
+                        acc[i][j][4 * q + 2] = fmaf(part[i][j][4 * q + 2], sa * sb.z, acc[i][j][4 * q + 2]);
+                        acc[i][j][4 * q + 3] = fmaf(part[i][j][4 * q + 3], sa * sb.w, acc[i][j][4 * q + 3]);
+                    }
                 }
         }
-        if (kb + 1 < kb1) MXL_BW_STASH(st ^ 1);   // the other stage was last read before the previous iteration's barrier
-        __syncthreads();
+        st = st == BWG_STAGES - 1 ? 0 : st + 1;
+        st2 = st2 == BWG_STAGES - 1 ? 0 : st2 + 1;
     }
-#undef MXL_BW_FETCH
-#undef MXL_BW_STASH
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int64_t m = row0 + wm * 64 + i * 32 + lr;
@@ -400,9 +465,11 @@ __global__ __launch_bounds__(BW_THREADS, 2) void bw_gemm_kernel(BwGemmArgs p) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
+                const int64_t col = col0 + wn * 64 + j * 32 + 8 * q + 4 * g;
+                if (col >= pn) continue;     // (n is a multiple of 128: a quad is in or out as a whole)
                 const bv4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
                                  (__bf16)acc[i][j][4 * q + 3]};
-                *(bv4bf*)(pc_out + m * pn + col0 + wn * 64 + j * 32 + 8 * q + 4 * g) = o;
+                *(bv4bf*)(pc_out + m * pn + col) = o;
             }
     }
 }
@@ -435,6 +502,25 @@ static int bw_quant(const void* x, int64_t rows, int64_t cols, int fmt, const in
                 : launch_bw_quant<false>(a, fmt, row_tiles, 1, (hipStream_t)stream);
 }
 
+// The dynamic LDS size is above the default limit.  The attribute belongs to the (kernel, device) pair and is set at
+// the first launch on a device -- not at every launch: a launch may be recorded by a stream capture, which is no
+// place for a call that changes function state.
+template <int AFMT, int BFMT, bool SBU>
+static int launch_bw_gemm(const BwGemmArgs& g, dim3 grid, hipStream_t st) {
+    static std::atomic<bool> attr_set[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MXL_ELAUNCH;
+    const int slot = dev & 63;
+    auto kern = bw_gemm_kernel<AFMT, BFMT, SBU>;
+    if (!attr_set[slot].load(std::memory_order_acquire)) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BW_GEMM_LDS) != hipSuccess)
+            return MXL_ELAUNCH;
+        attr_set[slot].store(true, std::memory_order_release);
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(BWG_THREADS), BW_GEMM_LDS, st, g);
+    return MXL_OK;
+}
+
 static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv, int b_fmt,
                    int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k, int mode, const int64_t* group_lens,
                    int num_groups, void* stream) {
@@ -451,23 +537,18 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
     // row tiles: exact for a dense GEMM and for wgrad; at most one ragged tile per group in the grouped forward
     const int64_t row_tiles = mode == 1 ? m / BW + num_groups : (m + BW - 1) / BW;
     if (row_tiles > 65535 || (mode == 2 && num_groups > 65535)) return MXL_EINVAL;
+    if (256 * k >= ((int64_t)1 << 31)) return MXL_EINVAL;     // byte offsets inside a tile's operand rows are 32-bit
     BwGemmArgs g{(const uint8_t*)a_codes, (const float*)a_sinv, (const uint8_t*)b_codes, (const float*)b_sinv, (uint16_t*)c_bf16,
                  m, n, k, b_rows_per_scale == 1 ? 0 : 7, mode, group_lens, num_groups};
-    const dim3 grid((unsigned)(n / BW), (unsigned)row_tiles, (unsigned)(mode == 2 ? num_groups : 1));
+    const dim3 grid((unsigned)((n + BWG_BN - 1) / BWG_BN), (unsigned)row_tiles, (unsigned)(mode == 2 ? num_groups : 1));
     hipStream_t st = (hipStream_t)stream;
-    // the dynamic LDS size is above the default limit: the attribute is set at every launch (a host-side table write)
-#define MXL_BW_GEMM(A, B)                                                                                                \
-    do {                                                                                                                 \
-        if (hipFuncSetAttribute((const void*)bw_gemm_kernel<A, B>, hipFuncAttributeMaxDynamicSharedMemorySize,          \
-                                BW_GEMM_LDS) != hipSuccess)                                                              \
-            return MXL_ELAUNCH;                                                                                          \
-        hipLaunchKernelGGL((bw_gemm_kernel<A, B>), grid, dim3(BW_THREADS), BW_GEMM_LDS, st, g);                          \
-    } while (0)
-    if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) MXL_BW_GEMM(MXL_FMT_E4M3, MXL_FMT_E4M3);
-    else if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) MXL_BW_GEMM(MXL_FMT_E5M2, MXL_FMT_E4M3);
-    else if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) MXL_BW_GEMM(MXL_FMT_E4M3, MXL_FMT_E5M2);
-    else MXL_BW_GEMM(MXL_FMT_E5M2, MXL_FMT_E5M2);
-#undef MXL_BW_GEMM
+    const bool sbu = b_rows_per_scale == BW;
+    int rc;
+    if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) rc = sbu ? launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, false>(g, grid, st);
+    else if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) rc = sbu ? launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, false>(g, grid, st);
+    else if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) rc = sbu ? launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E5M2, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E5M2, false>(g, grid, st);
+    else rc = sbu ? launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E5M2, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E5M2, false>(g, grid, st);
+    if (rc != MXL_OK) return rc;
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 

@@ -335,3 +335,41 @@ def test_megatron_grouped_linear_under_the_blockwise_recipe(gpu):
         pt.PrimusTurboLowPrecisionGlobalStateManager.reset()
         runtime.set_args()
         runtime.set_num_microbatches(1)
+
+
+def test_operator_replays_under_a_graph(gpu):
+    """Forward and backward of the dense operator captured once (after an eager pass, so every kernel's launch
+    attributes are in place before the capture) and replayed on new inputs: every replay equals the eager result."""
+    import primus_amd.pytorch as turbo
+    from primus_amd.pytorch.core import Float8QuantConfig, Format, ScalingGranularity
+
+    cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+    x = _x(1, 300, 256).to(gpu).requires_grad_()
+    w = (_x(2, 384, 256) * 0.05).bfloat16().to(gpu).requires_grad_()
+    dy = _x(3, 300, 384).to(gpu)
+
+    def step():
+        y = turbo.ops.gemm_fp8(x, w, config=cfg)
+        dx, dw = torch.autograd.grad(y, [x, w], dy)
+        return y, dx, dw
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for seed in (4, 5, 6):
+        with torch.no_grad():
+            x.copy_(_x(seed, 300, 256))
+            dy.copy_(_x(seed + 10, 300, 384))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()
+        torch.cuda.synchronize()
+        for u, v in zip(got, want):
+            assert torch.equal(u.view(torch.int16), v.view(torch.int16)), seed

@@ -257,9 +257,16 @@ int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_f
  *   mxl_grouped_gemm_bf16_wgrad: c[num_groups, m_out, n_out] = sum over the tokens t of group g of
  *     p[t, m_out] * q[t, n_out]  (p = dy, q = x gives the [n, k] weight gradient); a group without tokens yields zeros.
  *     bf16 output, or with MXL_BF_ACCUM_F32 c is float32 and the result is ADDED to it (the main_grad fusion).
- *     Requires m_out % 8 == 0, n_out % 8 == 0; an operand stays below 4 GiB. */
+ *     Requires m_out % 8 == 0, n_out % 8 == 0; an operand stays below 4 GiB.
+ * Output tiles are 256 columns wide and 256 or 128 rows high.  Without a tile flag the library picks by the average
+ * rows per group, total_m / num_groups (256 rows from 384 on for forward / dgrad, from 1024 on for the weight
+ * gradient, whose contraction runs over a group's rows); MXL_BF_TILE_128 / MXL_BF_TILE_256 state the choice (a caller
+ * who knows its groups are few and long, or many and short).  The result does not depend on the tile height beyond fp32 summation order -- it is the
+ * same: every output element adds its products in the same order in both. */
 #define MXL_BF_B_KN 1u
 #define MXL_BF_ACCUM_F32 2u
+#define MXL_BF_TILE_128 4u
+#define MXL_BF_TILE_256 8u
 int mxl_grouped_gemm_bf16(const void* a_bf16, const void* b_bf16, void* c_bf16, const int64_t* group_lens, int num_groups,
                           int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream);
 int mxl_grouped_gemm_bf16_wgrad(const void* p_bf16, const void* q_bf16, void* c, const int64_t* group_lens, int num_groups,
@@ -477,6 +484,9 @@ int mxl_calibrate_mfma(int a_fmt, int b_fmt, int64_t iters, void* stream);
  * is what that access pattern reaches on the board. */
 int mxl_calibrate_tile_copy(const void* in_bf16, int64_t rows, int64_t cols, void* out_row, void* out_colT, void* stream);
 int64_t mxl_calibrate_mfma_flops(int64_t iters);
+/* The same loop for the bf16 MFMA of the unquantised grouped GEMM (32 x 32 x 16, 32 per iteration and wave). */
+int mxl_calibrate_mfma_bf16(int64_t iters, void* stream);
+int64_t mxl_calibrate_mfma_bf16_flops(int64_t iters);
 /* mxl_calibrate_range_check makes the hardware rule observable on which the GEMM kernels' operand requests rely (a
  * request for rows past the end of an operand must read nothing): for each of num_cases triples of uint32
  * {voffset, soffset, num_records} (device array `cases`) one LDS-direct 16-byte buffer load goes through a raw

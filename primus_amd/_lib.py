@@ -33,7 +33,7 @@ GF_KSTEP = 4                                # ... K-step-major codes and scales 
 GF_ACCUM_F32 = 2                            # wgrad: the output is float32 and the result is added to it
 GF_B_SHUFFLED = 16                          # forward / dgrad, row-major E2M1: b's codes are in the pre-shuffled byte order
 GF_B_TRANSPOSED = 8                         # forward / dgrad: b's codes are those of the transposed matrices (row-wise weight copy)
-BF_B_KN, BF_ACCUM_F32 = 1, 2                # flags of the bf16 grouped GEMMs
+BF_B_KN, BF_ACCUM_F32, BF_TILE_128, BF_TILE_256 = 1, 2, 4, 8    # flags of the bf16 grouped GEMMs
 
 EXPORTS = (
     "mxl_version",
@@ -78,6 +78,8 @@ EXPORTS = (
     "mxl_shuffle_scales",
     "mxl_calibrate_mfma",
     "mxl_calibrate_mfma_flops",
+    "mxl_calibrate_mfma_bf16",
+    "mxl_calibrate_mfma_bf16_flops",
     "mxl_calibrate_tile_copy",
     "mxl_calibrate_range_check",
 )
@@ -195,6 +197,10 @@ def load() -> ctypes.CDLL:
         lib.mxl_calibrate_range_check.argtypes = [vp, i64, vp, i32, vp, i64, vp]
         lib.mxl_calibrate_mfma_flops.restype = i64
         lib.mxl_calibrate_mfma_flops.argtypes = [i64]
+        lib.mxl_calibrate_mfma_bf16.restype = i32
+        lib.mxl_calibrate_mfma_bf16.argtypes = [i64, vp]
+        lib.mxl_calibrate_mfma_bf16_flops.restype = i64
+        lib.mxl_calibrate_mfma_bf16_flops.argtypes = [i64]
         lib.mxl_gemm_nt_blockwise.restype = i32
         lib.mxl_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, i32, vp, i64, i64, i64, vp]
         _lib = lib

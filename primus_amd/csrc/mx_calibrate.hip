@@ -58,6 +58,50 @@ __global__ __launch_bounds__(256) void mfma_only_kernel(int iters) {
     if (s == 12345.678f) calibrate_sink[threadIdx.x & 63] = s;   // keeps the loop alive; practically never taken
 }
 
+// The same for the bf16 MFMA of the unquantised grouped GEMM (32 x 32 x 16): 32 MFMAs per iteration on the 128 x 128
+// accumulator tile, i.e. one K slot of 32 elements.
+typedef __bf16 cal_v8bf __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(256) void mfma_only_bf16_kernel(int iters) {
+    const uint32_t tid = blockIdx.x * 256 + threadIdx.x;
+    v4i a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            // two bf16 per word, exponents 0x3C .. 0x3F (magnitudes below 2, no NaN or Inf patterns)
+            a[i][e] = (int)((calib_hash(tid * 131u + i * 17u + e) & 0x81FF81FFu) | 0x3E003E00u);
+            b[i][e] = (int)((calib_hash(tid * 257u + i * 29u + e + 99u) & 0x81FF81FFu) | 0x3E003E00u);
+        }
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(cal_v8bf, b[j]), __builtin_bit_cast(cal_v8bf, a[i]),
+                                                                        acc[i][j], 0, 0, 0);
+            a[0][0] ^= (it & 0xFF);   // the operands change a little from step to step (mantissa bits only)
+            b[1][3] ^= (it & 0x1F) << 3;
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+    if (s == 12345.678f) calibrate_sink[threadIdx.x & 63] = s;
+}
+
 // The traffic of the dual quantiser without its arithmetic: every workgroup reads a 128 x 128 bf16 tile (16 bytes per
 // lane, rows adjacent) and writes one byte per element at the tile's place in a row-major array and one byte per
 // element at its place in the transposed array (16-byte stores; the bytes are XORs of the input, nothing is
@@ -176,6 +220,18 @@ extern "C" int mxl_calibrate_mfma(int a_fmt, int b_fmt, int64_t iters, void* str
     else if (a4) hipLaunchKernelGGL((mfma_only_kernel<4, 0>), grid, block, 0, st, (int)iters);
     else if (b4) hipLaunchKernelGGL((mfma_only_kernel<0, 4>), grid, block, 0, st, (int)iters);
     else hipLaunchKernelGGL((mfma_only_kernel<0, 0>), grid, block, 0, st, (int)iters);
+    return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
+}
+
+extern "C" int64_t mxl_calibrate_mfma_bf16_flops(int64_t iters) {
+    // 256 workgroups x 4 waves x iters x 32 MFMAs of 32 x 32 x 16
+    return iters < 0 ? -1 : 256 * 4 * iters * 32 * (2LL * 32 * 32 * 16);
+}
+
+extern "C" int mxl_calibrate_mfma_bf16(int64_t iters, void* stream) {
+    if (iters < 1 || iters > (1 << 24)) return MXL_EINVAL;
+    if (!device_is_gfx950()) return MXL_ENODEV;
+    hipLaunchKernelGGL(mfma_only_bf16_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, (int)iters);
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 

@@ -7,9 +7,12 @@
 //                                                                   or . b_g          b_g = [k, n]   (MXL_BF_B_KN)
 //   wgrad           :  c[g][m_out, n_out] = sum over the tokens t of group g of p[t, m_out] * q[t, n_out]
 //
-// One workgroup (4 waves, 2 x 2) per 128 x 256 output tile, a wave owns 64 x 128 = 2 x 4 MFMA tiles of 32 x 32 with
-// fp32 accumulators.  K advances in slots of 32 elements (64 bytes per row) through a 2-stage LDS buffer filled by
-// LDS-direct loads (buffer_load ... lds) one slot ahead.  An operand whose contraction dim is contiguous in memory is
+// One workgroup (4 waves, 2 x 2) per BM x 256 output tile, in two sizes chosen per launch: BM = 256 (a wave owns
+// 128 x 128 = 4 x 4 MFMA tiles of 32 x 32, 256 fp32 accumulators, one workgroup per CU, a ring of four 32 KiB LDS
+// stages filled three K slots ahead) for groups of many rows, and BM = 128 (64 x 128 per wave, two workgroups per CU,
+// two stages) for groups of a few hundred rows, where a 256-row tile would mostly hold padding.  K advances in slots
+// of 32 elements (64 bytes per row), filled by LDS-direct loads (buffer_load ... lds); loads complete in order, so a
+// partial s_waitcnt leaves the younger slots in flight, and there is one barrier per slot.  An operand whose contraction dim is contiguous in memory is
 // staged [rows][32] and read with ds_read_b128; one whose contraction dim is the slow one (the [k, n] weight, both
 // operands of wgrad) is staged as it lies, [32][columns], and read with the transposing LDS read ds_read_b64_tr_b16,
 // which hands every lane four consecutive contraction elements of its own column.  Measured lane mapping of that
@@ -19,12 +22,14 @@
 // for the largest tile count the sizes allow and surplus workgroups leave at once.
 #include "mx_device.h"
 
+#include <type_traits>
+
 namespace mxl {
 
-constexpr int BF_BM = 128, BF_BN = 256;
+constexpr int BF_BN = 256;
 constexpr int BF_KS = 32;                  // contraction elements per slot (two MFMA K steps of 16)
 constexpr int BF_THREADS = 256;
-constexpr int BF_A_BYTES = BF_BM * 64, BF_B_BYTES = BF_BN * 64, BF_STAGE = BF_A_BYTES + BF_B_BYTES;   // 8 + 16 KiB
+constexpr int BF_B_BYTES = BF_BN * 64;     // 16 KiB of b per stage; a: BM * 64
 constexpr int BF_CPITCH = 264;             // bytes per staged output row: 128 bf16 + 8 (rows spread over the banks)
 constexpr int BF_GROUP_M = 8;              // tile order: super-rows of this many row tiles
 
@@ -62,20 +67,29 @@ __device__ __forceinline__ void bf_dma16(v4i rsrc, uint32_t lds_off, uint32_t vo
                  : "memory");
 }
 
-constexpr int bf16_lds_bytes() {
-    return 2 * BF_STAGE + (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
+constexpr int bf16_lds_bytes(int bm, int nst) {
+    return nst * (bm * 64 + BF_B_BYTES) + (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
 }
-static_assert(BF_BM * BF_CPITCH <= 2 * BF_STAGE, "the output staging area reuses the operand stages");
+template <int N>
+__device__ __forceinline__ void bf_wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 // A_T / B_T: the operand's contraction dim is the slow one in memory (staged [32][cols], transposing reads).
 // WGRAD: contraction over the tokens of a group (both operands A_T / B_T), one output matrix per group.
 // ACCUM (wgrad): c is float32 and the result is added to it.
-template <bool A_T, bool B_T, bool WGRAD, bool ACCUM>
-__global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
+template <int BF_BM, int NST, bool A_T, bool B_T, bool WGRAD, bool ACCUM>
+__global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_kernel(Bf16Args p) {
     static_assert(!WGRAD || (A_T && B_T), "wgrad contracts over tokens: both operands are token-major");
     static_assert(!ACCUM || WGRAD, "only the weight gradient accumulates");
+    static_assert((BF_BM == 128 && NST == 2) || (BF_BM == 256 && NST == 4), "tile sizes built");
+    constexpr int BF_A_BYTES = BF_BM * 64, BF_STAGE = BF_A_BYTES + BF_B_BYTES;
+    constexpr int MI = BF_BM / 64;             // 32-row fragments per wave
+    constexpr int AR = BF_BM / 64;             // load rounds of 4 KiB for a (b: 4)
+    constexpr int LOADS = AR + 4;              // requests per wave and slot
+    static_assert(BF_BM * BF_CPITCH <= NST * BF_STAGE, "the output staging area reuses the operand stages");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    int* pre_tiles = (int*)(smem + 2 * BF_STAGE);
+    int* pre_tiles = (int*)(smem + NST * BF_STAGE);
     int64_t* pre_rows = (int64_t*)(pre_tiles + MXL_MAX_GROUPS + 2);
     const int t = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -131,7 +145,7 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
     int64_t c_row0;                 // first output row (forward: token row; wgrad: row inside the group's matrix)
     v4i ra, rb;
     uint32_t a_step, b_step;        // bytes from one K slot to the next
-    uint32_t va[2], vb[4];          // per-lane offsets of the load rounds
+    uint32_t va[AR], vb[4];         // per-lane offsets of the load rounds
     if (!WGRAD) {
         int lo = 0, hi = G;
         while (hi - lo > 1) {
@@ -149,7 +163,7 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
         ra = bf_rsrc(p.a + c_row0 * lda, (p.total_m - c_row0) * lda);
         a_step = 64;
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
+        for (int e = 0; e < AR; ++e) {
             const int row = (t >> 2) + 64 * e;
             va[e] = (uint32_t)(row * lda + 16 * ((t & 3) ^ ((row >> 2) & 3)));
         }
@@ -170,7 +184,7 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int row = (t >> 5) + 8 * e;
-                vb[e] = (uint32_t)(row * ldb + 16 * ((t & 31) ^ ((row & 3) << 1)));
+                vb[e] = (uint32_t)(row * ldb + 16 * ((t & 31) ^ ((row & 3) << 2)));
             }
         }
     } else {
@@ -186,15 +200,16 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
         rb = bf_rsrc(p.b + t0 * ldb + n0 * 2, len * ldb - n0 * 2);
         a_step = (uint32_t)(BF_KS * lda);
         b_step = (uint32_t)(BF_KS * ldb);
+        // a round of 4 KiB holds 32 / AR contraction rows of BM columns
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const int row = (t >> 4) + 16 * e;
-            va[e] = (uint32_t)(row * lda + 16 * ((t & 15) ^ ((row & 3) << 1)));
+        for (int e = 0; e < AR; ++e) {
+            const int row = t / (BF_BM / 8) + (32 / AR) * e;
+            va[e] = (uint32_t)(row * lda + 16 * ((t % (BF_BM / 8)) ^ ((row & 3) << 2)));
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = (t >> 5) + 8 * e;
-            vb[e] = (uint32_t)(row * ldb + 16 * ((t & 31) ^ ((row & 3) << 1)));
+            vb[e] = (uint32_t)(row * ldb + 16 * ((t & 31) ^ ((row & 3) << 2)));
         }
     }
     a_step = (uint32_t)__builtin_amdgcn_readfirstlane((int)a_step);
@@ -205,21 +220,21 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
         const uint32_t base = smem_base + (uint32_t)(stage * BF_STAGE) + (uint32_t)(w * 1024);
         const uint32_t sa = (uint32_t)slot * a_step, sb = (uint32_t)slot * b_step;
 #pragma unroll
-        for (int e = 0; e < 2; ++e) bf_dma16(ra, base + e * 4096, va[e], sa);
+        for (int e = 0; e < AR; ++e) bf_dma16(ra, base + e * 4096, va[e], sa);
 #pragma unroll
         for (int e = 0; e < 4; ++e) bf_dma16(rb, base + BF_A_BYTES + e * 4096, vb[e], sb);
     };
 
     // ---- per-lane constants of the fragment reads ----
     // contiguous operand, 64-byte rows: lane (row lr, half g) reads piece 2 ks + g, XOR (row / 4) % 4
-    const int ca_row = wm * 64 + lr, cb_row = wn * 128 + lr;
+    const int ca_row = wm * (BF_BM / 2) + lr, cb_row = wn * 128 + lr;
     // transposed operand: this lane ADDRESSES row j of a 4-row group, 8-byte piece `a4` of its 16-lane block's 16 columns
     const int tj = (l & 15) >> 2, ta4 = l & 3, tblk = (l >> 4) & 1;
     const int t_colbyte = 32 * tblk + 8 * ta4;     // byte offset of the piece inside a 32-column fragment
 
-    v16f acc[2][4];
+    v16f acc[MI][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -236,7 +251,7 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
         for (int h = 0; h < 2; ++h) {
             const int row = 16 * ks + 8 * g + 4 * h + tj;
             const int byte = 2 * col0 + t_colbyte;
-            uint8_t* ptr = base + row * pitch + 16 * ((byte >> 4) ^ ((row & 3) << 1)) + (byte & 15);
+            uint8_t* ptr = base + row * pitch + 16 * ((byte >> 4) ^ ((row & 3) << 2)) + (byte & 15);
             const v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)ptr);
             const v4bf vb4 = __builtin_bit_cast(v4bf, v);
             out[4 * h] = vb4[0]; out[4 * h + 1] = vb4[1]; out[4 * h + 2] = vb4[2]; out[4 * h + 3] = vb4[3];
@@ -244,27 +259,149 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
         return out;
     };
 
-    if (nslots > 0) issue(0, 0);
-    for (int s = 0; s < nslots; ++s) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();     // slot s has landed everywhere, and every wave has left the other stage
-        if (s + 1 < nslots) issue(s + 1, (s + 1) & 1);
-        uint8_t* sa = smem + (s & 1) * BF_STAGE;
-        uint8_t* sb = sa + BF_A_BYTES;
+    // row fragments of this wave that hold rows of the tile (the others are neither read nor multiplied)
+    int live = (m_valid - wm * (BF_BM / 2) + 31) >> 5;
+    live = __builtin_amdgcn_readfirstlane(live < 0 ? 0 : (live > MI ? MI : live));
+
+    // slot s has landed when at most the requests of the younger slots in flight are outstanding
+    auto wait_slot = [&](int s) __attribute__((always_inline)) {
+        const int younger = nslots - 1 - s;
+        if (NST >= 4 && younger >= 2) bf_wait_vm<2 * LOADS>();
+        else if (NST >= 3 && younger >= 1) bf_wait_vm<LOADS>();
+        else bf_wait_vm<0>();
+    };
+    auto read_a = [&](uint8_t* sa, int i, int ks) __attribute__((always_inline)) {
+        return A_T ? read_trans(sa, BF_BM * 2, wm * (BF_BM / 2) + 32 * i, ks) : read_contig(sa, ca_row + 32 * i, ks);
+    };
+    auto read_b = [&](uint8_t* sb, int j, int ks) __attribute__((always_inline)) {
+        return B_T ? read_trans(sb, 512, wn * 128 + 32 * j, ks) : read_contig(sb, cb_row + 32 * j, ks);
+    };
+    if constexpr (NST >= 4) {
+      if (live == MI && nslots > 0) {
+        // One wave per SIMD: nothing but this wave's own instruction order keeps the MFMA pipe fed, so the order is
+        // written out and pinned (sched_barrier): every fragment read and every load request sits between two MFMAs.
+        // A slot is two halves of 16 MFMAs (4 x 4 fragments, 16 contraction elements).  While the MFMAs of half 0 run,
+        // the fragments of half 1 are read; the first four MFMAs of half 1 are issued in front of the slot barrier (so
+        // the pipe has work while the waves meet), the fragments of the next slot's half 0 are read behind it.
+        // The 8 requests of slot s + 3 go out four per half, and the four waves -- which run in lockstep between the
+        // barriers, one per SIMD -- take turns: wave PH issues behind MFMA 4 e + PH, so the address unit sees one
+        // request per MFMA time instead of four at once and no wave waits at the unit's queue with its MFMA pipe
+        // running empty (a bf16 MFMA is over in 32 clocks, a request occupies the unit for about 16).
+        // Requests past the last slot fetch the last slot again (into a stage nobody reads any more): the request
+        // count per slot is then the same in every iteration and the partial waits are constants.
+        // The N-side fragment is MFMA source 0, so that a lane holds 4 consecutive output columns per register quad.
+        static_assert(MI == 4 && AR == 4, "written out for the 256-row tile");
+        const int last = nslots - 1;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            v8bf fa[2], fb[4];
+        for (int s = 0; s < NST - 1; ++s) issue(s < last ? s : last, s);
+        bf_wait_vm<2 * LOADS>();
+        __syncthreads();
+        auto run = [&](auto ph_tag) __attribute__((always_inline)) {
+            constexpr int PH = decltype(ph_tag)::value;
+            v8bf fa0[4], fb0[4], fa1[4], fb1[4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                fa[i] = A_T ? read_trans(sa, 256, wm * 64 + 32 * i, ks) : read_contig(sa, ca_row + 32 * i, ks);
+            for (int j = 0; j < 4; ++j) fb0[j] = read_b(smem + BF_A_BYTES, j, 0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                fb[j] = B_T ? read_trans(sb, 512, wn * 128 + 32 * j, ks) : read_contig(sb, cb_row + 32 * j, ks);
-            // the N-side fragment is MFMA source 0: a lane then holds 4 consecutive output columns per register quad
+            for (int i = 0; i < 4; ++i) fa0[i] = read_a(smem, i, 0);
+#define BF_PIN __builtin_amdgcn_sched_barrier(0)
+            // MFMA number M = 4 j + i of a half; behind it, wave PH issues request (M - PH) / 4 of the half
+#define BF_STEP(FA, FB, M, R, VO, SO, OFF)                                                                                \
+    acc[(M) & 3][(M) >> 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[(M) >> 2], FA[(M) & 3], acc[(M) & 3][(M) >> 2], 0, 0, 0); \
+    if constexpr (((M) & 3) == PH) bf_dma16(R, in_base + (OFF) + ((M) >> 2) * 4096, VO[(M) >> 2], SO);                       \
+    BF_PIN
+            int stage = 0;                            // stage of slot s; slot s + 3 goes into the stage in front of it
+            for (int s = 0; s < nslots; ++s) {
+                uint8_t* sa = smem + stage * BF_STAGE;
+                uint8_t* sb = sa + BF_A_BYTES;
+                const int in_slot = s + NST - 1 < last ? s + NST - 1 : last;
+                const uint32_t in_base = smem_base + (uint32_t)((stage == 0 ? NST - 1 : stage - 1) * BF_STAGE) + (uint32_t)(w * 1024);
+                const uint32_t in_sa = (uint32_t)in_slot * a_step, in_sb = (uint32_t)in_slot * b_step;
+                // ---- half 0 multiplies, half 1 is read; requests: the a rows of slot s + 3 ----
+                fb1[0] = read_b(sb, 0, 1); BF_STEP(fa0, fb0, 0, ra, va, in_sa, 0);
+                fa1[0] = read_a(sa, 0, 1); BF_STEP(fa0, fb0, 1, ra, va, in_sa, 0);
+                fa1[1] = read_a(sa, 1, 1); BF_STEP(fa0, fb0, 2, ra, va, in_sa, 0);
+                fa1[2] = read_a(sa, 2, 1); BF_STEP(fa0, fb0, 3, ra, va, in_sa, 0);
+                fa1[3] = read_a(sa, 3, 1); BF_STEP(fa0, fb0, 4, ra, va, in_sa, 0);
+                fb1[1] = read_b(sb, 1, 1); BF_STEP(fa0, fb0, 5, ra, va, in_sa, 0);
+                fb1[2] = read_b(sb, 2, 1); BF_STEP(fa0, fb0, 6, ra, va, in_sa, 0);
+                fb1[3] = read_b(sb, 3, 1); BF_STEP(fa0, fb0, 7, ra, va, in_sa, 0);
+                BF_STEP(fa0, fb0, 8, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 9, ra, va, in_sa, 0);
+                BF_STEP(fa0, fb0, 10, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 11, ra, va, in_sa, 0);
+                BF_STEP(fa0, fb0, 12, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 13, ra, va, in_sa, 0);
+                BF_STEP(fa0, fb0, 14, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 15, ra, va, in_sa, 0);
+                // ---- half 1 multiplies; behind the barrier the next slot's half 0 is read; requests: the b rows ----
+                BF_STEP(fa1, fb1, 0, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 1, rb, vb, in_sb, BF_A_BYTES);
+                BF_STEP(fa1, fb1, 2, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 3, rb, vb, in_sb, BF_A_BYTES);
+                stage = stage == NST - 1 ? 0 : stage + 1;
+                // slot s + 1 has landed when only slot s + 2, the a rows of slot s + 3 and its first b request are outstanding
+                // (waves of a ragged tile that run the generic loop below meet the same barriers: one per slot)
+                if (s + 1 < nslots) {
+                    bf_wait_vm<LOADS + AR + 1>();
+                    __syncthreads();   // slot s + 1 is in LDS for every wave; every wave holds its fragments of slot s
+                }
+                BF_PIN;
+                uint8_t* na = smem + stage * BF_STAGE;
+                uint8_t* nb = na + BF_A_BYTES;
+                fb0[0] = read_b(nb, 0, 0); BF_STEP(fa1, fb1, 4, rb, vb, in_sb, BF_A_BYTES);
+                fa0[0] = read_a(na, 0, 0); BF_STEP(fa1, fb1, 5, rb, vb, in_sb, BF_A_BYTES);
+                fa0[1] = read_a(na, 1, 0); BF_STEP(fa1, fb1, 6, rb, vb, in_sb, BF_A_BYTES);
+                fa0[2] = read_a(na, 2, 0); BF_STEP(fa1, fb1, 7, rb, vb, in_sb, BF_A_BYTES);
+                fa0[3] = read_a(na, 3, 0); BF_STEP(fa1, fb1, 8, rb, vb, in_sb, BF_A_BYTES);
+                fb0[1] = read_b(nb, 1, 0); BF_STEP(fa1, fb1, 9, rb, vb, in_sb, BF_A_BYTES);
+                fb0[2] = read_b(nb, 2, 0); BF_STEP(fa1, fb1, 10, rb, vb, in_sb, BF_A_BYTES);
+                fb0[3] = read_b(nb, 3, 0); BF_STEP(fa1, fb1, 11, rb, vb, in_sb, BF_A_BYTES);
+                BF_STEP(fa1, fb1, 12, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 13, rb, vb, in_sb, BF_A_BYTES);
+                BF_STEP(fa1, fb1, 14, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 15, rb, vb, in_sb, BF_A_BYTES);
+            }
+#undef BF_STEP
+#undef BF_PIN
+        };
+        if (w == 0) run(std::integral_constant<int, 0>{});
+        else if (w == 1) run(std::integral_constant<int, 1>{});
+        else if (w == 2) run(std::integral_constant<int, 2>{});
+        else run(std::integral_constant<int, 3>{});
+        bf_wait_vm<0>();     // the repeated requests of the last slots must not land in the output staging area
+      }
+    }
+    if (NST < 4 || live != MI) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+        for (int s = 0; s < NST - 1; ++s)
+            if (s < nslots) issue(s, s);
+        int stage = 0, stage_in = NST - 1;        // stage of slot s; stage that slot s + NST - 1 goes into
+        for (int s = 0; s < nslots; ++s) {
+            wait_slot(s);
+            __syncthreads();     // slot s is in LDS for every wave, and every wave has left the stage of slot s - 1
+            if (s + NST - 1 < nslots) issue(s + NST - 1, stage_in);
+            uint8_t* sa = smem + stage * BF_STAGE;
+            uint8_t* sb = sa + BF_A_BYTES;
+            if (live > 0) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                for (int ks = 0; ks < 2; ++ks) {
+                    v8bf fb[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) fb[j] = read_b(sb, j, ks);
+                    if (NST == 2 || live == MI) {
+                        v8bf fa[MI];
+#pragma unroll
+                        for (int i = 0; i < MI; ++i) fa[i] = read_a(sa, i, ks);
+#pragma unroll
+                        for (int i = 0; i < MI; ++i)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < MI; ++i) {
+                            if (i < live) {
+                                const v8bf fa = read_a(sa, i, ks);
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa, acc[i][j], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
+            stage = stage == NST - 1 ? 0 : stage + 1;
+            stage_in = stage_in == NST - 1 ? 0 : stage_in + 1;
         }
     }
     __syncthreads();         // every wave is done with the stages: they become the output staging area
@@ -273,8 +410,8 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
     if (ACCUM) {
         float* c = (float*)p.c + ((int64_t)grp * p.m + c_row0) * p.n + n0;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int row = wm * 64 + 32 * i + lr;
+        for (int i = 0; i < MI; ++i) {
+            const int row = wm * (BF_BM / 2) + 32 * i + lr;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -290,25 +427,25 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
         }
     } else {
         uint16_t* c = (uint16_t*)p.c + ((WGRAD ? (int64_t)grp * p.m : 0) + c_row0) * p.n + n0;
-        // two passes, one per 128-column half: its waves stage 128 x 128 bf16, then all threads store whole rows
+        // two passes, one per 128-column half: its waves stage BM x 128 bf16, then all threads store whole rows
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             if (h) __syncthreads();
             if (wn == h) {
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < MI; ++i)
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
                             const v4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
                                             (__bf16)acc[i][j][4 * q + 3]};
-                            *(v4bf*)(smem + (wm * 64 + 32 * i + lr) * BF_CPITCH + (32 * j + 8 * q + 4 * g) * 2) = o;
+                            *(v4bf*)(smem + (wm * (BF_BM / 2) + 32 * i + lr) * BF_CPITCH + (32 * j + 8 * q + 4 * g) * 2) = o;
                         }
             }
             __syncthreads();
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < BF_BM / 16; ++u) {
                 const int idx = u * BF_THREADS + t, row = idx >> 4, piece = idx & 15;
                 const int col = h * 128 + piece * 8;
                 if (row < m_valid && col < n_valid) {
@@ -321,14 +458,14 @@ __global__ __launch_bounds__(BF_THREADS, 2) void bf16_gemm_kernel(Bf16Args p) {
     }
 }
 
-template <bool A_T, bool B_T, bool WGRAD, bool ACCUM>
+template <int BM, int NST, bool A_T, bool B_T, bool WGRAD, bool ACCUM>
 static int launch_bf16(const Bf16Args& a, int64_t max_tiles, hipStream_t st) {
-    constexpr int lds = bf16_lds_bytes();
+    constexpr int lds = bf16_lds_bytes(BM, NST);
     if (!device_is_gfx950()) return MXL_ENODEV;
     static std::atomic<bool> attr_set[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return MXL_ELAUNCH;
-    auto kern = bf16_gemm_kernel<A_T, B_T, WGRAD, ACCUM>;
+    auto kern = bf16_gemm_kernel<BM, NST, A_T, B_T, WGRAD, ACCUM>;
     if (!attr_set[dev & 63].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return MXL_ELAUNCH;
         attr_set[dev & 63].store(true, std::memory_order_release);
@@ -340,13 +477,25 @@ static int launch_bf16(const Bf16Args& a, int64_t max_tiles, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
 
+// Tile height of a launch: the caller's choice (MXL_BF_TILE_128 / MXL_BF_TILE_256), else from the average number of
+// rows per group -- the counts live on the device, the average is all the host knows.  Measured crossovers: forward /
+// dgrad tiles are cut from a group's rows, and 256-row tiles win from about 400 rows per group on (below, most of a
+// group's last tile is padding); the weight gradient contracts over a group's rows, and the tall tile's longer
+// prologue and epilogue pay off from about 1000 rows per group on.
+static bool bf16_tall_tiles(uint32_t flags, int64_t rows_per_group, int64_t threshold) {
+    if (flags & MXL_BF_TILE_256) return true;
+    if (flags & MXL_BF_TILE_128) return false;
+    return rows_per_group >= threshold;
+}
+
 }  // namespace mxl
 
 using namespace mxl;
 
 extern "C" int mxl_grouped_gemm_bf16(const void* a_bf16, const void* b_bf16, void* c_bf16, const int64_t* group_lens,
                                      int num_groups, int64_t total_m, int64_t n, int64_t k, uint32_t flags, void* stream) {
-    if (flags & ~(uint32_t)MXL_BF_B_KN) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_BF_B_KN | MXL_BF_TILE_128 | MXL_BF_TILE_256)) return MXL_EINVAL;
+    if ((flags & MXL_BF_TILE_128) && (flags & MXL_BF_TILE_256)) return MXL_EINVAL;
     if (total_m < 0 || n <= 0 || k <= 0 || n % 8 != 0 || k % BF_KS != 0) return MXL_EINVAL;
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS || (num_groups > 1 && !group_lens)) return MXL_EINVAL;
     if (total_m == 0) return MXL_OK;
@@ -355,15 +504,19 @@ extern "C" int mxl_grouped_gemm_bf16(const void* a_bf16, const void* b_bf16, voi
     // offsets inside a tile's operand rows are 32-bit
     if (256 * k * 2 >= ((int64_t)1 << 31) || k * n * 2 >= ((int64_t)1 << 32)) return MXL_EINVAL;
     Bf16Args a{(const uint8_t*)a_bf16, (const uint8_t*)b_bf16, c_bf16, group_lens, num_groups, total_m, 0, n, k};
-    const int64_t max_tiles = (total_m / BF_BM + num_groups) * ((n + BF_BN - 1) / BF_BN);
-    if (flags & MXL_BF_B_KN) return launch_bf16<false, true, false, false>(a, max_tiles, (hipStream_t)stream);
-    return launch_bf16<false, false, false, false>(a, max_tiles, (hipStream_t)stream);
+    const bool tall = bf16_tall_tiles(flags, total_m / num_groups, 384);
+    const int64_t max_tiles = (total_m / (tall ? 256 : 128) + num_groups) * ((n + BF_BN - 1) / BF_BN);
+    hipStream_t st = (hipStream_t)stream;
+    if (flags & MXL_BF_B_KN)
+        return tall ? launch_bf16<256, 4, false, true, false, false>(a, max_tiles, st) : launch_bf16<128, 2, false, true, false, false>(a, max_tiles, st);
+    return tall ? launch_bf16<256, 4, false, false, false, false>(a, max_tiles, st) : launch_bf16<128, 2, false, false, false, false>(a, max_tiles, st);
 }
 
 extern "C" int mxl_grouped_gemm_bf16_wgrad(const void* p_bf16, const void* q_bf16, void* c, const int64_t* group_lens,
                                            int num_groups, int64_t total_m, int64_t m_out, int64_t n_out, uint32_t flags,
                                            void* stream) {
-    if (flags & ~(uint32_t)MXL_BF_ACCUM_F32) return MXL_EINVAL;
+    if (flags & ~(uint32_t)(MXL_BF_ACCUM_F32 | MXL_BF_TILE_128 | MXL_BF_TILE_256)) return MXL_EINVAL;
+    if ((flags & MXL_BF_TILE_128) && (flags & MXL_BF_TILE_256)) return MXL_EINVAL;
     if (total_m < 0 || m_out <= 0 || n_out <= 0 || m_out % 8 != 0 || n_out % 8 != 0) return MXL_EINVAL;
     if (num_groups < 1 || num_groups > MXL_MAX_GROUPS || (num_groups > 1 && !group_lens)) return MXL_EINVAL;
     if (!c || ((uintptr_t)c & 15) != 0) return MXL_EINVAL;
@@ -371,7 +524,12 @@ extern "C" int mxl_grouped_gemm_bf16_wgrad(const void* p_bf16, const void* q_bf1
     // the K-slot advance inside a group's token range is a 32-bit byte offset
     if (total_m * m_out * 2 >= ((int64_t)1 << 32) || total_m * n_out * 2 >= ((int64_t)1 << 32)) return MXL_EINVAL;
     Bf16Args a{(const uint8_t*)p_bf16, (const uint8_t*)q_bf16, c, group_lens, num_groups, total_m, m_out, n_out, 0};
-    const int64_t max_tiles = (int64_t)num_groups * ((m_out + BF_BM - 1) / BF_BM) * ((n_out + BF_BN - 1) / BF_BN);
-    if (flags & MXL_BF_ACCUM_F32) return launch_bf16<true, true, true, true>(a, max_tiles, (hipStream_t)stream);
-    return launch_bf16<true, true, true, false>(a, max_tiles, (hipStream_t)stream);
+    // the tiles are cut from the [m_out, n_out] matrix of every group; the contraction runs over the group's tokens
+    const bool tall = bf16_tall_tiles(flags, total_m / num_groups, 1024);
+    const int bm = tall ? 256 : 128;
+    const int64_t max_tiles = (int64_t)num_groups * ((m_out + bm - 1) / bm) * ((n_out + BF_BN - 1) / BF_BN);
+    hipStream_t st = (hipStream_t)stream;
+    if (flags & MXL_BF_ACCUM_F32)
+        return tall ? launch_bf16<256, 4, true, true, true, true>(a, max_tiles, st) : launch_bf16<128, 2, true, true, true, true>(a, max_tiles, st);
+    return tall ? launch_bf16<256, 4, true, true, true, false>(a, max_tiles, st) : launch_bf16<128, 2, true, true, true, false>(a, max_tiles, st);
 }

@@ -649,10 +649,20 @@ def _glu_args(x, probs, row_mask, activation):
     return _ACTS[activation], pd, row_mask
 
 
-def grouped_gemm_bf16_impl(a: torch.Tensor, b: torch.Tensor, group_lens: Optional[torch.Tensor], b_kn: bool = False) -> torch.Tensor:
+def _bf16_tile_flag(tile: Optional[int]) -> int:
+    if tile is None:
+        return 0
+    if tile not in (128, 256):
+        raise ValueError("tile must be None (the library picks), 128 or 256")
+    return _lib.BF_TILE_128 if tile == 128 else _lib.BF_TILE_256
+
+
+def grouped_gemm_bf16_impl(a: torch.Tensor, b: torch.Tensor, group_lens: Optional[torch.Tensor], b_kn: bool = False,
+                           tile: Optional[int] = None) -> torch.Tensor:
     """Grouped GEMM on unquantised bf16 operands: the rows of ``a [total_m, k]`` are split by ``group_lens`` (device,
     never read back) and group g is multiplied by ``b[g]^T`` with ``b [G, n, k]``, or by ``b[g]`` with ``b [G, k, n]``
-    when ``b_kn``.  ``group_lens`` None: one group (``b`` 2-D or with a leading 1)."""
+    when ``b_kn``.  ``group_lens`` None: one group (``b`` 2-D or with a leading 1).  ``tile``: height of the output
+    tiles, 128 or 256 rows (None: picked from the average rows per group); the result is the same bit for bit."""
     _require_cuda(a, b, group_lens)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.dim() != 2:
         raise ValueError("the bf16 grouped GEMM takes a 2-D bf16 activation and a bf16 weight")
@@ -670,13 +680,13 @@ def grouped_gemm_bf16_impl(a: torch.Tensor, b: torch.Tensor, group_lens: Optiona
     lib = _lib.load()
     with _hooked("grouped_gemm_bf16", m=total_m, n=n, k=k):
         rc = lib.mxl_grouped_gemm_bf16(_ptr(a), _ptr(b3), _ptr(out), _ptr(group_lens), G, total_m, n, k,
-                                       _lib.BF_B_KN if b_kn else 0, _stream())
+                                       (_lib.BF_B_KN if b_kn else 0) | _bf16_tile_flag(tile), _stream())
     _lib.check(rc, "mxl_grouped_gemm_bf16")
     return out
 
 
 def grouped_gemm_bf16_wgrad_impl(p: torch.Tensor, q: torch.Tensor, group_lens: Optional[torch.Tensor],
-                                 accum_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+                                 accum_into: Optional[torch.Tensor] = None, tile: Optional[int] = None) -> torch.Tensor:
     """``c[g] = p[rows of g]^T . q[rows of g]`` for bf16 ``p [total_m, m_out]``, ``q [total_m, n_out]``: ``[G, m_out,
     n_out]`` bf16, zeros for a group without tokens; or added to the float32 ``accum_into`` of that shape."""
     _require_cuda(p, q, group_lens, accum_into)
@@ -696,7 +706,7 @@ def grouped_gemm_bf16_wgrad_impl(p: torch.Tensor, q: torch.Tensor, group_lens: O
     lib = _lib.load()
     with _hooked("grouped_gemm_bf16_wgrad", m=total_m, n=m_out, k=n_out):
         rc = lib.mxl_grouped_gemm_bf16_wgrad(_ptr(p), _ptr(q), _ptr(out), _ptr(group_lens), G, total_m, m_out, n_out,
-                                             _lib.BF_ACCUM_F32 if accum_into is not None else 0, _stream())
+                                             (_lib.BF_ACCUM_F32 if accum_into is not None else 0) | _bf16_tile_flag(tile), _stream())
     _lib.check(rc, "mxl_grouped_gemm_bf16_wgrad")
     return out
 

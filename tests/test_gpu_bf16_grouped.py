@@ -159,3 +159,56 @@ def test_shapes_the_kernel_does_not_take_are_refused(gpu):
     b = torch.zeros(1, 16, 40, dtype=torch.bfloat16, device=gpu)
     with pytest.raises(ValueError):
         turbo.ops.grouped_gemm(a, b, gl)
+
+
+TILE_CASES = [
+    ([100, 0, 37, 300], 320, 256),
+    ([1, 129, 0, 0, 128, 255, 257], 288, 96),
+    ([1500, 3, 700], 544, 160),
+    ([0, 0, 5], 32, 32),
+    ([513, 256, 31], 2880, 64),
+]
+
+
+@pytest.mark.parametrize("lens,n,k", TILE_CASES)
+def test_both_tile_heights_give_the_same_bits_and_match_fp32(gpu, lens, n, k):
+    """The 256-row tiles (4-stage ring, one workgroup per CU) and the 128-row tiles (2 stages, two per CU) add every
+    output element's products in the same order: forward, dgrad, wgrad and the accumulating wgrad are bit-identical,
+    and each matches the fp32 matmul per expert."""
+    from primus_amd.pytorch import kernels as K
+
+    G, m = len(lens), sum(lens)
+    gen = torch.Generator().manual_seed(m + 3 * n + k)
+    a = torch.randn(m, k, generator=gen).bfloat16().to(gpu)
+    b = (torch.randn(G, n, k, generator=gen) * 0.1).bfloat16().to(gpu)
+    dy = torch.randn(m, n, generator=gen).bfloat16().to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    outs = {}
+    for tile in (128, 256):
+        y = K.grouped_gemm_bf16_impl(a, b, gl, tile=tile)
+        dx = K.grouped_gemm_bf16_impl(dy, b, gl, b_kn=True, tile=tile)
+        dw = K.grouped_gemm_bf16_wgrad_impl(dy, a, gl, tile=tile)
+        acc = torch.full((G, n, k), 0.5, dtype=torch.float32, device=gpu)
+        K.grouped_gemm_bf16_wgrad_impl(dy, a, gl, accum_into=acc, tile=tile)
+        outs[tile] = (y, dx, dw, acc)
+    for u, v in zip(outs[128], outs[256]):
+        assert torch.equal(u.view(torch.int16 if u.dtype == torch.bfloat16 else torch.int32),
+                           v.view(torch.int16 if v.dtype == torch.bfloat16 else torch.int32))
+    y, dx, dw, acc = outs[256]
+    _close(y, _ref(a, b, lens, True), _ref(a.abs(), b.abs(), lens, True), k)
+    _close(dx, _ref(dy, b, lens, False), _ref(dy.abs(), b.abs(), lens, False), n)
+    off = 0
+    for g, ln in enumerate(lens):
+        x_g, d_g = a[off:off + ln].float(), dy[off:off + ln].float()
+        _close(dw[g], d_g.t() @ x_g, d_g.abs().t() @ x_g.abs(), ln)
+        assert torch.allclose(acc[g], 0.5 + d_g.t() @ x_g, rtol=1e-5, atol=1e-3 * max(1, ln) ** 0.5)
+        off += ln
+
+
+def test_tile_flags_are_validated(gpu):
+    from primus_amd.pytorch import kernels as K
+
+    a = torch.zeros(64, 64, dtype=torch.bfloat16, device=gpu)
+    b = torch.zeros(1, 64, 64, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(ValueError):
+        K.grouped_gemm_bf16_impl(a, b, None, tile=64)

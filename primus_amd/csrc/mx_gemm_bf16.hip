@@ -18,8 +18,8 @@
 // which hands every lane four consecutive contraction elements of its own column.  Measured lane mapping of that
 // read: inside each block of 16 lanes, lane 4 a + e receives element e of the 8-byte pieces addressed by lanes a,
 // a + 4, a + 8, a + 12 (in this order).  16-byte pieces are XOR-swizzled on the global side so that both kinds of
-// read are spread over the LDS banks.  The tile list is derived from group_lens by every workgroup; the grid is sized
-// for the largest tile count the sizes allow and surplus workgroups leave at once.
+// read are spread over the LDS banks.  The tile list is derived from group_lens by every workgroup; the workgroups
+// are persistent and walk it in rounds.
 #include "mx_device.h"
 
 #include <type_traits>
@@ -69,6 +69,13 @@ __device__ __forceinline__ void bf_dma16(v4i rsrc, uint32_t lds_off, uint32_t vo
 
 constexpr int bf16_lds_bytes(int bm, int nst) {
     return nst * (bm * 64 + BF_B_BYTES) + (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
+}
+// number of gaps g in [first, m) that are not wave ph's request gaps (g % 4 == ph): the index of the fragment read
+// that the gap behind MFMA m holds
+constexpr int bf_read_index(int m, int first, int ph) {
+    int n = 0;
+    for (int g = first; g < m; ++g) n += (g & 3) != ph;
+    return n;
 }
 template <int N>
 __device__ __forceinline__ void bf_wait_vm() {
@@ -121,11 +128,16 @@ __global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_ke
     const int tiles_n = (int)((p.n + BF_BN - 1) / BF_BN);
     const int tiles_m = WGRAD ? (int)((p.m + BF_BM - 1) / BF_BM) : pre_tiles[G];
     const int total_tiles = WGRAD ? G * tiles_m * tiles_n : tiles_m * tiles_n;
-    // consecutive workgroup ids land on different XCDs: give every XCD a contiguous run of the tile order
+    // Persistent workgroups (one per CU for the 256-row tile, two for the 128-row one) walk the tile order in rounds:
+    // every workgroup starts its tile of a round at the same time and all tiles of a launch have the same contraction
+    // length, so the 32 tiles an XCD works on stay within a few K slots of each other and share their operand panels
+    // through that XCD's L2 (with one workgroup per tile, started whenever a CU fell free, the tiles of an XCD drifted
+    // apart and the launch filled the L2s with 1.75 times the bytes).  Consecutive workgroup ids land on different XCDs:
+    // XCD x takes the x-th run of gridDim / 8 tiles of every round.
     const int nwg = gridDim.x;
-    int tile = (nwg & 7) ? (int)blockIdx.x : ((int)(blockIdx.x & 7) * (nwg >> 3) + (int)(blockIdx.x >> 3));
-    if (tile >= total_tiles) return;
-
+    const int vwg = (nwg & 7) ? (int)blockIdx.x : ((int)(blockIdx.x & 7) * (nwg >> 3) + (int)(blockIdx.x >> 3));
+  for (int tile_id = vwg; tile_id < total_tiles; tile_id += nwg) {
+    int tile = tile_id;
     int grp = 0;
     if (WGRAD) {
         grp = tile / (tiles_m * tiles_n);
@@ -304,11 +316,23 @@ __global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_ke
 #pragma unroll
             for (int i = 0; i < 4; ++i) fa0[i] = read_a(smem, i, 0);
 #define BF_PIN __builtin_amdgcn_sched_barrier(0)
-            // MFMA number M = 4 j + i of a half; behind it, wave PH issues request (M - PH) / 4 of the half
-#define BF_STEP(FA, FB, M, R, VO, SO, OFF)                                                                                \
+            // The gap behind MFMA number M = 4 j + i of a half holds at most one other instruction of weight: wave PH's
+            // load request (M - PH) / 4 of the half when M % 4 == PH, else the next fragment read (eight per half,
+            // in the order the next half's MFMAs need them: b0, a0 .. a3, b1 .. b3), from gap FIRST on.
+            auto rd = [&](auto r_tag, v8bf (&fa)[4], v8bf (&fb)[4], uint8_t* pa, uint8_t* pb, int ks) __attribute__((always_inline)) {
+                constexpr int R = decltype(r_tag)::value;
+                if constexpr (R == 0) fb[0] = read_b(pb, 0, ks);
+                else if constexpr (R <= 4) fa[R - 1] = read_a(pa, R - 1, ks);
+                else fb[R - 4] = read_b(pb, R - 4, ks);
+            };
+#define BF_STEP(FA, FB, M, R, VO, SO, OFF, RFA, RFB, PA, PB, KS, FIRST)                                                    \
     acc[(M) & 3][(M) >> 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[(M) >> 2], FA[(M) & 3], acc[(M) & 3][(M) >> 2], 0, 0, 0); \
     if constexpr (((M) & 3) == PH) bf_dma16(R, in_base + (OFF) + ((M) >> 2) * 4096, VO[(M) >> 2], SO);                       \
+    else if constexpr ((M) >= (FIRST) && bf_read_index(M, FIRST, PH) < 8)                                                  \
+        rd(std::integral_constant<int, bf_read_index(M, FIRST, PH)>{}, RFA, RFB, PA, PB, KS);                              \
     BF_PIN
+#define BF_HALF0(M) BF_STEP(fa0, fb0, M, ra, va, in_sa, 0, fa1, fb1, sa, sb, 1, 0)
+#define BF_HALF1(M) BF_STEP(fa1, fb1, M, rb, vb, in_sb, BF_A_BYTES, fa0, fb0, na, nb, 0, 4)
             int stage = 0;                            // stage of slot s; slot s + 3 goes into the stage in front of it
             for (int s = 0; s < nslots; ++s) {
                 uint8_t* sa = smem + stage * BF_STAGE;
@@ -316,23 +340,14 @@ __global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_ke
                 const int in_slot = s + NST - 1 < last ? s + NST - 1 : last;
                 const uint32_t in_base = smem_base + (uint32_t)((stage == 0 ? NST - 1 : stage - 1) * BF_STAGE) + (uint32_t)(w * 1024);
                 const uint32_t in_sa = (uint32_t)in_slot * a_step, in_sb = (uint32_t)in_slot * b_step;
-                // ---- half 0 multiplies, half 1 is read; requests: the a rows of slot s + 3 ----
-                fb1[0] = read_b(sb, 0, 1); BF_STEP(fa0, fb0, 0, ra, va, in_sa, 0);
-                fa1[0] = read_a(sa, 0, 1); BF_STEP(fa0, fb0, 1, ra, va, in_sa, 0);
-                fa1[1] = read_a(sa, 1, 1); BF_STEP(fa0, fb0, 2, ra, va, in_sa, 0);
-                fa1[2] = read_a(sa, 2, 1); BF_STEP(fa0, fb0, 3, ra, va, in_sa, 0);
-                fa1[3] = read_a(sa, 3, 1); BF_STEP(fa0, fb0, 4, ra, va, in_sa, 0);
-                fb1[1] = read_b(sb, 1, 1); BF_STEP(fa0, fb0, 5, ra, va, in_sa, 0);
-                fb1[2] = read_b(sb, 2, 1); BF_STEP(fa0, fb0, 6, ra, va, in_sa, 0);
-                fb1[3] = read_b(sb, 3, 1); BF_STEP(fa0, fb0, 7, ra, va, in_sa, 0);
-                BF_STEP(fa0, fb0, 8, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 9, ra, va, in_sa, 0);
-                BF_STEP(fa0, fb0, 10, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 11, ra, va, in_sa, 0);
-                BF_STEP(fa0, fb0, 12, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 13, ra, va, in_sa, 0);
-                BF_STEP(fa0, fb0, 14, ra, va, in_sa, 0); BF_STEP(fa0, fb0, 15, ra, va, in_sa, 0);
-                // ---- half 1 multiplies; behind the barrier the next slot's half 0 is read; requests: the b rows ----
-                BF_STEP(fa1, fb1, 0, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 1, rb, vb, in_sb, BF_A_BYTES);
-                BF_STEP(fa1, fb1, 2, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 3, rb, vb, in_sb, BF_A_BYTES);
                 stage = stage == NST - 1 ? 0 : stage + 1;
+                uint8_t* na = smem + stage * BF_STAGE;
+                uint8_t* nb = na + BF_A_BYTES;
+                // ---- half 0 multiplies, half 1 is read; requests: the a rows of slot s + 3 ----
+                BF_HALF0(0); BF_HALF0(1); BF_HALF0(2); BF_HALF0(3); BF_HALF0(4); BF_HALF0(5); BF_HALF0(6); BF_HALF0(7);
+                BF_HALF0(8); BF_HALF0(9); BF_HALF0(10); BF_HALF0(11); BF_HALF0(12); BF_HALF0(13); BF_HALF0(14); BF_HALF0(15);
+                // ---- half 1 multiplies; behind the barrier the next slot's half 0 is read; requests: the b rows ----
+                BF_HALF1(0); BF_HALF1(1); BF_HALF1(2); BF_HALF1(3);
                 // slot s + 1 has landed when only slot s + 2, the a rows of slot s + 3 and its first b request are outstanding
                 // (waves of a ragged tile that run the generic loop below meet the same barriers: one per slot)
                 if (s + 1 < nslots) {
@@ -340,19 +355,11 @@ __global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_ke
                     __syncthreads();   // slot s + 1 is in LDS for every wave; every wave holds its fragments of slot s
                 }
                 BF_PIN;
-                uint8_t* na = smem + stage * BF_STAGE;
-                uint8_t* nb = na + BF_A_BYTES;
-                fb0[0] = read_b(nb, 0, 0); BF_STEP(fa1, fb1, 4, rb, vb, in_sb, BF_A_BYTES);
-                fa0[0] = read_a(na, 0, 0); BF_STEP(fa1, fb1, 5, rb, vb, in_sb, BF_A_BYTES);
-                fa0[1] = read_a(na, 1, 0); BF_STEP(fa1, fb1, 6, rb, vb, in_sb, BF_A_BYTES);
-                fa0[2] = read_a(na, 2, 0); BF_STEP(fa1, fb1, 7, rb, vb, in_sb, BF_A_BYTES);
-                fa0[3] = read_a(na, 3, 0); BF_STEP(fa1, fb1, 8, rb, vb, in_sb, BF_A_BYTES);
-                fb0[1] = read_b(nb, 1, 0); BF_STEP(fa1, fb1, 9, rb, vb, in_sb, BF_A_BYTES);
-                fb0[2] = read_b(nb, 2, 0); BF_STEP(fa1, fb1, 10, rb, vb, in_sb, BF_A_BYTES);
-                fb0[3] = read_b(nb, 3, 0); BF_STEP(fa1, fb1, 11, rb, vb, in_sb, BF_A_BYTES);
-                BF_STEP(fa1, fb1, 12, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 13, rb, vb, in_sb, BF_A_BYTES);
-                BF_STEP(fa1, fb1, 14, rb, vb, in_sb, BF_A_BYTES); BF_STEP(fa1, fb1, 15, rb, vb, in_sb, BF_A_BYTES);
+                BF_HALF1(4); BF_HALF1(5); BF_HALF1(6); BF_HALF1(7); BF_HALF1(8); BF_HALF1(9);
+                BF_HALF1(10); BF_HALF1(11); BF_HALF1(12); BF_HALF1(13); BF_HALF1(14); BF_HALF1(15);
             }
+#undef BF_HALF0
+#undef BF_HALF1
 #undef BF_STEP
 #undef BF_PIN
         };
@@ -456,6 +463,18 @@ __global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_ke
             }
         }
     }
+    __syncthreads();         // every wave has left the staging area: the next tile's requests may overwrite it
+  }
+}
+
+static int bf16_num_cus(int dev) {
+    static std::atomic<int> cached[64];
+    int v = cached[dev & 63].load(std::memory_order_relaxed);
+    if (v) return v;
+    hipDeviceProp_t pr;
+    if (hipGetDeviceProperties(&pr, dev) != hipSuccess || pr.multiProcessorCount <= 0) return 256;
+    cached[dev & 63].store(pr.multiProcessorCount, std::memory_order_relaxed);
+    return pr.multiProcessorCount;
 }
 
 template <int BM, int NST, bool A_T, bool B_T, bool WGRAD, bool ACCUM>
@@ -471,8 +490,12 @@ static int launch_bf16(const Bf16Args& a, int64_t max_tiles, hipStream_t st) {
         attr_set[dev & 63].store(true, std::memory_order_release);
     }
     if (max_tiles <= 0) return MXL_OK;
-    const int64_t grid = (max_tiles + 7) / 8 * 8;
-    if (grid > 0x7FFFFFFF) return MXL_EINVAL;
+    if (max_tiles > 0x7FFFFFFF) return MXL_EINVAL;
+    // persistent: as many workgroups as the device holds at once (a multiple of 8, one share per XCD), fewer for few tiles
+    int64_t grid = (int64_t)bf16_num_cus(dev) * (BM == 256 ? 1 : 2);
+    grid = grid / 8 * 8;
+    if (grid < 8) grid = 8;
+    if ((max_tiles + 7) / 8 * 8 < grid) grid = (max_tiles + 7) / 8 * 8;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(BF_THREADS), lds, st, a);
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }

@@ -258,10 +258,9 @@ int mxl_grouped_gemm_wgrad_ex(const void* a_codes, const void* a_scales, int a_f
  *     p[t, m_out] * q[t, n_out]  (p = dy, q = x gives the [n, k] weight gradient); a group without tokens yields zeros.
  *     bf16 output, or with MXL_BF_ACCUM_F32 c is float32 and the result is ADDED to it (the main_grad fusion).
  *     Requires m_out % 8 == 0, n_out % 8 == 0; an operand stays below 4 GiB.
- * Output tiles are 256 columns wide and 256 or 128 rows high.  Without a tile flag the library picks by the average
- * rows per group, total_m / num_groups (256 rows from 384 on for forward / dgrad, from 1024 on for the weight
- * gradient, whose contraction runs over a group's rows); MXL_BF_TILE_128 / MXL_BF_TILE_256 state the choice (a caller
- * who knows its groups are few and long, or many and short).  The result does not depend on the tile height beyond fp32 summation order -- it is the
+ * Output tiles are 256 columns wide and 256 or 128 rows high.  Without a tile flag the library picks: forward / dgrad
+ * 256 rows when total_m / num_groups is at least 256, else 128; the weight gradient 128.  MXL_BF_TILE_128 /
+ * MXL_BF_TILE_256 state the choice (a caller who knows its groups are few and long, or many and short).  The result does not depend on the tile height beyond fp32 summation order -- it is the
  * same: every output element adds its products in the same order in both. */
 #define MXL_BF_B_KN 1u
 #define MXL_BF_ACCUM_F32 2u

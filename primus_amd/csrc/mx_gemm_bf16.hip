@@ -501,10 +501,11 @@ static int launch_bf16(const Bf16Args& a, int64_t max_tiles, hipStream_t st) {
 }
 
 // Tile height of a launch: the caller's choice (MXL_BF_TILE_128 / MXL_BF_TILE_256), else from the average number of
-// rows per group -- the counts live on the device, the average is all the host knows.  Measured crossovers: forward /
-// dgrad tiles are cut from a group's rows, and 256-row tiles win from about 400 rows per group on (below, most of a
-// group's last tile is padding); the weight gradient contracts over a group's rows, and the tall tile's longer
-// prologue and epilogue pay off from about 1000 rows per group on.
+// rows per group -- the counts live on the device, the average is all the host knows.  Measured: forward / dgrad
+// tiles are cut from a group's rows, and 256-row tiles win from a few hundred rows per group on (512 rows: +7 %, 4096:
+// +18-24 %; below, most of a group's last tile is padding).  The weight gradient reads both operands through the
+// transposing LDS reads (twice the LDS instructions per MFMA): two workgroups per CU hide that better than one, and the
+// 128-row tile wins at every shape tried (+2 % at 4096 rows per group, +50 % at 512), so it is the default there.
 static bool bf16_tall_tiles(uint32_t flags, int64_t rows_per_group, int64_t threshold) {
     if (flags & MXL_BF_TILE_256) return true;
     if (flags & MXL_BF_TILE_128) return false;
@@ -527,7 +528,7 @@ extern "C" int mxl_grouped_gemm_bf16(const void* a_bf16, const void* b_bf16, voi
     // offsets inside a tile's operand rows are 32-bit
     if (256 * k * 2 >= ((int64_t)1 << 31) || k * n * 2 >= ((int64_t)1 << 32)) return MXL_EINVAL;
     Bf16Args a{(const uint8_t*)a_bf16, (const uint8_t*)b_bf16, c_bf16, group_lens, num_groups, total_m, 0, n, k};
-    const bool tall = bf16_tall_tiles(flags, total_m / num_groups, 384);
+    const bool tall = bf16_tall_tiles(flags, total_m / num_groups, 256);
     const int64_t max_tiles = (total_m / (tall ? 256 : 128) + num_groups) * ((n + BF_BN - 1) / BF_BN);
     hipStream_t st = (hipStream_t)stream;
     if (flags & MXL_BF_B_KN)
@@ -548,7 +549,7 @@ extern "C" int mxl_grouped_gemm_bf16_wgrad(const void* p_bf16, const void* q_bf1
     if (total_m * m_out * 2 >= ((int64_t)1 << 32) || total_m * n_out * 2 >= ((int64_t)1 << 32)) return MXL_EINVAL;
     Bf16Args a{(const uint8_t*)p_bf16, (const uint8_t*)q_bf16, c, group_lens, num_groups, total_m, m_out, n_out, 0};
     // the tiles are cut from the [m_out, n_out] matrix of every group; the contraction runs over the group's tokens
-    const bool tall = bf16_tall_tiles(flags, total_m / num_groups, 1024);
+    const bool tall = bf16_tall_tiles(flags, total_m / num_groups, INT64_MAX);
     const int bm = tall ? 256 : 128;
     const int64_t max_tiles = (int64_t)num_groups * ((m_out + bm - 1) / bm) * ((n_out + BF_BN - 1) / BF_BN);
     hipStream_t st = (hipStream_t)stream;

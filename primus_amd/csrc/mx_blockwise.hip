@@ -397,10 +397,12 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
         else if (f_any) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
         __syncthreads();       // block kb and its factors are in LDS for every wave; every wave has left block kb - 1
-        if (kb + 2 < k1) {
-            issue(kb + 2, st2);
-            issue_fac(kb + 2, st2);
-        }
+        // the requests of block kb + 2 go out one behind each MFMA of this block (six operand rounds, then the
+        // factors): all at once, the 8 waves' 56 requests queue at the CU's address unit for ~900 clocks with every
+        // wave waiting behind its own
+        const bool more = kb + 2 < k1;
+        const uint32_t in_koff = (uint32_t)__builtin_amdgcn_readfirstlane((kb + 2) * BW);
+        const uint32_t in_base = wave_lds + (uint32_t)(st2 * BWG_STAGE);
         const float* fac = fac_base + st * (BWG_BM + BWG_BN);
         const uint8_t* sa_ = bw_smem + st * BWG_STAGE;
         const uint8_t* sb_ = sa_ + BWG_A;
@@ -429,6 +431,12 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
                     // the b fragment is the first operand: a lane ends up with 4 consecutive output columns
                     part[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], ks == 0 ? zero : part[i][j], CB, BL, 0,
                                                                                127, 0, 127);
+                    const int mi = 4 * ks + 2 * i + j;      // (a constant after unrolling)
+                    if (more) {
+                        if (mi < 2) bw_dma16(ra, in_base + mi * 8192, ld_voff, in_koff + mi * round_bytes);
+                        else if (mi < 6) bw_dma16(rb, in_base + BWG_A + (mi - 2) * 8192, ld_voff, in_koff + (mi - 2) * round_bytes);
+                        else if (mi == 6) issue_fac(kb + 2, st2);
+                    }
                 }
         }
         // acc += part * (sa[row] * sb[col]): lane (lr, g), register e = 4 q + r of tile (i, j) is row i * 32 + lr,

@@ -885,15 +885,35 @@ def _alpha_ok(*alphas):
     _require_cuda(*alphas)
 
 
-def gemm_tw_nt_impl(a, a_unit, a_scale_inv, b, b_unit, b_scale_inv, group_lens=None, kchunk: bool = False) -> torch.Tensor:
+def gemm_tw_nt_impl(a, a_unit, a_scale_inv, b, b_unit, b_scale_inv, group_lens=None, kchunk: bool = False,
+                    b_transposed_n: Optional[int] = None) -> torch.Tensor:
     """``c = (a . b^T) * a_scale_inv * b_scale_inv`` on tensor-wise scaled codes, dense (``group_lens`` None,
     ``b [n, k]``) or grouped (``b [G, n, k]``); layouts and the unit block scales as the quantisers above
-    return them (``b_unit`` is ``[n, k/32]`` or ``[G, n, k/32]``).  The contraction dim must be padded to 128."""
+    return them (``b_unit`` is ``[n, k/32]`` or ``[G, n, k/32]``).  The contraction dim must be padded to 128.
+    ``b_transposed_n`` (K-step-major E4M3 weights): ``b`` holds the ROW-WISE codes of the weight ``[G, k, n]`` whose
+    transpose this GEMM multiplies by (its dgrad: one scale per tensor, so the transposed copy would be the same
+    codes transposed), ``[n_ld / 64, G * k, 64]``; the value is ``n``, the number of output columns."""
     _require_cuda(a, a_unit, b, b_unit, group_lens)
     _alpha_ok(a_scale_inv, b_scale_inv)
     G = _check_group_lens(group_lens, a.device)
     groups = max(G, 1)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
+    if b_transposed_n is not None:
+        if _layout(kchunk) != LAYOUT_KSTEP:
+            raise ValueError("b_transposed_n needs K-step-major operands")
+        total_m, k = _chunked_dims(a, a_fmt, kchunk)
+        bt_rows, n_ld = _chunked_dims(b, b_fmt, kchunk)
+        n = int(b_transposed_n)
+        if bt_rows != groups * k or _round_up(n, KCHUNK) != n_ld:
+            raise ValueError("b_transposed_n: b must be the K-step-major row-wise codes of a [num_groups, k, n] weight")
+        c = torch.empty((total_m, n), dtype=torch.bfloat16, device=a.device)
+        with _hooked("grouped_gemm_nt" if G else "gemm_nt", m=total_m, n=n, k=k):
+            rc = _lib.load().mxl_grouped_gemm_nt_scaled(
+                _ptr(a), _ptr(a_unit), a_fmt, _ptr(b), None, b_fmt, _ptr(c), _ptr(group_lens), groups, total_m, n, k,
+                _ptr(a_scale_inv), _ptr(b_scale_inv), _lib.GF_KSTEP | _lib.GF_B_TRANSPOSED, _stream(),
+            )
+        _lib.check(rc, "mxl_grouped_gemm_nt_scaled")
+        return c
     kstep = _paneled(kchunk)
     if kchunk:
         total_m, k = _chunked_dims(a, a_fmt, kchunk)

@@ -357,17 +357,25 @@ class _TWLinearFunction(torch.autograd.Function):
                 raise ValueError("the forward weight copy must be a tensor-wise scaled copy quantised along axis=-1")
             w_row, w_ru, w_si = _cached_codes(b, kc), _cached_scales(b, kc), b.tensor_scale_inv
             w_col = w_cu = None
+            bt = False
             if need_dgrad:
                 if b_t is not None:
                     w_col, w_cu = _cached_codes(b_t, kc), _cached_scales(b_t, kc)
                 else:
                     w_col, w_cu = _transposed_cache(b, kc)
         else:
+            # one scale per tensor: the transposed copy would be the row-wise codes transposed, so on the ring kernel
+            # dgrad reads the row-wise codes through its transposing LDS reads and no second copy is written
+            bt = (need_dgrad and _dgrad_reads_rowwise and kc == K.LAYOUT_KSTEP and fwd_fmt == _lib.FMT_E4M3
+                  and b.shape[-2] % K.GEMM_K_ALIGN == 0 and b.shape[-1] % K.GEMM_K_ALIGN == 0)
             w_row, w_ru, w_col, w_cu, w_si = K.quantize_weight_tensorwise_impl(
-                b.detach(), fwd_fmt, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
+                b.detach(), fwd_fmt, rowwise=True, colwise=need_dgrad and not bt, pad_to=K.GEMM_K_ALIGN, kchunk=kc)
+            if bt:
+                w_col, w_cu = w_row, w_ru
         y = K.gemm_tw_nt_impl(a_row, a_ru, a_si, w_row, w_ru, w_si, group_lens, kchunk=kc)
         ctx.save_for_backward(a_col, a_cu, a_si, w_col, w_cu, w_si, group_lens)
         ctx.cfg = (bwd_fmt, a.shape[0], need_dgrad, need_wgrad, tuple(b.shape), kc)
+        ctx.b_transposed = bt
         ctx.accum = accum
         return y
 
@@ -387,7 +395,8 @@ class _TWLinearFunction(torch.autograd.Function):
             side = _side_stream(dy.device)
             side.wait_stream(main)
         if need_dgrad:
-            grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc)
+            grad_a = K.gemm_tw_nt_impl(d_row, d_ru, d_si, w_col, w_cu, w_si, group_lens, kchunk=kc,
+                                       b_transposed_n=w_shape[-1] if ctx.b_transposed else None)
         if need_wgrad:
             target = ctx.accum[0] if ctx.accum is not None else None
             fused = _fusable(target) and kc != K.LAYOUT_ROWMAJOR

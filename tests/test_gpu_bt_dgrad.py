@@ -48,11 +48,15 @@ def test_dgrad_from_rowwise_codes_matches_the_transposed_copy(gpu, lens, n, k):
 
 
 @pytest.mark.parametrize("grouped", [True, False])
-def test_operator_gradients_do_not_depend_on_the_route(gpu, grouped):
+@pytest.mark.parametrize("recipe", ["mx", "tensorwise_e4m3", "tensorwise_hybrid"])
+def test_operator_gradients_do_not_depend_on_the_route(gpu, grouped, recipe):
     import primus_amd.pytorch as turbo
     from primus_amd.pytorch.core import Float8QuantConfig, Format, ScaleDtype, ScalingGranularity
 
-    cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0, block_size=32)
+    if recipe == "mx":
+        cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, scale_dtype=ScaleDtype.E8M0, block_size=32)
+    else:
+        cfg = Float8QuantConfig(format=Format.E4M3 if recipe.endswith("e4m3") else Format.HYBRID, granularity=ScalingGranularity.TENSORWISE)
     lens = [200, 0, 312] if grouped else [512]
     G, m, n, k = len(lens), sum(lens), 384, 256
     gen = torch.Generator().manual_seed(17)

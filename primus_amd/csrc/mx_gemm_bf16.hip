@@ -67,6 +67,16 @@ __device__ __forceinline__ void bf_dma16(v4i rsrc, uint32_t lds_off, uint32_t vo
                  : "memory");
 }
 
+// the same with the LDS address formed in the request's own scalar instruction (base + constant): two scalar
+// instructions per request instead of five
+template <int LDS_IMM>
+__device__ __forceinline__ void bf_dma16_at(v4i rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
+                 :
+                 : "s"(lds_base), "n"(LDS_IMM), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "scc");
+}
+
 constexpr int bf16_lds_bytes(int bm, int nst) {
     return nst * (bm * 64 + BF_B_BYTES) + (MXL_MAX_GROUPS + 2) * 4 + (MXL_MAX_GROUPS + 2) * 8;
 }
@@ -327,7 +337,7 @@ __global__ __launch_bounds__(BF_THREADS, BF_BM == 256 ? 1 : 2) void bf16_gemm_ke
             };
 #define BF_STEP(FA, FB, M, R, VO, SO, OFF, RFA, RFB, PA, PB, KS, FIRST)                                                    \
     acc[(M) & 3][(M) >> 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[(M) >> 2], FA[(M) & 3], acc[(M) & 3][(M) >> 2], 0, 0, 0); \
-    if constexpr (((M) & 3) == PH) bf_dma16(R, in_base + (OFF) + ((M) >> 2) * 4096, VO[(M) >> 2], SO);                       \
+    if constexpr (((M) & 3) == PH) bf_dma16_at<(OFF) + ((M) >> 2) * 4096>(R, in_base, VO[(M) >> 2], SO);                     \
     else if constexpr ((M) >= (FIRST) && bf_read_index(M, FIRST, PH) < 8)                                                  \
         rd(std::integral_constant<int, bf_read_index(M, FIRST, PH)>{}, RFA, RFB, PA, PB, KS);                              \
     BF_PIN

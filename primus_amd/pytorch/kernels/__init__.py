@@ -1213,12 +1213,14 @@ def _bw_scales(t, shape, what):
         raise ValueError(f"{what} must be contiguous float32 {tuple(shape)}")
 
 
-def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv, group_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv, group_lens: Optional[torch.Tensor] = None,
+                           b_rows_per_scale: Optional[int] = None) -> torch.Tensor:
     """``gemm_fp8_impl`` / ``grouped_gemm_fp8_impl`` with ``granularity=BLOCKWISE`` in NT form
     (primus_turbo_float8_local.py:1022-1033, zbpp_gemm.py:608-630):
     ``c[m, n] = sum_kb a_scale_inv[m, kb] * b_scale_inv[n or n / 128, kb] * (a[m, kb] . b[n, kb])``, bf16.
     Dense: ``b [n, k]``, ``b_scale_inv`` with one row per row of ``b`` (an activation copy) or one per 128 rows (a
-    weight).  Grouped: the rows of ``a`` are split by ``group_lens``, ``b [G, n, k]``, ``b_scale_inv [G, n / 128, k / 128]``."""
+    weight).  Grouped: the rows of ``a`` are split by ``group_lens``, ``b [G, n, k]``, ``b_scale_inv [G, n / 128, k / 128]``.
+    ``b_rows_per_scale`` (dense): 1 or 128, which of the two forms ``b_scale_inv`` has; None reads it off its shape."""
     _require_cuda(a, a_scale_inv, b, b_scale_inv, group_lens)
     G = _check_group_lens(group_lens, a.device)
     m, k = a.shape
@@ -1244,7 +1246,9 @@ def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv, group_lens: Optional[
         raise ValueError("dense blockwise GEMM expects b [n, k]")
     if b_scale_inv.dtype != torch.float32 or not b_scale_inv.is_contiguous() or tuple(b_scale_inv.shape) not in ((n, kb), (n // BW_BLOCK, kb)):
         raise ValueError("b_scale_inv must be contiguous float32 [n, k / 128] or [n / 128, k / 128]")
-    per = 1 if b_scale_inv.shape[0] == n else BW_BLOCK
+    per = (1 if b_scale_inv.shape[0] == n else BW_BLOCK) if b_rows_per_scale is None else int(b_rows_per_scale)
+    if per not in (1, BW_BLOCK) or b_scale_inv.shape[0] != n // per:
+        raise ValueError("b_rows_per_scale must be 1 or 128 and match the rows of b_scale_inv")
     with _hooked("gemm_blockwise_nt", m=m, n=n, k=k):
         rc = lib.mxl_gemm_nt_blockwise(_ptr(a), _ptr(a_scale_inv), _fp8_fmt_of(a), _ptr(b), _ptr(b_scale_inv),
                                        _fp8_fmt_of(b), per, _ptr(c), m, n, k, _stream())

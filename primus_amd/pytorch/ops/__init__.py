@@ -429,7 +429,7 @@ class _BWLinearFunction(torch.autograd.Function):
     def forward(ctx, a, b, group_lens, fwd_fmt, bwd_fmt, accum=None):
         a_row, a_s, _, _ = K.quantize_blockwise_impl(a, fwd_fmt, rowwise=True, colwise=False)
         w_row, w_s, _, _ = K.quantize_blockwise_weight_impl(b.detach(), fwd_fmt, rowwise=True, colwise=False)
-        y = K.gemm_blockwise_nt_impl(a_row, a_s, w_row, w_s, group_lens)
+        y = K.gemm_blockwise_nt_impl(a_row, a_s, w_row, w_s, group_lens, b_rows_per_scale=None if group_lens is not None else 128)
         ctx.save_for_backward(a, b, group_lens)
         ctx.cfg = (bwd_fmt, a.requires_grad, b.requires_grad)
         ctx.accum = accum
@@ -447,11 +447,11 @@ class _BWLinearFunction(torch.autograd.Function):
         grad_a = grad_b = None
         if need_dgrad:
             _, _, w_col, w_cs = K.quantize_blockwise_weight_impl(b.detach(), bwd_fmt, rowwise=False, colwise=True)
-            grad_a = K.gemm_blockwise_nt_impl(d_row, d_s, w_col, w_cs, group_lens)
+            grad_a = K.gemm_blockwise_nt_impl(d_row, d_s, w_col, w_cs, group_lens, b_rows_per_scale=None if group_lens is not None else 128)
         if need_wgrad:
             _, _, a_col, a_cs = K.quantize_blockwise_impl(a.detach(), bwd_fmt, rowwise=False, colwise=True, group_lens=group_lens)
             if group_lens is None:
-                grad_b = K.gemm_blockwise_nt_impl(d_col, d_cs, a_col, a_cs)
+                grad_b = K.gemm_blockwise_nt_impl(d_col, d_cs, a_col, a_cs, b_rows_per_scale=1)
             else:
                 grad_b = K.grouped_gemm_blockwise_wgrad_impl(d_col, d_cs, a_col, a_cs, group_lens, a.shape[0])
             grad_b = _finish_wgrad(grad_b, ctx.accum, False, tuple(b.shape))

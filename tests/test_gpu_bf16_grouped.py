@@ -212,3 +212,29 @@ def test_tile_flags_are_validated(gpu):
     b = torch.zeros(1, 64, 64, dtype=torch.bfloat16, device=gpu)
     with pytest.raises(ValueError):
         K.grouped_gemm_bf16_impl(a, b, None, tile=64)
+
+
+@pytest.mark.parametrize("tile", [128, 256])
+def test_many_rounds_of_tiles_are_exact_on_integers(gpu, tile):
+    """More tiles than persistent workgroups (several rounds per workgroup, ragged and empty groups in between):
+    integer operands make every partial sum exact, so forward, dgrad and wgrad equal the fp32 matmul bit for bit."""
+    from primus_amd.pytorch import kernels as K
+
+    lens = [3000, 0, 517, 4100, 1, 2600, 255, 9527]
+    n, k = 2048, 256
+    G, m = len(lens), sum(lens)
+    gen = torch.Generator().manual_seed(77)
+    a = torch.randint(-3, 4, (m, k), generator=gen).bfloat16().to(gpu)
+    b = torch.randint(-2, 3, (G, n, k), generator=gen).bfloat16().to(gpu)
+    dy = torch.randint(-2, 3, (m, n), generator=gen).bfloat16().to(gpu)
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    y = K.grouped_gemm_bf16_impl(a, b, gl, tile=tile)
+    dx = K.grouped_gemm_bf16_impl(dy, b, gl, b_kn=True, tile=tile)
+    dw = K.grouped_gemm_bf16_wgrad_impl(dy, a, gl, tile=tile)
+    assert torch.equal(y, _ref(a, b, lens, True).bfloat16())
+    assert torch.equal(dx, _ref(dy, b, lens, False).bfloat16())
+    off = 0
+    for g, ln in enumerate(lens):
+        want = (dy[off:off + ln].float().t() @ a[off:off + ln].float()).bfloat16()
+        assert torch.equal(dw[g], want), g
+        off += ln

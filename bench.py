@@ -250,7 +250,7 @@ def cpu_baseline(spec, lens, layers, sample_div=16):
     }
 
 
-def gemm_calibration(fp4_weights, dev, fp4_acts=False):
+def gemm_calibration(fp4_weights, dev, fp4_acts=False, bf16=False):
     """What this board's matrix cores deliver, measured in the same process, to read the GEMM figures against
     (the published peak assumes the 2.4 GHz boost clock; under load the board sits at its power limit):
     the library's register-only loop of the GEMM's own scaled MFMA (no memory traffic: the ceiling of any GEMM here),
@@ -283,6 +283,20 @@ def gemm_calibration(fp4_weights, dev, fp4_acts=False):
         torch.cuda.synchronize()
         return round(n * flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
 
+    if bf16:
+        # the unquantised workload: the register-only loop of the bf16 MFMA and torch's vendor dense bf16 GEMM
+        iters = 8192
+        flops = float(lib.mxl_calibrate_mfma_bf16_flops(iters))
+        out["mfma_only_loop_bf16_TFLOP/s"] = rate(lambda: _lib.check(lib.mxl_calibrate_mfma_bf16(iters, st), "mxl_calibrate_mfma_bf16"), flops)
+        out["mfma_only_loop"] = "mxl_calibrate_mfma_bf16: 256 workgroups x 4 waves, 32 MFMAs 32x32x16 bf16 per K slot on register operands, no memory traffic"
+        M, N, Kd = 32768, 28672, 4096
+        out["dense_gemm_shape_mnk"] = [M, N, Kd]
+        x = torch.randn(M, Kd, device=dev).bfloat16()
+        w = (torch.randn(N, Kd, device=dev) * 0.02).bfloat16()
+        from primus_amd.pytorch import kernels as K
+        out["this_library_bf16_one_group_TFLOP/s"] = rate(lambda: K.grouped_gemm_bf16_impl(x, w, None), 2.0 * M * N * Kd)
+        out["torch_matmul_bf16_TFLOP/s"] = rate(lambda: torch.matmul(x, w.t()), 2.0 * M * N * Kd)
+        return out
     iters = 4096
     flops = float(lib.mxl_calibrate_mfma_flops(iters))
     for name, (fa, fb) in (("fp8_x_fp8", (_lib.FMT_E4M3, _lib.FMT_E4M3)),) + ((("fp8_x_fp4", (_lib.FMT_E4M3, _lib.FMT_E2M1)),) if fp4_weights and not fp4_acts else ()) \
@@ -455,7 +469,7 @@ def main():
     torch.cuda.set_device(dev)
     spec = WORKLOADS[args.workload]
     if args.calibration_only:
-        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev, bool(spec.get("act_fp4"))), "quantizer_traffic_twin": quantizer_twin(dev)}))
+        print(json.dumps({"mfma_calibration": gemm_calibration(spec["fp4"], dev, bool(spec.get("act_fp4")), bool(spec.get("bf16"))), "quantizer_traffic_twin": quantizer_twin(dev)}))
         return
     lens = route(spec)
     G, M = spec["G"], sum(lens)
@@ -675,8 +689,8 @@ def main():
     if not args.no_gemm_calibration:
         out["hbm_stream_calibration"]["quantizer_traffic_twin"] = quantizer_twin(dev)
     if not args.no_gemm_calibration:
-        out["mfma_calibration"] = cal = gemm_calibration(spec["fp4"], dev, act_fp4)
-        ceiling = cal.get("mfma_only_loop_fp4_x_fp4_TFLOP/s" if act_fp4 else
+        out["mfma_calibration"] = cal = gemm_calibration(spec["fp4"], dev, act_fp4, bool(spec.get("bf16")))
+        ceiling = cal.get("mfma_only_loop_bf16_TFLOP/s" if spec.get("bf16") else "mfma_only_loop_fp4_x_fp4_TFLOP/s" if act_fp4 else
                           "mfma_only_loop_fp8_x_fp4_TFLOP/s" if spec["fp4"] else "mfma_only_loop_fp8_x_fp8_TFLOP/s")
         for name, entry in kernels.items():
             if "gemm" in name and "TFLOP/s" in entry and ceiling:

@@ -231,8 +231,10 @@ int mxl_grouped_gemm_wgrad(const void* a_codes, const void* a_scales, int a_fmt,
  * of the weight, so that no transposed copy of the weight's codes has to be written or cached (the reference keeps a
  * second quantised copy for it, _maybe_create_quantized_weight_buffers, primus_turbo.py:278-358).  Meaningful where a
  * transposed copy is the same codes transposed: 2-D 32 x 32 block scales (mxl_quantize_weight_2d_ex writes the transposed
- * copy's scales alone when q_colT is NULL and s_colT is not) or tensor-wise scaling.  E4M3 weights, E4M3 (or, scaled,
- * E5M2) rows, at most 256 groups; k % 128 == 0.  Bit-identical to the GEMM on the transposed copy. */
+ * copy's scales alone when q_colT is NULL and s_colT is not) or tensor-wise scaling.  E4M3 weights with E4M3 (or,
+ * scaled, E5M2) rows; or E2M1 weights with E2M1 rows, both in 128-element steps (MXL_QF_KSTEP128: b_codes are then
+ * [n_ld / 128][num_groups * k][64 bytes]).  At most 256 groups; k % 128 == 0.  Bit-identical to the GEMM on the
+ * transposed copy. */
 #define MXL_GF_B_TRANSPOSED 8u
 /* mxl_grouped_gemm_nt_ex only, alone (row-major operands): b_codes are E2M1 codes in the pre-shuffled byte order of
  * mxl_shuffle_codes -- what gemm_fp4_impl(..., preshuffled=True) of the reference is handed for its second operand

@@ -655,7 +655,7 @@ constexpr int ring_lds_bytes() {
 }
 
 
-// BT (forward / dgrad of FP8-format operands): b_codes hold the codes of the TRANSPOSED matrices -- [G, k, n] instead of
+// BT (forward / dgrad of FP8-format operands; E2M1 x E2M1 further down): b_codes hold the codes of the TRANSPOSED matrices -- [G, k, n] instead of
 // [G, n, k], K-step-major along n: [n_ld / 64][G * k][64] -- i.e. the row-wise copy of a weight serves its dgrad GEMM
 // and no transposed copy of the codes is ever written.  Valid where transposing the codes is all a transposed copy
 // amounts to: 2-D 32 x 32 block scales (the quantiser's transposed SCALES are still passed as b_scales, they are
@@ -664,9 +664,13 @@ constexpr int ring_lds_bytes() {
 // transposing read ds_read_b64_tr_b8, which hands a lane 8 consecutive contraction bytes of its own column.  Measured
 // lane mapping of that read: inside a block of 16 lanes, lane 8 a + e receives byte e of the 8-byte pieces
 // addressed by lanes a, a + 2, ..., a + 14 (in this order).
+// With both operands E2M1 (128-element steps, 64-byte rows) a plane of the row-wise codes holds 128 output columns, a K
+// step is 128 contraction rows of the tile's two planes (four rounds of 64 rows x 64 bytes), and the fragments come
+// through ds_read_b64_tr_b4, a 16 x 16 nibble transpose inside each block of 16 lanes.
 template <int AFMT, int BFMT, int MODE, bool ALPHA, bool ACCUM = false, bool BT = false>
 __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
-    static_assert(!BT || (MODE == MODE_FWD && AFMT != kFmtE2M1 && BFMT != kFmtE2M1), "transposed weight codes: forward / dgrad, FP8 formats");
+    static_assert(!BT || (MODE == MODE_FWD && ((AFMT != kFmtE2M1 && BFMT != kFmtE2M1) || (AFMT == kFmtE2M1 && BFMT == kFmtE2M1))),
+                  "transposed weight codes: forward / dgrad, both operands FP8 formats or both E2M1");
     // ACCUM (wgrad): p.c is a float32 buffer the result is ADDED to (one workgroup per output tile: no race, and the
     // sum does not depend on any order)
     static_assert(!ACCUM || MODE == MODE_WGRAD, "the accumulating epilogue belongs to the weight-gradient GEMM");
@@ -766,7 +770,8 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     // BT: the rows of b's code array are the contraction index (G * k of them); a K step moves on by 64 rows inside
     // a plane, and the four load rounds of a step are one plane apart
     const int64_t bt_rows = (int64_t)G * p.k;
-    const uint32_t b_cstride = BT ? (uint32_t)(64 * BK) : (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * B_ROW));
+    // (E2M1 x E2M1: a step is 128 contraction rows of a 128-column plane, and a tile's two planes take two rounds each)
+    const uint32_t b_cstride = BT ? (uint32_t)(KS * BK) : (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * B_ROW));
     const uint32_t a_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a_rows_total * 16));
     const uint32_t b_pstride = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b_rows_total * 16));
     // a load round covers 64 consecutive rows = 4 KiB: thread -> (row t / 4, 16-byte piece t % 4); the XOR swizzle of
@@ -782,7 +787,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         va[e] = addr::ring_code_lane(t, e, false);
-        vb[e] = BT ? addr::ring_bt_lane(t, e, bt_rows) : addr::ring_code_lane(t, e, B4);
+        vb[e] = !BT ? addr::ring_code_lane(t, e, B4) : F44 ? addr::ring_bt4_lane(t, e, bt_rows) : addr::ring_bt_lane(t, e, bt_rows);
     }
 
     struct Tile {
@@ -850,7 +855,7 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
         // row past the operand's last one is dropped in the last plane and reads a later plane's rows in the others.
         {
             const addr::Desc da = addr::ring_code_desc(a_rows_total, p.k / KS, a_row0, BK);
-            const addr::Desc db = BT ? addr::ring_bt_desc(bt_rows, (p.n + 127) / 128 * 2, (int64_t)grp * p.k, (int64_t)pid_n * (BN / 64))
+            const addr::Desc db = BT ? addr::ring_bt_desc(bt_rows, (p.n + 127) / 128 * (F44 ? 1 : 2), (int64_t)grp * p.k, (int64_t)pid_n * (F44 ? BN / 128 : BN / 64))
                                      : addr::ring_code_desc(b_rows_total, p.k / KS, b_row0, B_ROW);
             const addr::Desc dsa = addr::ring_panel_desc(a_rows_total, n_panels, a_row0), dsb = addr::ring_panel_desc(b_rows_total, n_panels, b_row0);
             d.ra = make_rsrc(p.a + da.base, da.records);
@@ -924,7 +929,12 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
          F.a[I][4] = hi_.x; F.a[I][5] = hi_.y; F.a[I][6] = hi_.z; F.a[I][7] = hi_.w; } } while (0)
 #define MXL_RD_B(F, J) \
     do { const uint8_t* r_ = sn + A_BYTES + b_frag + (J) * (32 * B_ROW); \
-         if (BT) { \
+         if (BT && F44) { \
+             _Pragma("unroll") for (int q_ = 0; q_ < 2; ++q_) _Pragma("unroll") for (int h_ = 0; h_ < 2; ++h_) { \
+                 const v2i v_ = __builtin_amdgcn_ds_read_tr4_b64_v2i32( \
+                     (__attribute__((address_space(3))) v2i*)((uint8_t*)sn + A_BYTES + (2 * wn + q_) * 4096 + (bt4_off[h_] ^ (16 * (J))))); \
+                 F.b[J][4 * q_ + 2 * h_] = v_[0]; F.b[J][4 * q_ + 2 * h_ + 1] = v_[1]; } \
+         } else if (BT) { \
              uint8_t* t_ = (uint8_t*)sn + A_BYTES + (2 * wn + ((J) >> 1)) * 4096; \
              _Pragma("unroll") for (int q_ = 0; q_ < 2; ++q_) _Pragma("unroll") for (int h_ = 0; h_ < 2; ++h_) { \
                  const v2i v_ = __builtin_amdgcn_ds_read_tr8_b64_v2i32( \
@@ -950,8 +960,20 @@ __global__ __launch_bounds__(GTHREADS) void mx_gemm_ring_kernel(GemmArgs p) {
     // BT: this lane ADDRESSES contraction row 16 g + 8 h + tj (+ 32 for the second half of the step) and the 8-byte
     // piece of its 16-lane block's 16 columns: bt_off[h][J & 1] inside a plane's 64 rows x 64 bytes (same swizzle
     // as the loads: 16-byte piece XOR (row / 4) % 4)
+    // BT, E2M1 x E2M1 (ds_read_b64_tr_b4: in a block of 16 lanes, lane i receives nibble i of the 8-byte pieces
+    // addressed by lanes 0 .. 15, in this order): this lane ADDRESSES contraction row 32 g + 16 h + l % 16 of a round's
+    // 64 rows and the 8-byte half (l / 16) % 2 of a fragment's 16 bytes; fragment J is 16-byte piece J of the 64-byte
+    // row, XOR (row / 4) % 4 as the loads placed it -- the XOR with 16 J is applied at the read.
+    int bt4_off[2] = {0, 0};
+    if (BT && F44) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = 32 * g + 16 * h + (l & 15);
+            bt4_off[h] = row * 64 + 16 * ((row >> 2) & 3) + 8 * ((l >> 4) & 1);
+        }
+    }
     int bt_off[2][2];
-    if (BT) {
+    if (BT && !F44) {
         const int tj = (l & 15) >> 1, ta = l & 1, tblk = (l >> 4) & 1;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
@@ -1427,9 +1449,15 @@ static int dispatch_wgrad_accum_ring(int afmt, int bfmt, const GemmArgs& a, int6
     return MXL_EINVAL;
 }
 
-// forward / dgrad on the row-wise codes of the transposed weight (MXL_GF_B_TRANSPOSED): E4M3 weights, E4M3 or E5M2 rows
+// forward / dgrad on the row-wise codes of the transposed weight (MXL_GF_B_TRANSPOSED): E4M3 weights with E4M3 or E5M2
+// rows, or E2M1 weights with E2M1 rows (128-element steps)
 static int dispatch_gemm_ring_bt(int afmt, int bfmt, const GemmArgs& a, int64_t max_tiles, hipStream_t st) {
-    if (bfmt != MXL_FMT_E4M3 || a.num_groups > RING_MAX_GROUPS) return MXL_EINVAL;
+    if (a.num_groups > RING_MAX_GROUPS) return MXL_EINVAL;
+    if (bfmt == MXL_FMT_E2M1) {
+        if (afmt != MXL_FMT_E2M1 || a.alpha_a != nullptr) return MXL_EINVAL;
+        return launch_gemm_ring<MXL_FMT_E2M1, MXL_FMT_E2M1, MODE_FWD, false, false, true>(a, max_tiles, st);
+    }
+    if (bfmt != MXL_FMT_E4M3) return MXL_EINVAL;
     if (a.alpha_a != nullptr) {
         if (afmt == MXL_FMT_E5M2) return launch_gemm_ring<MXL_FMT_E5M2, MXL_FMT_E4M3, MODE_FWD, true, false, true>(a, max_tiles, st);
         if (afmt == MXL_FMT_E4M3) return launch_gemm_ring<MXL_FMT_E4M3, MXL_FMT_E4M3, MODE_FWD, true, false, true>(a, max_tiles, st);

@@ -93,6 +93,12 @@ MXL_HD Desc ring_bt_desc(int64_t rows_total, int64_t planes, int64_t row0, int64
 MXL_HD uint32_t ring_bt_lane(int t, int e, int64_t rows_total) {
     return ring_code_lane(t, 0, false) + (uint32_t)e * (uint32_t)(rows_total * 64);
 }
+// The transposed read of E2M1 codes stored in 128-element steps (64-byte rows): [planes][rows_total][64] with 128
+// output columns per plane; a K step is 128 contraction rows, so a tile's 256 output columns take two planes and a
+// step's four load rounds are (plane e / 2, rows 64 (e % 2) .. + 63); the K step adds 128 rows * 64 bytes.
+MXL_HD uint32_t ring_bt4_lane(int t, int e, int64_t rows_total) {
+    return ring_code_lane(t, 0, false) + (uint32_t)(e >> 1) * (uint32_t)(rows_total * 64) + (uint32_t)(e & 1) * 4096u;
+}
 // Scale panels [panels][rows_total][16]: thread t fetches the 16 bytes of tile row t; the panel is chosen by the
 // scalar offset panel * rows_total * 16.
 MXL_HD Desc ring_panel_desc(int64_t rows_total, int64_t panels, int64_t row0) {

@@ -501,16 +501,18 @@ def grouped_gemm_mx_nt_impl(a, a_scale, b, b_scale, group_lens, out_dtype=torch.
     """Forward / dgrad grouped GEMM: rows of ``a[total_m, k]`` split by
     ``group_lens``; ``b`` is ``[G, n, k]``.  ``kchunk``: both code tensors are K-chunk-major,
     ``a [k / 128, total_m, 128]`` and ``b [k / 128, G * n, 128]``; ``b_scale`` is ``[G, n, k / 32]`` as always.
-    ``b_transposed`` (K-step-major FP8 operands): ``b`` holds the codes of the transposed matrices, ``[n_ld / 64,
-    G * k, 64]`` -- the row-wise copy of a weight ``[G, k, n]`` serving its dgrad GEMM -- and ``b_scale`` the scale
-    panels of ``[G * n, k]`` (the transposed copy's scales)."""
+    ``b_transposed`` (K-step-major FP8 operands, or E2M1 operands in 128-element steps): ``b`` holds the codes of the
+    transposed matrices, ``[n_ld / 64, G * k, 64]`` (E2M1: ``[n_ld / 128, G * k, 64 bytes]``) -- the row-wise copy of a
+    weight ``[G, k, n]`` serving its dgrad GEMM -- and ``b_scale`` the scale panels of ``[G * n, k]`` (the transposed
+    copy's scales)."""
     _check_out_dtype(out_dtype)
     _require_cuda(a, a_scale, b, b_scale, group_lens)
     G = _check_group_lens(group_lens, a.device)
     a_fmt, b_fmt = fmt_of(a), fmt_of(b)
     if b_transposed:
-        if _layout(kchunk) != LAYOUT_KSTEP:
-            raise ValueError("b_transposed needs K-step-major operands")
+        both4 = a_fmt == _lib.FMT_E2M1 and b_fmt == _lib.FMT_E2M1
+        if _layout(kchunk) != (LAYOUT_KSTEP128 if both4 else LAYOUT_KSTEP):
+            raise ValueError("b_transposed needs K-step-major operands (128-element steps when both are E2M1)")
         total_m, k = _chunked_dims(a, a_fmt, kchunk)
         groups = max(G, 1)
         bt_rows, n_ld = _chunked_dims(b, b_fmt, kchunk)           # rows = groups * k, width = n padded to 128

@@ -214,8 +214,10 @@ class _MXLinearFunction(torch.autograd.Function):
         else:
             # FP8 weights on the ring kernel: dgrad reads the ROW-WISE codes transposed (2-D blocks: the transposed
             # copy is the same codes transposed), so only that copy's scales are written next to the row-wise copy
-            bt = (need_dgrad and _dgrad_reads_rowwise and kc == K.LAYOUT_KSTEP and w_fmt == _lib.FMT_E4M3
-                  and act_fmt == _lib.FMT_E4M3 and b.shape[-2] % K.GEMM_K_ALIGN == 0 and b.shape[-1] % K.GEMM_K_ALIGN == 0)
+            # (the same for E2M1 weights against E2M1 rows in 128-element steps, through the 4-bit transposing read)
+            bt = (need_dgrad and _dgrad_reads_rowwise and b.shape[-2] % K.GEMM_K_ALIGN == 0 and b.shape[-1] % K.GEMM_K_ALIGN == 0
+                  and ((kc == K.LAYOUT_KSTEP and w_fmt == _lib.FMT_E4M3 and act_fmt == _lib.FMT_E4M3)
+                       or (kc == K.LAYOUT_KSTEP128 and w_fmt == _lib.FMT_E2M1 and act_fmt == _lib.FMT_E2M1)))
             w_row, w_rs, w_col, w_cs = K.quantize_mx_weight_2d_impl(
                 b.detach(), w_fmt, scale_mode, rowwise=True, colwise=need_dgrad, pad_to=K.GEMM_K_ALIGN, kchunk=kc,
                 col_scales_only=bt,

@@ -119,7 +119,24 @@ static void check_ring_bt(int64_t groups, int64_t kc, int64_t planes, int64_t gr
                 request(d, ring_bt_lane(t, e, rows_total), (uint32_t)(st * 64 * 64), bytes, plane0 + e < planes, "ring codes transposed");
 }
 
+// the same for E2M1 codes in 128-element steps: planes of 128 output columns, a K step = 128 rows, round e = plane e / 2,
+// rows 64 (e % 2) .. + 63 of the step
+static void check_ring_bt4(int64_t groups, int64_t kc, int64_t planes, int64_t grp, int64_t plane0) {
+    const int64_t rows_total = groups * kc, bytes = planes * rows_total * 64;
+    const Desc d = ring_bt_desc(rows_total, planes, grp * kc, plane0);
+    const int64_t steps = kc / 128;
+    for (int64_t st = 0; st < steps; ++st)
+        for (int e = 0; e < 4; ++e)
+            for (int t = 0; t < 256; ++t)
+                request(d, ring_bt4_lane(t, e, rows_total), (uint32_t)(st * 128 * 64), bytes, plane0 + (e >> 1) < planes, "ring E2M1 codes transposed");
+}
+
 int main() {
+    for (int64_t groups : {1, 3})
+        for (int64_t kc : {128, 384})
+            for (int64_t planes : {1, 2, 3, 5})
+                for (int64_t grp = 0; grp < groups; ++grp)
+                    for (int64_t plane0 = 0; plane0 < planes; plane0 += 2) check_ring_bt4(groups, kc, planes, grp, plane0);
     for (int64_t rows_total : {16, 48, 256, 272, 1008})
         for (int64_t row0 = 0; row0 < rows_total; row0 += 16)
             for (int64_t k_slots : {2, 6}) check_slot2_shuffled(rows_total, k_slots, row0);

@@ -47,6 +47,7 @@ struct BwQuantArgs {
     const int64_t* group_lens;
     int num_groups;
     int64_t W;
+    int tiles_r, tiles_c, super_c, n_super;   // the launch's tile grid and its 8 x 8 supertiles
 };
 
 constexpr int BW_MAX_GROUPS = 1024;
@@ -120,15 +121,23 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
     __shared__ int grp_pre[BW_MAX_GROUPS + 1];
     __shared__ int64_t grp_red[4];
     const int t = threadIdx.x;
-    const int64_t col0 = (int64_t)blockIdx.x * BW;
+    // Tile order: consecutive workgroup ids land on different XCDs, and every XCD walks whole 8 x 8 supertiles (column
+    // tile fastest): the 4-byte factors that 8 neighbouring tiles write into one row of sinv_row (32 contiguous bytes)
+    // then meet in one L2, and the resident workgroups of an XCD cover long contiguous row spans.
+    const int L = blockIdx.x, xcd = L & 7, kk = L >> 3;
+    const int sup = (kk >> 6) * 8 + xcd;
+    if (sup >= a.n_super) return;
+    const int bx = (sup % a.super_c) * 8 + (kk & 7), by = (sup / a.super_c) * 8 + ((kk >> 3) & 7);
+    if (bx >= a.tiles_c || by >= a.tiles_r) return;
+    const int64_t col0 = (int64_t)bx * BW;
     // the tile's rows: rows [row0, row0 + valid) of this matrix land in columns [prow0, prow0 + 128) of the transposed copy
-    const int64_t zoff = TWOD ? (int64_t)blockIdx.z : 0;          // matrix of a batch of weights
-    int64_t row0 = (int64_t)blockIdx.y * BW, prow0 = row0, rows_pad = (a.rows + BW - 1) / BW * BW;
+    const int64_t zoff = TWOD ? (int64_t)blockIdx.y : 0;          // matrix of a batch of weights
+    int64_t row0 = (int64_t)by * BW, prow0 = row0, rows_pad = (a.rows + BW - 1) / BW * BW;
     int64_t valid = a.rows - row0 < BW ? a.rows - row0 : BW;
     if (!TWOD && a.group_lens != nullptr) {
         int tile_in_group;
         int64_t before, len;
-        const int grp = bw_locate(a.group_lens, a.num_groups, (int)blockIdx.y, grp_pre, grp_red, tile_in_group, before, len);
+        const int grp = bw_locate(a.group_lens, a.num_groups, by, grp_pre, grp_red, tile_in_group, before, len);
         // bw_locate counts tiles per group exactly as the padded layout counts 128-column pieces per segment
         row0 = before + (int64_t)tile_in_group * BW;
         valid = grp >= 0 ? len - (int64_t)tile_in_group * BW : 0;
@@ -196,9 +205,9 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
                 o.w = bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(p[8 * i + 6], p[8 * i + 7], sc);
                 *(uint4*)(dst + 16 * i) = o;
             }
-            if (!TWOD && half == 0) a.sinv_row[r * kb_cols + blockIdx.x] = 1.0f / sc;
+            if (!TWOD && half == 0) a.sinv_row[r * kb_cols + bx] = 1.0f / sc;
         }
-        if (TWOD && t == 0) a.sinv_row[(zoff * kb_rows + blockIdx.y) * kb_cols + blockIdx.x] = 1.0f / sc;
+        if (TWOD && t == 0) a.sinv_row[(zoff * kb_rows + by) * kb_cols + bx] = 1.0f / sc;
     }
     // ---- transposed copy: half a column, 64 codes of row (col0 + own) of the output; rows past the end give zero codes ----
     if (a.q_colT != nullptr) {
@@ -219,8 +228,8 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
             }
             *(uint4*)(dst + 16 * i) = make_uint4(w[0], w[1], w[2], w[3]);
         }
-        if (!TWOD && half == 0) a.sinv_colT[(col0 + own) * kb_rows + blockIdx.y] = 1.0f / sc;
-        if (TWOD && t == 0) a.sinv_colT[(zoff * kb_cols + blockIdx.x) * kb_rows + blockIdx.y] = 1.0f / sc;
+        if (!TWOD && half == 0) a.sinv_colT[(col0 + own) * kb_rows + by] = 1.0f / sc;
+        if (TWOD && t == 0) a.sinv_colT[(zoff * kb_cols + bx) * kb_rows + by] = 1.0f / sc;
     }
 }
 
@@ -484,7 +493,9 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
 
 template <bool TWOD>
 static int launch_bw_quant(const BwQuantArgs& a, int fmt, int64_t row_tiles, int batch, hipStream_t st) {
-    const dim3 grid((unsigned)(a.cols / BW), (unsigned)row_tiles, (unsigned)batch);
+    const int64_t wgs = (int64_t)(a.n_super + 7) / 8 * 8 * 64;
+    if (wgs > 0x7FFFFFFF) return MXL_EINVAL;
+    const dim3 grid((unsigned)wgs, (unsigned)batch);
     if (fmt == MXL_FMT_E4M3) hipLaunchKernelGGL((bw_quant_kernel<MXL_FMT_E4M3, TWOD>), grid, dim3(BW_THREADS), 0, st, a);
     else hipLaunchKernelGGL((bw_quant_kernel<MXL_FMT_E5M2, TWOD>), grid, dim3(BW_THREADS), 0, st, a);
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
@@ -504,8 +515,10 @@ static int bw_quant(const void* x, int64_t rows, int64_t cols, int fmt, const in
     if (((uintptr_t)x & 15) != 0 || row_tiles > 65535) return MXL_EINVAL;
     if ((((uintptr_t)q_row | (uintptr_t)q_colT) & 15) != 0) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
+    const int tiles_c = (int)(cols / BW), super_c = (tiles_c + 7) / 8, super_r = (int)((row_tiles + 7) / 8);
+    if ((int64_t)super_c * super_r > 0x7FFFFFF) return MXL_EINVAL;
     BwQuantArgs a{(const uint16_t*)x, rows, cols, (uint8_t*)q_row, (float*)sinv_row, (uint8_t*)q_colT, (float*)sinv_colT,
-                  group_lens, num_groups, W};
+                  group_lens, num_groups, W, (int)row_tiles, tiles_c, super_c, super_c * super_r};
     return twod ? launch_bw_quant<true>(a, fmt, row_tiles, batch, (hipStream_t)stream)
                 : launch_bw_quant<false>(a, fmt, row_tiles, 1, (hipStream_t)stream);
 }

@@ -25,9 +25,14 @@ typedef int bv8i __attribute__((ext_vector_type(8)));
 typedef __bf16 bv4bf __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------------------------------------------------
-// Quantiser.  One workgroup per 128 x 128 tile of x[rows, cols] (cols % 128 == 0; rows ragged).  The tile sits in
-// LDS as bf16 with a pitch of 130 elements; thread t owns half a row (row t / 2, 64 columns) for the row-wise copy and
-// half a column (column t / 2, 64 rows) for the transposed one.
+// Quantiser.  One workgroup per 128 x 128 tile of x[rows, cols] (cols % 128 == 0; rows ragged).  The tile stays in
+// registers: lane (wave w, row group rg = lane / 16, c16 = lane % 16) holds rows 32 w + 8 rg + 0..7, columns
+// 8 c16 + 0..7, eight 16-byte loads that are all in flight together.  A row's largest magnitude is a maximum over the
+// 16 lanes of a DPP row, a column's goes through the row groups of a wave and then through LDS over the four waves;
+// the fp32 factors are computed once per row and column (a division each, by 256 of the workgroup's lanes for the tile)
+// and handed round through LDS.  Row-wise codes leave as 16-byte stores (a lane pair swaps 8-byte pieces of a row
+// pair); the transposed codes are converted straight into transposed order (the convert instruction takes any two
+// values), collected in an LDS tile and stored as 128 contiguous bytes per output row.
 //   ROW  : q_row[rows, cols], sinv_row[rows, cols / 128]
 //   COL  : q_colT[cols, rows_pad], sinv_colT[cols, rows_pad / 128], rows_pad = rows rounded up to 128 (zero codes)
 //   TWOD : one scale per tile for both copies: sinv_row[ceil(rows / 128), cols / 128], sinv_colT[cols / 128, ceil(rows / 128)]
@@ -109,18 +114,38 @@ __device__ __forceinline__ int bw_locate(const int64_t* lens, int groups, int y,
     return g;
 }
 
-constexpr int BW_PITCH = 130;
+constexpr int BW_TPITCH = BW + 16;   // bytes per LDS row of the transposed code tile
 
 template <int FMT> __device__ __forceinline__ float bw_fp8_max() { return FMT == kFmtE5M2 ? 57344.f : 448.f; }
+// fp8_max / max(amax, 1e-12) with the sign bit set when the block holds a NaN or an infinity (its codes are all NaN
+// then, and the factor, which is never negative, is not used for them)
+template <int FMT> __device__ __forceinline__ uint32_t bw_scale_word(uint32_t amax16, float& sinv) {
+    const float sc = bw_fp8_max<FMT>() / fmaxf(__uint_as_float(amax16 << 16), 1e-12f);
+    sinv = 1.0f / sc;
+    return __float_as_uint(sc) | (amax16 >= 0x7F80u ? 0x80000000u : 0u);
+}
+template <int FMT> __device__ __forceinline__ uint2 bw_cvt8(uint32_t p0, uint32_t p1, uint32_t p2, uint32_t p3, uint32_t scale_word) {
+    const float sc = __uint_as_float(scale_word & 0x7FFFFFFFu);
+    const bool bad = (scale_word >> 31) != 0;
+    uint2 o;
+    o.x = cvt4_fp8<FMT>(p0, p1, sc);
+    o.y = cvt4_fp8<FMT>(p2, p3, sc);
+    o.x = bad ? 0x7F7F7F7Fu : o.x;
+    o.y = bad ? 0x7F7F7F7Fu : o.y;
+    return o;
+}
 
 template <int FMT, bool TWOD>
 __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
-    __shared__ uint16_t tile[BW * BW_PITCH];
-    __shared__ uint32_t amax_r[BW], amax_c[BW];
-    __shared__ uint32_t amax_tile;
+    __shared__ __attribute__((aligned(16))) uint8_t t_tile[BW * BW_TPITCH];
+    __shared__ __attribute__((aligned(16))) uint32_t amax_r[BW];         // per row
+    __shared__ __attribute__((aligned(16))) uint32_t amax_c[4][BW / 2];  // per wave: column pairs, packed 16-bit maxima
+    __shared__ __attribute__((aligned(16))) uint32_t scale_r[BW], scale_c[BW];
+    __shared__ uint32_t amax_w[4];
     __shared__ int grp_pre[BW_MAX_GROUPS + 1];
     __shared__ int64_t grp_red[4];
     const int t = threadIdx.x;
+    const int w = t >> 6, l = t & 63, c16 = l & 15, rg = l >> 4, rbase = 32 * w + 8 * rg;
     // Tile order: consecutive workgroup ids land on different XCDs, and every XCD walks whole 8 x 8 supertiles (column
     // tile fastest): the 4-byte factors that 8 neighbouring tiles write into one row of sinv_row (32 contiguous bytes)
     // then meet in one L2, and the resident workgroups of an XCD cover long contiguous row spans.
@@ -133,103 +158,162 @@ __global__ __launch_bounds__(BW_THREADS) void bw_quant_kernel(BwQuantArgs a) {
     // the tile's rows: rows [row0, row0 + valid) of this matrix land in columns [prow0, prow0 + 128) of the transposed copy
     const int64_t zoff = TWOD ? (int64_t)blockIdx.y : 0;          // matrix of a batch of weights
     int64_t row0 = (int64_t)by * BW, prow0 = row0, rows_pad = (a.rows + BW - 1) / BW * BW;
-    int64_t valid = a.rows - row0 < BW ? a.rows - row0 : BW;
+    int64_t valid64 = a.rows - row0 < BW ? a.rows - row0 : BW;
     if (!TWOD && a.group_lens != nullptr) {
         int tile_in_group;
         int64_t before, len;
         const int grp = bw_locate(a.group_lens, a.num_groups, by, grp_pre, grp_red, tile_in_group, before, len);
         // bw_locate counts tiles per group exactly as the padded layout counts 128-column pieces per segment
         row0 = before + (int64_t)tile_in_group * BW;
-        valid = grp >= 0 ? len - (int64_t)tile_in_group * BW : 0;
-        valid = valid > BW ? BW : valid;
-        valid = row0 + valid > a.rows ? a.rows - row0 : valid;     // lens that claim more rows than there are
-        valid = valid < 0 ? 0 : valid;
+        valid64 = grp >= 0 ? len - (int64_t)tile_in_group * BW : 0;
+        valid64 = valid64 > BW ? BW : valid64;
+        valid64 = row0 + valid64 > a.rows ? a.rows - row0 : valid64;     // lens that claim more rows than there are
         rows_pad = a.W;
     }
+    const int valid = valid64 < 0 ? 0 : (int)valid64;
     const uint16_t* xin = a.x + zoff * a.rows * a.cols;
     const int64_t kb_cols = a.cols / BW, kb_rows = rows_pad / BW;
-    // load: 2048 pieces of 8 elements, 8 per thread; rows past the end read as zero
+    const bool want_row = a.q_row != nullptr, want_col = a.q_colT != nullptr;   // uniform
+
+    // ---- load 8 rows x 8 columns per lane; rows past the end read as zero ----
+    // (a row past the end fetches the tile's last row instead and drops it: eight loads without a branch between them)
+    uint4 d[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int pc = i * BW_THREADS + t, r = pc >> 4, c8 = (pc & 15) * 8;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (r < valid) v = *(const uint4*)(xin + (row0 + r) * a.cols + col0 + c8);
-        uint32_t* d = (uint32_t*)(tile + r * BW_PITCH + c8);   // pitch 130 elements: 4-byte aligned
-        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-    }
-    if (t == 0) amax_tile = 0u;
-    __syncthreads();
-    const int own = t >> 1, half = t & 1;
-    // largest magnitude (15-bit bf16 pattern) of the half row and of the half column this thread owns
-    uint32_t mr = 0u, mc = 0u;
-    {
-        const uint32_t* p = (const uint32_t*)(tile + own * BW_PITCH + half * 64);
-#pragma unroll 8
-        for (int i = 0; i < 32; ++i) mr = pk_absmax(mr, p[i]);
-        mr = hmax16(mr);
-        const uint16_t* q = tile + (half * 64) * BW_PITCH + own;
-#pragma unroll 8
-        for (int i = 0; i < 64; ++i) {
-            const uint32_t v = q[i * BW_PITCH] & 0x7FFFu;
-            mc = v > mc ? v : mc;
+    for (int it = 0; it < 8; ++it) d[it] = make_uint4(0u, 0u, 0u, 0u);
+    if (valid > 0) {
+        const uint16_t* src = xin + row0 * a.cols + col0 + 8 * c16;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int r = rbase + it;
+            const uint4 v = load16_streaming(src + (int64_t)(r < valid ? r : valid - 1) * a.cols);
+            d[it] = r < valid ? v : make_uint4(0u, 0u, 0u, 0u);
         }
     }
-    {
-        const uint32_t orr = __shfl_xor(mr, 1), occ = __shfl_xor(mc, 1);
-        mr = orr > mr ? orr : mr;
-        mc = occ > mc ? occ : mc;
-    }
-    if (half == 0) {
-        amax_r[own] = mr;
-        amax_c[own] = mc;
-        if (TWOD) atomicMax(&amax_tile, mr);
-    }
-    __syncthreads();
-    const float fmax = bw_fp8_max<FMT>();
-    auto scale_of = [&](uint32_t amax16) { return fmax / fmaxf(__uint_as_float(amax16 << 16), 1e-12f); };
-    // ---- row-wise copy: half a row, 64 codes = four 16-byte stores ----
-    if (a.q_row != nullptr) {
-        const uint32_t am = TWOD ? amax_tile : amax_r[own];
-        const float sc = scale_of(am);
-        const bool bad = am >= 0x7F80u;
-        const int64_t r = row0 + own;
-        if (own < valid) {
-            const uint32_t* p = (const uint32_t*)(tile + own * BW_PITCH + half * 64);
-            uint8_t* dst = a.q_row + (zoff * a.rows + r) * a.cols + col0 + half * 64;
+
+    // ---- largest magnitudes (15-bit bf16 patterns) ----
+    uint32_t rmax[8];                    // of the lane's rows, over the 128 columns
+    uint32_t cmax[4] = {0u, 0u, 0u, 0u}; // of the lane's column pairs (packed), over its 8 rows
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint4 o;
-                o.x = bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(p[8 * i + 0], p[8 * i + 1], sc);
-                o.y = bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(p[8 * i + 2], p[8 * i + 3], sc);
-                o.z = bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(p[8 * i + 4], p[8 * i + 5], sc);
-                o.w = bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(p[8 * i + 6], p[8 * i + 7], sc);
-                *(uint4*)(dst + 16 * i) = o;
-            }
-            if (!TWOD && half == 0) a.sinv_row[r * kb_cols + bx] = 1.0f / sc;
+    for (int it = 0; it < 8; ++it) {
+        const uint32_t p0 = d[it].x & 0x7FFF7FFFu, p1 = d[it].y & 0x7FFF7FFFu, p2 = d[it].z & 0x7FFF7FFFu,
+                       p3 = d[it].w & 0x7FFF7FFFu;
+        if (!TWOD) {
+            cmax[0] = pk_max16(cmax[0], p0);
+            cmax[1] = pk_max16(cmax[1], p1);
+            cmax[2] = pk_max16(cmax[2], p2);
+            cmax[3] = pk_max16(cmax[3], p3);
         }
-        if (TWOD && t == 0) a.sinv_row[(zoff * kb_rows + by) * kb_cols + bx] = 1.0f / sc;
+        uint32_t m = hmax16(pk_max16(pk_max16(p0, p1), pk_max16(p2, p3)));
+        m = max(m, dpp_xor1(m));
+        m = max(m, dpp_xor2(m));
+        if (!TWOD) {
+            m = max(m, dpp_half_mirror(m));
+            m = max(m, dpp_mirror(m));
+        }
+        rmax[it] = m;
     }
-    // ---- transposed copy: half a column, 64 codes of row (col0 + own) of the output; rows past the end give zero codes ----
-    if (a.q_colT != nullptr) {
-        const uint32_t am = TWOD ? amax_tile : amax_c[own];
-        const float sc = scale_of(am);
-        const bool bad = am >= 0x7F80u;
-        const uint16_t* q = tile + (half * 64) * BW_PITCH + own;
-        uint8_t* dst = a.q_colT + (zoff * a.cols + col0 + own) * rows_pad + prow0 + half * 64;
+    uint32_t tile_word = 0u;
+    if (TWOD) {
+        uint32_t m = rmax[0];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t w[4];
+        for (int it = 1; it < 8; ++it) m = max(m, rmax[it]);
+#pragma unroll
+        for (int dlt = 4; dlt < 64; dlt <<= 1) m = max(m, (uint32_t)__shfl_xor((int)m, dlt));
+        if (l == 0) amax_w[w] = m;
+        __syncthreads();
+        m = max(max(amax_w[0], amax_w[1]), max(amax_w[2], amax_w[3]));
+        float sinv;
+        tile_word = bw_scale_word<FMT>(m, sinv);
+        if (t == 0) {
+            if (want_row) a.sinv_row[(zoff * kb_rows + by) * kb_cols + bx] = sinv;
+            if (want_col) a.sinv_colT[(zoff * kb_cols + bx) * kb_rows + by] = sinv;
+        }
+    } else {
+        if (want_col) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int e = 16 * i + 4 * j;
-                const uint32_t p0 = (uint32_t)q[(e + 0) * BW_PITCH] | ((uint32_t)q[(e + 1) * BW_PITCH] << 16);
-                const uint32_t p1 = (uint32_t)q[(e + 2) * BW_PITCH] | ((uint32_t)q[(e + 3) * BW_PITCH] << 16);
-                w[j] = bad ? 0x7F7F7F7Fu : cvt4_fp8<FMT>(p0, p1, sc);
+                cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 16));
+                cmax[j] = pk_max16(cmax[j], (uint32_t)__shfl_xor((int)cmax[j], 32));
             }
-            *(uint4*)(dst + 16 * i) = make_uint4(w[0], w[1], w[2], w[3]);
+            if (rg == 0) *(uint4*)&amax_c[w][4 * c16] = make_uint4(cmax[0], cmax[1], cmax[2], cmax[3]);
         }
-        if (!TWOD && half == 0) a.sinv_colT[(col0 + own) * kb_rows + by] = 1.0f / sc;
-        if (TWOD && t == 0) a.sinv_colT[(zoff * kb_cols + bx) * kb_rows + by] = 1.0f / sc;
+        if (want_row && c16 == 0) {
+            *(uint4*)&amax_r[rbase] = make_uint4(rmax[0], rmax[1], rmax[2], rmax[3]);
+            *(uint4*)&amax_r[rbase + 4] = make_uint4(rmax[4], rmax[5], rmax[6], rmax[7]);
+        }
+        __syncthreads();
+        // one factor per row (waves 2 and 3) and per column (waves 0 and 1)
+        if (t >= BW) {
+            if (want_row) {
+                const int r = t - BW;
+                float sinv;
+                scale_r[r] = bw_scale_word<FMT>(amax_r[r], sinv);
+                if (r < valid) a.sinv_row[(row0 + r) * kb_cols + bx] = sinv;
+            }
+        } else if (want_col) {
+            const uint16_t* h = (const uint16_t*)&amax_c[0][0];
+            const uint32_t m = max(max((uint32_t)h[t], (uint32_t)h[BW + t]), max((uint32_t)h[2 * BW + t], (uint32_t)h[3 * BW + t]));
+            float sinv;
+            scale_c[t] = bw_scale_word<FMT>(m, sinv);
+            a.sinv_colT[(col0 + t) * kb_rows + by] = sinv;
+        }
+        __syncthreads();
+    }
+
+    // ---- row-wise copy: two rows at a time, 16 bytes per lane ----
+    if (want_row) {
+        uint32_t sw[8];
+        if (!TWOD) {
+            const uint4 s0 = *(const uint4*)&scale_r[rbase], s1 = *(const uint4*)&scale_r[rbase + 4];
+            sw[0] = s0.x; sw[1] = s0.y; sw[2] = s0.z; sw[3] = s0.w;
+            sw[4] = s1.x; sw[5] = s1.y; sw[6] = s1.z; sw[7] = s1.w;
+        }
+        const bool odd = (c16 & 1) != 0;
+        uint8_t* dst = a.q_row + (zoff * a.rows + row0 + rbase) * a.cols + col0 + 8 * (c16 & ~1);
+        uint2 o_even = make_uint2(0u, 0u);
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const uint2 o = bw_cvt8<FMT>(d[it].x, d[it].y, d[it].z, d[it].w, TWOD ? tile_word : sw[it]);
+            if ((it & 1) == 0) {
+                o_even = o;
+            } else {
+                // even lane: 16 codes of the even row; odd lane: 16 codes of the odd row
+                const uint2 send = odd ? o_even : o;
+                const uint2 recv = make_uint2(dpp_xor1(send.x), dpp_xor1(send.y));
+                const uint4 out = odd ? make_uint4(recv.x, recv.y, o.x, o.y) : make_uint4(o_even.x, o_even.y, recv.x, recv.y);
+                const int rr = odd ? it : it - 1;
+                if (rbase + rr < valid) store16_streaming(dst + (int64_t)rr * a.cols, out);
+            }
+        }
+    }
+
+    // ---- transposed copy: column 8 c16 + j of the lane's 8 rows = 8 bytes of output row col0 + 8 c16 + j ----
+    if (want_col) {
+        uint32_t sw[8];
+        if (!TWOD) {
+            const uint4 s0 = *(const uint4*)&scale_c[8 * c16], s1 = *(const uint4*)&scale_c[8 * c16 + 4];
+            sw[0] = s0.x; sw[1] = s0.y; sw[2] = s0.z; sw[3] = s0.w;
+            sw[4] = s1.x; sw[5] = s1.y; sw[6] = s1.z; sw[7] = s1.w;
+        }
+        const uint32_t* dw = (const uint32_t*)d;  // dw[it * 4 + j / 2]: columns j, j + 1 (j even) of row `it`
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t pr[4];   // rows (2 i, 2 i + 1) of column j
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t lo = dw[(2 * i) * 4 + (j >> 1)], hi = dw[(2 * i + 1) * 4 + (j >> 1)];
+                pr[i] = (j & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
+            }
+            *(uint2*)(t_tile + (8 * c16 + j) * BW_TPITCH + rbase) = bw_cvt8<FMT>(pr[0], pr[1], pr[2], pr[3], TWOD ? tile_word : sw[j]);
+        }
+        __syncthreads();
+        // rows past the end hold zero codes (or NaN codes in a block with a NaN or an infinity)
+        uint8_t* dst = a.q_colT + (zoff * a.cols + col0) * rows_pad + prow0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = (t >> 3) + 32 * i, ch = t & 7;
+            store16_streaming(dst + (int64_t)c * rows_pad + 16 * ch, *(const uint4*)(t_tile + c * BW_TPITCH + 16 * ch));
+        }
     }
 }
 

@@ -249,4 +249,38 @@ __device__ __forceinline__ uint4 norm8(const uint4& x, const uint4& wv, float rs
     return make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
+// ---- shared by the quantisers ----
+// The quantisers stream: every input byte is read once and every output byte written once, by one
+// workgroup.  Non-temporal accesses keep that traffic from displacing the scale words in L2, which
+// do have to wait there for their neighbours (the 8 x 8 supertile order of the quantisers' grids).
+typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store16_streaming(void* d, const uint4& v) {
+    const qu32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (qu32x4*)d);
+}
+__device__ __forceinline__ void store8_streaming(void* d, const uint2& v) {
+    const qu32x2 t = {v.x, v.y};
+    __builtin_nontemporal_store(t, (qu32x2*)d);
+}
+__device__ __forceinline__ void store4_streaming(void* d, uint32_t v) { __builtin_nontemporal_store(v, (uint32_t*)d); }
+__device__ __forceinline__ uint4 load16_streaming(const void* s) {
+    const qu32x4 t = __builtin_nontemporal_load((const qu32x4*)s);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+
+__device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+}
+// the other two steps of a maximum over the 16 lanes of a DPP row: lane i <-> 7 - i inside each half row, lane i <-> 15 - i
+__device__ __forceinline__ uint32_t dpp_half_mirror(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+}
+__device__ __forceinline__ uint32_t dpp_mirror(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true);  // row_mirror
+}
+
 }  // namespace mxl

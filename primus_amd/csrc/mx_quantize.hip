@@ -18,34 +18,8 @@
 
 namespace mxl {
 
-// The quantisers stream: every input byte is read once and every output byte written once, by one
-// workgroup.  Non-temporal accesses keep that traffic from displacing the E8M0 scale words in L2,
-// which do have to wait there for their neighbours (see quant_tile_of_workgroup).
-typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void store16_streaming(void* d, const uint4& v) {
-    const qu32x4 t = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(t, (qu32x4*)d);
-}
-__device__ __forceinline__ void store8_streaming(void* d, const uint2& v) {
-    const qu32x2 t = {v.x, v.y};
-    __builtin_nontemporal_store(t, (qu32x2*)d);
-}
-__device__ __forceinline__ void store4_streaming(void* d, uint32_t v) { __builtin_nontemporal_store(v, (uint32_t*)d); }
-__device__ __forceinline__ uint4 load16_streaming(const void* s) {
-    const qu32x4 t = __builtin_nontemporal_load((const qu32x4*)s);
-    return make_uint4(t.x, t.y, t.z, t.w);
-}
-
 constexpr int QT = 128;       // tile edge
 constexpr int QTHREADS = 256;
-
-__device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
-}
-__device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
-}
 
 struct QuantArgs {
     const uint16_t* x;

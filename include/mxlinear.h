@@ -453,6 +453,11 @@ int mxl_grouped_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a
 int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,
                                      int b_fmt, void* c_bf16, const int64_t* group_lens, int num_groups, int64_t total_m,
                                      int64_t n, int64_t k, void* stream);
+/* The blockwise GEMMs run on output tiles of 128 x 256 or 256 x 256 and pick by the shape (256 rows unless that leaves
+ * more of the chip idle than it gains; same bits either way).  mxl_blockwise_gemm_tile(128 / 256) forces one for every later
+ * call of the process, 0 returns to the choice by shape: a measuring and testing aid without counterpart in the
+ * reference.  MXL_EINVAL for any other value. */
+int mxl_blockwise_gemm_tile(int rows);
 
 /* ---- pre-shuffled MXFP4 layouts ----
  *

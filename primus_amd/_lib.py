@@ -74,6 +74,7 @@ EXPORTS = (
     "mxl_gemm_nt_blockwise",
     "mxl_grouped_gemm_nt_blockwise",
     "mxl_grouped_gemm_wgrad_blockwise",
+    "mxl_blockwise_gemm_tile",
     "mxl_shuffle_codes",
     "mxl_shuffle_scales",
     "mxl_calibrate_mfma",
@@ -203,6 +204,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_calibrate_mfma_bf16_flops.argtypes = [i64]
         lib.mxl_gemm_nt_blockwise.restype = i32
         lib.mxl_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, i32, vp, i64, i64, i64, vp]
+        lib.mxl_blockwise_gemm_tile.restype = i32
+        lib.mxl_blockwise_gemm_tile.argtypes = [i32]
         _lib = lib
     return _lib
 

@@ -57,18 +57,18 @@ struct BwQuantArgs {
 
 constexpr int BW_MAX_GROUPS = 1024;
 
-// Which group holds tile `y` when every group is cut into tiles of 128 rows (a group's last tile may be ragged):
+// Which group holds tile `y` when every group is cut into tiles of TR rows (a group's last tile may be ragged):
 // `pre` (LDS, BW_MAX_GROUPS + 1 ints) receives the prefix sum of the groups' tile counts, `red` (LDS, one word of 8
 // bytes per wave of the workgroup, NT / 64 of them) is scratch.  Returns the group (or -1 behind the last tile); tile_in_group, the rows in front of the group
 // and its length come back through the references.  Negative lens read as 0.  All threads of the workgroup call it.
-template <int NT = 256>
+template <int NT = 256, int TR = BW>
 __device__ __forceinline__ int bw_locate(const int64_t* lens, int groups, int y, int* pre, int64_t* red, int& tile_in_group,
                                          int64_t& rows_before, int64_t& len) {
     const int t = threadIdx.x;
     if (t == 0) pre[0] = 0;
     for (int j = t; j < groups; j += NT) {
         const int64_t l = lens[j] > 0 ? lens[j] : 0;
-        pre[j + 1] = (int)((l + BW - 1) / BW);
+        pre[j + 1] = (int)((l + TR - 1) / TR);
     }
     __syncthreads();
     if (t < 64) {   // in-place inclusive scan of pre[1 .. groups], a run of consecutive entries per lane
@@ -575,6 +575,237 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// The same GEMM on a 256 x 256 tile, for problems with enough of them to fill the chip: a third fewer operand bytes
+// per flop travel from L2 to LDS (what the 128 x 256 kernel waits for most) and half as many barriers and tiles.
+// 8 waves as 4 x 2, a wave owns 64 rows x 128 columns = 2 x 4 MFMA tiles (128 accumulator registers); the partial
+// sums of only ONE column of tiles (2 x 16 registers) exist at a time: for each of the four b fragments of a K block,
+// 4 MFMAs (both a fragments, both halves of the block) add up from zero and are multiplied into the accumulators
+// in the shadow of the following MFMAs.  Same MFMA and FMA order per output element as the 128 x 256 kernel, so the
+// same bits.  Two LDS stages of 64 KiB (a K block of both operands) + factors: the requests of block kb + 1 go out
+// behind the first nine MFMAs of block kb, into the stage block kb - 1 has left.
+// One workgroup per tile, like the 128 x 256 kernel (a persistent form, whose last K block requests the first block of
+// the workgroup's next tile, was built and measured: no faster -- workgroups in lockstep all reach their epilogues at
+// once, and the burst of stores costs what the saved dispatches gain).
+// ------------------------------------------------------------------------------------------------------------
+constexpr int BWH_BM = 256, BWH_BN = 256;
+constexpr int BWH_A = BWH_BM * BW, BWH_STAGE = (BWH_BM + BWH_BN) * BW;      // 32 + 32 KiB
+constexpr int BWH_FAC = (BWH_BM + BWH_BN) * 4;
+constexpr int BW_GEMM256_LDS = 2 * (BWH_STAGE + BWH_FAC);
+
+template <int AFMT, int BFMT, bool SBU>
+__global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
+    constexpr int CB = BFMT == kFmtE5M2 ? 1 : 0, BL = AFMT == kFmtE5M2 ? 1 : 0;
+    extern __shared__ __attribute__((aligned(16))) uint8_t bw_smem[];
+    float* fac_base = (float*)(bw_smem + 2 * BWH_STAGE);                 // [stage][a: 256 | b: 256]
+    __shared__ int grp_pre[BW_MAX_GROUPS + 1];
+    __shared__ int64_t grp_red[BWG_THREADS / 64];
+    const int t = threadIdx.x;
+    const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l = t & 63, lr = l & 31, g = l >> 5, wm = w >> 1, wn = w & 1;
+    const uint32_t smem_base = (uint32_t)(uintptr_t)bw_smem;
+    int64_t row0 = (int64_t)blockIdx.y * BWH_BM;
+    const int64_t col0 = (int64_t)blockIdx.x * BWH_BN;
+    const int64_t kb_n = p.k / BW;
+    int64_t m_end = p.m, b_group = 0, c_group = 0, kb0 = 0, kb1 = kb_n;
+    if (p.mode == 1) {
+        int tile_in_group;
+        int64_t before, len;
+        const int grp = bw_locate<BWG_THREADS, BWH_BM>(p.group_lens, p.num_groups, (int)blockIdx.y, grp_pre, grp_red, tile_in_group, before, len);
+        if (grp < 0) return;                     // the grid is sized for the worst case (every group with a ragged tile)
+        row0 = before + (int64_t)tile_in_group * BWH_BM;
+        m_end = before + len < p.m ? before + len : p.m;
+        if (row0 >= m_end) return;
+        b_group = grp;
+    } else if (p.mode == 2) {
+        // this group's segment of the contraction: [sum of the padded lens in front, + its own padded len), in blocks
+        const int grp = (int)blockIdx.z;
+        int64_t part = 0;
+        for (int j = t; j < grp; j += BWG_THREADS) part += ((p.group_lens[j] > 0 ? p.group_lens[j] : 0) + BW - 1) / BW;
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) part += __shfl_xor(part, d);
+        if ((t & 63) == 0) grp_red[t >> 6] = part;
+        __syncthreads();
+        kb0 = 0;
+#pragma unroll
+        for (int i = 0; i < BWG_THREADS / 64; ++i) kb0 += grp_red[i];
+        kb1 = kb0 + ((p.group_lens[grp] > 0 ? p.group_lens[grp] : 0) + BW - 1) / BW;
+        kb0 = kb0 > kb_n ? kb_n : kb0;           // lens that claim more than the operands hold
+        kb1 = kb1 > kb_n ? kb_n : kb1;
+        c_group = grp;
+    }
+    const int64_t pm = m_end, pk = p.k, pn = p.n;
+    const int sb_shift = p.sb_shift;
+    const float* const psb = p.sb + b_group * (pn >> sb_shift) * kb_n;
+    uint16_t* const pc_out = p.c + c_group * p.m * pn;
+    // descriptors: from the tile's first row to the last row that may be read (the group's / the operand's end for a,
+    // the end of the group's matrix for b); offsets inside them are 32-bit (the host bounds 256 rows x k)
+    const v4i ra = bw_rsrc(p.a + row0 * pk, (pm - row0) * pk);
+    const v4i rb = bw_rsrc(p.b + b_group * pn * pk + col0 * pk, (pn - col0) * pk);
+    // loader geometry as in the 128 x 256 kernel: a round = 64 rows x 128 bytes, piece (i % 8) ^ ((row / 2) % 8)
+    const int ld_row = t >> 3;
+    const uint32_t ld_voff = (uint32_t)(ld_row * pk + 16 * ((t & 7) ^ ((ld_row >> 1) & 7)));
+    const uint32_t round_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(64 * pk));
+    const uint32_t wave_lds = smem_base + (uint32_t)(w * 1024);
+    // factors: waves 0 .. 3 fetch a's 256 row factors, waves 4 .. 7 b's (lane i of wave w lands at word 64 w + i)
+    const bool f_a = w < 4;
+    const int frow = f_a ? t : t - BWH_BM;
+    const uint32_t fac_voff = (uint32_t)(((f_a ? frow : (frow >> sb_shift)) * kb_n) * 4);
+    const uint32_t fac_lds = smem_base + (uint32_t)(2 * BWH_STAGE + w * 256);
+    const v4i rfac = f_a ? bw_rsrc(p.sa + row0 * kb_n, (pm - row0) * kb_n * 4)
+                         : bw_rsrc(psb + (col0 >> sb_shift) * kb_n, (((pn - col0) + (1 << sb_shift) - 1) >> sb_shift) * kb_n * 4);
+    // round e of a block: 0 .. 3 the a rows, 4 .. 7 the b rows
+    auto issue_round = [&](uint32_t koff, uint32_t base, int e) __attribute__((always_inline)) {
+        if (e < 4) bw_dma16(ra, base + e * 8192, ld_voff, koff + e * round_bytes);
+        else bw_dma16(rb, base + BWH_A + (e - 4) * 8192, ld_voff, koff + (e - 4) * round_bytes);
+    };
+    auto issue_fac = [&](uint32_t soff, int stage) __attribute__((always_inline)) {
+        const uint32_t lds = fac_lds + (uint32_t)(stage * BWH_FAC);
+        asm volatile("" : "+s"(soff));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                     :
+                     : "s"(lds), "v"(fac_voff), "s"(rfac), "s"(soff)
+                     : "memory");
+    };
+    // fragment addressing: lane (lr, g) reads the 16-byte pieces 4 ks + 2 h + g of its row, swizzled by the row
+    const int swz = (lr >> 1) & 7;
+    uint32_t piece[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) piece[ks][h] = (uint32_t)(16 * ((4 * ks + 2 * h + g) ^ swz));
+    const uint32_t a_row = (uint32_t)((wm * 64 + lr) * BW), b_row = (uint32_t)(BWH_A + (wn * 128 + lr) * BW);
+
+    bv16f acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    const int k0 = __builtin_amdgcn_readfirstlane((int)kb0), k1 = __builtin_amdgcn_readfirstlane((int)kb1);
+    if (k0 < k1) {
+        const uint32_t koff = (uint32_t)__builtin_amdgcn_readfirstlane(k0 * BW);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) issue_round(koff, wave_lds, e);
+        issue_fac((uint32_t)__builtin_amdgcn_readfirstlane(k0 * 4), 0);
+    }
+    int st = 0;
+    for (int kb = k0; kb < k1; ++kb) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();   // block kb and its factors are in LDS for every wave; every wave has left the other stage
+        // The requests of block kb + 1 go out behind this block's MFMAs.  In the last block they go out as well, at
+        // an offset of 2 GiB: past the end of what the descriptor covers they are dropped (or, under an operand that
+        // large, fetch bytes of it that nobody reads) -- a branch between the MFMAs would split the block's
+        // instructions into basic blocks, and the order below, which the register budget depends on, would not
+        // survive that.
+        const bool follows = kb + 1 < k1;
+        const uint32_t in_koff = follows ? (uint32_t)__builtin_amdgcn_readfirstlane((kb + 1) * BW) : 0x80000000u;
+        const uint32_t in_fac = follows ? (uint32_t)__builtin_amdgcn_readfirstlane((kb + 1) * 4) : 0x80000000u;
+        const uint32_t in_base = wave_lds + (uint32_t)((st ^ 1) * BWH_STAGE);
+        const float* fac = fac_base + st * (BWH_BM + BWH_BN);
+        const uint8_t* stg = bw_smem + st * BWH_STAGE;
+        auto frag = [&](uint32_t row_off, int ks) __attribute__((always_inline)) {
+            const uint4 lo = *(const uint4*)(stg + row_off + piece[ks][0]);
+            const uint4 hi = *(const uint4*)(stg + row_off + piece[ks][1]);
+            return bv8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        };
+        bv8i fa8[2][2], fb8[2];      // [a fragment][ks], [ks]
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) fa8[i][ks] = frag(a_row + i * 32 * BW, ks);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) fb8[ks] = frag(b_row, ks);
+        const float sbu = SBU ? fac[BWH_BM + wn * 128] : 0.f;
+        float sa[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) sa[i] = fac[wm * 64 + i * 32 + lr];
+        bv16f zero;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) zero[e] = 0.f;
+        // acc += part * (sa[row] * sb[col]): lane (lr, g), register e = 4 q + r of tile (i, j) is row i * 32 + lr,
+        // column j * 32 + 8 q + 4 g + r of the wave's 64 x 128
+        auto scale_in = [&](const bv16f& part, int i, int j) __attribute__((always_inline)) {
+            const float sab = sa[i] * sbu;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (SBU) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = fmaf(part[4 * q + e], sab, acc[i][j][4 * q + e]);
+                } else {
+                    const float4 sb = *(const float4*)(&fac[BWH_BM + wn * 128 + j * 32 + 8 * q + 4 * g]);
+                    acc[i][j][4 * q + 0] = fmaf(part[4 * q + 0], sa[i] * sb.x, acc[i][j][4 * q + 0]);
+                    acc[i][j][4 * q + 1] = fmaf(part[4 * q + 1], sa[i] * sb.y, acc[i][j][4 * q + 1]);
+                    acc[i][j][4 * q + 2] = fmaf(part[4 * q + 2], sa[i] * sb.z, acc[i][j][4 * q + 2]);
+                    acc[i][j][4 * q + 3] = fmaf(part[4 * q + 3], sa[i] * sb.w, acc[i][j][4 * q + 3]);
+                }
+            }
+        };
+        // request number mi (one behind each of the block's first nine MFMAs): the eight operand rounds, then the factors
+#define REQ(mi)                                            \
+    do {                                                   \
+        if ((mi) < 8) issue_round(in_koff, in_base, (mi)); \
+        else if ((mi) == 8) issue_fac(in_fac, st ^ 1);     \
+    } while (0)
+        // Per b fragment j: the two MFMAs of a fragment 0, the FMAs of the previous fragment's second tile in their
+        // shadow, the two MFMAs of a fragment 1 (each half of the b fragment gives its registers to the next
+        // fragment's half as soon as its last MFMA has gone), the FMAs of this fragment's first tile.  The b
+        // fragment is the MFMA's first operand: a lane ends up with 4 consecutive output columns.
+        bv16f part0, part1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            part0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[0], fa8[0][0], zero, CB, BL, 0, 127, 0, 127);
+            REQ(4 * j);
+            part0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[1], fa8[0][1], part0, CB, BL, 0, 127, 0, 127);
+            REQ(4 * j + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j > 0) scale_in(part1, 1, j - 1);
+            __builtin_amdgcn_sched_barrier(0);
+            part1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[0], fa8[1][0], zero, CB, BL, 0, 127, 0, 127);
+            REQ(4 * j + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j < 3) fb8[0] = frag(b_row + (j + 1) * 32 * BW, 0);
+            part1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[1], fa8[1][1], part1, CB, BL, 0, 127, 0, 127);
+            REQ(4 * j + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j < 3) fb8[1] = frag(b_row + (j + 1) * 32 * BW, 1);
+            scale_in(part0, 0, j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#undef REQ
+        scale_in(part1, 1, 3);
+        st ^= 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // no request of any wave (the last block's dropped ones included) still writes LDS: the stages are free
+    // Output through a wave-private LDS patch of 32 rows x 256 bytes, one a fragment at a time: a lane's four
+    // consecutive bf16 go in as 8 bytes and come out as 16 bytes per lane, 4 rows x 256 contiguous bytes per store
+    // instruction (16-byte pieces XOR-swizzled by the row).  Stored straight from the accumulator layout, 16 bytes per
+    // row and instruction, the partial lines cost a K = 4096 tile 5 % of its time.
+    uint8_t* const patch = bw_smem + w * (32 * 256);
+    const bool cols_in = col0 + wn * 128 < pn;       // (n is a multiple of 128: the wave's columns are in or out as a whole)
+    const int er = l >> 4, ep = l & 15;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bv4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
+                                 (__bf16)acc[i][j][4 * q + 3]};
+                *(bv4bf*)(patch + lr * 256 + 16 * ((4 * j + q) ^ (lr & 15)) + 8 * g) = o;
+            }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int r = 4 * u + er;
+            const uint4 v = *(const uint4*)(patch + r * 256 + 16 * (ep ^ (r & 15)));
+            const int64_t m = row0 + wm * 64 + i * 32 + r;
+            if (cols_in && m < pm) store16_streaming(pc_out + m * pn + col0 + wn * 128 + 8 * ep, v);
+        }
+    }
+}
+
 template <bool TWOD>
 static int launch_bw_quant(const BwQuantArgs& a, int fmt, int64_t row_tiles, int batch, hipStream_t st) {
     const int64_t wgs = (int64_t)(a.n_super + 7) / 8 * 8 * 64;
@@ -610,21 +841,29 @@ static int bw_quant(const void* x, int64_t rows, int64_t cols, int fmt, const in
 // The dynamic LDS size is above the default limit.  The attribute belongs to the (kernel, device) pair and is set at
 // the first launch on a device -- not at every launch: a launch may be recorded by a stream capture, which is no
 // place for a call that changes function state.
-template <int AFMT, int BFMT, bool SBU>
+template <int AFMT, int BFMT, bool SBU, bool TALL>
 static int launch_bw_gemm(const BwGemmArgs& g, dim3 grid, hipStream_t st) {
     static std::atomic<bool> attr_set[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return MXL_ELAUNCH;
     const int slot = dev & 63;
-    auto kern = bw_gemm_kernel<AFMT, BFMT, SBU>;
+    constexpr int lds = TALL ? BW_GEMM256_LDS : BW_GEMM_LDS;
+    const void* kern = TALL ? (const void*)bw_gemm256_kernel<AFMT, BFMT, SBU> : (const void*)bw_gemm_kernel<AFMT, BFMT, SBU>;
     if (!attr_set[slot].load(std::memory_order_acquire)) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BW_GEMM_LDS) != hipSuccess)
-            return MXL_ELAUNCH;
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return MXL_ELAUNCH;
         attr_set[slot].store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL(kern, grid, dim3(BWG_THREADS), BW_GEMM_LDS, st, g);
+    if (TALL) hipLaunchKernelGGL((bw_gemm256_kernel<AFMT, BFMT, SBU>), grid, dim3(BWG_THREADS), lds, st, g);
+    else hipLaunchKernelGGL((bw_gemm_kernel<AFMT, BFMT, SBU>), grid, dim3(BWG_THREADS), lds, st, g);
     return MXL_OK;
 }
+template <int AFMT, int BFMT>
+static int launch_bw_gemm_fmt(const BwGemmArgs& g, dim3 grid, bool sbu, bool tall, hipStream_t st) {
+    if (tall) return sbu ? launch_bw_gemm<AFMT, BFMT, true, true>(g, grid, st) : launch_bw_gemm<AFMT, BFMT, false, true>(g, grid, st);
+    return sbu ? launch_bw_gemm<AFMT, BFMT, true, false>(g, grid, st) : launch_bw_gemm<AFMT, BFMT, false, false>(g, grid, st);
+}
+
+static std::atomic<int> bw_gemm_tile_rows{0};   // 0: by the shape; 128 or 256: forced (mxl_blockwise_gemm_tile)
 
 static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv, int b_fmt,
                    int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k, int mode, const int64_t* group_lens,
@@ -639,20 +878,31 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
     if (k == 0 && mode != 2) return MXL_EINVAL;
     if ((((uintptr_t)a_codes | (uintptr_t)b_codes) & 15) != 0) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
-    // row tiles: exact for a dense GEMM and for wgrad; at most one ragged tile per group in the grouped forward
-    const int64_t row_tiles = mode == 1 ? m / BW + num_groups : (m + BW - 1) / BW;
+    // Tile height: 256 x 256 tiles run a fifth to a quarter faster per flop than 128 x 256 ones (a third fewer operand
+    // bytes from L2 per flop), so they win unless the coarser tiles leave that much more of the chip idle -- in the
+    // last round of tiles, or in the ragged last tile of every group of a grouped forward (expected padding: half a
+    // tile per group, which a group of 512 rows pays back).  mxl_blockwise_gemm_tile overrides.
+    const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1;
+    auto row_tiles_of = [&](int64_t bm) { return mode == 1 ? m / bm + num_groups : (m + bm - 1) / bm; };
+    auto fill_of = [&](int64_t tiles) { const int64_t cus = 256; return (double)tiles / (double)((tiles + cus - 1) / cus * cus); };
+    const int64_t tiles_tall = ((m + BWH_BM - 1) / BWH_BM) * col_tiles * zs, tiles_low = ((m + BWG_BM - 1) / BWG_BM) * col_tiles * zs;
+    bool tall = fill_of(tiles_tall) * 1.2 >= fill_of(tiles_low) && (mode != 1 || m >= 512 * (int64_t)num_groups);
+    const int forced = bw_gemm_tile_rows.load(std::memory_order_relaxed);
+    if (forced == BWH_BM || forced == BWG_BM) tall = forced == BWH_BM;
+    tall = tall && ((uintptr_t)c_bf16 & 15) == 0;            // its epilogue stores 16 bytes per lane
+    const int64_t row_tiles = row_tiles_of(tall ? BWH_BM : BWG_BM);
     if (row_tiles > 65535 || (mode == 2 && num_groups > 65535)) return MXL_EINVAL;
     if (256 * k >= ((int64_t)1 << 31)) return MXL_EINVAL;     // byte offsets inside a tile's operand rows are 32-bit
     BwGemmArgs g{(const uint8_t*)a_codes, (const float*)a_sinv, (const uint8_t*)b_codes, (const float*)b_sinv, (uint16_t*)c_bf16,
                  m, n, k, b_rows_per_scale == 1 ? 0 : 7, mode, group_lens, num_groups};
-    const dim3 grid((unsigned)((n + BWG_BN - 1) / BWG_BN), (unsigned)row_tiles, (unsigned)(mode == 2 ? num_groups : 1));
+    const dim3 grid((unsigned)col_tiles, (unsigned)row_tiles, (unsigned)zs);
     hipStream_t st = (hipStream_t)stream;
     const bool sbu = b_rows_per_scale == BW;
     int rc;
-    if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) rc = sbu ? launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E4M3, false>(g, grid, st);
-    else if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) rc = sbu ? launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E4M3, false>(g, grid, st);
-    else if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) rc = sbu ? launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E5M2, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E4M3, MXL_FMT_E5M2, false>(g, grid, st);
-    else rc = sbu ? launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E5M2, true>(g, grid, st) : launch_bw_gemm<MXL_FMT_E5M2, MXL_FMT_E5M2, false>(g, grid, st);
+    if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) rc = launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
+    else if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) rc = launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
+    else if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) rc = launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
+    else rc = launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
     if (rc != MXL_OK) return rc;
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }
@@ -670,6 +920,12 @@ extern "C" int mxl_quantize_blockwise_weight(const void* w_bf16, int64_t batch, 
                                              void* q_T, void* sinv_T, void* stream) {
     if (batch < 1 || batch > 65535) return MXL_EINVAL;
     return bw_quant(w_bf16, n, k, fmt, nullptr, 0, (int)batch, q, sinv, q_T, sinv_T, true, stream);
+}
+
+extern "C" int mxl_blockwise_gemm_tile(int rows) {
+    if (rows != 0 && rows != BWG_BM && rows != BWH_BM) return MXL_EINVAL;
+    bw_gemm_tile_rows.store(rows, std::memory_order_relaxed);
+    return MXL_OK;
 }
 
 extern "C" int mxl_gemm_nt_blockwise(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv,

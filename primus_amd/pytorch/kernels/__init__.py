@@ -1215,6 +1215,12 @@ def _bw_scales(t, shape, what):
         raise ValueError(f"{what} must be contiguous float32 {tuple(shape)}")
 
 
+def set_blockwise_gemm_tile(rows: int) -> None:
+    """Output-tile height of the blockwise GEMMs for every later call: 128 or 256 rows, 0 = chosen by the shape (the
+    default).  Both give the same bits; a measuring and testing aid (``mxl_blockwise_gemm_tile``)."""
+    _lib.check(_lib.load().mxl_blockwise_gemm_tile(int(rows)), "mxl_blockwise_gemm_tile")
+
+
 def gemm_blockwise_nt_impl(a, a_scale_inv, b, b_scale_inv, group_lens: Optional[torch.Tensor] = None,
                            b_rows_per_scale: Optional[int] = None) -> torch.Tensor:
     """``gemm_fp8_impl`` / ``grouped_gemm_fp8_impl`` with ``granularity=BLOCKWISE`` in NT form

@@ -72,6 +72,16 @@ def test_zero_and_nonfinite_blocks(gpu):
     assert np.array_equal(s.cpu().numpy()[fin], ws[fin])
 
 
+@pytest.fixture(params=[128, 256])
+def tile(request):
+    """Runs the test once per output-tile height of the blockwise GEMMs (the library picks by the shape otherwise)."""
+    from primus_amd.pytorch import kernels as K
+
+    K.set_blockwise_gemm_tile(request.param)
+    yield request.param
+    K.set_blockwise_gemm_tile(0)
+
+
 def _bound(a_codes, sa, b_codes, sb, a_fmt, b_fmt, want32):
     da = np.abs(o.decode_fp8(a_codes, a_fmt)).astype(np.float64) * np.repeat(np.abs(sa).astype(np.float64), 128, axis=1)
     sbr = sb if sb.shape[0] == b_codes.shape[0] else np.repeat(sb, 128, axis=0)
@@ -82,7 +92,7 @@ def _bound(a_codes, sa, b_codes, sb, a_fmt, b_fmt, want32):
 
 @pytest.mark.parametrize("a_fmt,b_fmt", [(0, 0), (2, 2), (2, 0), (0, 2)])
 @pytest.mark.parametrize("m,n,k,per_row", [(70, 128, 128, False), (300, 256, 384, False), (129, 384, 1024, True), (1, 128, 256, True)])
-def test_gemm_against_the_oracle(gpu, a_fmt, b_fmt, m, n, k, per_row):
+def test_gemm_against_the_oracle(gpu, tile, a_fmt, b_fmt, m, n, k, per_row):
     from primus_amd.pytorch import kernels as K
 
     x = _x(m + n + k, m, k)
@@ -101,7 +111,7 @@ def test_gemm_against_the_oracle(gpu, a_fmt, b_fmt, m, n, k, per_row):
     assert err.max() <= 1e-2 * np.abs(want32).max()
 
 
-def test_gemm_is_exact_where_the_arithmetic_is(gpu):
+def test_gemm_is_exact_where_the_arithmetic_is(gpu, tile):
     """Small integers times power-of-two scales: every product and every sum is exact in float32 and in bf16."""
     from primus_amd.pytorch import kernels as K
 
@@ -116,6 +126,41 @@ def test_gemm_is_exact_where_the_arithmetic_is(gpu):
     got = K.gemm_blockwise_nt_impl(a.to(torch.float8_e4m3fn).to(gpu), sa.contiguous().to(gpu),
                                    b.to(torch.float8_e4m3fn).to(gpu), sb.contiguous().to(gpu))
     assert torch.equal(got.float().cpu(), want.bfloat16().float())
+
+
+def test_both_tile_heights_give_the_same_bits(gpu):
+    """Dense (weight factors and per-row factors), grouped forward and grouped weight gradient on shapes with ragged
+    row tiles, a half-empty last column tile and several K blocks: the 128 x 256 and the 256 x 256 kernel multiply and
+    add in the same order."""
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator().manual_seed(77)
+    m, n, k = 777, 640, 896
+    x = (torch.randn(m, k, generator=g) * torch.logspace(-2, 1, k)[None, :]).bfloat16().to(gpu)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(gpu)
+    lens = [300, 0, 1, 476]
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    wg = (torch.randn(len(lens), n, k, generator=g) * 0.05).bfloat16().to(gpu)
+    dy = torch.randn(m, n, generator=g).bfloat16().to(gpu)
+    xq, xs, _, _ = K.quantize_blockwise_impl(x, 0, rowwise=True, colwise=False)
+    wq, ws, _, _ = K.quantize_blockwise_weight_impl(w, 0, rowwise=True, colwise=False)
+    wr, wrs, _, _ = K.quantize_blockwise_impl(w, 0, rowwise=True, colwise=False)
+    wgq, wgs, _, _ = K.quantize_blockwise_weight_impl(wg, 0, rowwise=True, colwise=False)
+    _, _, xt, xts = K.quantize_blockwise_impl(x, 2, rowwise=False, colwise=True, group_lens=gl)
+    _, _, dt, dts = K.quantize_blockwise_impl(dy, 2, rowwise=False, colwise=True, group_lens=gl)
+    out = {}
+    try:
+        for rows in (128, 256):
+            K.set_blockwise_gemm_tile(rows)
+            out[rows] = (K.gemm_blockwise_nt_impl(xq, xs, wq, ws), K.gemm_blockwise_nt_impl(xq, xs, wr, wrs),
+                         K.gemm_blockwise_nt_impl(xq, xs, wgq, wgs, gl), K.grouped_gemm_blockwise_wgrad_impl(dt, dts, xt, xts, gl, m))
+    finally:
+        K.set_blockwise_gemm_tile(0)
+    for a, b in zip(out[128], out[256]):
+        assert torch.isfinite(a.float()).all() and a.float().abs().max() > 0
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    with pytest.raises(Exception):
+        K.set_blockwise_gemm_tile(64)
 
 
 def _cos(a, b):
@@ -245,7 +290,7 @@ def test_weight_batch_equals_the_oracle(gpu, fmt):
 
 @pytest.mark.parametrize("a_fmt,b_fmt", [(0, 0), (2, 2)])
 @pytest.mark.parametrize("lens,k", GROUPS)
-def test_grouped_gemms_against_the_oracle(gpu, a_fmt, b_fmt, lens, k):
+def test_grouped_gemms_against_the_oracle(gpu, tile, a_fmt, b_fmt, lens, k):
     from primus_amd.pytorch import kernels as K
 
     rows, G, n = sum(lens), len(lens), 256

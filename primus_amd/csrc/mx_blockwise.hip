@@ -710,17 +710,22 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
             const uint4 hi = *(const uint4*)(stg + row_off + piece[ks][1]);
             return bv8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
         };
-        bv8i fa8[2][2], fb8[2];      // [a fragment][ks], [ks]
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) fa8[i][ks] = frag(a_row + i * 32 * BW, ks);
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) fb8[ks] = frag(b_row, ks);
+        // fragment reads in the order the MFMAs want them: all eight waves read at once behind the barrier, and the
+        // first MFMA should wait for 4 of a wave's 12 reads, not for 10
         const float sbu = SBU ? fac[BWH_BM + wn * 128] : 0.f;
         float sa[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) sa[i] = fac[wm * 64 + i * 32 + lr];
+        __builtin_amdgcn_sched_barrier(0);
+        bv8i fa8[2][2], fb8[2];      // [a fragment][ks], [ks]
+        fb8[0] = frag(b_row, 0);
+        fa8[0][0] = frag(a_row, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        fb8[1] = frag(b_row, 1);
+        fa8[0][1] = frag(a_row, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        fa8[1][0] = frag(a_row + 32 * BW, 0);
+        fa8[1][1] = frag(a_row + 32 * BW, 1);
         bv16f zero;
 #pragma unroll
         for (int e = 0; e < 16; ++e) zero[e] = 0.f;

@@ -886,28 +886,54 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
     // Tile height: 256 x 256 tiles run a fifth to a quarter faster per flop than 128 x 256 ones (a third fewer operand
     // bytes from L2 per flop), so they win unless the coarser tiles leave that much more of the chip idle -- in the
     // last round of tiles, or in the ragged last tile of every group of a grouped forward (expected padding: half a
-    // tile per group, which a group of 512 rows pays back).  mxl_blockwise_gemm_tile overrides.
-    const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1;
-    auto row_tiles_of = [&](int64_t bm) { return mode == 1 ? m / bm + num_groups : (m + bm - 1) / bm; };
-    auto fill_of = [&](int64_t tiles) { const int64_t cus = 256; return (double)tiles / (double)((tiles + cus - 1) / cus * cus); };
-    const int64_t tiles_tall = ((m + BWH_BM - 1) / BWH_BM) * col_tiles * zs, tiles_low = ((m + BWG_BM - 1) / BWG_BM) * col_tiles * zs;
-    bool tall = fill_of(tiles_tall) * 1.2 >= fill_of(tiles_low) && (mode != 1 || m >= 512 * (int64_t)num_groups);
+    // tile per group, which a group of 512 rows pays back).  A dense GEMM may take both: the first rows on 256-row
+    // tiles in whole rounds, the rest on 128-row tiles (a second launch), whichever split has the lowest cost in
+    // rounds of tiles (a round of 128-row tiles = 0.5 x 1.25 rounds of 256-row tiles).  mxl_blockwise_gemm_tile overrides.
+    const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1, cus = 256;
+    auto rounds_of = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
+    const int64_t rt_tall = (m + BWH_BM - 1) / BWH_BM;
+    int64_t tall_tiles = 0;                                   // row tiles of 256 rows; the rows behind them take 128-row tiles
     const int forced = bw_gemm_tile_rows.load(std::memory_order_relaxed);
-    if (forced == BWH_BM || forced == BWG_BM) tall = forced == BWH_BM;
-    tall = tall && ((uintptr_t)c_bf16 & 15) == 0;            // its epilogue stores 16 bytes per lane
-    const int64_t row_tiles = row_tiles_of(tall ? BWH_BM : BWG_BM);
-    if (row_tiles > 65535 || (mode == 2 && num_groups > 65535)) return MXL_EINVAL;
+    if (((uintptr_t)c_bf16 & 15) != 0 || forced == BWG_BM) {
+        tall_tiles = 0;                                       // (the 256-row kernel's epilogue stores 16 bytes per lane)
+    } else if (forced == BWH_BM) {
+        tall_tiles = rt_tall;
+    } else if (mode == 0) {
+        double best = 1e30;
+        for (int64_t low = 0; low <= rt_tall && low <= 4 * cus; ++low) {       // `low` of the 256-row tiles cut in two
+            const int64_t low_rows = low == rt_tall ? m : low * BWH_BM;
+            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.625 * rounds_of((low_rows + BWG_BM - 1) / BWG_BM * col_tiles);
+            if (cost < best) {
+                best = cost;
+                tall_tiles = rt_tall - low;
+            }
+        }
+        const double all_low = 0.625 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles);
+        if (all_low <= best) tall_tiles = 0;
+    } else {
+        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.625 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles * zs);
+        if (cost_tall < cost_low && (mode != 1 || m >= 512 * (int64_t)num_groups)) tall_tiles = rt_tall;
+    }
     if (256 * k >= ((int64_t)1 << 31)) return MXL_EINVAL;     // byte offsets inside a tile's operand rows are 32-bit
-    BwGemmArgs g{(const uint8_t*)a_codes, (const float*)a_sinv, (const uint8_t*)b_codes, (const float*)b_sinv, (uint16_t*)c_bf16,
-                 m, n, k, b_rows_per_scale == 1 ? 0 : 7, mode, group_lens, num_groups};
-    const dim3 grid((unsigned)col_tiles, (unsigned)row_tiles, (unsigned)zs);
     hipStream_t st = (hipStream_t)stream;
     const bool sbu = b_rows_per_scale == BW;
-    int rc;
-    if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) rc = launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
-    else if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) rc = launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
-    else if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) rc = launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
-    else rc = launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
+    // rows [r0, r1) of a (dense: a sub-range; grouped: everything) on tiles of `tall ? 256 : 128` rows
+    auto run = [&](bool tall, int64_t r0, int64_t r1) {
+        const int64_t bm = tall ? BWH_BM : BWG_BM, rows = r1 - r0;
+        const int64_t row_tiles = mode == 1 ? rows / bm + num_groups : (rows + bm - 1) / bm;
+        if (row_tiles > 65535 || (mode == 2 && num_groups > 65535)) return (int)MXL_EINVAL;
+        BwGemmArgs g{(const uint8_t*)a_codes + r0 * k, (const float*)a_sinv + r0 * (k / BW), (const uint8_t*)b_codes, (const float*)b_sinv,
+                     (uint16_t*)c_bf16 + r0 * n, rows, n, k, b_rows_per_scale == 1 ? 0 : 7, mode, group_lens, num_groups};
+        const dim3 grid((unsigned)col_tiles, (unsigned)row_tiles, (unsigned)zs);
+        if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) return launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
+        if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) return launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
+        if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) return launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
+        return launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
+    };
+    int rc = MXL_OK;
+    const int64_t split = tall_tiles >= rt_tall ? m : tall_tiles * BWH_BM;     // (only a dense GEMM is ever split)
+    if (split > 0) rc = run(true, 0, split);
+    if (rc == MXL_OK && split < m) rc = run(false, split, m);
     if (rc != MXL_OK) return rc;
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }

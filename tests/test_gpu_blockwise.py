@@ -163,6 +163,28 @@ def test_both_tile_heights_give_the_same_bits(gpu):
         K.set_blockwise_gemm_tile(64)
 
 
+def test_a_dense_gemm_split_over_both_tile_heights_gives_the_same_bits(gpu):
+    """56.3 x 16 tiles of 256 x 256 are 3.5 rounds on 256 CUs: left to itself the library runs the first 48 row tiles
+    on 256-row tiles and the remaining rows (a ragged end included) on 128-row tiles, in two launches."""
+    from primus_amd.pytorch import kernels as K
+
+    g = torch.Generator().manual_seed(78)
+    m, n, k = 56 * 256 + 77, 4096, 256
+    x = torch.randn(m, k, generator=g).bfloat16().to(gpu)
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(gpu)
+    xq, xs, _, _ = K.quantize_blockwise_impl(x, 0, rowwise=True, colwise=False)
+    wr, wrs, _, _ = K.quantize_blockwise_impl(w, 2, rowwise=True, colwise=False)
+    auto = K.gemm_blockwise_nt_impl(xq, xs, wr, wrs)
+    try:
+        K.set_blockwise_gemm_tile(128)
+        low = K.gemm_blockwise_nt_impl(xq, xs, wr, wrs)
+    finally:
+        K.set_blockwise_gemm_tile(0)
+    assert auto.float().abs().max() > 0 and torch.equal(auto.view(torch.int16), low.view(torch.int16))
+    want = x[-300:].float() @ w.float().t()
+    assert _cos(auto[-300:], want) > 0.998
+
+
 def _cos(a, b):
     return torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item()
 

@@ -55,6 +55,8 @@ WORKLOADS = {
     "mixtral_8x7b_moe_fp8_tensorwise": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, tensorwise=True),
     # the 128-blockwise FP8 recipe (1 x 128 activation blocks, 128 x 128 weight blocks, fp32 scales; HYBRID formats) on the Llama MLP
     "llama3_8b_mlp_fp8_blockwise": dict(G=1, topk=1, tokens=8192, hidden=4096, fc1_out=14336, fc2_in=14336, routing="dense", seed=1002, fp4=False, blockwise=True, outliers=True),
+    # the same recipe on the headline shapes: grouped forward / dgrad (a row tile per group) and the grouped weight gradient
+    "mixtral_8x7b_moe_fp8_blockwise": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, blockwise=True),
     # the unquantised bf16 grouped GEMM (ops.grouped_gemm: what a layer outside the low-precision autocast runs) on the headline shapes
     "mixtral_8x7b_moe_bf16": dict(G=8, topk=2, tokens=16384, hidden=4096, fc1_out=28672, fc2_in=14336, routing="gauss_bias", seed=1003, fp4=False, bf16=True),
     # the same MLP with the RMSNorm that precedes fc1 in the layer (LayerNormColumnParallelLinear), folded into fc1's quantiser
@@ -602,7 +604,7 @@ def main():
     roofline = {
         # the MX and tensor-wise workloads run on the 4-slot ring kernel
         "kernel": "bf16_gemm_kernel<fwd/dgrad> (grouped_gemm_bf16)" if spec.get("bf16") else
-                  "bw_gemm_kernel<e4m3|e5m2,e4m3> (%s)" % fwd_name if spec.get("blockwise") else
+                  "bw_gemm256_kernel<e4m3|e5m2,weight factors> (%s)" % fwd_name if spec.get("blockwise") else
                   "%s<%s,%s,fwd/dgrad%s> (%s)" % ("mx_gemm_ring_kernel",
                                                    "e4m3|e5m2" if spec.get("tensorwise") else "e2m1" if act_fp4 else "e4m3",
                                                    "e2m1" if spec["fp4"] else "e4m3",

@@ -10,9 +10,10 @@
 //
 // scale = fp8_max / max(amax, 1e-12), codes = cast(clamp(x * scale)), scale_inv = 1 / scale, all fp32: the formula the
 // reference restates for its tensor-wise quantiser (:194-207) applied per block.  Arbitrary fp32 factors cannot ride on
-// the MFMA's E8M0 scale inputs, so this GEMM keeps two accumulator sets: the MFMAs of one K block of 128 add up in
-// the first (from zero), which is then multiplied into the second with the block's factors.  That takes registers
-// the 256 x 256 kernels do not have: the tile is 128 x 256 for 8 waves, 64 x 64 per wave, two waves per SIMD.
+// the MFMA's E8M0 scale inputs, so these GEMMs keep two kinds of accumulators: the MFMAs of one K block of 128 add up
+// in partial tiles (from zero), which are then multiplied into the real accumulators with the block's factors.  Two
+// kernels, both of 8 waves, two per SIMD: a 128 x 256 tile with all four partial tiles of a wave's 64 x 64 at once
+// (small problems), and a 256 x 256 tile whose waves own 64 x 128 and keep one column of partial tiles at a time.
 #include "mx_device.h"
 
 namespace mxl {

@@ -691,6 +691,7 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
         for (int e = 0; e < 8; ++e) issue_round(koff, wave_lds, e);
         issue_fac((uint32_t)__builtin_amdgcn_readfirstlane(k0 * 4), 0);
     }
+    const bool wave_live = __builtin_amdgcn_readfirstlane((int)(row0 + wm * 64 < pm && col0 + wn * 128 < pn)) != 0;
     int st = 0;
     for (int kb = k0; kb < k1; ++kb) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -704,6 +705,15 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
         const uint32_t in_koff = follows ? (uint32_t)__builtin_amdgcn_readfirstlane((kb + 1) * BW) : 0x80000000u;
         const uint32_t in_fac = follows ? (uint32_t)__builtin_amdgcn_readfirstlane((kb + 1) * 4) : 0x80000000u;
         const uint32_t in_base = wave_lds + (uint32_t)((st ^ 1) * BWH_STAGE);
+        if (!wave_live) {
+            // all of this wave's rows (or columns) lie past the end of the tile: it only keeps its share of the requests
+            // going, and the wave it shares a SIMD with has the MFMA pipe to itself
+#pragma unroll
+            for (int e = 0; e < 8; ++e) issue_round(in_koff, in_base, e);
+            issue_fac(in_fac, st ^ 1);
+            st ^= 1;
+            continue;
+        }
         const float* fac = fac_base + st * (BWH_BM + BWH_BN);
         const uint8_t* stg = bw_smem + st * BWH_STAGE;
         auto frag = [&](uint32_t row_off, int ks) __attribute__((always_inline)) {

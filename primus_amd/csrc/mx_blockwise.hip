@@ -438,8 +438,7 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
     const uint32_t ld_voff = (uint32_t)(ld_row * pk + 16 * ((t & 7) ^ ((ld_row >> 1) & 7)));
     const uint32_t round_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(64 * pk));
     const uint32_t wave_lds = smem_base + (uint32_t)(w * 1024);
-    auto issue = [&](int kb, int stage) __attribute__((always_inline)) {
-        const uint32_t koff = (uint32_t)__builtin_amdgcn_readfirstlane(kb * BW);
+    auto issue = [&](uint32_t koff, int stage) __attribute__((always_inline)) {
         const uint32_t base = wave_lds + (uint32_t)(stage * BWG_STAGE);
 #pragma unroll
         for (int e = 0; e < 2; ++e) bw_dma16(ra, base + e * 8192, ld_voff, koff + e * round_bytes);
@@ -447,23 +446,23 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
         for (int e = 0; e < 4; ++e) bw_dma16(rb, base + BWG_A + e * 8192, ld_voff, koff + e * round_bytes);
     };
     // Factors of a K block, one dword per lane straight into LDS (lane i of wave w lands at word 64 w + i): waves 0, 1
-    // fetch a's 128 row factors, waves 2 .. 5 b's 256 (per row of b, or one per 128 rows), waves 6, 7 nothing.  Rows
-    // past the end of the group or of b are dropped by the descriptors and read as zero.
-    const bool f_a = w < 2, f_any = w < 6;
-    const int frow = f_a ? t : t - BWG_BM;
+    // fetch a's 128 row factors, waves 2 .. 5 b's 256 (per row of b, or one per 128 rows); waves 6, 7 repeat the
+    // requests of waves 4, 5 (the same bytes to the same place), so that every wave has the same number of requests in
+    // flight.  Rows past the end of the group or of b are dropped by the descriptors and read as zero.
+    const int fw = w < 6 ? w : w - 2;
+    const bool f_a = fw < 2;
+    const int frow = f_a ? fw * 64 + l : fw * 64 + l - BWG_BM;
     const v4i rfac = f_a ? bw_rsrc(psa + row0 * kb_n, (pm - row0) * kb_n * 4)
                          : bw_rsrc(psb + (col0 >> sb_shift) * kb_n, (((pn - col0) + (1 << sb_shift) - 1) >> sb_shift) * kb_n * 4);
     const uint32_t fac_voff = (uint32_t)(((f_a ? frow : (frow >> sb_shift)) * kb_n) * 4);
-    const uint32_t fac_lds = smem_base + (uint32_t)(BWG_STAGES * BWG_STAGE + w * 256);
-    auto issue_fac = [&](int kb, int stage) __attribute__((always_inline)) {
-        if (f_any) {
-            uint32_t soff = (uint32_t)__builtin_amdgcn_readfirstlane(kb * 4);
-            const uint32_t lds = fac_lds + (uint32_t)(stage * BWG_FAC);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
-                         :
-                         : "s"(lds), "v"(fac_voff), "s"(rfac), "s"(soff)
-                         : "memory");
-        }
+    const uint32_t fac_lds = smem_base + (uint32_t)(BWG_STAGES * BWG_STAGE + fw * 256);
+    auto issue_fac = [&](uint32_t soff, int stage) __attribute__((always_inline)) {
+        const uint32_t lds = fac_lds + (uint32_t)(stage * BWG_FAC);
+        asm volatile("" : "+s"(soff));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                     :
+                     : "s"(lds), "v"(fac_voff), "s"(rfac), "s"(soff)
+                     : "memory");
     };
 
     bv16f acc[2][2];
@@ -474,91 +473,139 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    // pipeline: two blocks ahead.  A wave's requests for a block are its six operand rounds, then (waves 0 .. 5) one
-    // factor request; at the top of block kb everything but the requests of block kb + 1 has landed.
-    const int k0 = (int)kb0, k1 = (int)kb1;      // (block indices: k is below 2^23)
+    // pipeline: two blocks ahead.  A wave's requests for a block are its six operand rounds and one factor request; at the
+    // top of block kb everything but the seven requests of block kb + 1 has landed.  Requests for blocks past the range go
+    // out as well, at an offset of 2 GiB, where the descriptors' range check drops them (or, under an operand that large,
+    // they fetch bytes of it that nobody reads): the request count per block is then a constant, and the block's
+    // instructions stay one basic block whose order can be pinned (a branch around the requests lets the compiler sink
+    // the MFMAs behind every load).
+    constexpr uint32_t DROP = 0x80000000u;
+    const int k0 = __builtin_amdgcn_readfirstlane((int)kb0), k1 = __builtin_amdgcn_readfirstlane((int)kb1);   // (k is below 2^23)
     if (k0 < k1) {
-        issue(k0, 0);
-        issue_fac(k0, 0);
-        if (k0 + 1 < k1) {
-            issue(k0 + 1, 1);
-            issue_fac(k0 + 1, 1);
-        }
+        issue((uint32_t)(k0 * BW), 0);
+        issue_fac((uint32_t)(k0 * 4), 0);
+        const bool two = k0 + 1 < k1;
+        issue(two ? (uint32_t)((k0 + 1) * BW) : DROP, 1);
+        issue_fac(two ? (uint32_t)((k0 + 1) * 4) : DROP, 1);
     }
+    // fragment addressing: lane (lr, g) reads the 16-byte pieces 4 ks + 2 h + g of its row, swizzled by the row
+    const int swz = (lr >> 1) & 7;
+    uint32_t piece[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) piece[ks][h] = (uint32_t)(16 * ((4 * ks + 2 * h + g) ^ swz));
+    const uint32_t a_row = (uint32_t)((wm * 64 + lr) * BW), b_row = (uint32_t)(BWG_A + (wn * 64 + lr) * BW);
     int st = 0, st2 = 2;                          // stage of block kb, stage of block kb + 2
     for (int kb = k0; kb < k1; ++kb) {
-        if (kb + 1 >= k1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else if (f_any) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
         __syncthreads();       // block kb and its factors are in LDS for every wave; every wave has left block kb - 1
-        // the requests of block kb + 2 go out one behind each MFMA of this block (six operand rounds, then the
-        // factors): all at once, the 8 waves' 56 requests queue at the CU's address unit for ~900 clocks with every
-        // wave waiting behind its own
         const bool more = kb + 2 < k1;
-        const uint32_t in_koff = (uint32_t)__builtin_amdgcn_readfirstlane((kb + 2) * BW);
+        const uint32_t in_koff = more ? (uint32_t)__builtin_amdgcn_readfirstlane((kb + 2) * BW) : DROP;
+        const uint32_t in_fac = more ? (uint32_t)__builtin_amdgcn_readfirstlane((kb + 2) * 4) : DROP;
         const uint32_t in_base = wave_lds + (uint32_t)(st2 * BWG_STAGE);
         const float* fac = fac_base + st * (BWG_BM + BWG_BN);
-        const uint8_t* sa_ = bw_smem + st * BWG_STAGE;
-        const uint8_t* sb_ = sa_ + BWG_A;
-        bv16f part[2][2];
+        const uint8_t* stg = bw_smem + st * BWG_STAGE;
+        auto frag = [&](uint32_t row_off, int ks) __attribute__((always_inline)) {
+            const uint4 lo = *(const uint4*)(stg + row_off + piece[ks][0]);
+            const uint4 hi = *(const uint4*)(stg + row_off + piece[ks][1]);
+            return bv8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        };
+        const float sbu = SBU ? fac[BWG_BM + wn * 64] : 0.f;
+        float sa[2];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            bv8i fa8[2], fb8[2];
+        for (int i = 0; i < 2; ++i) sa[i] = fac[wm * 64 + i * 32 + lr];
+        __builtin_amdgcn_sched_barrier(0);
+        // fragment reads in the order the MFMAs want them (tile (0, 0) first)
+        bv8i fa8[2][2], fb8[2][2];      // [fragment][ks]
+        fb8[0][0] = frag(b_row, 0);
+        fa8[0][0] = frag(a_row, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        fb8[0][1] = frag(b_row, 1);
+        fa8[0][1] = frag(a_row, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        fb8[1][0] = frag(b_row + 32 * BW, 0);
+        fb8[1][1] = frag(b_row + 32 * BW, 1);
+        fa8[1][0] = frag(a_row + 32 * BW, 0);
+        fa8[1][1] = frag(a_row + 32 * BW, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        bv16f zero;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                // lane (lr, g) of a 32-row fragment holds bytes 16 g .. 16 g + 15 and 32 + 16 g .. of the K step
-                const int ra_ = wm * 64 + i * 32 + lr, rb_ = wn * 64 + i * 32 + lr;
-                const uint4 alo = *(const uint4*)(sa_ + ra_ * BW + 16 * ((4 * ks + g) ^ ((ra_ >> 1) & 7)));
-                const uint4 ahi = *(const uint4*)(sa_ + ra_ * BW + 16 * ((4 * ks + 2 + g) ^ ((ra_ >> 1) & 7)));
-                const uint4 blo = *(const uint4*)(sb_ + rb_ * BW + 16 * ((4 * ks + g) ^ ((rb_ >> 1) & 7)));
-                const uint4 bhi = *(const uint4*)(sb_ + rb_ * BW + 16 * ((4 * ks + 2 + g) ^ ((rb_ >> 1) & 7)));
-                fa8[i] = bv8i{(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
-                fb8[i] = bv8i{(int)blo.x, (int)blo.y, (int)blo.z, (int)blo.w, (int)bhi.x, (int)bhi.y, (int)bhi.z, (int)bhi.w};
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    bv16f zero;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) zero[e] = 0.f;
-                    // the b fragment is the first operand: a lane ends up with 4 consecutive output columns
-                    part[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j], fa8[i], ks == 0 ? zero : part[i][j], CB, BL, 0,
-                                                                               127, 0, 127);
-                    const int mi = 4 * ks + 2 * i + j;      // (a constant after unrolling)
-                    if (more) {
-                        if (mi < 2) bw_dma16(ra, in_base + mi * 8192, ld_voff, in_koff + mi * round_bytes);
-                        else if (mi < 6) bw_dma16(rb, in_base + BWG_A + (mi - 2) * 8192, ld_voff, in_koff + (mi - 2) * round_bytes);
-                        else if (mi == 6) issue_fac(kb + 2, st2);
-                    }
-                }
-        }
+        for (int e = 0; e < 16; ++e) zero[e] = 0.f;
         // acc += part * (sa[row] * sb[col]): lane (lr, g), register e = 4 q + r of tile (i, j) is row i * 32 + lr,
         // column j * 32 + 8 q + 4 g + r of the wave's 64 x 64
-        const float sbu = SBU ? fac[BWG_BM + wn * 64] : 0.f;
+        auto scale_in = [&](const bv16f& part, int i, int j) __attribute__((always_inline)) {
+            const float sab = sa[i] * sbu;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (SBU) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = fmaf(part[4 * q + e], sab, acc[i][j][4 * q + e]);
+                } else {
+                    const float4 sb = *(const float4*)(&fac[BWG_BM + wn * 64 + j * 32 + 8 * q + 4 * g]);
+                    acc[i][j][4 * q + 0] = fmaf(part[4 * q + 0], sa[i] * sb.x, acc[i][j][4 * q + 0]);
+                    acc[i][j][4 * q + 1] = fmaf(part[4 * q + 1], sa[i] * sb.y, acc[i][j][4 * q + 1]);
+                    acc[i][j][4 * q + 2] = fmaf(part[4 * q + 2], sa[i] * sb.z, acc[i][j][4 * q + 2]);
+                    acc[i][j][4 * q + 3] = fmaf(part[4 * q + 3], sa[i] * sb.w, acc[i][j][4 * q + 3]);
+                }
+            }
+        };
+        // request number mi of block kb + 2, one behind each of this block's first seven MFMAs: six operand rounds, the factors
+#define REQ(mi)                                                                                                        \
+    do {                                                                                                               \
+        if ((mi) < 2) bw_dma16(ra, in_base + (mi) * 8192, ld_voff, in_koff + (mi) * round_bytes);                          \
+        else if ((mi) < 6) bw_dma16(rb, in_base + BWG_A + ((mi) - 2) * 8192, ld_voff, in_koff + ((mi) - 2) * round_bytes); \
+        else if ((mi) == 6) issue_fac(in_fac, st2);                                                                    \
+    } while (0)
+        // The four 32 x 32 tiles one after the other, two MFMAs each (the b fragment is the first operand: a lane ends up
+        // with 4 consecutive output columns); the FMAs of a tile run in the shadow of the next tile's MFMAs.
+        bv16f part[4];
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            const int i = tl >> 1, j = tl & 1;
+            part[tl] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j][0], fa8[i][0], zero, CB, BL, 0, 127, 0, 127);
+            REQ(2 * tl);
+            part[tl] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[j][1], fa8[i][1], part[tl], CB, BL, 0, 127, 0, 127);
+            REQ(2 * tl + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (tl > 0) scale_in(part[tl - 1], (tl - 1) >> 1, (tl - 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#undef REQ
+        scale_in(part[3], 1, 1);
+        st = st == BWG_STAGES - 1 ? 0 : st + 1;
+        st2 = st2 == BWG_STAGES - 1 ? 0 : st2 + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // (dropped requests included: none may outlive the workgroup's LDS)
+    if ((((uintptr_t)pc_out) & 15) == 0) {
+        __syncthreads();   // no request of any wave still writes LDS: the stages are free
+        // Output through a wave-private LDS patch of 32 rows x 128 bytes, one a fragment at a time: a lane's four
+        // consecutive bf16 go in as 8 bytes and come out as 16 bytes per lane, 8 rows x 128 contiguous bytes per store
+        // instruction (16-byte pieces XOR-swizzled by the row).
+        uint8_t* const patch = bw_smem + w * (32 * 128);
+        const bool cols_in = col0 + wn * 64 < pn;        // (n is a multiple of 128: the wave's columns are in or out as a whole)
+        const int er = l >> 3, ep = l & 7;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const float sa = fac[wm * 64 + i * 32 + lr];
-            const float sab = sa * sbu;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    if (SBU) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = fmaf(part[i][j][4 * q + e], sab, acc[i][j][4 * q + e]);
-                    } else {
-                        const float4 sb = *(const float4*)(&fac[BWG_BM + wn * 64 + j * 32 + 8 * q + 4 * g]);
-                        acc[i][j][4 * q + 0] = fmaf(part[i][j][4 * q + 0], sa * sb.x, acc[i][j][4 * q + 0]);
-                        acc[i][j][4 * q + 1] = fmaf(part[i][j][4 * q + 1], sa * sb.y, acc[i][j][4 * q + 1]);
-                        acc[i][j][4 * q + 2] = fmaf(part[i][j][4 * q + 2], sa * sb.z, acc[i][j][4 * q + 2]);
-                        acc[i][j][4 * q + 3] = fmaf(part[i][j][4 * q + 3], sa * sb.w, acc[i][j][4 * q + 3]);
-                    }
+                    const bv4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
+                                     (__bf16)acc[i][j][4 * q + 3]};
+                    *(bv4bf*)(patch + lr * 128 + 16 * ((4 * j + q) ^ ((lr >> 1) & 7)) + 8 * g) = o;
                 }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int r = 8 * u + er;
+                const uint4 v = *(const uint4*)(patch + r * 128 + 16 * (ep ^ ((r >> 1) & 7)));
+                const int64_t m = row0 + wm * 64 + i * 32 + r;
+                if (cols_in && m < pm) store16_streaming(pc_out + m * pn + col0 + wn * 64 + 8 * ep, v);
+            }
         }
-        st = st == BWG_STAGES - 1 ? 0 : st + 1;
-        st2 = st2 == BWG_STAGES - 1 ? 0 : st2 + 1;
+        return;
     }
+    // an output that is only 8-byte aligned: stored straight from the accumulator layout
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int64_t m = row0 + wm * 64 + i * 32 + lr;
@@ -894,12 +941,12 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
     if (k == 0 && mode != 2) return MXL_EINVAL;
     if ((((uintptr_t)a_codes | (uintptr_t)b_codes) & 15) != 0) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
-    // Tile height: 256 x 256 tiles run a fifth to a quarter faster per flop than 128 x 256 ones (a third fewer operand
+    // Tile height: 256 x 256 tiles run about 15 % faster per flop than 128 x 256 ones (a third fewer operand
     // bytes from L2 per flop), so they win unless the coarser tiles leave that much more of the chip idle -- in the
     // last round of tiles, or in the ragged last tile of every group of a grouped forward (expected padding: half a
     // tile per group, which a group of 512 rows pays back).  A dense GEMM may take both: the first rows on 256-row
     // tiles in whole rounds, the rest on 128-row tiles (a second launch), whichever split has the lowest cost in
-    // rounds of tiles (a round of 128-row tiles = 0.5 x 1.25 rounds of 256-row tiles).  mxl_blockwise_gemm_tile overrides.
+    // rounds of tiles (a round of 128-row tiles = 0.5 x 1.15 rounds of 256-row tiles).  mxl_blockwise_gemm_tile overrides.
     const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1, cus = 256;
     auto rounds_of = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
     const int64_t rt_tall = (m + BWH_BM - 1) / BWH_BM;
@@ -913,16 +960,16 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
         double best = 1e30;
         for (int64_t low = 0; low <= rt_tall && low <= 4 * cus; ++low) {       // `low` of the 256-row tiles cut in two
             const int64_t low_rows = low == rt_tall ? m : low * BWH_BM;
-            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.625 * rounds_of((low_rows + BWG_BM - 1) / BWG_BM * col_tiles);
+            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.575 * rounds_of((low_rows + BWG_BM - 1) / BWG_BM * col_tiles);
             if (cost < best) {
                 best = cost;
                 tall_tiles = rt_tall - low;
             }
         }
-        const double all_low = 0.625 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles);
+        const double all_low = 0.575 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles);
         if (all_low <= best) tall_tiles = 0;
     } else {
-        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.625 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles * zs);
+        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.575 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles * zs);
         if (cost_tall < cost_low && (mode != 1 || m >= 512 * (int64_t)num_groups)) tall_tiles = rt_tall;
     }
     if (256 * k >= ((int64_t)1 << 31)) return MXL_EINVAL;     // byte offsets inside a tile's operand rows are 32-bit

@@ -340,6 +340,7 @@ struct BwGemmArgs {
     const float* sb;
     uint16_t* c;
     int64_t m, n, k;
+    int64_t ldc;        // elements between rows of c (n, unless the launch covers a range of a wider output's columns)
     int sb_shift;
     // mode 0: one dense GEMM.  mode 1 (forward / dgrad of a grouped linear): the rows of a are split by group_lens, b is
     // [num_groups, n, k] with its factors per group, a row tile belongs to one group.  mode 2 (wgrad of a grouped
@@ -423,7 +424,8 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
     const int sb_shift = p.sb_shift;
     const float* const psa = p.sa;
     const float* const psb = p.sb + b_group * (pn >> sb_shift) * kb_n;
-    uint16_t* const pc_out = p.c + c_group * p.m * pn;
+    uint16_t* const pc_out = p.c + c_group * p.m * p.ldc;
+    const int64_t ldc = p.ldc;
     // descriptors: from the tile's first row to the last row that may be read (the group's / the operand's end for a,
     // the end of the group's matrix for b); offsets inside them are 32-bit (the host bounds 256 rows x k)
     const uint8_t* const b_mat = p.b + b_group * pn * pk;
@@ -600,7 +602,7 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
                 const int r = 8 * u + er;
                 const uint4 v = *(const uint4*)(patch + r * 128 + 16 * (ep ^ ((r >> 1) & 7)));
                 const int64_t m = row0 + wm * 64 + i * 32 + r;
-                if (cols_in && m < pm) store16_streaming(pc_out + m * pn + col0 + wn * 64 + 8 * ep, v);
+                if (cols_in && m < pm) store16_streaming(pc_out + m * ldc + col0 + wn * 64 + 8 * ep, v);
             }
         }
         return;
@@ -618,7 +620,7 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
                 if (col >= pn) continue;     // (n is a multiple of 128: a quad is in or out as a whole)
                 const bv4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
                                  (__bf16)acc[i][j][4 * q + 3]};
-                *(bv4bf*)(pc_out + m * pn + col) = o;
+                *(bv4bf*)(pc_out + m * ldc + col) = o;
             }
     }
 }
@@ -685,7 +687,8 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
     const int64_t pm = m_end, pk = p.k, pn = p.n;
     const int sb_shift = p.sb_shift;
     const float* const psb = p.sb + b_group * (pn >> sb_shift) * kb_n;
-    uint16_t* const pc_out = p.c + c_group * p.m * pn;
+    uint16_t* const pc_out = p.c + c_group * p.m * p.ldc;
+    const int64_t ldc = p.ldc;
     // descriptors: from the tile's first row to the last row that may be read (the group's / the operand's end for a,
     // the end of the group's matrix for b); offsets inside them are 32-bit (the host bounds 256 rows x k)
     const v4i ra = bw_rsrc(p.a + row0 * pk, (pm - row0) * pk);
@@ -864,7 +867,7 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
             const int r = 4 * u + er;
             const uint4 v = *(const uint4*)(patch + r * 256 + 16 * (ep ^ (r & 15)));
             const int64_t m = row0 + wm * 64 + i * 32 + r;
-            if (cols_in && m < pm) store16_streaming(pc_out + m * pn + col0 + wn * 128 + 8 * ep, v);
+            if (cols_in && m < pm) store16_streaming(pc_out + m * ldc + col0 + wn * 128 + 8 * ep, v);
         }
     }
 }
@@ -944,54 +947,66 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
     // Tile height: 256 x 256 tiles run about 15 % faster per flop than 128 x 256 ones (a third fewer operand
     // bytes from L2 per flop), so they win unless the coarser tiles leave that much more of the chip idle -- in the
     // last round of tiles, or in the ragged last tile of every group of a grouped forward (expected padding: half a
-    // tile per group, which a group of 512 rows pays back).  A dense GEMM may take both: the first rows on 256-row
-    // tiles in whole rounds, the rest on 128-row tiles (a second launch), whichever split has the lowest cost in
-    // rounds of tiles (a round of 128-row tiles = 0.5 x 1.15 rounds of 256-row tiles).  mxl_blockwise_gemm_tile overrides.
+    // tile per group, which a group of 512 rows pays back).  A dense GEMM may take both: most of the output on 256-row
+    // tiles in whole rounds, its last rows or its last columns on 128-row tiles (a second launch), whichever split has
+    // the lowest cost in rounds of tiles (a round of 128-row tiles = 0.5 x 1.15 rounds of 256-row tiles).
+    // mxl_blockwise_gemm_tile overrides.
     const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1, cus = 256;
     auto rounds_of = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
-    const int64_t rt_tall = (m + BWH_BM - 1) / BWH_BM;
-    int64_t tall_tiles = 0;                                   // row tiles of 256 rows; the rows behind them take 128-row tiles
+    const int64_t rt_tall = (m + BWH_BM - 1) / BWH_BM, rt_low = (m + BWG_BM - 1) / BWG_BM;
+    int64_t low_rows = 0, low_cols = 0;                       // what the 128-row tiles take: the last rows, or the last columns
+    bool all_low = false;
     const int forced = bw_gemm_tile_rows.load(std::memory_order_relaxed);
     if (((uintptr_t)c_bf16 & 15) != 0 || forced == BWG_BM) {
-        tall_tiles = 0;                                       // (the 256-row kernel's epilogue stores 16 bytes per lane)
+        all_low = true;                                       // (the 256-row kernel's epilogue stores 16 bytes per lane)
     } else if (forced == BWH_BM) {
-        tall_tiles = rt_tall;
     } else if (mode == 0) {
-        double best = 1e30;
-        for (int64_t low = 0; low <= rt_tall && low <= 4 * cus; ++low) {       // `low` of the 256-row tiles cut in two
-            const int64_t low_rows = low == rt_tall ? m : low * BWH_BM;
-            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.575 * rounds_of((low_rows + BWG_BM - 1) / BWG_BM * col_tiles);
-            if (cost < best) {
-                best = cost;
-                tall_tiles = rt_tall - low;
-            }
+        double best = rounds_of(rt_tall * col_tiles);
+        for (int64_t low = 1; low < rt_tall && low <= 4 * cus; ++low) {        // `low` of the 256-row tiles cut in two
+            const int64_t rows = m - (rt_tall - low) * BWH_BM;
+            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.575 * rounds_of((rows + BWG_BM - 1) / BWG_BM * col_tiles);
+            if (cost < best) best = cost, low_rows = rows, low_cols = 0;
         }
-        const double all_low = 0.575 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles);
-        if (all_low <= best) tall_tiles = 0;
+        for (int64_t low = 1; low < col_tiles && low <= 4 * cus; ++low) {      // the last `low` column tiles
+            const double cost = rounds_of(rt_tall * (col_tiles - low)) + 0.575 * rounds_of(rt_low * low);
+            if (cost < best) best = cost, low_rows = 0, low_cols = n - (col_tiles - low) * BWG_BN;
+        }
+        if (0.575 * rounds_of(rt_low * col_tiles) <= best) all_low = true;
     } else {
-        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.575 * rounds_of((m + BWG_BM - 1) / BWG_BM * col_tiles * zs);
-        if (cost_tall < cost_low && (mode != 1 || m >= 512 * (int64_t)num_groups)) tall_tiles = rt_tall;
+        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.575 * rounds_of(rt_low * col_tiles * zs);
+        all_low = !(cost_tall < cost_low && (mode != 1 || m >= 512 * (int64_t)num_groups));
     }
     if (256 * k >= ((int64_t)1 << 31)) return MXL_EINVAL;     // byte offsets inside a tile's operand rows are 32-bit
     hipStream_t st = (hipStream_t)stream;
     const bool sbu = b_rows_per_scale == BW;
-    // rows [r0, r1) of a (dense: a sub-range; grouped: everything) on tiles of `tall ? 256 : 128` rows
-    auto run = [&](bool tall, int64_t r0, int64_t r1) {
-        const int64_t bm = tall ? BWH_BM : BWG_BM, rows = r1 - r0;
+    const int sb_shift = sbu ? 7 : 0;
+    // rows [r0, r1) x columns [c0, c1) of the output (a dense GEMM: any range whose c0 is a multiple of 256; grouped:
+    // everything) on tiles of `tall ? 256 : 128` rows
+    auto run = [&](bool tall, int64_t r0, int64_t r1, int64_t c0, int64_t c1) {
+        const int64_t bm = tall ? BWH_BM : BWG_BM, rows = r1 - r0, cols = c1 - c0;
         const int64_t row_tiles = mode == 1 ? rows / bm + num_groups : (rows + bm - 1) / bm;
         if (row_tiles > 65535 || (mode == 2 && num_groups > 65535)) return (int)MXL_EINVAL;
-        BwGemmArgs g{(const uint8_t*)a_codes + r0 * k, (const float*)a_sinv + r0 * (k / BW), (const uint8_t*)b_codes, (const float*)b_sinv,
-                     (uint16_t*)c_bf16 + r0 * n, rows, n, k, b_rows_per_scale == 1 ? 0 : 7, mode, group_lens, num_groups};
-        const dim3 grid((unsigned)col_tiles, (unsigned)row_tiles, (unsigned)zs);
+        BwGemmArgs g{(const uint8_t*)a_codes + r0 * k, (const float*)a_sinv + r0 * (k / BW), (const uint8_t*)b_codes + c0 * k,
+                     (const float*)b_sinv + (c0 >> sb_shift) * (k / BW), (uint16_t*)c_bf16 + r0 * n + c0, rows, cols, k, n, sb_shift, mode,
+                     group_lens, num_groups};
+        const dim3 grid((unsigned)((cols + BWG_BN - 1) / BWG_BN), (unsigned)row_tiles, (unsigned)zs);
         if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E4M3) return launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
         if (a_fmt == MXL_FMT_E5M2 && b_fmt == MXL_FMT_E4M3) return launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E4M3>(g, grid, sbu, tall, st);
         if (a_fmt == MXL_FMT_E4M3 && b_fmt == MXL_FMT_E5M2) return launch_bw_gemm_fmt<MXL_FMT_E4M3, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
         return launch_bw_gemm_fmt<MXL_FMT_E5M2, MXL_FMT_E5M2>(g, grid, sbu, tall, st);
     };
-    int rc = MXL_OK;
-    const int64_t split = tall_tiles >= rt_tall ? m : tall_tiles * BWH_BM;     // (only a dense GEMM is ever split)
-    if (split > 0) rc = run(true, 0, split);
-    if (rc == MXL_OK && split < m) rc = run(false, split, m);
+    int rc;
+    if (all_low) {
+        rc = run(false, 0, m, 0, n);
+    } else if (low_rows > 0) {
+        rc = run(true, 0, m - low_rows, 0, n);
+        if (rc == MXL_OK) rc = run(false, m - low_rows, m, 0, n);
+    } else if (low_cols > 0) {
+        rc = run(true, 0, m, 0, n - low_cols);
+        if (rc == MXL_OK) rc = run(false, 0, m, n - low_cols, n);
+    } else {
+        rc = run(true, 0, m, 0, n);
+    }
     if (rc != MXL_OK) return rc;
     return hipGetLastError() == hipSuccess ? MXL_OK : MXL_ELAUNCH;
 }

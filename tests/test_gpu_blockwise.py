@@ -163,13 +163,15 @@ def test_both_tile_heights_give_the_same_bits(gpu):
         K.set_blockwise_gemm_tile(64)
 
 
-def test_a_dense_gemm_split_over_both_tile_heights_gives_the_same_bits(gpu):
+@pytest.mark.parametrize("m,n", [(56 * 256 + 77, 4096), (4096, 14336)])
+def test_a_dense_gemm_split_over_both_tile_heights_gives_the_same_bits(gpu, m, n):
     """56.3 x 16 tiles of 256 x 256 are 3.5 rounds on 256 CUs: left to itself the library runs the first 48 row tiles
-    on 256-row tiles and the remaining rows (a ragged end included) on 128-row tiles, in two launches."""
+    on 256-row tiles and the remaining rows (a ragged end included) on 128-row tiles, in two launches; with 16 x 56
+    tiles it is the last 8 column tiles that go to the 128-row kernel."""
     from primus_amd.pytorch import kernels as K
 
     g = torch.Generator().manual_seed(78)
-    m, n, k = 56 * 256 + 77, 4096, 256
+    k = 256
     x = torch.randn(m, k, generator=g).bfloat16().to(gpu)
     w = (torch.randn(n, k, generator=g) * 0.05).bfloat16().to(gpu)
     xq, xs, _, _ = K.quantize_blockwise_impl(x, 0, rowwise=True, colwise=False)

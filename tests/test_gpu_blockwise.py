@@ -442,3 +442,69 @@ def test_operator_replays_under_a_graph(gpu):
         torch.cuda.synchronize()
         for u, v in zip(got, want):
             assert torch.equal(u.view(torch.int16), v.view(torch.int16)), seed
+
+
+def _exact_operands(gen, m, n, k, per_row, dev):
+    """Small integers times power-of-two factors: every product and partial sum is exact in float32 whatever the order."""
+    a = torch.randint(-2, 3, (m, k), generator=gen, device=dev).float()
+    b = torch.randint(-2, 3, (n, k), generator=gen, device=dev).float()
+    sa = torch.tensor([0.5, 1.0, 2.0, 4.0], device=dev)[torch.randint(0, 4, (m, k // 128), generator=gen, device=dev)]
+    sb_rows = n if per_row else n // 128
+    sb = torch.tensor([0.25, 1.0, 2.0], device=dev)[torch.randint(0, 3, (sb_rows, k // 128), generator=gen, device=dev)]
+    bs = b * (sb if per_row else sb.repeat_interleave(128, 0)).repeat_interleave(128, 1)
+    want = ((a * sa.repeat_interleave(128, 1)) @ bs.t()).bfloat16()
+    return a, sa.contiguous(), b, sb.contiguous(), want
+
+
+@pytest.mark.parametrize("m,n,k,per_row", [(8192, 14336, 4096, False), (8192, 4096, 14336, False), (14336, 4096, 8192, True)])
+def test_llama_mlp_shapes_at_full_size_are_exact(gpu, m, n, k, per_row):
+    """The three GEMMs of the Llama-3-8B MLP under this recipe at their real sizes (forward, dgrad, weight gradient: the
+    last one is split over both tile heights) on operands whose exact result does not depend on the order of the sums."""
+    from primus_amd.pytorch import kernels as K
+
+    gen = torch.Generator(device=gpu).manual_seed(m + n + k)
+    a, sa, b, sb, want = _exact_operands(gen, m, n, k, per_row, gpu)
+    fa, fb = (torch.float8_e5m2, torch.float8_e5m2) if per_row else (torch.float8_e4m3fn, torch.float8_e4m3fn)
+    got = K.gemm_blockwise_nt_impl(a.to(fa), sa, b.to(fb), sb, b_rows_per_scale=1 if per_row else 128)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_seeded_sweep_of_ragged_gemms_under_every_tile_height(gpu):
+    """40 random shapes (dense with either kind of b factors, grouped forward with empty and ragged groups): the 128-row
+    kernel, the 256-row kernel and the library's choice give the same bits, and they are the exact result."""
+    import random
+
+    from primus_amd.pytorch import kernels as K
+
+    rnd = random.Random(2024)
+    gen = torch.Generator(device=gpu).manual_seed(2024)
+    try:
+        for case in range(40):
+            n, k = 128 * rnd.randint(1, 10), 128 * rnd.randint(1, 5)
+            if case % 2 == 0:
+                m, per_row = rnd.choice([1, 127, 129, 255, 257, 700, rnd.randint(1, 3000)]), rnd.random() < 0.5
+                a, sa, b, sb, want = _exact_operands(gen, m, n, k, per_row, gpu)
+                run = lambda: K.gemm_blockwise_nt_impl(a.to(torch.float8_e4m3fn), sa, b.to(torch.float8_e5m2), sb,
+                                                       b_rows_per_scale=1 if per_row else 128)
+            else:
+                lens = [rnd.choice([0, 1, 128, 129, 255, 256, 257, 513, rnd.randint(1, 900)]) for _ in range(rnd.randint(1, 7))]
+                lens[rnd.randrange(len(lens))] += 1
+                m, G = sum(lens), len(lens)
+                a, sa, _, _, _ = _exact_operands(gen, m, 128, k, False, gpu)
+                ws = [_exact_operands(gen, 1, n, k, False, gpu) for _ in range(G)]
+                b, sb = torch.stack([w[2] for w in ws]), torch.stack([w[3] for w in ws])
+                asc, rows, off = a * sa.repeat_interleave(128, 1), [], 0
+                for e, ln in enumerate(lens):
+                    rows.append(asc[off:off + ln] @ (b[e] * sb[e].repeat_interleave(128, 0).repeat_interleave(128, 1)).t())
+                    off += ln
+                want = torch.cat(rows).bfloat16()
+                gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+                run = lambda: K.gemm_blockwise_nt_impl(a.to(torch.float8_e4m3fn), sa, b.to(torch.float8_e4m3fn), sb, gl)
+            outs = []
+            for rows_ in (128, 256, 0):
+                K.set_blockwise_gemm_tile(rows_)
+                outs.append(run())
+            for o_ in outs:
+                assert torch.equal(o_.view(torch.int16), want.view(torch.int16)), (case, m, n, k)
+    finally:
+        K.set_blockwise_gemm_tile(0)

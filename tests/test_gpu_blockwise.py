@@ -508,3 +508,23 @@ def test_seeded_sweep_of_ragged_gemms_under_every_tile_height(gpu):
                 assert torch.equal(o_.view(torch.int16), want.view(torch.int16)), (case, m, n, k)
     finally:
         K.set_blockwise_gemm_tile(0)
+
+
+def test_mixtral_routing_at_full_row_count_is_exact(gpu):
+    """32 768 routed rows in the benchmark's eight ragged groups against per-group weights (n and k of fc2's dgrad):
+    the grouped forward kernel on 256-row tiles, exact on exactly representable operands."""
+    from primus_amd.pytorch import kernels as K
+
+    lens = [3615, 1451, 2686, 6852, 6436, 4634, 1493, 5601]
+    m, G, n, k = sum(lens), len(lens), 4096, 4096
+    gen = torch.Generator(device=gpu).manual_seed(11)
+    a, sa, _, _, _ = _exact_operands(gen, m, 128, k, False, gpu)
+    ws = [_exact_operands(gen, 1, n, k, False, gpu) for _ in range(G)]
+    b, sb = torch.stack([w[2] for w in ws]), torch.stack([w[3] for w in ws])
+    gl = torch.tensor(lens, dtype=torch.int64, device=gpu)
+    got = K.gemm_blockwise_nt_impl(a.to(torch.float8_e4m3fn), sa, b.to(torch.float8_e4m3fn), sb, gl)
+    asc, off = a * sa.repeat_interleave(128, 1), 0
+    for e, ln in enumerate(lens):
+        want = (asc[off:off + ln] @ (b[e] * sb[e].repeat_interleave(128, 0).repeat_interleave(128, 1)).t()).bfloat16()
+        assert torch.equal(got[off:off + ln].view(torch.int16), want.view(torch.int16)), e
+        off += ln

@@ -528,3 +528,35 @@ def test_mixtral_routing_at_full_row_count_is_exact(gpu):
         want = (asc[off:off + ln] @ (b[e] * sb[e].repeat_interleave(128, 0).repeat_interleave(128, 1)).t()).bfloat16()
         assert torch.equal(got[off:off + ln].view(torch.int16), want.view(torch.int16)), e
         off += ln
+
+
+def test_a_split_launch_replays_under_a_graph(gpu):
+    """The GEMM whose output the library splits over the two tile heights (two launches per call) captured once, after
+    an eager call, and replayed on new operands: every replay equals the eager result."""
+    from primus_amd.pytorch import kernels as K
+
+    gen = torch.Generator(device=gpu).manual_seed(5)
+    m, n, k = 56 * 256 + 77, 4096, 256
+    a, sa, b, sb, _ = _exact_operands(gen, m, n, k, True, gpu)
+    aq, bq = a.to(torch.float8_e5m2), b.to(torch.float8_e5m2)
+    run = lambda: K.gemm_blockwise_nt_impl(aq, sa, bq, sb, b_rows_per_scale=1)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        run()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = run()
+    for seed in (6, 7, 8):
+        a2, sa2, _, _, _ = _exact_operands(torch.Generator(device=gpu).manual_seed(seed), m, 128, k, True, gpu)
+        with torch.no_grad():
+            aq.copy_(a2.to(torch.float8_e5m2))
+            sa.copy_(sa2)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = run()
+        torch.cuda.synchronize()
+        assert want.float().abs().max() > 0 and torch.equal(got.view(torch.int16), want.view(torch.int16)), seed

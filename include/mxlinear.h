@@ -458,6 +458,11 @@ int mxl_grouped_gemm_wgrad_blockwise(const void* a_codes, const void* a_sinv, in
  * call of the process, 0 returns to the choice by shape: a measuring and testing aid without counterpart in the
  * reference.  MXL_EINVAL for any other value. */
 int mxl_blockwise_gemm_tile(int rows);
+/* What the choice by shape comes to (a host-side calculation, no GPU needed; no counterpart in the reference): the 256-row
+ * tiles take rows [0, *tall_rows) x columns [0, *tall_cols) of an m x n output, the 128-row tiles the rest (the last rows
+ * or the last columns of a dense GEMM, in a second launch; 0 x 0: everything on 128-row tiles).  mode 0: dense, 1: grouped
+ * forward / dgrad (m = total rows), 2: grouped weight gradient (m, n = rows and columns of one group's matrix). */
+int mxl_blockwise_gemm_plan(int64_t m, int64_t n, int mode, int num_groups, int64_t* tall_rows, int64_t* tall_cols);
 
 /* ---- pre-shuffled MXFP4 layouts ----
  *

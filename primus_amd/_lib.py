@@ -75,6 +75,7 @@ EXPORTS = (
     "mxl_grouped_gemm_nt_blockwise",
     "mxl_grouped_gemm_wgrad_blockwise",
     "mxl_blockwise_gemm_tile",
+    "mxl_blockwise_gemm_plan",
     "mxl_shuffle_codes",
     "mxl_shuffle_scales",
     "mxl_calibrate_mfma",
@@ -206,6 +207,8 @@ def load() -> ctypes.CDLL:
         lib.mxl_gemm_nt_blockwise.argtypes = [vp, vp, i32, vp, vp, i32, i32, vp, i64, i64, i64, vp]
         lib.mxl_blockwise_gemm_tile.restype = i32
         lib.mxl_blockwise_gemm_tile.argtypes = [i32]
+        lib.mxl_blockwise_gemm_plan.restype = i32
+        lib.mxl_blockwise_gemm_plan.argtypes = [i64, i64, i32, i32, vp, vp]
         _lib = lib
     return _lib
 

@@ -931,6 +931,45 @@ static int launch_bw_gemm_fmt(const BwGemmArgs& g, dim3 grid, bool sbu, bool tal
 
 static std::atomic<int> bw_gemm_tile_rows{0};   // 0: by the shape; 128 or 256: forced (mxl_blockwise_gemm_tile)
 
+// Tile height of a launch.  256 x 256 tiles run about 15 % faster per flop than 128 x 256 ones (a third fewer operand
+// bytes from L2 per flop), so they win unless the coarser tiles leave that much more of the chip idle -- in the last
+// round of tiles, or in the ragged last tile of every group of a grouped forward (expected padding: half a tile per
+// group, which a group of 512 rows pays back).  A dense GEMM may take both: most of the output on 256-row tiles in
+// whole rounds, its last rows or its last columns on 128-row tiles (a second launch), whichever split has the lowest
+// cost in rounds of tiles over the chip's 256 CUs (a round of 128-row tiles = 0.5 x 1.15 rounds of 256-row tiles).
+// mxl_blockwise_gemm_tile overrides.
+struct BwPlan {
+    bool all_low;                 // everything on 128-row tiles
+    int64_t low_rows, low_cols;   // otherwise: what the 128-row tiles take, the last rows or the last columns (0, 0: nothing)
+};
+static BwPlan bw_plan(int64_t m, int64_t n, int mode, int num_groups) {
+    BwPlan pl{false, 0, 0};
+    const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1, cus = 256;
+    auto rounds_of = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
+    const int64_t rt_tall = (m + BWH_BM - 1) / BWH_BM, rt_low = (m + BWG_BM - 1) / BWG_BM;
+    const int forced = bw_gemm_tile_rows.load(std::memory_order_relaxed);
+    if (forced == BWG_BM) {
+        pl.all_low = true;
+    } else if (forced == BWH_BM) {
+    } else if (mode == 0) {
+        double best = rounds_of(rt_tall * col_tiles);
+        for (int64_t low = 1; low < rt_tall && low <= 4 * cus; ++low) {        // `low` of the 256-row tiles cut in two
+            const int64_t rows = m - (rt_tall - low) * BWH_BM;
+            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.575 * rounds_of((rows + BWG_BM - 1) / BWG_BM * col_tiles);
+            if (cost < best) best = cost, pl.low_rows = rows, pl.low_cols = 0;
+        }
+        for (int64_t low = 1; low < col_tiles && low <= 4 * cus; ++low) {      // the last `low` column tiles
+            const double cost = rounds_of(rt_tall * (col_tiles - low)) + 0.575 * rounds_of(rt_low * low);
+            if (cost < best) best = cost, pl.low_rows = 0, pl.low_cols = n - (col_tiles - low) * BWG_BN;
+        }
+        if (0.575 * rounds_of(rt_low * col_tiles) <= best) pl = BwPlan{true, 0, 0};
+    } else {
+        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.575 * rounds_of(rt_low * col_tiles * zs);
+        pl.all_low = !(cost_tall < cost_low && (mode != 1 || m >= 512 * (int64_t)num_groups));
+    }
+    return pl;
+}
+
 static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const void* b_codes, const void* b_sinv, int b_fmt,
                    int b_rows_per_scale, void* c_bf16, int64_t m, int64_t n, int64_t k, int mode, const int64_t* group_lens,
                    int num_groups, void* stream) {
@@ -944,38 +983,11 @@ static int bw_gemm(const void* a_codes, const void* a_sinv, int a_fmt, const voi
     if (k == 0 && mode != 2) return MXL_EINVAL;
     if ((((uintptr_t)a_codes | (uintptr_t)b_codes) & 15) != 0) return MXL_EINVAL;
     if (!device_is_gfx950()) return MXL_ENODEV;
-    // Tile height: 256 x 256 tiles run about 15 % faster per flop than 128 x 256 ones (a third fewer operand
-    // bytes from L2 per flop), so they win unless the coarser tiles leave that much more of the chip idle -- in the
-    // last round of tiles, or in the ragged last tile of every group of a grouped forward (expected padding: half a
-    // tile per group, which a group of 512 rows pays back).  A dense GEMM may take both: most of the output on 256-row
-    // tiles in whole rounds, its last rows or its last columns on 128-row tiles (a second launch), whichever split has
-    // the lowest cost in rounds of tiles (a round of 128-row tiles = 0.5 x 1.15 rounds of 256-row tiles).
-    // mxl_blockwise_gemm_tile overrides.
-    const int64_t col_tiles = (n + BWG_BN - 1) / BWG_BN, zs = mode == 2 ? num_groups : 1, cus = 256;
-    auto rounds_of = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
-    const int64_t rt_tall = (m + BWH_BM - 1) / BWH_BM, rt_low = (m + BWG_BM - 1) / BWG_BM;
-    int64_t low_rows = 0, low_cols = 0;                       // what the 128-row tiles take: the last rows, or the last columns
-    bool all_low = false;
-    const int forced = bw_gemm_tile_rows.load(std::memory_order_relaxed);
-    if (((uintptr_t)c_bf16 & 15) != 0 || forced == BWG_BM) {
-        all_low = true;                                       // (the 256-row kernel's epilogue stores 16 bytes per lane)
-    } else if (forced == BWH_BM) {
-    } else if (mode == 0) {
-        double best = rounds_of(rt_tall * col_tiles);
-        for (int64_t low = 1; low < rt_tall && low <= 4 * cus; ++low) {        // `low` of the 256-row tiles cut in two
-            const int64_t rows = m - (rt_tall - low) * BWH_BM;
-            const double cost = rounds_of((rt_tall - low) * col_tiles) + 0.575 * rounds_of((rows + BWG_BM - 1) / BWG_BM * col_tiles);
-            if (cost < best) best = cost, low_rows = rows, low_cols = 0;
-        }
-        for (int64_t low = 1; low < col_tiles && low <= 4 * cus; ++low) {      // the last `low` column tiles
-            const double cost = rounds_of(rt_tall * (col_tiles - low)) + 0.575 * rounds_of(rt_low * low);
-            if (cost < best) best = cost, low_rows = 0, low_cols = n - (col_tiles - low) * BWG_BN;
-        }
-        if (0.575 * rounds_of(rt_low * col_tiles) <= best) all_low = true;
-    } else {
-        const double cost_tall = rounds_of(rt_tall * col_tiles * zs), cost_low = 0.575 * rounds_of(rt_low * col_tiles * zs);
-        all_low = !(cost_tall < cost_low && (mode != 1 || m >= 512 * (int64_t)num_groups));
-    }
+    BwPlan plan = bw_plan(m, n, mode, num_groups);
+    if (((uintptr_t)c_bf16 & 15) != 0) plan = BwPlan{true, 0, 0};      // (the 256-row kernel's epilogue stores 16 bytes per lane)
+    const bool all_low = plan.all_low;
+    const int64_t low_rows = plan.low_rows, low_cols = plan.low_cols;
+    const int64_t zs = mode == 2 ? num_groups : 1;
     if (256 * k >= ((int64_t)1 << 31)) return MXL_EINVAL;     // byte offsets inside a tile's operand rows are 32-bit
     hipStream_t st = (hipStream_t)stream;
     const bool sbu = b_rows_per_scale == BW;
@@ -1029,6 +1041,14 @@ extern "C" int mxl_quantize_blockwise_weight(const void* w_bf16, int64_t batch, 
 extern "C" int mxl_blockwise_gemm_tile(int rows) {
     if (rows != 0 && rows != BWG_BM && rows != BWH_BM) return MXL_EINVAL;
     bw_gemm_tile_rows.store(rows, std::memory_order_relaxed);
+    return MXL_OK;
+}
+
+extern "C" int mxl_blockwise_gemm_plan(int64_t m, int64_t n, int mode, int num_groups, int64_t* tall_rows, int64_t* tall_cols) {
+    if (m <= 0 || n <= 0 || n % BW != 0 || mode < 0 || mode > 2 || (mode != 0 && num_groups < 1) || !tall_rows || !tall_cols) return MXL_EINVAL;
+    const BwPlan pl = bw_plan(m, n, mode, num_groups);
+    *tall_rows = pl.all_low ? 0 : m - pl.low_rows;
+    *tall_cols = pl.all_low ? 0 : n - pl.low_cols;
     return MXL_OK;
 }
 

@@ -130,3 +130,27 @@ def test_newer_entry_points_validate_before_they_touch_the_device(lib):
     assert lib.mxl_grouped_gemm_wgrad_ex(p, p, 0, p, p, 0, p, None, 0, 128, 128, 128, _lib.GF_ACCUM_F32, None) == -1   # needs KCHUNK
     assert lib.mxl_grouped_gemm_wgrad_ex(p, p, 0, p, p, 0, p, None, 0, 128, 128, 128, 64, None) == -1                   # unknown flag
     assert lib.mxl_grouped_gemm_wgrad_ex(p, p, 0, p, p, 0, p, None, 0, 128, 128, 128, _lib.GF_ACCUM_F32 | _lib.GF_KCHUNK, None) == -3
+
+
+def test_blockwise_gemm_plan(lib):
+    """The tile-height choice of the blockwise GEMMs is a host calculation: the Llama-3-8B MLP's three GEMMs at 8192
+    tokens, a problem too small for 256-row tiles, grouped shapes, the override and the argument checks."""
+    def plan(m, n, mode=0, groups=0):
+        rows, cols = ctypes.c_int64(-1), ctypes.c_int64(-1)
+        rc = lib.mxl_blockwise_gemm_plan(m, n, mode, groups, ctypes.byref(rows), ctypes.byref(cols))
+        return rc, rows.value, cols.value
+
+    assert plan(8192, 14336) == (0, 8192, 14336)          # forward: 32 x 56 tiles = 7 rounds, all on 256-row tiles
+    assert plan(8192, 4096) == (0, 8192, 4096)            # dgrad: 2 rounds
+    assert plan(14336, 4096) == (0, 12288, 4096)          # wgrad of fc1: 3 whole rounds, the last 2048 rows on 128-row tiles
+    assert plan(4096, 14336) == (0, 4096, 12288)          # wgrad of fc2: the last 8 column tiles
+    assert plan(2048, 4096) == (0, 0, 0)                  # half a round of 256-row tiles: 128-row tiles fill the chip
+    assert plan(1, 128) == (0, 0, 0)
+    assert plan(32768, 28672, 1, 8) == (0, 32768, 28672)  # grouped forward, 4096 rows per group
+    assert plan(4096, 1024, 1, 64) == (0, 0, 0)           # 64 rows per group: the ragged last tiles would be mostly padding
+    assert plan(28672, 4096, 2, 8) == (0, 28672, 4096)    # grouped weight gradient
+    assert lib.mxl_blockwise_gemm_tile(128) == 0 and plan(8192, 14336) == (0, 0, 0)
+    assert lib.mxl_blockwise_gemm_tile(256) == 0 and plan(2048, 4096) == (0, 2048, 4096)
+    assert lib.mxl_blockwise_gemm_tile(0) == 0 and plan(8192, 14336) == (0, 8192, 14336)
+    assert lib.mxl_blockwise_gemm_tile(64) != 0
+    assert plan(0, 128)[0] != 0 and plan(128, 100)[0] != 0 and plan(128, 128, 3)[0] != 0 and plan(128, 128, 1, 0)[0] != 0

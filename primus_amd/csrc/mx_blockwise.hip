@@ -849,27 +849,28 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm256_kernel(BwGemmArgs p) {
     // consecutive bf16 go in as 8 bytes and come out as 16 bytes per lane, 4 rows x 256 contiguous bytes per store
     // instruction (16-byte pieces XOR-swizzled by the row).  Stored straight from the accumulator layout, 16 bytes per
     // row and instruction, the partial lines cost a K = 4096 tile 5 % of its time.
-    uint8_t* const patch = bw_smem + w * (32 * 256);
+    uint8_t* const patch = bw_smem + w * (2 * 32 * 256);     // (one patch per a fragment: the two stages hold all sixteen)
     const bool cols_in = col0 + wn * 128 < pn;       // (n is a multiple of 128: the wave's columns are in or out as a whole)
     const int er = l >> 4, ep = l & 15;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const bv4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
                                  (__bf16)acc[i][j][4 * q + 3]};
-                *(bv4bf*)(patch + lr * 256 + 16 * ((4 * j + q) ^ (lr & 15)) + 8 * g) = o;
+                *(bv4bf*)(patch + i * (32 * 256) + lr * 256 + 16 * ((4 * j + q) ^ (lr & 15)) + 8 * g) = o;
             }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int r = 4 * u + er;
-            const uint4 v = *(const uint4*)(patch + r * 256 + 16 * (ep ^ (r & 15)));
+            const uint4 v = *(const uint4*)(patch + i * (32 * 256) + r * 256 + 16 * (ep ^ (r & 15)));
             const int64_t m = row0 + wm * 64 + i * 32 + r;
             if (cols_in && m < pm) store16_streaming(pc_out + m * ldc + col0 + wn * 128 + 8 * ep, v);
         }
-    }
 }
 
 template <bool TWOD>

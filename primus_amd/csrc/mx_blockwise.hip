@@ -584,27 +584,28 @@ __global__ __launch_bounds__(BWG_THREADS) void bw_gemm_kernel(BwGemmArgs p) {
         // Output through a wave-private LDS patch of 32 rows x 128 bytes, one a fragment at a time: a lane's four
         // consecutive bf16 go in as 8 bytes and come out as 16 bytes per lane, 8 rows x 128 contiguous bytes per store
         // instruction (16-byte pieces XOR-swizzled by the row).
-        uint8_t* const patch = bw_smem + w * (32 * 128);
+        uint8_t* const patch = bw_smem + w * (2 * 32 * 128);   // (one patch per a fragment, both written before the first is read back)
         const bool cols_in = col0 + wn * 64 < pn;        // (n is a multiple of 128: the wave's columns are in or out as a whole)
         const int er = l >> 3, ep = l & 7;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const bv4bf o = {(__bf16)acc[i][j][4 * q], (__bf16)acc[i][j][4 * q + 1], (__bf16)acc[i][j][4 * q + 2],
                                      (__bf16)acc[i][j][4 * q + 3]};
-                    *(bv4bf*)(patch + lr * 128 + 16 * ((4 * j + q) ^ ((lr >> 1) & 7)) + 8 * g) = o;
+                    *(bv4bf*)(patch + i * (32 * 128) + lr * 128 + 16 * ((4 * j + q) ^ ((lr >> 1) & 7)) + 8 * g) = o;
                 }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int r = 8 * u + er;
-                const uint4 v = *(const uint4*)(patch + r * 128 + 16 * (ep ^ ((r >> 1) & 7)));
+                const uint4 v = *(const uint4*)(patch + i * (32 * 128) + r * 128 + 16 * (ep ^ ((r >> 1) & 7)));
                 const int64_t m = row0 + wm * 64 + i * 32 + r;
                 if (cols_in && m < pm) store16_streaming(pc_out + m * ldc + col0 + wn * 64 + 8 * ep, v);
             }
-        }
         return;
     }
     // an output that is only 8-byte aligned: stored straight from the accumulator layout

@@ -560,3 +560,29 @@ def test_a_split_launch_replays_under_a_graph(gpu):
         want = run()
         torch.cuda.synchronize()
         assert want.float().abs().max() > 0 and torch.equal(got.view(torch.int16), want.view(torch.int16)), seed
+
+
+def test_an_output_that_is_only_8_byte_aligned(gpu):
+    """The C entry point accepts an output pointer aligned to 8 bytes: such a call stays on the 128-row kernel and stores
+    straight from the accumulator layout, with the same bits as the aligned call (and a misaligned one is refused)."""
+    from primus_amd import _lib
+    from primus_amd.pytorch import kernels as K
+
+    gen = torch.Generator(device=gpu).manual_seed(21)
+    m, n, k = 777, 384, 512
+    a, sa, b, sb, want = _exact_operands(gen, m, n, k, False, gpu)
+    aq, bq = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+    buf = torch.zeros(m * n + 16, dtype=torch.bfloat16, device=gpu)
+    lib, stream = _lib.load(), torch.cuda.current_stream().cuda_stream
+    for tile in (0, 256):
+        K.set_blockwise_gemm_tile(tile)
+        try:
+            buf.zero_()
+            rc = lib.mxl_gemm_nt_blockwise(aq.data_ptr(), sa.data_ptr(), 0, bq.data_ptr(), sb.data_ptr(), 0, 128, buf.data_ptr() + 8, m, n, k, stream)
+        finally:
+            K.set_blockwise_gemm_tile(0)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(buf[4:4 + m * n].view(m, n).view(torch.int16), want.view(torch.int16))
+        assert not buf[:4].any() and not buf[4 + m * n:].any()
+    assert lib.mxl_gemm_nt_blockwise(aq.data_ptr(), sa.data_ptr(), 0, bq.data_ptr(), sb.data_ptr(), 0, 128, buf.data_ptr() + 2, m, n, k, stream) != 0
